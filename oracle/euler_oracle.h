@@ -1,0 +1,125 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.
+ *
+ * CPU restatement ("oracle") of the reference's quantized-convolution arithmetic.  Only the
+ * tests, the smoke check and the benchmark's cpu_baseline leg may load it; the product
+ * library never does.  Every function names the reference file:line it restates.
+ *
+ * Conventions
+ *   - activations are nChw16c: [n][C/16][h][w][16]; user weights are OIhw16i16o f32:
+ *     [OC/16][IC/16][kh][kw][16 ic][16 oc]; depthwise user weights are goihw f32 [g][kh][kw].
+ *   - quantized weights leave the oracle in a plain order ([OCp][ICp][kh][kw] s8, OCp/ICp =
+ *     channel counts rounded up to 16) so that they can be compared with any packed layout.
+ *   - float glue is written with explicit fmaf() exactly where the reference's compiled code
+ *     (g++ -O2, default -ffp-contract=fast) performs one fused rounding; this file is built
+ *     with -ffp-contract=off so nothing else fuses.
+ *
+ * Pinning status (what checks each part; see tests/test_oracle_*.py):
+ *   - fused-rounding pattern of the GEMM/conv/depthwise epilogues, depthwise floor/round split,
+ *     unsigned saturation, Winograd F(4,3) input/weights/output transforms: pinned against the
+ *     reference's own kernel templates compiled from /root/reference (oracle/ref_kernels.cpp).
+ *   - integer contractions: pinned by brute-force integer convolution in numpy.
+ *   - weight quantization (abs-max, (w*127)/absmax, round-half-even) and scale/shift folding:
+ *     pure IEEE mul/div/rint sequences, pinned by an independent numpy float32 evaluation.
+ *     For input_z != 0 or sum_z != 0 the folding contains a product-difference whose fusion
+ *     is compiler-chosen and no compiled reference code is available for it here:
+ *     PARITY UNPINNED for non-zero input/sum zero points (all configured layers use 0).
+ *   - reorders: closed-form index maps, pinned by numpy transposes.
+ */
+#ifndef EULER_ORACLE_H
+#define EULER_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* same numbering as the reference's data-type enum (include/euler.hpp:66-73) */
+enum { ORC_F32 = 1, ORC_U8 = 3, ORC_S8 = 4, ORC_S32 = 5 };
+
+typedef struct orc_conv_params {
+  int32_t n, g, ic, oc, ih, iw, oh, ow, kh, kw;
+  int32_t pad_t, pad_l, stride_h, stride_w;
+  int32_t out_type;            /* ORC_F32 / ORC_U8 / ORC_S8 */
+  int32_t with_bias, with_relu, with_sum;
+  int32_t T;                   /* width-block size (flatting.t); only depthwise u8 output depends on it */
+  float in_scale, in_z;        /* input_quant  */
+  float out_scale, out_z;      /* output_quant */
+  float sum_scale, sum_z;      /* sum_quant    */
+  float tin_scale, tin_z;      /* wino_tinput_quant */
+  float relu_lo, relu_hi;      /* relu_bound   */
+} orc_conv_params;
+
+/* ---- layout reorders: src/elx_reorder.cpp:35-93 ---- */
+void orc_reorder_nchw_to_blocked_f32(float *dst, const float *src, int n, int c, int h, int w);
+void orc_reorder_nchw_to_blocked_u8(uint8_t *dst, const uint8_t *src, int n, int c, int h, int w);
+void orc_reorder_blocked_to_nchw_f32(float *dst, const float *src, int n, int c, int h, int w);
+void orc_reorder_blocked_to_nchw_u8(uint8_t *dst, const uint8_t *src, int n, int c, int h, int w);
+void orc_reorder_oihw_to_blocked_f32(float *dst, const float *src, int o, int i, int h, int w);
+void orc_reorder_blocked_to_oihw_f32(float *dst, const float *src, int o, int i, int h, int w);
+
+/* ---- harness-side input quantization: tests/elt_conv_utils.cpp:354-401 ---- */
+void orc_quantize_input_u8(uint8_t *dst, const float *src, size_t count, float scale, float z);
+
+/* ---- direct 1x1 / KxK ----
+ * weight quantization + scale/shift folding:
+ *   src/elx_int8_conv_direct_1x1.cpp:234-355, src/elx_int8_conv_direct.cpp:311-500.
+ * wq [OCp][ICp][kh][kw] s8, scale/shift [OCp] f32, wsum [OCp] s32. */
+int orc_direct_prepare(const orc_conv_params *p, const float *w_blocked, const float *bias,
+                       int8_t *wq, float *scale, float *shift, int32_t *wsum);
+/* contraction + epilogue: src/kernel/elk_u8s8_gemm.hxx:168-266,269-406,
+ * src/kernel/elk_u8s8_conv.hxx:190-252,679-901, src/elx_int8_conv_direct.cpp:574-718.
+ * `output` is nChw16c of out_type and, with_sum, also holds the sum operand on entry.
+ * `acc` (optional) receives the raw s32 accumulators, nChw16c. */
+int orc_direct_execute(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
+                       const float *scale, const float *shift, void *output, int32_t *acc);
+
+/* ---- depthwise 3x3 ----
+ * src/elx_int8_conv_direct_depthwise.cpp:200-292; wq [G][3][3], scale/shift [G], G = g up to 16. */
+int orc_depthwise_prepare(const orc_conv_params *p, const float *w_goihw, const float *bias,
+                          int8_t *wq, float *scale, float *shift, int32_t *wsum);
+/* src/kernel/elk_u8s8_depthwise_conv.hxx:219-286,288-474 */
+int orc_depthwise_execute(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
+                          const float *scale, const float *shift, void *output, int32_t *acc);
+
+/* ---- Winograd F(4x4,3x3), int8 GEMM, fp32 user tensors ----
+ * tiles: t = n*ht*wt + th*wt + tw (src/elx_conv_wino_trans_input.cpp:10-24).
+ * twq [36][OCp][ICp] s8; tscale/tshift [36][OCp];
+ * tinput [36][ICp/16][t][16] u8; toutput [36][OCp/16][t][16] f32. */
+int orc_wino_tiles(const orc_conv_params *p);
+/* fp32 transform only (what the reference harness dumps to calibrate wino_tinput_quant,
+ * tests/elt_conv_utils.cpp:222-262): min/max over all transformed-input elements. */
+int orc_wino_tinput_range(const orc_conv_params *p, const float *input, float *min_out, float *max_out);
+/* src/kernel/elk_conv_wino_4x4_3x3_weights.hxx:18-72 + src/elx_conv_wino_trans_weights.cpp:437-535 */
+int orc_wino_prepare(const orc_conv_params *p, const float *w_blocked, int8_t *twq,
+                     float *tscale, float *tshift);
+/* src/kernel/elk_conv_wino_4x4_3x3_input.hxx:13-352 + src/elx_conv_wino_trans_input.cpp:599-654 */
+int orc_wino_trans_input(const orc_conv_params *p, const float *input, uint8_t *tinput);
+/* src/elx_int8_conv_wino_gemm.cpp:23-76 + src/kernel/elk_u8s8_gemm.hxx:200-208 */
+int orc_wino_gemm(const orc_conv_params *p, const uint8_t *tinput, const int8_t *twq,
+                  const float *tscale, const float *tshift, float *toutput, int32_t *acc);
+/* src/kernel/elk_conv_wino_4x4_3x3_output.hxx:19-201 + src/elx_conv_wino_trans_output.cpp:212-277 */
+int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const float *bias,
+                          float *output);
+
+/* single 6x6 / 3x3 / 4x4 tile transforms, exposed so they can be compared one-to-one with the
+ * reference's compiled kernel templates */
+void orc_wino_tile_input(const float d[36], float v[36]);         /* interior tiles */
+void orc_wino_tile_input_border(const float d[36], float v[36]);  /* tiles that touch the zero border */
+void orc_wino_tile_weights(const float g[9], float u[36]);
+void orc_wino_tile_output(const float m[36], float y[16]);
+
+/* epilogue on one value, exposed for the same reason (out_kind ORC_*; returns the f32 result
+ * for ORC_F32 through *fout, else the quantized byte through the return value) */
+int orc_epilogue(int out_kind, int32_t acc, float scale, float shift, int with_sum, int old_q,
+                 float sum_scale, int with_relu, float lo, float hi, float *fout);
+
+int orc_num_threads(void);
+int orc_has_vnni(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,265 @@
+// TEST INFRASTRUCTURE ONLY -- never linked into, imported by, or called from the product path.
+//
+// Thin C-ABI driver around the reference's own AVX-512 micro-kernel templates.  It is
+// compiled (by oracle/Makefile, target `ref`) against the header files where they lie under
+// /root/reference with the GNU flags of the reference's cmake/flags.cmake:77-87
+// (-std=c++11 -O2 -DNDEBUG -mavx512f -mavx512dq -mavx512bw -mfma -mavx512vl, WITH_VNNI),
+// so that the float glue of the reference (which a*b+c become one fused rounding, the
+// floor/round-to-nearest split of the depthwise store, the unsigned saturation) is pinned by
+// the reference's compiled code and not by a reading of it.  Nothing of the reference is
+// copied: the templates are instantiated straight from
+//   src/kernel/elk_u8s8_gemm.hxx, elk_u8s8_conv.hxx, elk_u8s8_depthwise_conv.hxx,
+//   src/kernel/elk_conv_wino_4x4_3x3_{input,weights,output}.hxx.
+// The executor classes (src/elx_int8_conv_*.cpp) are NOT built: they bind kernels through
+// tables that the reference's build generates with shell scripts at configure time.
+//
+// The only accommodation: the reference uses the "aligned" 512-bit integer load/store
+// intrinsics on addresses that are only 16-byte aligned (depthwise kernel); the intrinsic
+// headers are included first and those two names are redirected to the unaligned forms.
+// This changes no arithmetic.
+#include <immintrin.h>
+#include <x86intrin.h>
+#define _mm512_load_epi32(p) _mm512_loadu_si512(p)
+#define _mm512_store_epi32(p, v) _mm512_storeu_si512(p, v)
+
+#include <cstdint>
+#include <cstring>
+#include <string>
+#include <cfloat>
+
+#include "euler.hpp"
+#include "el_def.hpp"
+#include "elk_def.hpp"
+#include "elx_conv.hpp"
+#include "elk_u8s8_gemm.hxx"
+#include "elk_u8s8_conv.hxx"
+#include "elk_u8s8_depthwise_conv.hxx"
+#include "elk_conv_wino.hpp"
+#include "elk_conv_wino_4x4_3x3_input.hxx"
+#include "elk_conv_wino_4x4_3x3_weights.hxx"
+#include "elk_conv_wino_4x4_3x3_output.hxx"
+
+using namespace euler;
+
+namespace {
+
+void fill_common(elx_param_t &ep, float relu_lo, float relu_hi, float sum_S)
+{
+  ep.V1 = 4; ep.Vx = 4;
+  ep.O = 1; ep.O1 = 1; ep.O2 = 1; ep.O3 = 1; ep.O4 = 1;
+  ep.I2 = 1; ep.I3 = 1; ep.I4 = 1;
+  ep.Ir = 4; ep.Or = 16;
+  ep.hs = ep.ws = 1; ep.hd = ep.wd = 1;
+  ep.lp = ep.rp = ep.tp = ep.bp = 0;
+  ep.kh = ep.kw = 1;
+  ep.g = 1; ep.G2 = 1; ep.G3 = 1;
+  ep.streaming_input = ep.streaming_output = 0;
+  ep.sampling_kind = CALIBRATED;
+  ep.relu_bound_lower = relu_lo;
+  ep.relu_bound_upper = relu_hi;
+  ep.sum_quant_S = sum_S;
+  for (int i = 0; i < 16; ++i) {
+    ep.relu_bound_lower_vec[i] = relu_lo;
+    ep.relu_bound_upper_vec[i] = relu_hi;
+    ep.sum_quant_S_vec[i] = sum_S;
+  }
+}
+
+template <typename OT, int O, int T>
+void run_gemm_ccc(elx_param_t &ep, float *toutput, void *ooutput, uint8_t *input,
+    int8_t *weights, int attr, float *wscale, float *wshift)
+{
+  using ker = u8s8_gemm_kernel<conv_impl::INT8_F32, OT, 16, 4, ISA_AVX512,
+      estl::integer_sequence<1, GKF_CCC, O, T, 1>>;
+  ker::gemm(ep, toutput, (OT *)ooutput, input, weights, nullptr, attr,
+      nullptr, nullptr, wscale, wshift);
+}
+
+template <typename OT, int T>
+void run_dw(elx_param_t &ep, void *routput, uint8_t *input, int8_t *weights,
+    float *wscale, float *wshift, int khs, int khe, int pad_l, int pad_r, int attr)
+{
+  using ker = u8s8_depthwise_conv_kernel<conv_impl::INT8_F32, OT, 16, 4, ISA_AVX512,
+      estl::integer_sequence<1, GKF_DCD, 1, T, 3>>;
+  ker::conv(ep, nullptr, (OT *)routput, input, weights, nullptr, nullptr, nullptr,
+      wscale, wshift, khs, khe, 0, 3, pad_l, pad_r, attr);
+}
+
+template <typename OT, int T>
+void run_conv3(elx_param_t &ep, float *toutput, void *routput, uint8_t *input,
+    int8_t *weights, float *wscale, float *wshift, int khs, int khe, int kws,
+    int kwe, int pad_l, int pad_r, int attr)
+{
+  using ker = u8s8_conv_kernel<conv_impl::INT8_F32, OT, 16, 4, ISA_AVX512,
+      estl::integer_sequence<1, GKF_DCD, 1, T, 3>>;
+  ker::conv(ep, toutput, (OT *)routput, input, weights, nullptr, nullptr, nullptr,
+      wscale, wshift, khs, khe, kws, kwe, pad_l, pad_r, attr);
+}
+
+} // namespace
+
+extern "C" {
+
+// u8s8 GEMM micro-kernel, compact layout (GKF_CCC, src/kernel/elk_def.hpp:36-41):
+//   input   [I2][T][16]  u8,   weights [I2][4][O][16 oc][4 ic] s8  (O1 = 1),
+//   toutput [O][T][16]   f32-typed (holds s32 partials or the f32 result),
+//   ooutput [O][T][16]   u8/s8 (out_kind 1/2; also the in-place sum operand).
+// out_kind: 0 = f32, 1 = u8, 2 = s8.  (O,T) in {(1,4),(2,6)}.
+int ref_u8s8_gemm(int out_kind, int O, int T, int I2, int attr, float relu_lo,
+    float relu_hi, float sum_S, float *toutput, void *ooutput, uint8_t *input,
+    int8_t *weights, float *wscale, float *wshift)
+{
+  elx_param_t ep;
+  fill_common(ep, relu_lo, relu_hi, sum_S);
+  ep.I2 = I2; ep.O = O; ep.O2 = O; ep.T = T;
+  ep.IC = I2 * 16; ep.ic = ep.IC; ep.OC = O * 16; ep.oc = ep.OC;
+  ep.ic2 = I2; ep.ic34 = 1;
+  ep.oh = 1; ep.ow = T; ep.ih = 1; ep.iw = T;
+#define GEMM_CASE(k, OT, o, t)                                                  \
+  if (out_kind == k && O == o && T == t) {                                      \
+    run_gemm_ccc<OT, o, t>(ep, toutput, ooutput, input, weights, attr, wscale,  \
+        wshift);                                                                \
+    return 0;                                                                   \
+  }
+  GEMM_CASE(0, float, 1, 4) GEMM_CASE(0, float, 2, 6)
+  GEMM_CASE(1, uint8_t, 1, 4) GEMM_CASE(1, uint8_t, 2, 6)
+  GEMM_CASE(2, int8_t, 1, 4) GEMM_CASE(2, int8_t, 2, 6)
+#undef GEMM_CASE
+  return -1;
+}
+
+// Depthwise 3x3 stride-1 micro-kernel (src/kernel/elk_u8s8_depthwise_conv.hxx:288-474) on
+// one width block of T outputs of one output row, all G2 channel groups:
+//   input   [G2][ih][iw][16] u8 (whole plane; the kernel is handed the pointer of the
+//           block's first centre pixel, as conv_c160 does,
+//           src/elx_int8_conv_direct_depthwise.cpp:294-319),
+//   weights [G2][3][16][4] s8, wscale/wshift [G2][16], routput [G2][oh*ow][16].
+// out_kind: 1 = u8, 2 = s8.  T is the layer's width-block size, Tz the size of THIS block
+// (T, or ow % T for the last one); the kernel is instantiated for Tz in {4,5,6,7,8,11,14}.
+int ref_u8s8_depthwise(int out_kind, int T, int Tz, int G2, int ih, int iw, int oh, int ow,
+    int _ht, int _wt, int tp, int lp, int rp, int with_relu, float relu_lo,
+    float relu_hi, void *routput, uint8_t *input, int8_t *weights, float *wscale,
+    float *wshift)
+{
+  elx_param_t ep;
+  fill_common(ep, relu_lo, relu_hi, 0.f);
+  ep.kh = ep.kw = 3; ep.G2 = G2; ep.ic2 = G2; ep.oc2 = G2; ep.I2 = G2;
+  ep.ih = ih; ep.iw = iw; ep.oh = oh; ep.ow = ow; ep.T = T;
+  ep.tp = tp; ep.lp = lp; ep.rp = rp;
+  const int wt = (ow + T - 1) / T;
+  int khs = tp - _ht > 0 ? tp - _ht : 0;
+  int khe = 3 < ih + tp - _ht ? 3 : ih + tp - _ht;
+  int pad_l = (_wt == 0) && lp > 0;
+  int pad_r = (_wt == wt - 1) && rp > 0;
+  int cih = _ht + 1 - tp, ciw = _wt * T + 1 - lp;
+  uint8_t *in = input + ((size_t)cih * iw + ciw) * 16;
+  char *out = (char *)routput + ((size_t)_ht * ow + _wt * T) * 16;
+  int attr = with_relu ? (int)AT_RELU_MASK : 0;
+#define DW_CASE(k, OT, t)                                                       \
+  if (out_kind == k && Tz == t) {                                                \
+    run_dw<OT, t>(ep, out, in, weights, wscale, wshift, khs, khe, pad_l, pad_r, \
+        attr);                                                                  \
+    return 0;                                                                   \
+  }
+  DW_CASE(1, uint8_t, 4) DW_CASE(1, uint8_t, 5) DW_CASE(1, uint8_t, 6)
+  DW_CASE(1, uint8_t, 7) DW_CASE(1, uint8_t, 8) DW_CASE(1, uint8_t, 11)
+  DW_CASE(1, uint8_t, 14)
+  DW_CASE(2, int8_t, 7) DW_CASE(2, int8_t, 14)
+#undef DW_CASE
+  return -1;
+}
+
+// Direct 3x3 stride-1 micro-kernel (src/kernel/elk_u8s8_conv.hxx:679-901), O = O1 = 1, one
+// width block of T outputs of one output row, one 16-wide OC block:
+//   input   [I2][ih][iw][16] u8,  weights [3][3][I2][4][16 oc][4 ic] s8,
+//   wscale [16], wshift [T][16], routput [oh*ow][16] (u8/s8) or toutput (f32).
+// out_kind: 0 = f32 (toutput), 1 = u8, 2 = s8.  T in {7, 14}.
+int ref_u8s8_conv3x3(int out_kind, int T, int I2, int ih, int iw, int oh, int ow,
+    int _ht, int _wt, int pad, int with_relu, float relu_lo, float relu_hi,
+    float *toutput, void *routput, uint8_t *input, int8_t *weights, float *wscale,
+    float *wshift)
+{
+  elx_param_t ep;
+  fill_common(ep, relu_lo, relu_hi, 0.f);
+  ep.kh = ep.kw = 3; ep.I2 = I2; ep.ic2 = I2; ep.IC = ep.ic = 16 * I2;
+  ep.OC = ep.oc = 16; ep.oc2 = 1;
+  ep.ih = ih; ep.iw = iw; ep.oh = oh; ep.ow = ow; ep.T = T;
+  ep.tp = ep.lp = ep.rp = ep.bp = pad;
+  const int wt = (ow + T - 1) / T;
+  int khs = pad - _ht > 0 ? pad - _ht : 0;
+  int khe = 3 < ih + pad - _ht ? 3 : ih + pad - _ht;
+  int kws = _wt == 0 ? pad : 0;
+  int kwe = _wt == wt - 1 ? 3 - pad : 3;
+  int pad_l = _wt == 0 ? pad : 0;
+  int pad_r = _wt == wt - 1 ? pad : 0;
+  int cih = _ht + 1 - pad, ciw = _wt * T + 1 - pad;
+  uint8_t *in = input + ((size_t)cih * iw + ciw) * 16;
+  size_t ooff = ((size_t)_ht * ow + _wt * T) * 16;
+  int attr = AT_CLEAR_OUTPUT_MASK | AT_RESTORE_OUTPUT_MASK
+      | (with_relu ? (int)AT_RELU_MASK : 0);
+#define CV_CASE(k, OT, t)                                                       \
+  if (out_kind == k && T == t) {                                                \
+    run_conv3<OT, t>(ep, toutput ? toutput + ooff : nullptr,                    \
+        routput ? (char *)routput + ooff * sizeof(OT) : nullptr, in, weights,   \
+        wscale, wshift, khs, khe, kws, kwe, pad_l, pad_r, attr);                \
+    return 0;                                                                   \
+  }
+  CV_CASE(0, float, 7) CV_CASE(0, float, 14)
+  CV_CASE(1, uint8_t, 7) CV_CASE(1, uint8_t, 14)
+  CV_CASE(2, int8_t, 7) CV_CASE(2, int8_t, 14)
+#undef CV_CASE
+  return -1;
+}
+
+// Winograd F(4x4,3x3) input transform of one 6x6 tile of 16 channels
+// (src/kernel/elk_conv_wino_4x4_3x3_input.hxx:13-352).  `tile` points at element (0,0) of
+// the tile inside an [ih][iw][16] f32 plane; rows/cols outside [hs,he]x[ws,we] read as zero
+// when border != 0.  tinput is [6][6][16] f32.
+void ref_wino_trans_input(int border, int ih, int iw, float *tinput, float *tile,
+    int hs, int he, int ws, int we)
+{
+  elx_param_t ep;
+  fill_common(ep, 0.f, FLT_MAX, 0.f);
+  ep.ih = ih; ep.iw = iw;
+  if (border)
+    elk_conv_wino_trans_input<float, float, TKF_BLOCKED, true, ISA_AVX512, 6,
+        16>::execute(ep, tinput, tile, hs, he, ws, we);
+  else
+    elk_conv_wino_trans_input<float, float, TKF_BLOCKED, false, ISA_AVX512, 6,
+        16>::execute(ep, tinput, tile, 0, 5, 0, 5);
+}
+
+// Winograd F(4x4,3x3) weights transform of one 16ic x 16oc block
+// (src/kernel/elk_conv_wino_4x4_3x3_weights.hxx:18-72): in [3][3][16 ic][16 oc],
+// out [6][6][16 ic][16 oc], both f32, 64-byte aligned.
+void ref_wino_trans_weights(float *tweights, float *weights)
+{
+  elk_conv_wino_trans_weights<float, float, ISA_AVX512, 6, 3, 16>::execute(
+      *(float(*)[6][6][16][16])tweights, *(float(*)[3][3][16][16])weights);
+}
+
+// Winograd F(4x4,3x3) output transform of one tile of 16 channels
+// (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:19-201), f32 output in an [oh][ow][16] plane.
+// `out` points at the tile's first output element, toutput is [6][6][16] f32, rows > h_end or
+// cols > w_end are not written when border != 0.
+void ref_wino_trans_output(int border, int with_bias, int with_relu, int oh, int ow,
+    float *out, float *toutput, float *bias, int h_end, int w_end)
+{
+  elx_param_t ep;
+  fill_common(ep, 0.f, FLT_MAX, 0.f);
+  ep.oh = oh; ep.ow = ow;
+#define WO_CASE(b, wb, wr)                                                      \
+  if (!!border == b && !!with_bias == wb && !!with_relu == wr) {                \
+    elk_conv_wino_trans_output<float, float, float, TKF_BLOCKED, b, wb, wr,     \
+        false, ISA_AVX512, 6, 3, 16>::execute(ep, out, toutput, bias, h_end,    \
+        w_end);                                                                 \
+    return;                                                                     \
+  }
+  WO_CASE(false, false, false) WO_CASE(false, true, false)
+  WO_CASE(false, true, true) WO_CASE(false, false, true)
+  WO_CASE(true, false, false) WO_CASE(true, true, false)
+  WO_CASE(true, true, true) WO_CASE(true, false, true)
+#undef WO_CASE
+}
+
+} // extern "C"
