@@ -1,0 +1,78 @@
+"""Builds libeuler_hip.so (HIP kernels + C-ABI + the C++ euler:: API) for gfx950 with hipcc.
+
+    python deep-learning-math-kernel-research_amd/build.py
+
+The library is written next to this file so that it travels with the source tree.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libeuler_hip.so")
+
+SOURCES = [
+    "ehip_gemm.hip",
+    "ehip_conv3x3.hip",
+    "ehip_depthwise.hip",
+    "ehip_wino.hip",
+    "ehip_prepare.hip",
+    "ehip_api.hip",
+    "euler_api.hip",
+]
+
+# -ffp-contract=off: every single-rounding multiply-add of the reference is written as an explicit
+#   fma; nothing else may fuse, or float results stop being bit-identical.
+# packed-fp32-ops off: keep the compiler from forming packed fp32 instructions.
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+]
+
+
+def build(verbose=True, jobs=8):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    procs = []
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src + ".o")
+        objs.append(obj)
+        cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        if len(procs) >= jobs:
+            _wait(procs)
+    _wait(procs)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB
+
+
+def _wait(procs):
+    failed = []
+    for src, p in procs:
+        out, _ = p.communicate()
+        text = out.decode(errors="replace")
+        # the host pass does not know the packed-fp32 feature name; that warning is harmless
+        text = "\n".join(l for l in text.splitlines() if "packed-fp32-ops" not in l)
+        if text.strip():
+            print(text)
+        if p.returncode != 0:
+            failed.append(src)
+    procs.clear()
+    if failed:
+        raise RuntimeError("hipcc failed for: " + ", ".join(failed))
+
+
+if __name__ == "__main__":
+    build()
+    print("built", LIB)

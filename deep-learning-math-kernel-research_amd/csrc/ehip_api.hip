@@ -1,0 +1,605 @@
+// C-ABI layer (include/euler_hip.h): descriptor validation and executor choice, device
+// workspace, weight preparation, launches.  No kernels here.
+#include <cfloat>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "ehip_internal.hpp"
+
+using namespace ehip;
+
+namespace {
+thread_local std::string g_last_error;
+}
+
+namespace ehip {
+void set_error(const std::string &msg) { g_last_error = msg; }
+}  // namespace ehip
+
+#define HIP_TRY(expr)                                                                              \
+  do {                                                                                             \
+    hipError_t _e = (expr);                                                                        \
+    if (_e != hipSuccess) {                                                                        \
+      set_error(std::string(#expr) + ": " + hipGetErrorString(_e));                                \
+      return EHIP_HIP_ERROR;                                                                       \
+    }                                                                                              \
+  } while (0)
+
+struct ehip_conv {
+  ehip_conv_desc_t d;
+  int family = 0;
+  int variant = 0;
+  bool prepared = false;
+  std::string kernel_name;
+
+  int ic2 = 0, oc2 = 0, ocpp = 0, units_pad = 0, taps = 1, nbatch = 1;
+  int8_t *wpacked = nullptr;
+  size_t wpacked_bytes = 0;
+  float *scale = nullptr, *shift = nullptr, *absmax = nullptr;
+  int *wsum = nullptr, *comp = nullptr;
+  size_t per_oc = 0;  // elements in scale/shift/wsum/comp
+
+  // 3x3
+  int halo_rows = 0;
+  size_t lds_bytes = 0;
+  // depthwise
+  int T = 1, Tr = 1, wtb = 1;
+  // Winograd
+  int ht = 0, wt = 0, nt = 0, t = 0;
+  uint8_t *tin = nullptr;
+  float *tout = nullptr;
+  size_t tin_bytes = 0, tout_bytes = 0;
+};
+
+namespace {
+
+const float kNoCali = FLT_MAX;  // EL_NO_CALI
+
+int fail(int code, const std::string &msg)
+{
+  set_error(msg);
+  return code;
+}
+
+void free_all(ehip_conv *c)
+{
+  void *ptrs[] = {c->wpacked, c->scale, c->shift, c->absmax, c->wsum, c->comp, c->tin, c->tout};
+  for (void *p : ptrs)
+    if (p) (void)hipFree(p);
+}
+
+template <typename T>
+int dev_alloc(T **p, size_t count, bool zero)
+{
+  HIP_TRY(hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T)));
+  if (zero) HIP_TRY(hipMemset(*p, 0, count * sizeof(T)));
+  return EHIP_OK;
+}
+
+// mirrors the dispatch of eld_conv_t::setup (src/eld_conv.cpp:148-313) for the int8 executors
+int classify(ehip_conv *c)
+{
+  ehip_conv_desc_t &d = c->d;
+  if (d.g <= 0 || d.ic % d.g || d.oc % d.g) return fail(EHIP_GENERAL_ERROR, "dims: groups: ic|oc != g * x");
+  const bool depthwise = d.g == d.ic && d.g == d.oc && d.g > 1;
+  const int icg = d.ic / d.g;
+  if (d.dilation_h != 1 || d.dilation_w != 1) return fail(EHIP_UNIMPLEMENTED, "dilation is not supported by the int8 path");
+
+  if (d.algorithm == EHIP_CONV_AUTO) {
+    if (d.kh == 1 && d.kw == 1) d.algorithm = EHIP_CONV_DIRECT_1X1;
+    else if (icg >= 16 && d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.pad_l == 1 &&
+             d.pad_r == 1 && d.pad_t == 1 && d.pad_b == 1)
+      d.algorithm = EHIP_CONV_WINOGRAD;
+    else d.algorithm = EHIP_CONV_DIRECT;
+  }
+
+  const bool in_u8 = d.input_type == EHIP_U8 && d.weights_type == EHIP_F32 && d.bias_type == EHIP_F32;
+  const bool out_q = d.output_type == EHIP_U8 || d.output_type == EHIP_S8;
+  const bool all_f32 = d.input_type == EHIP_F32 && d.weights_type == EHIP_F32 && d.output_type == EHIP_F32 &&
+      d.bias_type == EHIP_F32;
+
+  if (d.algorithm != EHIP_CONV_WINOGRAD) {
+    if (!in_u8) return fail(EHIP_UNIMPLEMENTED, "only the u8-input int8 executors are built (fp32 paths are out of scope)");
+    if (d.sampling_kind != 2) return fail(EHIP_UNIMPLEMENTED, "int8 direct: non-calibrated sampling_kind not supported");
+    if (d.input_scale == kNoCali || d.input_z == kNoCali) return fail(EHIP_GENERAL_ERROR, "input_quant is not set");
+    if (out_q && (d.output_scale == kNoCali || d.output_z == kNoCali || d.output_scale == 0.0f))
+      return fail(EHIP_GENERAL_ERROR, "output_quant is not set");
+    if (d.input_fmt != EHIP_NCHW16C || d.output_fmt != EHIP_NCHW16C)
+      return fail(EHIP_UNIMPLEMENTED, "only the blocked nChw16c activation format is built");
+  }
+
+  if (d.algorithm == EHIP_CONV_DIRECT_1X1) {
+    if (d.kh != 1 || d.kw != 1) return fail(EHIP_GENERAL_ERROR, "Algorithm CONV_DIRECT_1X1 not supported for this shape.");
+    if (!(out_q || d.output_type == EHIP_S32)) return fail(EHIP_UNIMPLEMENTED, "direct_1x1: int8: only u8/s8 output");
+    if (d.g != 1) return fail(EHIP_UNIMPLEMENTED, "direct_1x1: groups are not supported");
+    if (d.pad_l || d.pad_t || d.stride_h * (d.oh - 1) + 1 > d.ih || d.stride_w * (d.ow - 1) + 1 > d.iw)
+      return fail(EHIP_UNIMPLEMENTED, "no support for padding in 1x1 u8s8 conv");
+    if (d.stride_h > 2 || d.stride_w > 2 || d.stride_h != d.stride_w)
+      return fail(EHIP_UNIMPLEMENTED, "direct_1x1: int8: Shape not supported");
+    if (d.stride_w == 2 && d.flatting_t > 0 && d.ow % d.flatting_t)
+      return fail(EHIP_UNIMPLEMENTED, "direct_1x1: int8: No Tr support for ws == 2");
+    if (d.weights_fmt != EHIP_OIHW16I16O) return fail(EHIP_UNIMPLEMENTED, "weights must be OIhw16i16o");
+    if (d.with_ip_sum && d.output_type == EHIP_S32) return fail(EHIP_UNIMPLEMENTED, "s32 output has no sum fusion");
+    c->family = FAM_GEMM_1X1;
+    return EHIP_OK;
+  }
+
+  if (d.algorithm == EHIP_CONV_DIRECT) {
+    if (depthwise) {
+      if (!(out_q || d.output_type == EHIP_S32)) return fail(EHIP_UNIMPLEMENTED, "depthwise: only u8/s8 output");
+      if (d.kh != 3 || d.kw != 3 || d.pad_l > 1 || d.pad_t > 1)
+        return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: int8: shape not supported");
+      if (d.stride_h != 1 || d.stride_w != 1) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: stride 2 is not built");
+      if (d.g % 16) return fail(EHIP_UNIMPLEMENTED, "conv: g blocking error for depthwise conv");
+      if (d.weights_fmt != EHIP_GOIHW) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: format not supported");
+      if (d.with_ip_sum) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: no sum fusion");
+      if (d.input_z != 0.0f) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: input zero point with padding");
+      c->family = FAM_DEPTHWISE;
+      return EHIP_OK;
+    }
+    if (d.g != 1) return fail(EHIP_UNIMPLEMENTED, "direct: groups are not supported");
+    if (!(out_q || d.output_type == EHIP_F32 || d.output_type == EHIP_S32))
+      return fail(EHIP_UNIMPLEMENTED, "direct: output type not supported");
+    if (d.weights_fmt != EHIP_OIHW16I16O) return fail(EHIP_UNIMPLEMENTED, "direct: format not supported");
+    // the reference's direct executor silently drops with_ip_sum (src/elx_int8_conv_direct.cpp:121);
+    // refuse instead of computing something else than asked
+    if (d.with_ip_sum) return fail(EHIP_UNIMPLEMENTED, "direct: sum fusion is only available in CONV_DIRECT_1X1");
+    if (d.kh == 1 && d.kw == 1) {
+      if (d.pad_l || d.pad_t || d.stride_h * (d.oh - 1) + 1 > d.ih || d.stride_w * (d.ow - 1) + 1 > d.iw)
+        return fail(EHIP_UNIMPLEMENTED, "direct: a160: padding is not built");
+      if (d.stride_h > 2 || d.stride_w > 2) return fail(EHIP_UNIMPLEMENTED, "direct: a160: stride not supported");
+      c->family = FAM_GEMM_1X1;
+      return EHIP_OK;
+    }
+    if (d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.pad_l <= 1 && d.pad_t <= 1) {
+      if (d.input_z != 0.0f && (d.pad_l || d.pad_t))
+        return fail(EHIP_UNIMPLEMENTED, "direct: input zero point with padding is not built");
+      if (d.flatting_t > 0 && d.ow % (d.flatting_t > d.ow ? d.ow : d.flatting_t))
+        return fail(EHIP_UNIMPLEMENTED, "direct: c160: ow must be a multiple of T (the reference mis-indexes shift for Tr != T)");
+      c->family = FAM_CONV_3X3;
+      return EHIP_OK;
+    }
+    return fail(EHIP_UNIMPLEMENTED, "direct: c160: shape not supported");
+  }
+
+  if (d.algorithm == EHIP_CONV_WINOGRAD) {
+    if (d.stride_h != 1 || d.stride_w != 1 || d.kh != 3 || d.kw != 3)
+      return fail(EHIP_UNIMPLEMENTED, "Algorithm CONV_WINOGRAD: data shape not supported");
+    if (d.g != 1) return fail(EHIP_UNIMPLEMENTED, "winograd: groups are not supported");
+    if (!all_f32) return fail(EHIP_UNIMPLEMENTED, "winograd: only fp32 user tensors are built");
+    if ((d.execution_mode & 0xF00) != 0x100)
+      return fail(EHIP_UNIMPLEMENTED, "winograd: only the int8 implementation (execution_mode 0xa1xx) is built");
+    if (d.tile_size == 0) {
+      const int t = d.n * ((d.oh + 3) / 4) * ((d.ow + 3) / 4);
+      const int ocp = up(d.oc, 16);
+      const float mac_per_read = (float)((double)t * ocp) / (float)(t + ocp);
+      d.tile_size = mac_per_read > 25.0f ? 6 : 4;
+    }
+    if (d.tile_size != 6) return fail(EHIP_UNIMPLEMENTED, "winograd: only tile_size 6 (F(4x4,3x3)) is built");
+    if (d.sampling_kind != 2) return fail(EHIP_UNIMPLEMENTED, "Winograd: to enable sampling from elk_u8s8_gemm");
+    if (d.input_scale == kNoCali || d.input_z == kNoCali)
+      return fail(EHIP_UNIMPLEMENTED, "winograd: input_quant must be set (FINE sampling is not built)");
+    if (d.tinput_scale == kNoCali || d.tinput_scale == 0.0f) return fail(EHIP_GENERAL_ERROR, "wino_tinput_quant is not set");
+    if (d.input_fmt != EHIP_NCHW16C || d.output_fmt != EHIP_NCHW16C || d.weights_fmt != EHIP_OIHW16I16O)
+      return fail(EHIP_UNIMPLEMENTED, "winograd: only blocked formats are built");
+    if (d.with_ip_sum) return fail(EHIP_UNIMPLEMENTED, "winograd: sum fusion is not built");
+    if (d.pad_t > 1 || d.pad_l > 1) return fail(EHIP_UNIMPLEMENTED, "winograd: pads > 1");
+    c->family = FAM_WINOGRAD;
+    return EHIP_OK;
+  }
+  return fail(EHIP_UNIMPLEMENTED, "algorithm not supported");
+}
+
+int setup_workspace(ehip_conv *c)
+{
+  const ehip_conv_desc_t &d = c->d;
+  c->ic2 = up(d.ic, 16) / 16;
+  c->oc2 = up(d.oc, 16) / 16;
+  int rc;
+  switch (c->family) {
+  case FAM_GEMM_1X1: {
+    c->taps = 1;
+    c->nbatch = 1;
+    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2, 1);
+    c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
+    c->kernel_name = gemm_variant_name(c->variant);
+    break;
+  }
+  case FAM_CONV_3X3: {
+    c->taps = 9;
+    c->nbatch = 1;
+    c->units_pad = up(c->ic2, 4);
+    int v = conv3x3_pick_variant(d.oh, d.ow, c->oc2);
+    // the staged tile (4 units x halo rows x (ow+2) cells) must fit the per-thread staging budget
+    for (int tries = 0; tries < 8; ++tries) {
+      const int p_t = conv3x3_variant_pixels(v);
+      int rows = (p_t + d.ow - 2) / d.ow + 1;
+      if (p_t % d.ow == 0) rows = p_t / d.ow;
+      if (rows > d.oh) rows = d.oh;
+      c->halo_rows = rows + 2;
+      const int items = 4 * c->halo_rows * (d.ow + 2);
+      if (items <= 8 * kBlock) break;
+      if (v == 4) return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too wide for the staged tile");
+      v = (v == 2 || v == 5) ? 4 : 2;
+    }
+    c->variant = v;
+    c->lds_bytes = (size_t)2 * 4 * c->halo_rows * (d.ow + 2) * 16;
+    c->kernel_name = conv3x3_variant_name(c->variant);
+    break;
+  }
+  case FAM_DEPTHWISE: {
+    c->taps = 9;
+    c->oc2 = c->ic2 = up(d.g, 16) / 16;
+    c->T = d.flatting_t > 0 ? (d.flatting_t > d.ow ? d.ow : d.flatting_t) : 1;
+    c->wtb = (d.ow + c->T - 1) / c->T;
+    c->Tr = d.ow % c->T ? d.ow % c->T : c->T;
+    c->kernel_name = "k_depthwise3x3_u8s8";
+    break;
+  }
+  case FAM_WINOGRAD: {
+    c->taps = 1;
+    c->nbatch = 36;
+    c->ht = (d.oh + 3) / 4;
+    c->wt = (d.ow + 3) / 4;
+    c->nt = c->ht * c->wt;
+    c->t = c->nt * d.n;
+    c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, 36);
+    c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
+    c->kernel_name = std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output_f32";
+    c->tin_bytes = (size_t)36 * c->ic2 * c->t * 16;
+    c->tout_bytes = (size_t)36 * c->oc2 * c->t * 16 * sizeof(float);
+    if ((rc = dev_alloc(&c->tin, c->tin_bytes, false)) != EHIP_OK) return rc;
+    if ((rc = dev_alloc(reinterpret_cast<uint8_t **>(&c->tout), c->tout_bytes, false)) != EHIP_OK) return rc;
+    break;
+  }
+  default:
+    return fail(EHIP_GENERAL_ERROR, "internal: no executor");
+  }
+
+  if (c->family == FAM_DEPTHWISE) {
+    c->ocpp = c->oc2 * 16;
+    c->wpacked_bytes = (size_t)c->oc2 * 9 * 16;
+  } else {
+    c->ocpp = up(c->oc2 * 16, kOcTile);
+    c->wpacked_bytes = (size_t)c->nbatch * c->taps * c->units_pad * c->ocpp * 16;
+  }
+  c->per_oc = (size_t)c->nbatch * c->ocpp;
+  if ((rc = dev_alloc(&c->wpacked, c->wpacked_bytes, true)) != EHIP_OK) return rc;
+  if ((rc = dev_alloc(&c->scale, c->per_oc, true)) != EHIP_OK) return rc;
+  if ((rc = dev_alloc(&c->shift, c->per_oc, true)) != EHIP_OK) return rc;
+  if ((rc = dev_alloc(&c->absmax, c->per_oc, true)) != EHIP_OK) return rc;
+  if ((rc = dev_alloc(&c->wsum, c->per_oc, true)) != EHIP_OK) return rc;
+  if ((rc = dev_alloc(&c->comp, c->per_oc, true)) != EHIP_OK) return rc;
+  return EHIP_OK;
+}
+
+Epilogue make_epilogue(const ehip_conv *c, int out_type, bool sum, bool relu)
+{
+  Epilogue e;
+  e.scale = c->scale;
+  e.shift = c->shift;
+  e.comp = c->comp;
+  e.sum_scale = c->d.sum_scale;
+  e.lo = c->d.relu_lower;
+  e.hi = c->d.relu_upper;
+  e.out_type = out_type;
+  e.with_sum = sum ? 1 : 0;
+  e.with_relu = relu ? 1 : 0;
+  return e;
+}
+
+WinoArgs make_wino_args(const ehip_conv_desc_t &d, int ic2, int oc2)
+{
+  WinoArgs w;
+  memset(&w, 0, sizeof(w));
+  w.n = d.n; w.ic2 = ic2; w.oc2 = oc2;
+  w.ih = d.ih; w.iw = d.iw; w.oh = d.oh; w.ow = d.ow;
+  w.ht = (d.oh + 3) / 4; w.wt = (d.ow + 3) / 4;
+  w.nt = w.ht * w.wt; w.t = w.nt * d.n;
+  w.pad_t = d.pad_t; w.pad_l = d.pad_l;
+  w.with_bias = d.with_bias; w.with_relu = d.with_relu;
+  return w;
+}
+
+}  // namespace
+
+extern "C" {
+
+EHIP_API const char *ehip_last_error(void) { return g_last_error.c_str(); }
+
+EHIP_API int ehip_init(int device)
+{
+  HIP_TRY(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(EHIP_GENERAL_ERROR, std::string("this library is built for gfx950 only, device is ") + prop.gcnArchName);
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_conv_create(const ehip_conv_desc_t *desc, ehip_conv_t **out)
+{
+  if (!desc || !out) return fail(EHIP_GENERAL_ERROR, "null argument");
+  *out = nullptr;
+  ehip_conv *c = new ehip_conv();
+  c->d = *desc;
+  int rc = classify(c);
+  if (rc == EHIP_OK) rc = setup_workspace(c);
+  if (rc != EHIP_OK) {
+    free_all(c);
+    delete c;
+    return rc;
+  }
+  *out = c;
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_conv_destroy(ehip_conv_t *c)
+{
+  if (!c) return EHIP_OK;
+  free_all(c);
+  delete c;
+  return EHIP_OK;
+}
+
+EHIP_API const char *ehip_conv_kernel_name(ehip_conv_t *c) { return c ? c->kernel_name.c_str() : ""; }
+
+EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const void *bias_dev, void *hip_stream)
+{
+  if (!c || !weights_dev) return fail(EHIP_GENERAL_ERROR, "Parameter error. Invalid input data!");
+  if (c->d.with_bias && !bias_dev) return fail(EHIP_GENERAL_ERROR, "Parameter error. Invalid input data!");
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  const ehip_conv_desc_t &d = c->d;
+  const float *w = static_cast<const float *>(weights_dev);
+  const float *b = static_cast<const float *>(bias_dev);
+  switch (c->family) {
+  case FAM_GEMM_1X1:
+  case FAM_CONV_3X3:
+    HIP_TRY(launch_prepare_direct(w, b, d.oc, d.ic, d.kh, d.kw, c->units_pad, c->ocpp, d, c->absmax, c->wpacked,
+                                  c->scale, c->shift, c->wsum, c->comp, s));
+    break;
+  case FAM_DEPTHWISE:
+    HIP_TRY(launch_prepare_depthwise(w, b, d.g, d, c->wpacked, c->scale, c->shift, c->wsum, s));
+    break;
+  case FAM_WINOGRAD: {
+    float *u_tmp = nullptr;
+    const size_t n = (size_t)36 * up(d.oc, 16) * up(d.ic, 16);
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&u_tmp), n * sizeof(float)));
+    hipError_t e = launch_prepare_wino(w, d.oc, d.ic, c->units_pad, c->ocpp, d, u_tmp, c->wpacked, c->scale,
+                                       c->shift, c->wsum, c->comp, s);
+    hipError_t e2 = hipStreamSynchronize(s);
+    (void)hipFree(u_tmp);
+    HIP_TRY(e);
+    HIP_TRY(e2);
+    break;
+  }
+  default:
+    return fail(EHIP_GENERAL_ERROR, "internal: no executor");
+  }
+  c->prepared = true;
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *input_dev, const void *weights_dev,
+                               const void *bias_dev, void *hip_stream)
+{
+  if (!c || !output_dev || !input_dev) return fail(EHIP_GENERAL_ERROR, "Parameter error. Invalid input data!");
+  if (!c->prepared) {
+    int rc = ehip_conv_prepare(c, weights_dev, bias_dev, hip_stream);
+    if (rc != EHIP_OK) return rc;
+  }
+  hipStream_t s = static_cast<hipStream_t>(hip_stream);
+  const ehip_conv_desc_t &d = c->d;
+  switch (c->family) {
+  case FAM_GEMM_1X1: {
+    GemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.in = static_cast<const uint8_t *>(input_dev);
+    a.w = c->wpacked;
+    a.out = output_dev;
+    a.ep = make_epilogue(c, d.output_type, d.with_ip_sum && d.algorithm == EHIP_CONV_DIRECT_1X1, d.with_relu);
+    a.p_total = d.n * d.oh * d.ow;
+    a.ohw = d.oh * d.ow; a.ow = d.ow;
+    a.ihw = d.ih * d.iw; a.iw = d.iw;
+    a.stride_h = d.stride_h; a.stride_w = d.stride_w;
+    a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    HIP_TRY(launch_gemm(a, 1, c->variant, s));
+    break;
+  }
+  case FAM_CONV_3X3: {
+    Conv3x3Args a;
+    memset(&a, 0, sizeof(a));
+    a.in = static_cast<const uint8_t *>(input_dev);
+    a.w = c->wpacked;
+    a.out = output_dev;
+    a.ep = make_epilogue(c, d.output_type, false, d.with_relu);
+    a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
+    a.pad_t = d.pad_t; a.pad_l = d.pad_l;
+    a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    a.halo_rows = c->halo_rows; a.chunk_units = 4;
+    HIP_TRY(launch_conv3x3(a, d.n, c->variant, c->lds_bytes, s));
+    break;
+  }
+  case FAM_DEPTHWISE: {
+    DepthwiseArgs a;
+    memset(&a, 0, sizeof(a));
+    a.in = static_cast<const uint8_t *>(input_dev);
+    a.w = c->wpacked;
+    a.out = output_dev;
+    a.scale = c->scale; a.shift = c->shift;
+    a.n = d.n; a.g2 = c->oc2; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
+    a.pad_t = d.pad_t; a.pad_l = d.pad_l;
+    a.T = c->T; a.Tr = c->Tr; a.wt = c->wtb;
+    a.out_type = d.output_type; a.with_relu = d.with_relu;
+    a.lo = d.relu_lower; a.hi = d.relu_upper;
+    HIP_TRY(launch_depthwise(a, s));
+    break;
+  }
+  case FAM_WINOGRAD: {
+    WinoArgs w = make_wino_args(d, c->ic2, c->oc2);
+    w.in = static_cast<const float *>(input_dev);
+    w.tin = c->tin;
+    w.tout = c->tout;
+    w.out = static_cast<float *>(output_dev);
+    w.bias = static_cast<const float *>(bias_dev);
+    if (d.with_bias && !bias_dev) return fail(EHIP_GENERAL_ERROR, "Parameter error. Invalid input data!");
+    // mrepS = input_S * (1 / tinput_S), z = ceil(tinput_z)
+    // (src/elx_conv_wino_trans_input.cpp:617-618, src/elx_int8_conv_wino.cpp:270-276)
+    const float tin_repS = 1.0f / d.tinput_scale;
+    w.mrepS = d.input_scale * tin_repS;
+    w.mz = ceilf(d.tinput_z);
+    HIP_TRY(launch_wino_trans_input(w, s));
+    GemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.in = c->tin;
+    a.w = c->wpacked;
+    a.out = c->tout;
+    a.ep = make_epilogue(c, EHIP_F32, false, false);
+    a.p_total = c->t;
+    a.ohw = c->t; a.ow = c->t; a.ihw = c->t; a.iw = c->t;
+    a.stride_h = 1; a.stride_w = 1;
+    a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    a.in_batch_stride = (long long)c->ic2 * c->t * 16;
+    a.out_batch_stride = (long long)c->oc2 * c->t * 16;
+    HIP_TRY(launch_gemm(a, 36, c->variant, s));
+    HIP_TRY(launch_wino_trans_output(w, s));
+    break;
+  }
+  default:
+    return fail(EHIP_GENERAL_ERROR, "internal: no executor");
+  }
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *bytes)
+{
+  if (!c) return fail(EHIP_GENERAL_ERROR, "null handle");
+  const ehip_conv_desc_t &d = c->d;
+  const int ocp = c->oc2 * 16, icp = c->ic2 * 16;
+  HIP_TRY(hipDeviceSynchronize());
+  auto want = [&](size_t n) {
+    if (bytes) *bytes = n;
+    return host_dst != nullptr;
+  };
+  switch (what) {
+  case EHIP_Q_WEIGHTS_S8: {
+    if (!c->prepared) return fail(EHIP_GENERAL_ERROR, "not prepared");
+    std::vector<int8_t> packed(c->wpacked_bytes);
+    if (c->family == FAM_DEPTHWISE) {
+      if (!want((size_t)ocp * 9)) return EHIP_OK;
+      HIP_TRY(hipMemcpy(packed.data(), c->wpacked, c->wpacked_bytes, hipMemcpyDeviceToHost));
+      int8_t *dst = static_cast<int8_t *>(host_dst);
+      for (int g = 0; g < ocp; ++g)
+        for (int k = 0; k < 9; ++k) dst[(size_t)g * 9 + k] = packed[((size_t)(g >> 4) * 9 + k) * 16 + (g & 15)];
+      return EHIP_OK;
+    }
+    const int taps = c->taps;
+    if (!want((size_t)c->nbatch * ocp * icp * taps)) return EHIP_OK;
+    HIP_TRY(hipMemcpy(packed.data(), c->wpacked, c->wpacked_bytes, hipMemcpyDeviceToHost));
+    int8_t *dst = static_cast<int8_t *>(host_dst);
+    for (int b = 0; b < c->nbatch; ++b)
+      for (int oc = 0; oc < ocp; ++oc)
+        for (int ic = 0; ic < icp; ++ic)
+          for (int tap = 0; tap < taps; ++tap)
+            dst[(((size_t)b * ocp + oc) * icp + ic) * taps + tap] =
+                packed[((((size_t)b * taps + tap) * c->units_pad + (ic >> 4)) * c->ocpp + oc) * 16 + (ic & 15)];
+    return EHIP_OK;
+  }
+  case EHIP_Q_SCALE:
+  case EHIP_Q_SHIFT:
+  case EHIP_Q_WSUM: {
+    if (!c->prepared) return fail(EHIP_GENERAL_ERROR, "not prepared");
+    if (!want((size_t)c->nbatch * ocp * 4)) return EHIP_OK;
+    const void *src = what == EHIP_Q_SCALE ? (const void *)c->scale
+        : what == EHIP_Q_SHIFT ? (const void *)c->shift : (const void *)c->wsum;
+    std::vector<uint32_t> tmp(c->per_oc);
+    HIP_TRY(hipMemcpy(tmp.data(), src, c->per_oc * 4, hipMemcpyDeviceToHost));
+    uint32_t *dst = static_cast<uint32_t *>(host_dst);
+    for (int b = 0; b < c->nbatch; ++b)
+      for (int oc = 0; oc < ocp; ++oc) dst[(size_t)b * ocp + oc] = tmp[(size_t)b * c->ocpp + oc];
+    return EHIP_OK;
+  }
+  case EHIP_Q_TINPUT_U8:
+    if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "not a Winograd handle");
+    if (!want(c->tin_bytes)) return EHIP_OK;
+    HIP_TRY(hipMemcpy(host_dst, c->tin, c->tin_bytes, hipMemcpyDeviceToHost));
+    return EHIP_OK;
+  case EHIP_Q_TOUTPUT_F32:
+    if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "not a Winograd handle");
+    if (!want(c->tout_bytes)) return EHIP_OK;
+    HIP_TRY(hipMemcpy(host_dst, c->tout, c->tout_bytes, hipMemcpyDeviceToHost));
+    return EHIP_OK;
+  default:
+    (void)d;
+    return fail(EHIP_GENERAL_ERROR, "unknown query");
+  }
+}
+
+EHIP_API int ehip_quantize_input_u8(void *dst_dev, const void *src_dev, size_t count, float scale, float z,
+                                    void *hip_stream)
+{
+  if (!dst_dev || !src_dev) return fail(EHIP_GENERAL_ERROR, "null argument");
+  if (scale == 0.0f) return fail(EHIP_GENERAL_ERROR, "scale is zero");
+  HIP_TRY(launch_quantize_input(static_cast<uint8_t *>(dst_dev), static_cast<const float *>(src_dev), count, scale, z,
+                                static_cast<hipStream_t>(hip_stream)));
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev, float *min_out,
+                                    float *max_out)
+{
+  if (!desc || !input_dev || !min_out || !max_out) return fail(EHIP_GENERAL_ERROR, "null argument");
+  const ehip_conv_desc_t &d = *desc;
+  if (d.kh != 3 || d.kw != 3 || d.stride_h != 1 || d.stride_w != 1 || d.input_type != EHIP_F32 ||
+      d.input_fmt != EHIP_NCHW16C)
+    return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 blocked 3x3 stride-1 layers only");
+  WinoArgs w = make_wino_args(d, up(d.ic, 16) / 16, up(d.oc, 16) / 16);
+  w.in = static_cast<const float *>(input_dev);
+  unsigned *mm = nullptr;
+  HIP_TRY(hipMalloc(reinterpret_cast<void **>(&mm), 2 * sizeof(unsigned)));
+  const unsigned init[2] = {0xffffffffu, 0u};
+  hipError_t e = hipMemcpy(mm, init, sizeof(init), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = launch_wino_range(w, d.ic, mm, nullptr);
+  unsigned res[2] = {0, 0};
+  if (e == hipSuccess) e = hipMemcpy(res, mm, sizeof(res), hipMemcpyDeviceToHost);
+  (void)hipFree(mm);
+  HIP_TRY(e);
+  auto ord2f = [](unsigned u) {
+    u = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+  };
+  *min_out = ord2f(res[0]);
+  *max_out = ord2f(res[1]);
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_reorder_nchw_to_blocked(void *dst_dev, const void *src_dev, int elem_size, int n, int c, int h,
+                                          int w, void *hip_stream)
+{
+  if (!dst_dev || !src_dev || (elem_size != 1 && elem_size != 4)) return fail(EHIP_GENERAL_ERROR, "bad argument");
+  HIP_TRY(launch_reorder_nchw_to_blocked(dst_dev, src_dev, elem_size, n, c, h, w, static_cast<hipStream_t>(hip_stream)));
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_reorder_blocked_to_nchw(void *dst_dev, const void *src_dev, int elem_size, int n, int c, int h,
+                                          int w, void *hip_stream)
+{
+  if (!dst_dev || !src_dev || (elem_size != 1 && elem_size != 4)) return fail(EHIP_GENERAL_ERROR, "bad argument");
+  HIP_TRY(launch_reorder_blocked_to_nchw(dst_dev, src_dev, elem_size, n, c, h, w, static_cast<hipStream_t>(hip_stream)));
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_reorder_oihw_to_blocked(void *dst_dev, const void *src_dev, int o, int i, int h, int w,
+                                          void *hip_stream)
+{
+  if (!dst_dev || !src_dev) return fail(EHIP_GENERAL_ERROR, "bad argument");
+  HIP_TRY(launch_reorder_oihw_to_blocked(static_cast<float *>(dst_dev), static_cast<const float *>(src_dev), o, i, h, w,
+                                         static_cast<hipStream_t>(hip_stream)));
+  return EHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,135 @@
+/*
+ * C-ABI of the MI355X (gfx950) implementation of Euler's int8 convolution path.
+ *
+ * This is the boundary a host-language binding (the C++ `euler::` API in euler.hpp, a ctypes /
+ * cgo / JNI stub ...) talks to: plain pointers, sizes and PODs, no C++ or torch types.  Every
+ * pointer named *_dev is a DEVICE pointer; the caller owns input/weights/bias/output, the
+ * handle owns its workspace (packed s8 weights, per-channel scale/shift, Winograd
+ * intermediates).  All functions return EHIP_OK (0) or an EHIP_* error code and never abort;
+ * ehip_last_error() gives the text of the calling thread's last failure.
+ *
+ * Enum values are the reference's (include/euler.hpp:35-103) so that a descriptor can be
+ * copied field by field.
+ */
+#ifndef EULER_HIP_H
+#define EULER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EHIP_API __attribute__((visibility("default")))
+
+/* status codes: 0/1/2 match ELD_OK / ELD_UNIMPLEMENTED / ELD_GENERAL_ERROR and the ELX_* trio
+ * (include/euler.hpp:44-56) */
+enum { EHIP_OK = 0, EHIP_UNIMPLEMENTED = 1, EHIP_GENERAL_ERROR = 2, EHIP_HIP_ERROR = 3 };
+
+/* data types (include/euler.hpp:66-73) */
+enum { EHIP_DT_UNDEF = 0, EHIP_F32 = 1, EHIP_F16 = 2, EHIP_U8 = 3, EHIP_S8 = 4, EHIP_S32 = 5 };
+
+/* algorithms (include/euler.hpp:35-42) */
+enum { EHIP_CONV_AUTO = 0, EHIP_CONV_DIRECT_1X1 = 1, EHIP_CONV_DIRECT = 2, EHIP_CONV_WINOGRAD = 4 };
+
+/* formats (include/euler.hpp:75-89) */
+enum {
+  EHIP_FMT_UNDEF = 0, EHIP_NCHW = 1, EHIP_NHWC = 2, EHIP_NCHW16C = 3, EHIP_OIHW = 5,
+  EHIP_OIHW16I16O = 7, EHIP_GOIHW = 9
+};
+
+/* The fields of eld_conv_t (include/euler.hpp:110-172) that the int8 path reads, as a POD.
+ * output_type EHIP_S32 is an extension: the raw s32 accumulators are written instead of the
+ * requantized result (used to check the contraction on its own). */
+typedef struct ehip_conv_desc {
+  int32_t n, g, ic, oc, ih, iw, oh, ow, kh, kw;      /* dims                     */
+  int32_t pad_l, pad_r, pad_t, pad_b;                /* pads                     */
+  int32_t stride_h, stride_w, dilation_h, dilation_w;
+  int32_t input_type, weights_type, output_type, bias_type;
+  int32_t input_fmt, weights_fmt, output_fmt;
+  int32_t algorithm, tile_size, execution_mode;
+  int32_t with_relu, with_bias, with_ip_sum;
+  int32_t flatting_o, flatting_t;                    /* flatting.{o,t}: t is the width block T;
+                                                        only the depthwise u8 store depends on it */
+  int32_t sampling_kind;                             /* must be CALIBRATED (2)   */
+  float input_scale, input_z;                        /* input_quant              */
+  float tinput_scale, tinput_z;                      /* wino_tinput_quant        */
+  float output_scale, output_z;                      /* output_quant             */
+  float sum_scale, sum_z;                            /* sum_quant                */
+  float relu_lower, relu_upper;                      /* relu_bound               */
+} ehip_conv_desc_t;
+
+typedef struct ehip_conv ehip_conv_t;
+
+/* what ehip_conv_query copies out (host buffers, canonical plain layouts) */
+enum {
+  EHIP_Q_WEIGHTS_S8 = 1,   /* direct: [OCp][ICp][kh][kw]; depthwise: [G][3][3]; winograd: [36][OCp][ICp] */
+  EHIP_Q_SCALE = 2,        /* f32 [OCp] (winograd [36][OCp])                                            */
+  EHIP_Q_SHIFT = 3,        /* f32, same shape                                                           */
+  EHIP_Q_WSUM = 4,         /* s32, same shape: sum of the quantized weights                              */
+  EHIP_Q_TINPUT_U8 = 5,    /* winograd: transformed+quantized input of the last execute [36][ICp/16][t][16] */
+  EHIP_Q_TOUTPUT_F32 = 6   /* winograd: GEMM result of the last execute [36][OCp/16][t][16]             */
+};
+
+/* Binds the calling thread to `device` and checks that it is a gfx950.  Optional: the other
+ * entry points use the current device. */
+EHIP_API int ehip_init(int device);
+EHIP_API const char *ehip_last_error(void);
+
+/* Replaces eld_conv_t::setup(): validates the descriptor, picks the executor
+ * (src/eld_conv.cpp:166-313: direct 1x1 / direct KxK / depthwise / Winograd F(4,3) int8) and
+ * allocates the device workspace.  Unsupported shapes return EHIP_UNIMPLEMENTED where the
+ * reference calls el_error()/abort(). */
+EHIP_API int ehip_conv_create(const ehip_conv_desc_t *desc, ehip_conv_t **out);
+EHIP_API int ehip_conv_destroy(ehip_conv_t *conv);
+
+/* Replaces the first-run branch of every executor (`is_first_run_`,
+ * e.g. src/elx_int8_conv_direct_1x1_xopt.hpp:27-35): per-channel abs-max quantization of the f32
+ * weights to s8, packing for the MFMA kernels, and folding of the quantization scales, bias and
+ * zero points into one scale/shift pair per output channel
+ * (src/elx_int8_conv_direct_1x1.cpp:234-355, src/elx_int8_conv_direct.cpp:311-500,
+ *  src/elx_int8_conv_direct_depthwise.cpp:200-292, src/elx_conv_wino_trans_weights.cpp:437-553).
+ * weights_dev: f32 OIhw16i16o (depthwise: goihw); bias_dev: f32 [OCp] or NULL. */
+EHIP_API int ehip_conv_prepare(ehip_conv_t *conv, const void *weights_dev, const void *bias_dev,
+                               void *hip_stream);
+
+/* Replaces elx_conv_t::execute() (src/elx_conv.hpp:125, src/elx_conv.cpp:213-240) for the
+ * steady state.  Asynchronous on `hip_stream` (NULL = the default stream).  With with_ip_sum the
+ * output buffer also holds the sum operand.  If the handle has not been prepared yet,
+ * weights_dev/bias_dev are used to do so first (the reference's lazy first run); afterwards
+ * they are ignored and may be NULL. */
+EHIP_API int ehip_conv_execute(ehip_conv_t *conv, void *output_dev, const void *input_dev,
+                               const void *weights_dev, const void *bias_dev, void *hip_stream);
+
+/* Copies workspace contents to a host buffer in a canonical layout (see EHIP_Q_*).  Synchronous.
+ * Returns the number of bytes through *bytes when host_dst is NULL. */
+EHIP_API int ehip_conv_query(ehip_conv_t *conv, int what, void *host_dst, size_t *bytes);
+
+/* Name of the kernel variant execute() launches (for profiles), and its launch geometry. */
+EHIP_API const char *ehip_conv_kernel_name(ehip_conv_t *conv);
+
+/* Replaces the harness-side fp32 -> u8 activation quantization
+ * (tests/elt_conv_utils.cpp:354-401): dst = (uint8_t) round(src / scale + z) with that helper's
+ * tie rule. */
+EHIP_API int ehip_quantize_input_u8(void *dst_dev, const void *src_dev, size_t count, float scale,
+                                    float z, void *hip_stream);
+
+/* Replaces the harness-side calibration of wino_tinput_quant (tests/elt_conv_utils.cpp:222-262):
+ * min and max over the fp32 Winograd-transformed input.  Synchronous. */
+EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev,
+                                    float *min_out, float *max_out);
+
+/* Device-side layout reorders with the index maps of src/elx_reorder.cpp:35-93
+ * (elem_size 1 or 4).  nchw <-> nChw16c and oihw -> OIhw16i16o; channel tails are zero-filled. */
+EHIP_API int ehip_reorder_nchw_to_blocked(void *dst_dev, const void *src_dev, int elem_size, int n,
+                                          int c, int h, int w, void *hip_stream);
+EHIP_API int ehip_reorder_blocked_to_nchw(void *dst_dev, const void *src_dev, int elem_size, int n,
+                                          int c, int h, int w, void *hip_stream);
+EHIP_API int ehip_reorder_oihw_to_blocked(void *dst_dev, const void *src_dev, int o, int i, int h,
+                                          int w, void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EULER_HIP_H */

@@ -58,7 +58,7 @@ inline void fold_scale_shift(const orc_conv_params *p, float w_S, float wsum, fl
                              float *scale, float *shift)
 {
   float s, z;
-  if (p->out_type == ORC_F32) {
+  if (p->out_type == ORC_F32 || p->out_type == ORC_S32) {
     s = p->in_scale * w_S;
     z = fmaf(-(p->in_z * wsum), s, bias);
   } else {

@@ -1,0 +1,119 @@
+"""Shared helpers for the GPU parity tests: seeded layer generation, oracle evaluation and the call
+through the C-ABI (via the package's ctypes binding).  torch is used only to own device memory."""
+import importlib
+
+import numpy as np
+
+import oracle_lib as ol
+
+f32 = np.float32
+
+
+def pkg():
+    return importlib.import_module("deep-learning-math-kernel-research_amd")
+
+
+def dev(arr):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(arr)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def bits(a):
+    """flat byte view, for bit-exact comparisons of float arrays"""
+    a = np.ascontiguousarray(a).ravel()
+    return a.view(np.uint8)
+
+
+class Layer:
+    """One seeded synthetic layer: tensors in the reference's blocked formats, the oracle's
+    parameters and the product's descriptor side by side."""
+
+    def __init__(self, n, ic, oc, hw, k=1, pad=0, stride=1, out_type=ol.U8, algorithm=None, with_sum=False,
+                 depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None):
+        E = pkg()
+        rng = np.random.default_rng(seed)
+        self.E = E
+        self.n, self.ic, self.oc, self.hw, self.k = n, ic, oc, hw, k
+        self.depthwise = depthwise
+        g = ic if depthwise else 1
+        x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
+        self.x_u8 = ol.quantize_input_u8(x, 1.0 / 255.0, 0.0)
+        self.xb = ol.to_blocked(self.x_u8)
+        if depthwise:
+            self.w = rng.normal(0, w_sigma, (ic, k, k)).astype(f32)
+            self.wb = self.w
+        else:
+            self.w = rng.normal(0, w_sigma, (oc, ic, k, k)).astype(f32)
+            self.wb = ol.weights_to_blocked(self.w)
+        self.bias = np.zeros(ol.up16(oc), f32)
+        self.bias[:oc] = rng.normal(0, 0.01, oc).astype(f32)
+        # output scale from the float result range (what the reference harness derives by running fp32)
+        fan = ic * k * k if not depthwise else k * k
+        out_scale = float(f32(4.0 * w_sigma * np.sqrt(fan) * 0.6 / 255.0)) if out_type in (ol.U8, ol.S8) else 1.0
+        if depthwise:
+            out_scale = float(f32(6.0 / 255.0))
+        if relu_hi is None:
+            relu_hi = 255.0 if (depthwise and out_type == ol.U8) else (127.0 if out_type == ol.S8 else ol.FLT_MAX)
+        sum_scale = 0.0
+        self.old = None
+        if with_sum:
+            r = rng.normal(0, 1, (n, oc, (hw - k + 2 * pad) // stride + 1, (hw - k + 2 * pad) // stride + 1)).astype(f32)
+            s_r = float(np.abs(r).max() / 127.0)
+            np_t = ol.NP_OF[out_type]
+            q = np.rint(r / f32(s_r))
+            if out_type == ol.U8:
+                q = np.abs(q)
+            self.old = ol.to_blocked(q.astype(np_t))
+            sum_scale = float(f32(s_r) / f32(out_scale))
+        self.p = ol.make_params(n, ic, oc, hw, hw, k, k, pad, stride, g=g, out_type=out_type, with_bias=with_bias,
+                                with_relu=with_relu, with_sum=with_sum, T=T, out_scale=out_scale, sum_scale=sum_scale,
+                                relu_hi=relu_hi)
+        if algorithm is None:
+            algorithm = E.CONV_DIRECT_1X1 if (k == 1 and out_type in (ol.U8, ol.S8, ol.S32)) else E.CONV_DIRECT
+        self.desc = E.make_desc(n, ic, oc, hw, hw, k, k, pad, stride, g=g, algorithm=algorithm,
+                                output_type=out_type, with_bias=with_bias, with_relu=with_relu, with_ip_sum=with_sum,
+                                output_quant=(out_scale, 0.0), sum_quant=(sum_scale, 0.0),
+                                relu_bound=(0.0, relu_hi), flatting_t=T)
+
+    # ---- oracle -----------------------------------------------------------------------------
+    def oracle(self):
+        p = self.p
+        if self.depthwise:
+            wq, scale, shift, wsum = ol.depthwise_prepare(p, self.wb, self.bias)
+            out, acc = ol.depthwise_execute(p, self.xb, wq, scale, shift)
+        else:
+            wq, scale, shift, wsum = ol.direct_prepare(p, self.wb, self.bias)
+            if p.out_type == ol.S32:
+                q = ol.ConvParams.from_buffer_copy(p)
+                q.out_type = ol.U8
+                _, acc = ol.direct_execute(q, self.xb, wq, scale, shift)
+                out = acc
+            else:
+                out, acc = ol.direct_execute(p, self.xb, wq, scale, shift, out_init=self.old)
+        return dict(wq=wq, scale=scale, shift=shift, wsum=wsum, out=out, acc=acc)
+
+    # ---- product ----------------------------------------------------------------------------
+    def run_gpu(self, lazy_prepare=False):
+        import torch
+        E = self.E
+        conv = E.Conv(self.desc)
+        d_x, d_w, d_b = dev(self.xb), dev(self.wb), dev(self.bias)
+        oc2 = ol.up16(self.oc) // 16
+        shape = (self.n, oc2, self.desc.oh, self.desc.ow, 16)
+        tdt = {ol.U8: torch.uint8, ol.S8: torch.int8, ol.F32: torch.float32, ol.S32: torch.int32}[self.p.out_type]
+        if self.old is not None:
+            d_out = dev(self.old)
+        else:
+            d_out = torch.full(shape, 77, dtype=tdt, device="cuda")
+        if lazy_prepare:
+            conv.execute(d_out, d_x, d_w, d_b)
+        else:
+            conv.prepare(d_w, d_b)
+            conv.execute(d_out, d_x)
+        torch.cuda.synchronize()
+        res = dict(out=host(d_out), conv=conv)
+        return res

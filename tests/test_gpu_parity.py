@@ -1,0 +1,148 @@
+"""GPU parity: the HIP path, called through the C-ABI, against the CPU oracle on the same seeded
+inputs.  Bars: s32 accumulators, quantized weights and u8/s8 outputs bit-exact; f32 scale/shift and
+f32 outputs bit-exact as well (the north-star tolerance is 1 ULP; the tests hold the tighter bar)."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_common import Layer, bits, dev, host, pkg
+
+pytestmark = pytest.mark.gpu
+
+
+def check_prepare(res, orc, E):
+    conv = res["conv"]
+    wq = conv.query(E.Q_WEIGHTS_S8)
+    assert np.array_equal(wq, orc["wq"].ravel()), "quantized weights differ"
+    assert np.array_equal(conv.query(E.Q_WSUM), orc["wsum"])
+    assert np.array_equal(bits(conv.query(E.Q_SCALE)), bits(orc["scale"])), "scale differs"
+    assert np.array_equal(bits(conv.query(E.Q_SHIFT)), bits(orc["shift"])), "shift differs"
+
+
+def run_and_compare(layer, lazy=False):
+    E = pkg()
+    orc = layer.oracle()
+    res = layer.run_gpu(lazy_prepare=lazy)
+    check_prepare(res, orc, E)
+    got, exp = res["out"], orc["out"]
+    assert got.shape == exp.shape
+    if not np.array_equal(bits(got), bits(exp)):
+        bad = np.argwhere(got != exp)
+        raise AssertionError("output differs at %d of %d positions, first %s: got %s expected %s (kernel %s)" % (
+            len(bad), got.size, bad[0], got[tuple(bad[0])], exp[tuple(bad[0])], res["conv"].kernel_name))
+    return res
+
+
+# ---- 1x1 (CONV_DIRECT_1X1 a160; f32 output goes through CONV_DIRECT a160) ----------------------
+@pytest.mark.parametrize("out_type", [ol.S32, ol.U8, ol.S8, ol.F32])
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 64, 64, 9), (1, 80, 48, 7), (3, 128, 272, 5)])
+def test_conv1x1_s1(out_type, n, ic, oc, hw):
+    run_and_compare(Layer(n, ic, oc, hw, out_type=out_type, seed=11 + ic + out_type))
+
+
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
+def test_conv1x1_sum_relu(out_type):
+    run_and_compare(Layer(2, 96, 64, 14, out_type=out_type, with_sum=True, seed=5))
+
+
+@pytest.mark.parametrize("out_type", [ol.S32, ol.S8])
+def test_conv1x1_stride2(out_type):
+    run_and_compare(Layer(2, 64, 96, 14, stride=2, out_type=out_type, with_sum=(out_type == ol.S8), seed=6))
+
+
+def test_conv1x1_lazy_first_run_and_no_bias():
+    run_and_compare(Layer(1, 64, 32, 6, out_type=ol.U8, with_bias=False, seed=8), lazy=True)
+
+
+@pytest.mark.parametrize("variant", range(8))
+def test_conv1x1_every_kernel_variant(variant, monkeypatch):
+    monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
+    res = run_and_compare(Layer(2, 128, 80, 11, out_type=ol.S8, with_sum=True, seed=40 + variant))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
+# ---- 3x3 direct (c160) ------------------------------------------------------------------------------
+@pytest.mark.parametrize("out_type", [ol.S32, ol.U8, ol.S8, ol.F32])
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 14), (1, 128, 128, 28), (2, 48, 80, 10), (1, 64, 16, 7)])
+def test_conv3x3(out_type, n, ic, oc, hw):
+    run_and_compare(Layer(n, ic, oc, hw, k=3, pad=1, out_type=out_type, seed=21 + hw + out_type))
+
+
+def test_conv3x3_no_padding():
+    run_and_compare(Layer(2, 32, 32, 12, k=3, pad=0, out_type=ol.U8, seed=3))
+
+
+@pytest.mark.parametrize("variant", range(6))
+def test_conv3x3_every_kernel_variant(variant, monkeypatch):
+    monkeypatch.setenv("EHIP_CONV3X3_VARIANT", str(variant))
+    run_and_compare(Layer(2, 64, 144, 13, k=3, pad=1, out_type=ol.U8, seed=60 + variant))
+
+
+# ---- depthwise 3x3 ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
+@pytest.mark.parametrize("g,hw,T", [(32, 14, 7), (144, 56, 14), (64, 7, 7), (16, 28, 11), (32, 9, 4), (32, 5, 0)])
+def test_depthwise(out_type, g, hw, T):
+    n = 2 if hw < 56 else 1
+    run_and_compare(Layer(n, g, g, hw, k=3, pad=1, out_type=out_type, depthwise=True, seed=g + hw + T, w_sigma=0.1,
+                          T=T))
+
+
+# ---- input quantizer and reorders ---------------------------------------------------------------------
+def test_quantize_input_u8():
+    import torch
+    E = pkg()
+    rng = np.random.default_rng(1)
+    x = rng.uniform(0, 1, 1 << 16).astype(np.float32)
+    x[:8] = [0.0, 1.0, 0.5 / 255, 1.5 / 255, 2.5 / 255, 254.5 / 255, 0.999999, 1e-9]
+    for count in (x.size, x.size - 3, 5):
+        d_x = dev(x[:count])
+        d_q = torch.zeros(count, dtype=torch.uint8, device="cuda")
+        E.quantize_input_u8(d_q, d_x, count, 1.0 / 255.0, 0.0)
+        torch.cuda.synchronize()
+        assert np.array_equal(host(d_q), ol.quantize_input_u8(x[:count], 1.0 / 255.0, 0.0))
+    # exact ties go to the odd neighbour, as in the reference's helper
+    t = np.array([0.5, 1.5, 2.5, 3.5, 4.5], np.float32)
+    d_q = torch.zeros(5, dtype=torch.uint8, device="cuda")
+    E.quantize_input_u8(d_q, dev(t), 5, 1.0, 0.0)
+    assert host(d_q).tolist() == [1, 1, 3, 3, 5]
+
+
+def test_device_reorders():
+    import torch
+    E = pkg()
+    rng = np.random.default_rng(2)
+    x = rng.normal(size=(2, 20, 5, 3)).astype(np.float32)
+    d = torch.zeros((2, 2, 5, 3, 16), dtype=torch.float32, device="cuda")
+    E.reorder_nchw_to_blocked(d, dev(x), 4, 2, 20, 5, 3)
+    assert np.array_equal(host(d), ol.to_blocked(x))
+    back = torch.zeros((2, 20, 5, 3), dtype=torch.float32, device="cuda")
+    E.reorder_blocked_to_nchw(back, d, 4, 2, 20, 5, 3)
+    assert np.array_equal(host(back), x)
+    u = rng.integers(0, 256, (1, 17, 4, 4)).astype(np.uint8)
+    du = torch.zeros((1, 2, 4, 4, 16), dtype=torch.uint8, device="cuda")
+    E.reorder_nchw_to_blocked(du, dev(u), 1, 1, 17, 4, 4)
+    assert np.array_equal(host(du), ol.to_blocked(u))
+    w = rng.normal(size=(20, 35, 3, 3)).astype(np.float32)
+    dw = torch.zeros((2, 3, 3, 3, 16, 16), dtype=torch.float32, device="cuda")
+    E.reorder_oihw_to_blocked(dw, dev(w), 20, 35, 3, 3)
+    assert np.array_equal(host(dw), ol.weights_to_blocked(w))
+
+
+# ---- error behaviour of setup ---------------------------------------------------------------------------
+def test_setup_rejects_what_the_reference_rejects():
+    E = pkg()
+    bad = [
+        E.make_desc(1, 64, 64, 8, 8, 1, 1, pad=1, algorithm=E.CONV_DIRECT_1X1),            # padding in 1x1
+        E.make_desc(1, 64, 64, 8, 8, 3, 3, pad=1, algorithm=E.CONV_DIRECT_1X1),            # not a 1x1
+        E.make_desc(1, 64, 64, 8, 8, 5, 5, pad=2, algorithm=E.CONV_DIRECT),                # 5x5 not built
+        E.make_desc(1, 64, 64, 8, 8, 3, 3, pad=1, algorithm=E.CONV_DIRECT, sampling_kind=E.FINE),
+        E.make_desc(1, 24, 24, 8, 8, 3, 3, pad=1, g=24, algorithm=E.CONV_DIRECT),          # g % 16
+        E.make_desc(1, 64, 64, 8, 8, 1, 1, algorithm=E.CONV_DIRECT_1X1, output_type=E.F32),
+    ]
+    for d in bad:
+        with pytest.raises(E.EulerHipError) as ei:
+            E.Conv(d)
+        assert ei.value.code in (E.EHIP_UNIMPLEMENTED, E.EHIP_GENERAL_ERROR)
+    conv = E.Conv(E.make_desc(1, 64, 64, 8, 8))
+    with pytest.raises(E.EulerHipError):
+        conv.execute(None, None)

@@ -1,0 +1,78 @@
+"""GPU parity of the Winograd F(4x4,3x3) int8 pipeline, stage by stage, against the CPU oracle:
+calibration range, transformed+quantized weights, u8 transformed input, f32 GEMM result and the
+final fp32 output -- all compared bit for bit (the north-star tolerance for fp32 is 1 ULP)."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_common import bits, dev, host, pkg
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def make_wino(n, ic, oc, hw, seed, with_bias=True, with_relu=True):
+    E = pkg()
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
+    w = rng.normal(0, 0.02, (oc, ic, 3, 3)).astype(f32)
+    bias = np.zeros(ol.up16(oc), f32)
+    bias[:oc] = rng.normal(0, 0.01, oc)
+    xb, wb = ol.to_blocked(x), ol.weights_to_blocked(w)
+    p = ol.make_params(n, ic, oc, hw, hw, 3, 3, 1, out_type=ol.F32, in_scale=1.0, with_bias=with_bias,
+                       with_relu=with_relu)
+    d = E.make_desc(n, ic, oc, hw, hw, 3, 3, 1, algorithm=E.CONV_WINOGRAD, input_type=E.F32, output_type=E.F32,
+                    with_bias=with_bias, with_relu=with_relu, input_quant=(1.0, 0.0), tile_size=6,
+                    execution_mode=0xa161, wino_tinput_quant=(1.0, 0.0))
+    return E, p, d, xb, wb, bias
+
+
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 10), (1, 64, 48, 12), (3, 16, 80, 7), (1, 32, 32, 28)])
+def test_wino_pipeline(n, ic, oc, hw):
+    import torch
+    E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 100 + hw)
+    d_x = dev(xb)
+    # calibration of wino_tinput_quant from the fp32 transformed input
+    mn, mx = E.wino_tinput_range(d, d_x)
+    omn, omx = ol.wino_tinput_range(p, xb)
+    assert (f32(mn), f32(mx)) == (f32(omn), f32(omx))
+    diff = f32(mx) - f32(mn) + f32(0.000001)
+    s_t, z_t = float(diff / f32(255.0)), float(-f32(mn) * f32(255.0) / diff)
+    p.tin_scale, p.tin_z = s_t, z_t
+    d.tinput_scale, d.tinput_z = s_t, z_t
+
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tin = ol.wino_trans_input(p, xb)
+    tout, _ = ol.wino_gemm(p, tin, twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias)
+
+    conv = E.Conv(d)
+    d_w, d_b = dev(wb), dev(bias)
+    d_out = torch.full(exp.shape, -7.0, dtype=torch.float32, device="cuda")
+    conv.prepare(d_w, d_b)
+    conv.execute(d_out, d_x, None, d_b)
+    torch.cuda.synchronize()
+    assert np.array_equal(conv.query(E.Q_WEIGHTS_S8), twq.ravel()), "transformed weights differ"
+    assert np.array_equal(bits(conv.query(E.Q_SCALE)), bits(tscale))
+    assert np.array_equal(bits(conv.query(E.Q_SHIFT)), bits(tshift))
+    g_tin = conv.query(E.Q_TINPUT_U8).reshape(tin.shape)
+    assert np.array_equal(g_tin, tin), "u8 transformed input differs at %d cells" % int((g_tin != tin).sum())
+    g_tout = conv.query(E.Q_TOUTPUT_F32).reshape(tout.shape)
+    assert np.array_equal(bits(g_tout), bits(tout)), "GEMM result differs"
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d" % int((got != exp).sum())
+
+
+def test_wino_no_bias_no_relu():
+    import torch
+    E, p, d, xb, wb, bias = make_wino(1, 32, 32, 9, seed=4, with_bias=False, with_relu=False)
+    p.tin_scale, p.tin_z = 0.04, 100.3
+    d.tinput_scale, d.tinput_z = 0.04, 100.3
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xb), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias)
+    conv = E.Conv(d)
+    d_out = torch.zeros(exp.shape, dtype=torch.float32, device="cuda")
+    conv.execute(d_out, dev(xb), dev(wb), None)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(host(d_out)), bits(exp))
