@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 convolution hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--layers all|none|C1,C3a,...]
+
+A step is one pass of the hot path (one elx_conv-equivalent execute) over one batch of synthetic,
+device-resident tensors of the named layer.  The headline workload is C2 (int8 3x3 direct conv,
+ResNet-50 res3 shape, N=32).  Prints ONE JSON line: effective INT8 TOPS (2 x direct-conv MACs /
+time, the reference's accounting), the roofline of the dominant kernel from HIP-event timing, the
+host-CPU baseline of the same layer, and -- under "layers" -- the other configured layers.
+"""
+import argparse
+import ctypes
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+PKG = "deep-learning-math-kernel-research_amd"
+
+
+def measure(layer, steps, warmup):
+    """(wall seconds per step, HIP-event seconds per step).  Both regions hold exactly `steps`
+    executions enqueued back to back on the stream the kernels run on (the default stream)."""
+    import torch
+    layer.run(warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    layer.run(steps)
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def single_launch_latency(layer, reps=20):
+    import torch
+    best = 1e9
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        layer.run(1)
+        torch.cuda.synchronize()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def roofline_of(wl, sec_per_launch, traffic):
+    from importlib import import_module
+    W = import_module(PKG + ".workloads")
+    kind, _ = wl.bound()
+    if kind == "mfma":
+        achieved = wl.ops() / sec_per_launch / 1e12
+        peak, unit = W.PEAK_INT8_TOPS, "TFLOP/s"
+    else:
+        achieved = wl.algorithmic_bytes() / sec_per_launch / 1e9
+        peak, unit = W.PEAK_HBM_GBS, "GB/s"
+    return {"bound": kind, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 5), "traffic": traffic}
+
+
+def cpu_baseline(wl, budget_s=12.0):
+    """The CPU oracle (a port of the reference's loop nest; AVX-512-VNNI inner loop when the host
+    has it) timed on this host's cores on the same layer.  Bounded: as many passes as fit ~budget."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import numpy as np
+    import oracle_lib as ol
+    rng = np.random.default_rng(7)
+    n = wl.n
+    # keep one pass in the low seconds even on a scalar host: sample a slice of the batch
+    lib = ol.oracle()
+    vnni = bool(lib.orc_has_vnni())
+    threads = int(lib.orc_num_threads())
+    if wl.algorithm != 2 or wl.depthwise or wl.k not in (1, 3):
+        return None
+    if not vnni:
+        n = max(1, n // 8)
+    x = rng.integers(0, 256, (n, ol.up16(wl.ic) // 16, wl.hw, wl.hw, 16)).astype(np.uint8)
+    w = rng.normal(0, wl.w_sigma, (wl.oc, wl.ic, wl.k, wl.k)).astype(np.float32)
+    b = rng.normal(0, 0.01, ol.up16(wl.oc)).astype(np.float32)
+    p = ol.make_params(n, wl.ic, wl.oc, wl.hw, wl.hw, wl.k, wl.k, wl.pad, wl.stride, out_type=wl.out_type,
+                       out_scale=0.02)
+    wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(w), b)   # first run, excluded from timing
+    out = np.zeros((n, ol.up16(wl.oc) // 16, wl.oh, wl.oh, 16), ol.NP_OF[wl.out_type])
+    args = (ctypes.byref(p), ol.ptr(x), ol.ptr(wq), ol.ptr(scale), ol.ptr(shift), ol.ptr(out), None)
+    lib.orc_direct_execute(*args)  # warm-up
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        lib.orc_direct_execute(*args)
+        passes += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or passes >= 1024:
+            break
+    sec = el / passes
+    ops = wl.ops() * n / wl.n
+    return {"value": round(ops / sec / 1e12, 4), "unit": "TOPS", "cores": threads, "kind": "port",
+            "isa": "avx512-vnni" if vnni else "scalar/auto-vectorised",
+            "sample": "%d passes of %s with N=%d of %d in %.1f s (weight preparation excluded)" % (
+                passes, wl.key, n, wl.n, el),
+            "ms_per_pass": round(sec * 1e3, 3), "images_per_s": round(n / sec, 1)}
+
+
+def load_traffic():
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            return json.load(f)
+    return {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="C2")
+    ap.add_argument("--layers", default="all", help="other layers to report: all, none or a comma list")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU: every layer is a single-device kernel and nothing here "
+              "shards across devices (batch-parallel sharding is described in DESIGN.md); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    E = importlib.import_module(PKG)
+    W = importlib.import_module(PKG + ".workloads")
+    rc = E.lib.ehip_init(0)
+    if rc != 0:
+        print("bench.py: " + E.lib.ehip_last_error().decode(), file=sys.stderr)
+        sys.exit(1)
+    traffic = load_traffic()
+
+    wl = W.WORKLOADS[args.workload]
+    layer = W.DeviceLayer(wl)
+    wall, ev = measure(layer, args.steps, args.warmup)
+    lat = single_launch_latency(layer)
+    tops = wl.ops() / wall / 1e12
+    result = {
+        "metric": "effective_int8_tops", "value": round(tops, 3), "unit": "TOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "%s: %s" % (wl.key, wl.title), "ops_per_step": wl.ops(),
+                   "algorithmic_bytes_per_step": wl.algorithmic_bytes(), "kernel": layer.conv.kernel_name},
+        "images_per_s": round(wl.n / wall, 1),
+        "single_launch_latency_us": round(lat * 1e6, 2),
+        "event_ms_per_step": round(ev * 1e3, 6),
+        "roofline": roofline_of(wl, ev, traffic.get(wl.key)),
+    }
+    del layer
+    torch.cuda.empty_cache()
+
+    layers = {}
+    keys = [] if args.layers == "none" else (
+        [k for k in W.WORKLOADS if k != wl.key] if args.layers == "all" else args.layers.split(","))
+    for k in keys:
+        w2 = W.WORKLOADS[k]
+        l2 = W.DeviceLayer(w2)
+        steps = 200
+        wall2, ev2 = measure(l2, steps, 10)
+        layers[k] = {"title": w2.title, "tops": round(w2.ops() / wall2 / 1e12, 3),
+                     "images_per_s": round(w2.n / wall2, 1), "ms_per_step": round(wall2 * 1e3, 5),
+                     "event_ms_per_step": round(ev2 * 1e3, 5), "kernel": l2.conv.kernel_name,
+                     "roofline": roofline_of(w2, ev2, traffic.get(k))}
+        del l2
+        torch.cuda.empty_cache()
+    if layers:
+        result["layers"] = layers
+
+    if not args.no_cpu:
+        try:
+            result["cpu_baseline"] = cpu_baseline(wl)
+        except Exception as exc:  # the baseline is a report, never a reason to lose the GPU number
+            result["cpu_baseline"] = {"value": None, "unit": "TOPS", "cores": 0, "kind": "port",
+                                      "sample": "failed: %r" % (exc,)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -473,6 +473,17 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
   return EHIP_OK;
 }
 
+EHIP_API int ehip_conv_execute_repeat(ehip_conv_t *c, void *output_dev, const void *input_dev,
+                                      const void *bias_dev, int count, void *hip_stream)
+{
+  if (!c || !c->prepared) return fail(EHIP_GENERAL_ERROR, "execute_repeat needs a prepared handle");
+  for (int i = 0; i < count; ++i) {
+    const int rc = ehip_conv_execute(c, output_dev, input_dev, nullptr, bias_dev, hip_stream);
+    if (rc != EHIP_OK) return rc;
+  }
+  return EHIP_OK;
+}
+
 EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *bytes)
 {
   if (!c) return fail(EHIP_GENERAL_ERROR, "null handle");

@@ -1,0 +1,144 @@
+"""The configured int8 layers (ResNet-50 / VGG-16 / MobileNet-v2 shapes) with their operation and
+byte accounting, and synthetic-tensor setup on the device.
+
+Operations follow the reference's benchmark accounting (tests/elt_conv_utils.cpp:638-659):
+2 x multiply-accumulates of the DIRECT algorithm with padded taps left out -- so Winograd figures
+are "effective" TOPS.  Algorithmic bytes = every user tensor touched once (input, packed s8
+weights, output, sum operand, per-channel f32 scale + shift); Winograd intermediates are not
+algorithmic.
+"""
+import math
+
+from . import (CONV_DIRECT, CONV_DIRECT_1X1, CONV_WINOGRAD, EL_NO_CALI, F32, FLT_MAX, S8, U8, Conv, make_desc,
+               up16, wino_tinput_range)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+
+
+class Workload:
+    def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
+                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False):
+        self.key, self.title = key, title
+        self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
+        self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
+        self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
+        self.oh = (hw + 2 * pad - k) // stride + 1
+
+    # 2 * MACs, padded taps excluded
+    def ops(self):
+        def valid(o_len, i_len):
+            tot = 0
+            for o in range(o_len):
+                for kk in range(self.k):
+                    i = o * self.stride + kk - self.pad
+                    tot += 0 <= i < i_len
+            return tot
+        v = valid(self.oh, self.hw)
+        per_pair = v * v
+        g = self.ic if self.depthwise else 1
+        return 2.0 * self.n * per_pair * (self.ic // g) * self.oc
+
+    def algorithmic_bytes(self):
+        esz = {U8: 1, S8: 1, F32: 4}
+        n_in = self.n * up16(self.ic) * self.hw * self.hw
+        if self.stride == 2 and self.k == 1:
+            n_in //= 4  # a stride-2 1x1 only samples every other row and column
+        n_out = self.n * up16(self.oc) * self.oh * self.oh
+        if self.depthwise:
+            w = up16(self.oc) * 9
+        elif self.algorithm == CONV_WINOGRAD:
+            w = 36 * up16(self.ic) * up16(self.oc)
+        else:
+            w = up16(self.ic) * up16(self.oc) * self.k * self.k
+        b = n_in * esz[self.in_type] + w + n_out * esz[self.out_type] + 8 * up16(self.oc)
+        if self.with_sum:
+            b += n_out * esz[self.out_type]
+        return float(b)
+
+    def bound(self):
+        t_mfma = self.ops() / (PEAK_INT8_TOPS * 1e12)
+        t_hbm = self.algorithmic_bytes() / (PEAK_HBM_GBS * 1e9)
+        return ("mfma", t_mfma) if t_mfma >= t_hbm else ("hbm", t_hbm)
+
+    def descriptor(self, out_scale=None, tinput_quant=(EL_NO_CALI, EL_NO_CALI)):
+        fan = self.k * self.k * (1 if self.depthwise else self.ic)
+        if out_scale is None:
+            # u8 in [0,255]/255 ~ U[0,1): E[x^2] = 1/3; four sigmas of the pre-activation over the code range
+            out_scale = 4.0 * self.w_sigma * math.sqrt(fan / 3.0) / (127.0 if self.out_type == S8 else 255.0)
+        relu = (0.0, FLT_MAX)
+        if self.relu6:
+            out_scale = 6.0 / 255.0
+            relu = (0.0, 255.0)   # ReLU6 in the quantized output domain
+        if self.out_type == S8:
+            relu = (0.0, 127.0)
+        g = self.ic if self.depthwise else 1
+        return make_desc(self.n, self.ic, self.oc, self.hw, self.hw, self.k, self.k, self.pad, self.stride, g=g,
+                         algorithm=self.algorithm, input_type=self.in_type, output_type=self.out_type,
+                         with_bias=True, with_relu=True, with_ip_sum=self.with_sum,
+                         input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, 0.0),
+                         output_quant=(out_scale, 0.0), sum_quant=(0.7, 0.0) if self.with_sum else (0.0, 0.0),
+                         wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
+                         tile_size=6 if self.algorithm == CONV_WINOGRAD else 0,
+                         execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
+
+
+WORKLOADS = {w.key: w for w in [
+    Workload("C1", "1x1 64->256 @56x56 N=1, ReLU, f32 out (ResNet-50 res2 expand)", 1, 64, 256, 56, out_type=F32),
+    Workload("C2", "3x3 128->128 @28x28 N=32 pad 1, bias+ReLU, u8 out (ResNet-50 res3)", 32, 128, 128, 28, k=3, pad=1,
+             T=14),
+    Workload("C3a", "1x1 1024->256 @14x14 N=64, sum+ReLU, s8 out (ResNet-50 res4 reduce)", 64, 1024, 256, 14,
+             algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True),
+    Workload("C3b", "1x1 s2 512->1024 28x28->14x14 N=64, sum+ReLU, s8 out (ResNet-50 res4 projection)", 64, 512, 1024,
+             28, stride=2, algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True),
+    Workload("C4a", "Winograd F(4,3) 256->256 @56x56 N=64, fp32 in/out (VGG-16 conv3)", 64, 256, 256, 56, k=3, pad=1,
+             algorithm=CONV_WINOGRAD, in_type=F32, out_type=F32, w_sigma=0.02),
+    Workload("C4b", "Winograd F(4,3) 512->512 @28x28 N=64, fp32 in/out (VGG-16 conv4)", 64, 512, 512, 28, k=3, pad=1,
+             algorithm=CONV_WINOGRAD, in_type=F32, out_type=F32, w_sigma=0.02),
+    Workload("C5a", "depthwise 3x3 C=144 @56x56 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 144, 144, 56, k=3, pad=1,
+             depthwise=True, w_sigma=0.1, T=14, relu6=True),
+    Workload("C5b", "depthwise 3x3 C=960 @7x7 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 960, 960, 7, k=3, pad=1,
+             depthwise=True, w_sigma=0.1, T=7, relu6=True),
+]}
+
+
+class DeviceLayer:
+    """Synthetic device-resident tensors of one workload (torch owns the memory) and its prepared
+    convolution handle."""
+
+    def __init__(self, wl, seed=1234):
+        import torch
+        self.wl = wl
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+        ic2, oc2 = up16(wl.ic) // 16, up16(wl.oc) // 16
+        if wl.in_type == U8:
+            # fp32 U[0,1) activations quantized with scale 1/255 are uniform codes 0..255
+            self.x = torch.randint(0, 256, (wl.n, ic2, wl.hw, wl.hw, 16), dtype=torch.uint8, device="cuda",
+                                   generator=gen)
+        else:
+            self.x = torch.rand((wl.n, ic2, wl.hw, wl.hw, 16), dtype=torch.float32, device="cuda", generator=gen)
+        if wl.depthwise:
+            self.w = torch.randn((wl.ic, 3, 3), dtype=torch.float32, device="cuda", generator=gen) * wl.w_sigma
+        else:
+            self.w = torch.randn((oc2, ic2, wl.k, wl.k, 16, 16), dtype=torch.float32, device="cuda",
+                                 generator=gen) * wl.w_sigma
+        self.bias = torch.randn(oc2 * 16, dtype=torch.float32, device="cuda", generator=gen) * 0.01
+        tdt = {U8: torch.uint8, S8: torch.int8, F32: torch.float32}[wl.out_type]
+        shape = (wl.n, oc2, wl.oh, wl.oh, 16)
+        if wl.with_sum:
+            self.out = torch.randint(-127, 128, shape, dtype=torch.int8, device="cuda", generator=gen).to(tdt)
+        else:
+            self.out = torch.zeros(shape, dtype=tdt, device="cuda")
+        tq = (EL_NO_CALI, EL_NO_CALI)
+        if wl.algorithm == CONV_WINOGRAD:
+            mn, mx = wino_tinput_range(wl.descriptor(tinput_quant=(1.0, 0.0)), self.x)
+            diff = mx - mn + 1e-6
+            tq = (diff / 255.0, -mn * 255.0 / diff)
+        self.desc = wl.descriptor(tinput_quant=tq)
+        self.conv = Conv(self.desc)
+        self.conv.prepare(self.w, self.bias)
+        torch.cuda.synchronize()
+
+    def run(self, count=1):
+        self.conv.execute_repeat(self.out, self.x, count, bias=self.bias)

@@ -102,6 +102,12 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *conv, const void *weights_dev, const
 EHIP_API int ehip_conv_execute(ehip_conv_t *conv, void *output_dev, const void *input_dev,
                                const void *weights_dev, const void *bias_dev, void *hip_stream);
 
+/* Steady-state driver: enqueues `count` back-to-back executions of a prepared handle on
+ * `hip_stream` without returning to the caller in between (what the reference's benchmark loop
+ * around elx_conv() does, tests/elt_conv.cpp:445-448).  No counterpart inside the library. */
+EHIP_API int ehip_conv_execute_repeat(ehip_conv_t *conv, void *output_dev, const void *input_dev,
+                                      const void *bias_dev, int count, void *hip_stream);
+
 /* Copies workspace contents to a host buffer in a canonical layout (see EHIP_Q_*).  Synchronous.
  * Returns the number of bytes through *bytes when host_dst is NULL. */
 EHIP_API int ehip_conv_query(ehip_conv_t *conv, int what, void *host_dst, size_t *bytes);
