@@ -94,7 +94,7 @@ def cpu_baseline(wl, budget_s=12.0):
         lib.orc_direct_execute(*args)
         passes += 1
         el = time.perf_counter() - t0
-        if el > budget_s or passes >= 1024:
+        if el > budget_s or passes >= 20000:
             break
     sec = el / passes
     ops = wl.ops() * n / wl.n
@@ -121,6 +121,9 @@ def main():
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--layers", default="all", help="other layers to report: all, none or a comma list")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="instead of a layer, run 20 plain device copies of MIB MiB (known traffic, used to "
+                         "scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU: every layer is a single-device kernel and nothing here "
@@ -139,6 +142,16 @@ def main():
         print("bench.py: " + E.lib.ehip_last_error().decode(), file=sys.stderr)
         sys.exit(1)
     traffic = load_traffic()
+
+    if args.calibrate_copy:
+        n = args.calibrate_copy << 20
+        src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": n, "launches": 20}))
+        return
 
     wl = W.WORKLOADS[args.workload]
     layer = W.DeviceLayer(wl)

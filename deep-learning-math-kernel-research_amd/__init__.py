@@ -14,7 +14,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libeuler_hip.so")
+LIB_PATH = os.environ.get("EULER_HIP_LIB") or os.path.join(_HERE, "libeuler_hip.so")
 
 # ---- enum values of include/euler_hip.h (== the reference's include/euler.hpp) -----------------
 EHIP_OK, EHIP_UNIMPLEMENTED, EHIP_GENERAL_ERROR, EHIP_HIP_ERROR = 0, 1, 2, 3

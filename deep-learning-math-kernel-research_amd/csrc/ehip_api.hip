@@ -200,6 +200,8 @@ int setup_workspace(ehip_conv *c)
   int rc;
   switch (c->family) {
   case FAM_GEMM_1X1: {
+    if ((long long)d.n * d.oh * d.ow * d.oh * d.ow >= (1ll << 32))
+      return fail(EHIP_UNIMPLEMENTED, "1x1: n*oh*ow*oh*ow must stay below 2^32");
     c->taps = 1;
     c->nbatch = 1;
     c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2, 1);
@@ -211,21 +213,27 @@ int setup_workspace(ehip_conv *c)
     c->taps = 9;
     c->nbatch = 1;
     c->units_pad = up(c->ic2, 4);
-    int v = conv3x3_pick_variant(d.oh, d.ow, c->oc2);
-    // the staged tile (4 units x halo rows x (ow+2) cells) must fit the per-thread staging budget
-    for (int tries = 0; tries < 8; ++tries) {
+    int v = conv3x3_pick_variant(d.oh, d.ow, c->oc2) & ~1;
+    // the staged tile (4 units x halo rows x (ow+2) cells) must fit the variant's staging budget:
+    // variants come in pairs (small, large budget); fall back to the 64-pixel tile if neither fits
+    bool ok = false;
+    for (int tries = 0; tries < 2 && !ok; ++tries) {
       const int p_t = conv3x3_variant_pixels(v);
       int rows = (p_t + d.ow - 2) / d.ow + 1;
       if (p_t % d.ow == 0) rows = p_t / d.ow;
       if (rows > d.oh) rows = d.oh;
       c->halo_rows = rows + 2;
       const int items = 4 * c->halo_rows * (d.ow + 2);
-      if (items <= 8 * kBlock) break;
-      if (v == 4) return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too wide for the staged tile");
-      v = (v == 2 || v == 5) ? 4 : 2;
+      for (int k = 0; k < 2; ++k)
+        if (!ok && items <= conv3x3_variant_slots(v + k)) {
+          v += k;
+          ok = true;
+        }
+      if (!ok) v = 8;
     }
+    if (!ok) return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too wide for the staged tile");
     c->variant = v;
-    c->lds_bytes = (size_t)2 * 4 * c->halo_rows * (d.ow + 2) * 16;
+    c->lds_bytes = (size_t)2 * conv3x3_variant_slots(v) * 16;
     c->kernel_name = conv3x3_variant_name(c->variant);
     break;
   }
@@ -402,6 +410,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ep = make_epilogue(c, d.output_type, d.with_ip_sum && d.algorithm == EHIP_CONV_DIRECT_1X1, d.with_relu);
     a.p_total = d.n * d.oh * d.ow;
     a.ohw = d.oh * d.ow; a.ow = d.ow;
+    a.ohw_magic = div_magic(a.ohw); a.ow_magic = div_magic(a.ow);
     a.ihw = d.ih * d.iw; a.iw = d.iw;
     a.stride_h = d.stride_h; a.stride_w = d.stride_w;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
@@ -419,6 +428,8 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.pad_t = d.pad_t; a.pad_l = d.pad_l;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
     a.halo_rows = c->halo_rows; a.chunk_units = 4;
+    a.dbg = getenv("EHIP_DBG") ? atoi(getenv("EHIP_DBG")) : 0;
+    a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
     HIP_TRY(launch_conv3x3(a, d.n, c->variant, c->lds_bytes, s));
     break;
   }
@@ -459,6 +470,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ep = make_epilogue(c, EHIP_F32, false, false);
     a.p_total = c->t;
     a.ohw = c->t; a.ow = c->t; a.ihw = c->t; a.iw = c->t;
+    a.ohw_magic = div_magic(a.ohw); a.ow_magic = div_magic(a.ow);
     a.stride_h = 1; a.stride_w = 1;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
     a.in_batch_stride = (long long)c->ic2 * c->t * 16;

@@ -16,15 +16,28 @@
 // waves of a workgroup split the output channels and share the staged pixels.
 #include "ehip_internal.hpp"
 
+// Development aid (compile with -DEHIP_TRACE): lane 0 of every wave records the shader clock at
+// phase boundaries into Conv3x3Args::trace.
+#ifdef EHIP_TRACE
+#define TRACE_POINT(i)                                                                             \
+  do {                                                                                             \
+    if (a.trace && lane == 0) a.trace[((size_t)(blockIdx.z * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
+  } while (0)
+#else
+#define TRACE_POINT(i) do { } while (0)
+#endif
+
 namespace ehip {
 
-constexpr int kMaxStage = 8;  // 16-byte cells a thread may stage per LDS fill
-
-template <int MO, int NP>
+// Every global load of the main loop is unconditional (addresses are clamped, unwanted values
+// are replaced afterwards): with no branch between a load and its use the compiler can count
+// outstanding loads exactly, so waiting for one operand does not drain the prefetches behind it.
+template <int MO, int NP, int NS>
 __global__ __launch_bounds__(kBlock) void k_conv3x3_u8s8(Conv3x3Args a)
 {
   constexpr int OC_T = 4 * MO * 16;
   constexpr int P_T = NP * 16;
+  constexpr int SLOTS = NS * kBlock;         // 16-byte cells per LDS buffer (>= cells of one fill)
   extern __shared__ uint4 lds[];
 
   const int tid = threadIdx.x;
@@ -43,47 +56,46 @@ __global__ __launch_bounds__(kBlock) void k_conv3x3_u8s8(Conv3x3Args a)
   const int items = 4 * cells_per_unit;      // one fill = 4 units = one k-step per tap
   const long long plane = (long long)a.ih * a.iw * 16;
   const uint8_t *inb = a.in + (long long)n * a.ic2 * plane;
+  TRACE_POINT(0);
 
   // ---- staging plan (the same cells for every fill) -------------------------------------------
-  int goff[kMaxStage];   // byte offset of the cell inside the chunk's first plane, -1 = frame
-  int gunit[kMaxStage];
+  int goff[NS];      // byte offset of the cell inside a unit's plane (clamped into the image)
+  int gunit[NS];
+  bool gin[NS];      // false: frame cell, staged as the u8 value 0
 #pragma unroll
-  for (int j = 0; j < kMaxStage; ++j) {
-    const int id = tid + j * kBlock;
-    goff[j] = -2;  // not mine
-    gunit[j] = 0;
-    if (id < items) {
-      const int u = id / cells_per_unit;
-      const int rem = id - u * cells_per_unit;
-      const int hr = rem / WP2;
-      const int hc = rem - hr * WP2;
-      const int ih = r0 - a.pad_t + hr;
-      const int iw = hc - a.pad_l;
-      gunit[j] = u;
-      goff[j] = (ih >= 0 && ih < a.ih && iw >= 0 && iw < a.iw) ? (ih * a.iw + iw) * 16 : -1;
-    }
+  for (int j = 0; j < NS; ++j) {
+    int id = tid + j * kBlock;
+    id = id < items ? id : items - 1;        // surplus slots re-stage the last cell into spare LDS
+    const int u = id / cells_per_unit;
+    const int rem = id - u * cells_per_unit;
+    const int hr = rem / WP2;
+    const int hc = rem - hr * WP2;
+    const int ih = r0 - a.pad_t + hr;
+    const int iw = hc - a.pad_l;
+    gunit[j] = u;
+    gin[j] = ih >= 0 && ih < a.ih && iw >= 0 && iw < a.iw;
+    const int ihc = ih < 0 ? 0 : (ih >= a.ih ? a.ih - 1 : ih);
+    const int iwc = iw < 0 ? 0 : (iw >= a.iw ? a.iw - 1 : iw);
+    goff[j] = (ihc * a.iw + iwc) * 16;
   }
-  uint4 stage[kMaxStage];
+  uint4 stage[NS];
   auto load_stage = [&](int chunk) {
 #pragma unroll
-    for (int j = 0; j < kMaxStage; ++j) {
-      if (goff[j] >= 0) {
-        int u = chunk * 4 + gunit[j];
-        u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights
-        stage[j] = *reinterpret_cast<const uint4 *>(inb + (long long)u * plane + goff[j]);
-      } else {
-        stage[j] = make_uint4(0u, 0u, 0u, 0u);
-      }
+    for (int j = 0; j < NS; ++j) {
+      int u = chunk * 4 + gunit[j];
+      u = u < a.ic2 ? u : a.ic2 - 1;         // padded units multiply zero weights
+      stage[j] = *reinterpret_cast<const uint4 *>(inb + (long long)u * plane + goff[j]);
     }
   };
   auto store_stage = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < kMaxStage; ++j) {
-      if (goff[j] >= -1) {
-        uint4 v = stage[j];
-        v.x ^= 0x80808080u; v.y ^= 0x80808080u; v.z ^= 0x80808080u; v.w ^= 0x80808080u;
-        lds[buf * items + tid + j * kBlock] = v;
-      }
+    for (int j = 0; j < NS; ++j) {
+      uint4 v = stage[j];
+      v.x = gin[j] ? v.x ^ 0x80808080u : 0x80808080u;
+      v.y = gin[j] ? v.y ^ 0x80808080u : 0x80808080u;
+      v.z = gin[j] ? v.z ^ 0x80808080u : 0x80808080u;
+      v.w = gin[j] ? v.w ^ 0x80808080u : 0x80808080u;
+      lds[buf * SLOTS + tid + j * kBlock] = v;
     }
   };
 
@@ -96,6 +108,14 @@ __global__ __launch_bounds__(kBlock) void k_conv3x3_u8s8(Conv3x3Args a)
     const int r = p / a.ow;
     const int c = p - r * a.ow;
     cellbase[np] = (lg * a.halo_rows + (r - r0)) * WP2 + c;
+  }
+
+  // per-channel scale/shift of this lane's channels: requested now, needed in the epilogue
+  float4 sc[MO], sh[MO];
+#pragma unroll
+  for (int mo = 0; mo < MO; ++mo) {
+    sc[mo] = *reinterpret_cast<const float4 *>(a.ep.scale + ocw0 + mo * 16 + 4 * lg);
+    sh[mo] = *reinterpret_cast<const float4 *>(a.ep.shift + ocw0 + mo * 16 + 4 * lg);
   }
 
   v4i acc[MO][NP];
@@ -111,66 +131,97 @@ __global__ __launch_bounds__(kBlock) void k_conv3x3_u8s8(Conv3x3Args a)
   const long long w_unit = (long long)a.ocpp * 16;
   const int nchunks = a.units_pad / 4;
   auto load_a = [&](v4i (&dst)[MO], int chunk, int tap) {
+    chunk = chunk < nchunks ? chunk : nchunks - 1;   // the last fill re-reads its own operands
     const int8_t *p = wb + ((long long)tap * a.units_pad + chunk * 4) * w_unit;
 #pragma unroll
     for (int mo = 0; mo < MO; ++mo) dst[mo] = *reinterpret_cast<const v4i *>(p + mo * 256);
   };
 
-  v4i a_cur[MO], a_nxt[MO];
+  // Software pipeline (one wave per SIMD has nobody else to hide its latencies behind):
+  //   - the weight operands of all nine taps of a fill live in registers; each slot is refilled
+  //     with the next fill's operand right after its last use, i.e. a whole fill ahead;
+  //   - the pixel operands of tap t+1 are read from LDS while the MFMAs of tap t run;
+  //   - the next fill's global loads are in flight during the whole fill.
+  v4i a_reg[9][MO];
   load_stage(0);
-  load_a(a_cur, 0, 0);
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap) load_a(a_reg[tap], 0, tap);
+  TRACE_POINT(1);
   int buf = 0;
   for (int c = 0; c < nchunks; ++c) {
     store_stage(buf);
+    TRACE_POINT(2 + 3 * (c < 3 ? c : 3));
     __syncthreads();
-    if (c + 1 < nchunks) load_stage(c + 1);
-    const v4i *tile = reinterpret_cast<const v4i *>(lds + buf * items);
+    TRACE_POINT(3 + 3 * (c < 3 ? c : 3));
+    load_stage(c + 1 < nchunks ? c + 1 : c);
+    const v4i *tile = reinterpret_cast<const v4i *>(lds + buf * SLOTS);
+    v4i bq[2][NP];
+#pragma unroll
+    for (int np = 0; np < NP; ++np) bq[0][np] = tile[cellbase[np]];
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap) {
-      if (tap < 8) load_a(a_nxt, c, tap + 1);
-      else if (c + 1 < nchunks) load_a(a_nxt, c + 1, 0);
-      const int toff = (tap / 3) * WP2 + (tap % 3);
+      if (tap < 8) {
+        const int toff = ((tap + 1) / 3) * WP2 + ((tap + 1) % 3);
+#ifdef EHIP_TRACE
+        if (a.dbg & 1) {
 #pragma unroll
-      for (int np = 0; np < NP; ++np) {
-        const v4i bq = tile[cellbase[np] + toff];
+          for (int np = 0; np < NP; ++np) bq[(tap + 1) & 1][np] = bq[tap & 1][np];
+        } else
+#endif
+#pragma unroll
+        for (int np = 0; np < NP; ++np) bq[(tap + 1) & 1][np] = tile[cellbase[np] + toff];
+      }
+      // keep the compiler from sinking these reads next to their use: they must be in flight
+      // while the MFMAs below run
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int np = 0; np < NP; ++np)
 #pragma unroll
         for (int mo = 0; mo < MO; ++mo)
-          acc[mo][np] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_cur[mo], bq, acc[mo][np], 0, 0, 0);
-      }
-#pragma unroll
-      for (int mo = 0; mo < MO; ++mo) a_cur[mo] = a_nxt[mo];
+          acc[mo][np] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_reg[tap][mo], bq[tap & 1][np], acc[mo][np], 0, 0, 0);
+#ifdef EHIP_TRACE
+      if (!(a.dbg & 2))
+#endif
+      load_a(a_reg[tap], c + 1, tap);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    TRACE_POINT(4 + 3 * (c < 3 ? c : 3));
     buf ^= 1;
   }
 
+  size_t pix[NP];
+  bool pvalid[NP];
 #pragma unroll
   for (int np = 0; np < NP; ++np) {
     const int p = p0 + np * 16 + l16;
-    if (p >= ohw) continue;
-#pragma unroll
-    for (int mo = 0; mo < MO; ++mo) {
-      const int oc = ocw0 + mo * 16 + 4 * lg;
-      if (oc >= oc_real) continue;
-      const size_t elem = (((size_t)n * a.oc2 + (oc >> 4)) * ohw + p) * 16 + (oc & 15);
-      store_quad(a.ep, a.ep.scale, a.ep.shift, acc[mo][np], oc, a.out, elem);
-    }
+    pvalid[np] = p < ohw;
+    pix[np] = ((size_t)n * a.oc2 * ohw + (pvalid[np] ? p : 0)) * 16;
   }
+  TRACE_POINT(14);
+  int oc_of[MO];
+#pragma unroll
+  for (int mo = 0; mo < MO; ++mo) oc_of[mo] = ocw0 + mo * 16 + 4 * lg;
+  epilogue_dispatch<MO, NP>(a.ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, (size_t)ohw * 16, a.out);
+  TRACE_POINT(15);
 }
 
 namespace {
 struct Variant {
   const char *name;
-  int oc_t, p_t;
+  int oc_t, p_t, ns;
   void (*kernel)(Conv3x3Args);
 };
-#define V(MO, NP) { "k_conv3x3_u8s8<" #MO "," #NP ">", 4 * MO * 16, NP * 16, k_conv3x3_u8s8<MO, NP> }
+#define V(MO, NP, NS)                                                                              \
+  { "k_conv3x3_u8s8<" #MO "," #NP "," #NS ">", 4 * MO * 16, NP * 16, NS, k_conv3x3_u8s8<MO, NP, NS> }
+// every (oc tile, pixel tile) comes with a small and a large staging budget NS (cells per thread
+// and fill); the launcher takes the first entry of the chosen tile whose budget fits the layer
 const Variant kVariants[] = {
-    V(2, 7),  // 0: 128 oc x 112 px (4 rows of 28, 2 rows of 56, 8 rows of 14)
-    V(2, 8),  // 1: 128 oc x 128 px
-    V(2, 4),  // 2: 128 oc x  64 px
-    V(1, 7),  // 3:  64 oc x 112 px
-    V(1, 4),  // 4:  64 oc x  64 px
-    V(4, 4),  // 5: 256 oc x  64 px
+    V(2, 7, 3), V(2, 7, 8),  // 0,1: 128 oc x 112 px (4 rows of 28, 2 rows of 56, 8 rows of 14)
+    V(2, 8, 4), V(2, 8, 8),  // 2,3: 128 oc x 128 px
+    V(2, 4, 3), V(2, 4, 8),  // 4,5: 128 oc x  64 px
+    V(1, 7, 3), V(1, 7, 8),  // 6,7:  64 oc x 112 px
+    V(1, 4, 3), V(1, 4, 8),  // 8,9:  64 oc x  64 px
+    V(4, 4, 3), V(4, 4, 8),  // 10,11: 256 oc x 64 px
 };
 #undef V
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -178,6 +229,8 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 const char *conv3x3_variant_name(int v) { return kVariants[v].name; }
 int conv3x3_variant_pixels(int v) { return kVariants[v].p_t; }
+int conv3x3_variant_slots(int v) { return kVariants[v].ns * kBlock; }
+int conv3x3_num_variants() { return kNumVariants; }
 
 int conv3x3_pick_variant(int oh, int ow, int oc2)
 {
@@ -189,7 +242,7 @@ int conv3x3_pick_variant(int oh, int ow, int oc2)
   const int oc = oc2 * 16, ohw = oh * ow;
   int best = 0;
   double best_score = -1;
-  for (int v = 0; v < kNumVariants; ++v) {
+  for (int v = 0; v < kNumVariants; v += 2) {
     const Variant &k = kVariants[v];
     const int tiles = (ohw + k.p_t - 1) / k.p_t;
     const double putil = (double)ohw / ((double)tiles * k.p_t);

@@ -7,152 +7,201 @@
 // elx_int8_conv_wino_gemm_t::execute (src/elx_int8_conv_wino_gemm.cpp:23-76) and the
 // u8s8 micro-kernel with its epilogue (src/kernel/elk_u8s8_gemm.hxx:168-406).
 //
-// Mapping.  D[oc][pixel] += W[oc][k] * X[k][pixel] with v_mfma_i32_16x16x64_i8:
-//   A operand = weights, one lane = 16 consecutive input channels of one output channel,
-//   B operand = activations, one lane = the 16 channels of one nChw16c pixel cell (16 bytes that
-//               are contiguous in memory, so no layout change is needed on the way in),
-//   D         = lane holds 4 consecutive output channels of one pixel, i.e. one dword of u8/s8
-//               output or one float4 of f32 output, and a wave stores 16 pixels x 16 channels as
-//               one contiguous run of the nChw16c output.
+// Mapping.  D[oc][pixel] += W[oc][k] * X[k][pixel] with v_mfma_i32_32x32x32_i8:
+//   A operand = weights: lane l holds 16 consecutive input channels (unit 2*kstep + l/32) of
+//               output channel l%32,
+//   B operand = activations: lane l holds the 16 channels of one nChw16c pixel cell (pixel l%32,
+//               unit 2*kstep + l/32) -- 16 bytes that are contiguous in memory, so no layout
+//               change is needed on the way in,
+//   D         = lane l holds, for pixel l%32, four runs of 4 consecutive output channels
+//               (8*g + 4*(l/32) .. +3, g = 0..3): one dword of u8/s8 output or one float4 of f32
+//               output per run.
 // The MFMA is signed x signed: activations are remapped u8 -> s8 by flipping the top bit when a
 // tile is staged into LDS, and the accumulators start at 128 * sum(weights) per output channel,
 // which makes the s32 result identical to the unsigned product.
 //
-// A workgroup (4 waves) owns OC_T output channels x P_T pixels.  The pixel tile is staged through
-// LDS (double buffered, KC units of 16 channels per fill) and shared by the waves that own different
-// output channels; every wave streams its own weight rows straight from L2 into registers, one
-// k-step ahead of the MFMAs that use them.
+// A workgroup (4 waves, WM x WN) owns OC_T output channels x P_T pixels; a wave owns TM x TN MFMA
+// tiles of 32 x 32.  Both operands go global -> registers -> LDS (double buffered, KC units of 16
+// channels per fill; the loads of fill c+1 are in flight while fill c is multiplied) and every
+// wave reads its operands from LDS one k-step ahead of the MFMAs that use them.  Two workgroups
+// share a CU, so one can multiply while the other waits at its barrier.
 #include "ehip_internal.hpp"
 
 namespace ehip {
 
-template <int MO, int NP, int WO, int WPX, int KC>
-__global__ __launch_bounds__(kBlock) void k_gemm_u8s8(GemmArgs a)
-{
-  constexpr int OC_T = WO * MO * 16;
-  constexpr int P_T = WPX * NP * 16;
-  constexpr int ITEMS = KC * P_T;  // 16-byte cells per LDS fill
-  constexpr int NI = (ITEMS + kBlock - 1) / kBlock;
-  constexpr int KS = KC / 4;       // MFMA k-steps per fill
-  static_assert(WO * WPX == 4, "four waves per workgroup");
-  static_assert(KC % 4 == 0, "a k-step is four units");
+typedef int v16i __attribute__((ext_vector_type(16)));
 
-  __shared__ uint4 lds[2][ITEMS];
+template <int WM, int WN, int TM, int TN, int KC>
+__global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
+{
+  constexpr int OC_T = WM * TM * 32;
+  constexpr int P_T = WN * TN * 32;
+  constexpr int KS = KC / 2;               // MFMA k-steps per fill
+  constexpr int A_CELLS = OC_T * KC;       // 16-byte cells per fill
+  constexpr int B_CELLS = P_T * KC;
+  constexpr int NA = A_CELLS / kBlock;
+  constexpr int NB = B_CELLS / kBlock;
+  constexpr int BU = kBlock / P_T;         // units covered by one pass of the workgroup over B
+  static_assert(WM * WN == 4, "four waves per workgroup");
+  static_assert(KC % 2 == 0, "a k-step is two units");
+  static_assert(A_CELLS % kBlock == 0 && B_CELLS % kBlock == 0, "whole passes of the workgroup");
+  static_assert(kBlock % P_T == 0 && OC_T <= kOcTile, "tile limits");
+
+  __shared__ v4i lds_a[2][A_CELLS];      // [unit][row]
+  __shared__ v4i lds_b[2][B_CELLS];      // [unit][pixel]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int l16 = lane & 15;
-  const int lg = lane >> 4;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
   const int b = blockIdx.z;
   const int pix0 = blockIdx.x * P_T;
-  const int ocw0 = blockIdx.y * OC_T + (wave % WO) * MO * 16;
-  const int pw0 = (wave / WO) * NP * 16;
+  const int oc0 = blockIdx.y * OC_T;
+  const int mw0 = (wave % WM) * TM * 32;   // wave's first row / pixel inside the workgroup tile
+  const int pw0 = (wave / WM) * TN * 32;
   const int oc_real = a.oc2 * 16;
+  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
 
-  // ---- staging plan: which pixel/unit cells this thread copies ---------------------------
+  // ---- staging plan ---------------------------------------------------------------------------
+  // B: a thread always copies the same pixel (tid % P_T), units tid / P_T + j * BU of a fill.
   const uint8_t *inb = a.in + (long long)b * a.in_batch_stride;
-  long long poff[NI];
-  int ucell[NI];
-#pragma unroll
-  for (int j = 0; j < NI; ++j) {
-    const int id = tid + j * kBlock;
-    const int p = id % P_T;
-    ucell[j] = id / P_T;
-    int gp = pix0 + p;
+  {
+    int gp = pix0 + tid % P_T;
     gp = gp < a.p_total ? gp : a.p_total - 1;
-    const int n = gp / a.ohw;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv(gp, a.ohw, a.ohw_magic);
     const int r = gp - n * a.ohw;
-    const int oh = r / a.ow;
-    const int ow = r - oh * a.ow;
-    poff[j] = ((long long)n * a.ic2 * a.ihw + (long long)(oh * a.stride_h) * a.iw + ow * a.stride_w) * 16;
+    long long off;
+    if (dense) {
+      off = (long long)n * a.ic2 * a.ihw + r;
+    } else {
+      const int oh = fastdiv(r, a.ow, a.ow_magic);
+      const int ow = r - oh * a.ow;
+      off = (long long)n * a.ic2 * a.ihw + (long long)(oh * a.stride_h) * a.iw + ow * a.stride_w;
+    }
+    inb += off * 16;
   }
+  const int bu0 = tid / P_T;
   const long long unit_stride = (long long)a.ihw * 16;
-  uint4 stage[NI];
+  // A: cell id = tid + j * 256 -> unit id / OC_T, row id % OC_T; rows of a unit are contiguous.
+  const int8_t *wb = a.w + (long long)b * a.units_pad * a.ocpp * 16 + (long long)oc0 * 16;
+  const long long w_unit = (long long)a.ocpp * 16;
+
+  v4i sta[NA], stb[NB];
+  // All global loads of the main loop are unconditional (indices clamped): without branches
+  // between a load and its use the compiler counts outstanding loads exactly.
   auto load_stage = [&](int chunk) {
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      if (NI * kBlock == ITEMS || tid + j * kBlock < ITEMS) {
-        int u = chunk * KC + ucell[j];
-        u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
-        stage[j] = *reinterpret_cast<const uint4 *>(inb + poff[j] + (long long)u * unit_stride);
-      }
+    for (int j = 0; j < NA; ++j) {
+      const int id = tid + j * kBlock;
+      sta[j] = *reinterpret_cast<const v4i *>(wb + (long long)(chunk * KC + id / OC_T) * w_unit + (id % OC_T) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      int u = chunk * KC + bu0 + j * BU;
+      u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
+      stb[j] = *reinterpret_cast<const v4i *>(inb + (long long)u * unit_stride);
     }
   };
   auto store_stage = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      if (NI * kBlock == ITEMS || tid + j * kBlock < ITEMS) {
-        uint4 v = stage[j];
-        v.x ^= 0x80808080u; v.y ^= 0x80808080u; v.z ^= 0x80808080u; v.w ^= 0x80808080u;
-        lds[buf][tid + j * kBlock] = v;
-      }
+    for (int j = 0; j < NA; ++j) lds_a[buf][tid + j * kBlock] = sta[j];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      lds_b[buf][tid + j * kBlock] = stb[j] ^ (int)0x80808080;
     }
   };
 
   // ---- accumulators start at the u8->s8 compensation -------------------------------------
-  v4i acc[MO][NP];
+  const long long per_oc = (long long)b * a.ocpp + oc0 + mw0 + 4 * lh;
+  v16i acc[TM][TN];
 #pragma unroll
-  for (int mo = 0; mo < MO; ++mo) {
-    const v4i c = *reinterpret_cast<const v4i *>(a.ep.comp + (long long)b * a.ocpp + ocw0 + mo * 16 + 4 * lg);
+  for (int mt = 0; mt < TM; ++mt) {
+    v16i c;
 #pragma unroll
-    for (int np = 0; np < NP; ++np) acc[mo][np] = c;
+    for (int g = 0; g < 4; ++g) {
+      const v4i c4 = *reinterpret_cast<const v4i *>(a.ep.comp + per_oc + mt * 32 + 8 * g);
+      c[4 * g + 0] = c4.x; c[4 * g + 1] = c4.y; c[4 * g + 2] = c4.z; c[4 * g + 3] = c4.w;
+    }
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) acc[mt][nt] = c;
   }
 
-  // ---- weights: each wave streams its own rows ---------------------------------------------
-  const int8_t *wb = a.w + (long long)b * a.units_pad * a.ocpp * 16 + ((long long)lg * a.ocpp + ocw0 + l16) * 16;
-  const long long w_kstep = (long long)4 * a.ocpp * 16;
-  auto load_a = [&](v4i (&dst)[MO], int kstep) {
+  // ---- main loop ------------------------------------------------------------------------------
+  v4i opa[2][TM], opb[2][TN];
+  auto read_ops = [&](int buf, int ks, int slot) {
+    const v4i *pa = &lds_a[buf][(2 * ks + lh) * OC_T + mw0 + l32];
+    const v4i *pb = &lds_b[buf][(2 * ks + lh) * P_T + pw0 + l32];
 #pragma unroll
-    for (int mo = 0; mo < MO; ++mo)
-      dst[mo] = *reinterpret_cast<const v4i *>(wb + (long long)kstep * w_kstep + mo * 256);
+    for (int mt = 0; mt < TM; ++mt) opa[slot][mt] = pa[mt * 32];
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) opb[slot][nt] = pb[nt * 32];
+  };
+  // The scheduling barriers keep the compiler from sinking the operand prefetch next to its use.
+  auto multiply = [&](int buf) {
+    read_ops(buf, 0, 0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) read_ops(buf, ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < TN; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(opa[ks & 1][mt], opb[ks & 1][nt], acc[mt][nt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   const int nchunks = a.units_pad / KC;
-  const int nksteps = nchunks * KS;
-  v4i a_cur[MO], a_nxt[MO];
   load_stage(0);
-  load_a(a_cur, 0);
   int buf = 0;
-  for (int c = 0; c < nchunks; ++c) {
+  for (int c = 0; c + 1 < nchunks; ++c) {
     store_stage(buf);
     __syncthreads();
-    if (c + 1 < nchunks) load_stage(c + 1);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int kstep = c * KS + ks;
-      if (kstep + 1 < nksteps) load_a(a_nxt, kstep + 1);
-      const v4i *bl = reinterpret_cast<const v4i *>(&lds[buf][(ks * 4 + lg) * P_T + pw0 + l16]);
-#pragma unroll
-      for (int np = 0; np < NP; ++np) {
-        const v4i bq = bl[np * 16];
-#pragma unroll
-        for (int mo = 0; mo < MO; ++mo)
-          acc[mo][np] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_cur[mo], bq, acc[mo][np], 0, 0, 0);
-      }
-#pragma unroll
-      for (int mo = 0; mo < MO; ++mo) a_cur[mo] = a_nxt[mo];
-    }
+    load_stage(c + 1);
+    multiply(buf);
     buf ^= 1;
   }
+  // last fill: nothing left to prefetch but the epilogue's per-channel constants
+  store_stage(buf);
+  __syncthreads();
+  float4 sc[TM][4], sh[TM][4];
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      sc[mt][g] = *reinterpret_cast<const float4 *>(a.ep.scale + per_oc + mt * 32 + 8 * g);
+      sh[mt][g] = *reinterpret_cast<const float4 *>(a.ep.shift + per_oc + mt * 32 + 8 * g);
+    }
+  multiply(buf);
 
   // ---- epilogue ------------------------------------------------------------------------------
-  const float *scale = a.ep.scale + (long long)b * a.ocpp;
-  const float *shift = a.ep.shift + (long long)b * a.ocpp;
+  size_t pix[TN];
+  bool pvalid[TN];
 #pragma unroll
-  for (int np = 0; np < NP; ++np) {
-    const int gp = pix0 + pw0 + np * 16 + l16;
-    if (gp >= a.p_total) continue;
-    const int n = gp / a.ohw;
-    const int r = gp - n * a.ohw;
+  for (int nt = 0; nt < TN; ++nt) {
+    const int gp = pix0 + pw0 + nt * 32 + l32;
+    pvalid[nt] = gp < a.p_total;
+    const int gpc = pvalid[nt] ? gp : 0;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv(gpc, a.ohw, a.ohw_magic);
+    const int r = gpc - n * a.ohw;
+    pix[nt] = (size_t)b * a.out_batch_stride + ((size_t)n * a.oc2 * a.ohw + r) * 16;
+  }
 #pragma unroll
-    for (int mo = 0; mo < MO; ++mo) {
-      const int oc = ocw0 + mo * 16 + 4 * lg;
-      if (oc >= oc_real) continue;
-      const size_t elem = (size_t)b * a.out_batch_stride +
-          (((size_t)n * a.oc2 + (oc >> 4)) * a.ohw + r) * 16 + (oc & 15);
-      store_quad(a.ep, scale, shift, acc[mo][np], oc, a.out, elem);
+  for (int mt = 0; mt < TM; ++mt) {
+    v4i quad[4][TN];
+    int oc_of[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      oc_of[g] = oc0 + mw0 + mt * 32 + 8 * g + 4 * lh;
+#pragma unroll
+      for (int nt = 0; nt < TN; ++nt) {
+        const v16i &d = acc[mt][nt];
+        quad[g][nt] = v4i{d[4 * g], d[4 * g + 1], d[4 * g + 2], d[4 * g + 3]};
+      }
     }
+    epilogue_dispatch<4, TN>(a.ep, quad, sc[mt], sh[mt], pix, pvalid, oc_of, oc_real, (size_t)a.ohw * 16, a.out);
   }
 }
 
@@ -162,18 +211,19 @@ struct Variant {
   int oc_t, p_t, kc;
   void (*kernel)(GemmArgs);
 };
-#define V(MO, NP, WO, WPX, KC)                                                                   \
-  { "k_gemm_u8s8<" #MO "," #NP "," #WO "," #WPX "," #KC ">", WO * MO * 16, WPX * NP * 16, KC,     \
-    k_gemm_u8s8<MO, NP, WO, WPX, KC> }
+#define V(WM, WN, TM, TN, KC)                                                                    \
+  { "k_gemm_u8s8<" #WM "," #WN "," #TM "," #TN "," #KC ">", WM * TM * 32, WN * TN * 32, KC,       \
+    k_gemm_u8s8<WM, WN, TM, TN, KC> }
 const Variant kVariants[] = {
-    V(4, 4, 4, 1, 8),  // 0: 256 oc x  64 px
-    V(2, 4, 4, 1, 8),  // 1: 128 oc x  64 px
-    V(4, 2, 4, 1, 8),  // 2: 256 oc x  32 px
-    V(2, 2, 4, 1, 4),  // 3: 128 oc x  32 px
-    V(4, 1, 4, 1, 4),  // 4: 256 oc x  16 px
-    V(4, 4, 2, 2, 8),  // 5: 128 oc x 128 px
-    V(2, 4, 2, 2, 8),  // 6:  64 oc x 128 px
-    V(1, 4, 4, 1, 4),  // 7:  64 oc x  64 px
+    V(2, 2, 2, 2, 8),  // 0: 128 oc x 128 px
+    V(2, 2, 2, 1, 8),  // 1: 128 oc x  64 px
+    V(4, 1, 2, 2, 8),  // 2: 256 oc x  64 px
+    V(2, 2, 1, 1, 8),  // 3:  64 oc x  64 px
+    V(4, 1, 2, 1, 8),  // 4: 256 oc x  32 px
+    V(2, 2, 1, 2, 8),  // 5:  64 oc x 128 px
+    V(2, 2, 1, 1, 4),  // 6:  64 oc x  64 px, short K
+    V(2, 2, 2, 4, 4),  // 7: 128 oc x 256 px
+    V(4, 1, 2, 4, 4),  // 8: 256 oc x 128 px
 };
 #undef V
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -181,9 +231,10 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 const char *gemm_variant_name(int v) { return kVariants[v].name; }
 int gemm_variant_chunk(int v) { return kVariants[v].kc; }
+int gemm_num_variants() { return kNumVariants; }
 
-// Largest tile that still gives every CU at least two workgroups; ties go to the tile that
-// re-reads the pixel tile least (all output channels in one workgroup).
+// Score = useful fraction of the padded tile grid x how well the grid fills the chip (two
+// workgroups per CU) x operand reuse of the tile.
 int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch)
 {
   const char *env = getenv("EHIP_GEMM_VARIANT");
@@ -196,12 +247,14 @@ int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch)
   double best_score = -1;
   for (int v = 0; v < kNumVariants; ++v) {
     const Variant &k = kVariants[v];
-    if (k.kc > up(ic2, 4) && k.kc > 4) continue;
-    const long long wgs = (long long)((p_total + k.p_t - 1) / k.p_t) * ((oc + k.oc_t - 1) / k.oc_t) * nbatch;
-    const double util = (double)oc / (double)(((oc + k.oc_t - 1) / k.oc_t) * k.oc_t);
-    const double fill = wgs >= 512 ? 1.0 : (double)wgs / 512.0;
-    const double tile = (double)k.oc_t * k.p_t / (256.0 * 128.0);
-    const double score = util * fill * (0.5 + tile);
+    const int gx = (p_total + k.p_t - 1) / k.p_t, gy = (oc + k.oc_t - 1) / k.oc_t;
+    const long long wgs = (long long)gx * gy * nbatch;
+    const double util = ((double)oc / ((double)gy * k.oc_t)) * ((double)p_total / ((double)gx * k.p_t)) *
+                        ((double)ic2 / (double)up(ic2, k.kc));
+    const long long rounds = (wgs + 511) / 512;
+    const double fill = (double)wgs / (double)(rounds * 512);
+    const double reuse = (double)k.oc_t * k.p_t / (double)(k.oc_t + k.p_t) / 64.0;  // 1.0 for 128 x 128
+    const double score = util * fill * (0.25 + reuse);
     if (score > best_score) { best_score = score; best = v; }
   }
   return best;
