@@ -42,8 +42,7 @@ struct ehip_conv {
   size_t per_oc = 0;  // elements in scale/shift/wsum/comp
 
   // 3x3
-  int halo_rows = 0;
-  size_t lds_bytes = 0;
+  int chunk_units = 2;
   // depthwise
   int T = 1, Tr = 1, wtb = 1;
   // Winograd
@@ -212,29 +211,15 @@ int setup_workspace(ehip_conv *c)
   case FAM_CONV_3X3: {
     c->taps = 9;
     c->nbatch = 1;
-    c->units_pad = up(c->ic2, 4);
-    int v = conv3x3_pick_variant(d.oh, d.ow, c->oc2) & ~1;
-    // the staged tile (4 units x halo rows x (ow+2) cells) must fit the variant's staging budget:
-    // variants come in pairs (small, large budget); fall back to the 64-pixel tile if neither fits
-    bool ok = false;
-    for (int tries = 0; tries < 2 && !ok; ++tries) {
-      const int p_t = conv3x3_variant_pixels(v);
-      int rows = (p_t + d.ow - 2) / d.ow + 1;
-      if (p_t % d.ow == 0) rows = p_t / d.ow;
-      if (rows > d.oh) rows = d.oh;
-      c->halo_rows = rows + 2;
-      const int items = 4 * c->halo_rows * (d.ow + 2);
-      for (int k = 0; k < 2; ++k)
-        if (!ok && items <= conv3x3_variant_slots(v + k)) {
-          v += k;
-          ok = true;
-        }
-      if (!ok) v = 8;
-    }
-    if (!ok) return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too wide for the staged tile");
-    c->variant = v;
-    c->lds_bytes = (size_t)2 * conv3x3_variant_slots(v) * 16;
-    c->kernel_name = conv3x3_variant_name(c->variant);
+    if (d.ow != d.iw + d.pad_l + d.pad_r - 2 || d.oh != d.ih + d.pad_t + d.pad_b - 2)
+      return fail(EHIP_GENERAL_ERROR, "direct 3x3: output size does not match input size and padding");
+    if ((long long)(d.oh + 2) * (d.ow + 2) * (d.ow + 2) >= (1ll << 31))
+      return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too large");
+    c->variant = conv3x3v_pick_variant(d.n, d.oh, d.ow, c->oc2);
+    if (c->variant < 0) return fail(EHIP_UNIMPLEMENTED, "direct 3x3: rows too wide for the staged tile");
+    c->chunk_units = conv3x3v_chunk_units(c->variant, c->ic2);
+    c->units_pad = up(c->ic2, c->chunk_units);
+    c->kernel_name = conv3x3v_variant_name(c->variant);
     break;
   }
   case FAM_DEPTHWISE: {
@@ -427,10 +412,11 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
     a.pad_t = d.pad_t; a.pad_l = d.pad_l;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
-    a.halo_rows = c->halo_rows; a.chunk_units = 4;
-    a.dbg = getenv("EHIP_DBG") ? atoi(getenv("EHIP_DBG")) : 0;
+    a.chunk_units = c->chunk_units;
+    a.vw = d.ow + 2;
+    a.vw_magic = div_magic(a.vw);
     a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
-    HIP_TRY(launch_conv3x3(a, d.n, c->variant, c->lds_bytes, s));
+    HIP_TRY(launch_conv3x3v(a, d.n, c->variant, s));
     break;
   }
   case FAM_DEPTHWISE: {
@@ -527,7 +513,7 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
         for (int ic = 0; ic < icp; ++ic)
           for (int tap = 0; tap < taps; ++tap)
             dst[(((size_t)b * ocp + oc) * icp + ic) * taps + tap] =
-                packed[((((size_t)b * taps + tap) * c->units_pad + (ic >> 4)) * c->ocpp + oc) * 16 + (ic & 15)];
+                packed[((((size_t)b * taps + tap) * c->units_pad + (ic >> 4)) * c->ocpp + packed_row_of_oc(oc)) * 16 + (ic & 15)];
     return EHIP_OK;
   }
   case EHIP_Q_SCALE:

@@ -1,0 +1,280 @@
+// Direct 3x3 stride-1 u8 x s8 -> s32 convolution on gfx950 matrix cores as an implicit GEMM
+// (K = 9 taps x IC) over "virtual rows", requantization epilogue fused.
+//
+// Replaces elx_int8_conv_direct_t::__execute_c160 + conv_c160
+// (src/elx_int8_conv_direct_xopt.hpp:20-110, src/elx_int8_conv_direct.cpp:502-571) and the 3x3
+// micro-kernel with its epilogue (src/kernel/elk_u8s8_conv.hxx:190-252,679-901).
+//
+// Virtual rows.  An image is addressed as if every row were VW = ow + 2 cells wide (the input row
+// with its left/right frame): virtual cell v = r * VW + c.  Output pixel v then reads, for tap
+// (kh, kw), input cell v + kh * VW + kw -- one constant offset per tap for ANY run of consecutive
+// virtual pixels, whatever its alignment to the image rows.  So a workgroup takes P_T consecutive
+// virtual pixels (a multiple of the 32-pixel MFMA tile, not of the row width), stages the
+// P_T + 2 * VW + 2 input cells they touch for ALL input channels into LDS once, and all nine taps of
+// all channel pairs read that one staged run at shifted positions.  Two of every VW virtual pixels
+// are the frame columns: they are computed and not stored.
+//
+// Frame cells hold the u8 value 0: after the u8 -> s8 remap (top bit flipped) a zero activation is
+// -128, whose product with a weight is cancelled exactly by the 128 * sum(weights) the accumulators
+// start from, so skipped border taps of the reference and zero taps here give the same s32.
+//
+// MFMA mapping as in the 1x1 kernel (v_mfma_i32_32x32x32_i8; A = weights in packed row order,
+// B = pixels, a lane's D = 16 consecutive output channels of one pixel).  A wave owns TM x TN tiles of 32 x 32; its
+// weight operands (9 taps x TM) live in registers and every slot is refilled with the next channel
+// pair's operand right after its last use, i.e. nine taps ahead; pixel operands come from LDS one
+// tap ahead.  Two workgroups share a CU.
+#include "ehip_internal.hpp"
+
+// Development aid (compile with -DEHIP_TRACE): lane 0 of every wave records the shader clock at
+// phase boundaries into Conv3x3Args::trace.
+#ifdef EHIP_TRACE
+#define TRACE_POINT(i)                                                                             \
+  do {                                                                                             \
+    if (a.trace && lane == 0) a.trace[((size_t)(blockIdx.z * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
+  } while (0)
+#else
+#define TRACE_POINT(i) do { } while (0)
+#endif
+
+namespace ehip {
+
+template <int WM, int WN, int TM, int TN, int CT, int NPASS>
+__global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
+{
+  constexpr int OC_T = WM * TM * 32;
+  constexpr int P_T = WN * TN * 32;
+  constexpr int STRIDE = CT * NPASS;   // LDS cells per unit
+  constexpr int G = kBlock / CT;       // thread groups that split the units of a fill
+  static_assert(WM * WN == 4, "four waves per workgroup");
+  static_assert(kBlock % CT == 0, "cells per pass");
+  extern __shared__ v4i lds[];         // [chunk_units][STRIDE]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int n = blockIdx.z;
+  const int v0 = blockIdx.x * P_T;
+  const int oc0 = blockIdx.y * OC_T;
+  const int mw0 = (wave % WM) * TM * 32;
+  const int pw0 = (wave / WM) * TN * 32;
+  const int oc_real = a.oc2 * 16;
+  const int VW = a.vw;
+  const int ohw = a.oh * a.ow;
+  const long long plane = (long long)a.ih * a.iw * 16;
+  const uint8_t *inb = a.in + (long long)n * a.ic2 * plane;
+  TRACE_POINT(0);
+
+  // ---- staging plan: the same cells for every fill ------------------------------------------
+  const int ug = tid / CT;
+  int goff[NPASS];
+  bool gin[NPASS];
+#pragma unroll
+  for (int p = 0; p < NPASS; ++p) {
+    const int v = v0 + tid % CT + p * CT;
+    const int r = fastdiv(v, VW, a.vw_magic);
+    const int c = v - r * VW;
+    const int ih = r - a.pad_t, iw = c - a.pad_l;
+    gin[p] = ih >= 0 && ih < a.ih && iw >= 0 && iw < a.iw;
+    goff[p] = gin[p] ? (ih * a.iw + iw) * 16 : 0;
+  }
+
+  // ---- weights [9][units_pad][ocpp][16]: lane = packed row l32 of unit 2 * pair + lh ---------
+  const int8_t *wb = a.w + ((long long)lh * a.ocpp + oc0 + mw0 + l32) * 16;
+  const long long w_unit = (long long)a.ocpp * 16;
+  const long long w_tap = (long long)a.units_pad * w_unit;
+  v4i a_reg[9][TM];
+  auto load_a = [&](int tap, int pair) {
+    const int8_t *p = wb + tap * w_tap + (long long)(2 * pair) * w_unit;
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) a_reg[tap][mt] = *reinterpret_cast<const v4i *>(p + mt * 512);
+  };
+
+  // All global loads are unconditional (clamped indices, unwanted values replaced afterwards).
+  // `first`: the weight operands of pair 0 are requested right behind the first batch of pixel
+  // loads -- loads return in order, and the pixels are needed first (LDS store, barrier).
+  const int nk = a.chunk_units / G;    // units per thread and pass
+  auto stage = [&](int chunk, bool first) {
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+      for (int k0 = 0; k0 < nk; k0 += 4) {
+        v4i t[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = k0 + j < nk ? k0 + j : nk - 1;
+          int u = chunk * a.chunk_units + ug + G * k;
+          u = u < a.ic2 ? u : a.ic2 - 1;   // padded units multiply zero weights
+          t[j] = *reinterpret_cast<const v4i *>(inb + (long long)u * plane + goff[p]);
+        }
+        if (first && p == 0 && k0 == 0) {
+#pragma unroll
+          for (int tap = 0; tap < 9; ++tap) load_a(tap, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (k0 + j < nk) {
+            const v4i x = t[j] ^ (int)0x80808080;
+            const v4i z = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+            lds[(ug + G * (k0 + j)) * STRIDE + tid % CT + p * CT] = gin[p] ? x : z;
+          }
+        }
+      }
+    }
+  };
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
+
+  // one channel pair (32 input channels) x nine taps; `last` = nothing left to prefetch
+  auto pair_taps = [&](int pl, int pair, bool last) {
+    const v4i *tile = lds + (2 * pl + lh) * STRIDE + pw0 + l32;
+    v4i bq[2][TN];
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) bq[0][nt] = tile[nt * 32];
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) {
+      if (tap < 8) {
+        const int toff = ((tap + 1) / 3) * VW + (tap + 1) % 3;
+#pragma unroll
+        for (int nt = 0; nt < TN; ++nt) bq[(tap + 1) & 1][nt] = tile[nt * 32 + toff];
+      }
+      // keep the compiler from sinking these reads next to their use
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < TN; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[tap][mt], bq[tap & 1][nt], acc[mt][nt], 0, 0, 0);
+      if (!last) load_a(tap, pair + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const int ppc = a.chunk_units / 2;
+  const int nchunks = a.units_pad / a.chunk_units;
+  const long long cidx = oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
+  OcConsts k0;
+  stage(0, true);
+  TRACE_POINT(2);
+  __syncthreads();
+  TRACE_POINT(3);
+  for (int chunk = 0; chunk < nchunks; ++chunk) {
+    if (chunk) {
+      __syncthreads();
+      stage(chunk, false);
+      __syncthreads();
+    }
+    const int npl = chunk + 1 < nchunks ? ppc : ppc - 1;
+    for (int pl = 0; pl < npl; ++pl) pair_taps(pl, chunk * ppc + pl, false);
+    TRACE_POINT(4);
+    if (chunk + 1 == nchunks) {
+      // the epilogue's per-channel constants travel while the last pair is multiplied
+      load_consts(k0, a.ep, cidx);
+      pair_taps(ppc - 1, chunk * ppc + ppc - 1, true);
+    }
+  }
+  TRACE_POINT(5);
+
+  // ---- epilogue ------------------------------------------------------------------------------
+  size_t pix[TN];
+  bool pvalid[TN];
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) {
+    const int v = v0 + pw0 + nt * 32 + l32;
+    const int r = fastdiv(v, VW, a.vw_magic);
+    const int c = v - r * VW;
+    pvalid[nt] = r < a.oh && c < a.ow;
+    pix[nt] = ((size_t)n * a.oc2 * ohw + (pvalid[nt] ? r * a.ow + c : 0)) * 16;
+  }
+  TRACE_POINT(14);
+  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, (int)cidx, pix, pvalid, oc_real, (size_t)ohw * 16, a.out);
+  TRACE_POINT(15);
+}
+
+namespace {
+struct Variant {
+  const char *name;
+  int oc_t, p_t, cells;
+  void (*kernel)(Conv3x3Args);
+};
+#define V(WM, WN, TM, TN, CT, NPASS)                                                              \
+  { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
+    CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS> }
+const Variant kVariants[] = {
+    V(2, 2, 2, 1, 128, 1),  // 0: 128 oc x  64 px, rows up to  31 cells
+    V(2, 2, 2, 1, 256, 1),  // 1: 128 oc x  64 px, rows up to  95 cells
+    V(2, 2, 2, 2, 256, 1),  // 2: 128 oc x 128 px, rows up to  63 cells
+    V(2, 2, 2, 2, 256, 3),  // 3: 128 oc x 128 px, rows up to 319 cells
+    V(1, 4, 2, 1, 256, 1),  // 4:  64 oc x 128 px, rows up to  63 cells
+    V(1, 4, 2, 1, 256, 3),  // 5:  64 oc x 128 px, rows up to 319 cells
+    V(1, 4, 1, 1, 256, 1),  // 6:  32 oc x 128 px, rows up to  63 cells
+    V(1, 4, 1, 1, 256, 3),  // 7:  32 oc x 128 px, rows up to 319 cells
+    V(4, 1, 1, 1, 128, 1),  // 8: 128 oc x  32 px, rows up to  47 cells
+    V(4, 1, 1, 4, 256, 1),  // 9: 128 oc x 128 px, rows up to  63 cells, every wave all pixels
+    V(4, 1, 1, 2, 128, 1),  // 10: 128 oc x 64 px, rows up to  31 cells, every wave all pixels
+};
+#undef V
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+constexpr int kLdsBudget = 64 * 1024;
+}  // namespace
+
+const char *conv3x3v_variant_name(int v) { return kVariants[v].name; }
+int conv3x3v_num_variants() { return kNumVariants; }
+bool conv3x3v_fits(int v, int ow) { return kVariants[v].p_t + 2 * (ow + 2) + 2 <= kVariants[v].cells; }
+
+// units of 16 input channels staged per LDS fill: all of them if they fit the budget
+int conv3x3v_chunk_units(int v, int ic2)
+{
+  int cu = (kLdsBudget / (kVariants[v].cells * 16)) & ~1;
+  const int all = up(ic2, 2);
+  return cu < all ? cu : all;
+}
+
+// -1: no variant fits the row width
+int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
+{
+  const char *env = getenv("EHIP_CONV3X3V_VARIANT");
+  if (env && env[0]) {
+    int v = atoi(env);
+    if (v >= 0 && v < kNumVariants && conv3x3v_fits(v, ow)) return v;
+    return -1;
+  }
+  const int oc = oc2 * 16, vpx = oh * (ow + 2);
+  int best = -1;
+  double best_score = -1;
+  for (int v = 0; v < kNumVariants; ++v) {
+    if (!conv3x3v_fits(v, ow)) continue;
+    const Variant &k = kVariants[v];
+    const int gx = (vpx + k.p_t - 1) / k.p_t, gy = (oc + k.oc_t - 1) / k.oc_t;
+    const long long wgs = (long long)gx * gy * n;
+    const double util = ((double)oc / ((double)gy * k.oc_t)) * ((double)(oh * ow) / ((double)gx * k.p_t));
+    const long long rounds = (wgs + 511) / 512;
+    const double fill = (double)wgs / (double)(rounds * 512);
+    const double lean = (double)(k.p_t + 2 * (ow + 2) + 2) / (double)k.cells;  // unused LDS costs occupancy
+    const double score = util * (0.5 + 0.5 * fill) * (0.75 + 0.25 * lean) * (k.oc_t >= 64 ? 1.0 : 0.8);
+    if (score > best_score) { best_score = score; best = v; }
+  }
+  return best;
+}
+
+hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s)
+{
+  const Variant &k = kVariants[variant];
+  const size_t lds_bytes = (size_t)a.chunk_units * k.cells * 16;
+  dim3 grid((a.oh * a.vw + k.p_t - 1) / k.p_t, (a.oc2 * 16 + k.oc_t - 1) / k.oc_t, n);
+  if (lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k.kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(k.kernel, grid, dim3(kBlock), lds_bytes, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace ehip

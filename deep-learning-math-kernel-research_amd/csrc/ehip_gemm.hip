@@ -9,16 +9,16 @@
 //
 // Mapping.  D[oc][pixel] += W[oc][k] * X[k][pixel] with v_mfma_i32_32x32x32_i8:
 //   A operand = weights: lane l holds 16 consecutive input channels (unit 2*kstep + l/32) of
-//               output channel l%32,
+//               packed row l%32 (rows are packed in the order that makes a lane's results 16
+//               consecutive output channels, see packed_row_of_oc),
 //   B operand = activations: lane l holds the 16 channels of one nChw16c pixel cell (pixel l%32,
 //               unit 2*kstep + l/32) -- 16 bytes that are contiguous in memory, so no layout
 //               change is needed on the way in,
-//   D         = lane l holds, for pixel l%32, four runs of 4 consecutive output channels
-//               (8*g + 4*(l/32) .. +3, g = 0..3): one dword of u8/s8 output or one float4 of f32
-//               output per run.
+//   D         = lane l holds, for pixel l%32, 16 consecutive output channels (16*(l/32) .. +15 of
+//               the 32-row tile): one 16-byte cell of u8/s8 output, four float4 of f32 output.
 // The MFMA is signed x signed: activations are remapped u8 -> s8 by flipping the top bit when a
-// tile is staged into LDS, and the accumulators start at 128 * sum(weights) per output channel,
-// which makes the s32 result identical to the unsigned product.
+// tile is staged into LDS, and 128 * sum(weights) per output channel is added to the sums,
+// which makes the s32 result identical to the unsigned product (the epilogue adds that term).
 //
 // A workgroup (4 waves, WM x WN) owns OC_T output channels x P_T pixels; a wave owns TM x TN MFMA
 // tiles of 32 x 32.  Both operands go global -> registers -> LDS (double buffered, KC units of 16
@@ -29,10 +29,8 @@
 
 namespace ehip {
 
-typedef int v16i __attribute__((ext_vector_type(16)));
-
 template <int WM, int WN, int TM, int TN, int KC>
-__global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
+__global__ __launch_bounds__(kBlock, (TM * TN >= 8 ? 1 : 2)) void k_gemm_u8s8(GemmArgs a)
 {
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
@@ -112,20 +110,13 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     }
   };
 
-  // ---- accumulators start at the u8->s8 compensation -------------------------------------
-  const long long per_oc = (long long)b * a.ocpp + oc0 + mw0 + 4 * lh;
   v16i acc[TM][TN];
 #pragma unroll
-  for (int mt = 0; mt < TM; ++mt) {
-    v16i c;
+  for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const v4i c4 = *reinterpret_cast<const v4i *>(a.ep.comp + per_oc + mt * 32 + 8 * g);
-      c[4 * g + 0] = c4.x; c[4 * g + 1] = c4.y; c[4 * g + 2] = c4.z; c[4 * g + 3] = c4.w;
-    }
+    for (int nt = 0; nt < TN; ++nt)
 #pragma unroll
-    for (int nt = 0; nt < TN; ++nt) acc[mt][nt] = c;
-  }
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
 
   // ---- main loop ------------------------------------------------------------------------------
   v4i opa[2][TM], opb[2][TN];
@@ -166,14 +157,9 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   // last fill: nothing left to prefetch but the epilogue's per-channel constants
   store_stage(buf);
   __syncthreads();
-  float4 sc[TM][4], sh[TM][4];
-#pragma unroll
-  for (int mt = 0; mt < TM; ++mt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      sc[mt][g] = *reinterpret_cast<const float4 *>(a.ep.scale + per_oc + mt * 32 + 8 * g);
-      sh[mt][g] = *reinterpret_cast<const float4 *>(a.ep.shift + per_oc + mt * 32 + 8 * g);
-    }
+  const long long cidx = (long long)b * a.ocpp + oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
+  OcConsts k0;
+  load_consts(k0, a.ep, cidx);
   multiply(buf);
 
   // ---- epilogue ------------------------------------------------------------------------------
@@ -188,21 +174,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     const int r = gpc - n * a.ohw;
     pix[nt] = (size_t)b * a.out_batch_stride + ((size_t)n * a.oc2 * a.ohw + r) * 16;
   }
-#pragma unroll
-  for (int mt = 0; mt < TM; ++mt) {
-    v4i quad[4][TN];
-    int oc_of[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      oc_of[g] = oc0 + mw0 + mt * 32 + 8 * g + 4 * lh;
-#pragma unroll
-      for (int nt = 0; nt < TN; ++nt) {
-        const v16i &d = acc[mt][nt];
-        quad[g][nt] = v4i{d[4 * g], d[4 * g + 1], d[4 * g + 2], d[4 * g + 3]};
-      }
-    }
-    epilogue_dispatch<4, TN>(a.ep, quad, sc[mt], sh[mt], pix, pvalid, oc_of, oc_real, (size_t)a.ohw * 16, a.out);
-  }
+  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real, (size_t)a.ohw * 16, a.out);
 }
 
 namespace {

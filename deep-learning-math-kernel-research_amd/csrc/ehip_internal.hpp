@@ -57,10 +57,10 @@ struct Conv3x3Args {
   int ih, iw, oh, ow;
   int pad_t, pad_l;
   int ic2, units_pad, oc2, ocpp;
-  int halo_rows;        // input rows staged per tile
-  int chunk_units;      // ic2 units staged per LDS fill (multiple of 4)
+  int chunk_units;      // ic2 units staged per LDS fill (even)
+  int vw;               // virtual row width ow + 2
+  unsigned vw_magic;    // div_magic(vw)
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
-  int dbg;              // development aid: bit 0 = skip LDS operand reads, bit 1 = skip weight reloads
 };
 
 struct DepthwiseArgs {
@@ -92,12 +92,11 @@ int gemm_variant_chunk(int variant);
 int gemm_num_variants();
 const char *gemm_variant_name(int variant);
 
-hipError_t launch_conv3x3(const Conv3x3Args &a, int n, int variant, size_t lds_bytes, hipStream_t s);
-int conv3x3_pick_variant(int oh, int ow, int oc2);
-int conv3x3_variant_pixels(int variant);
-int conv3x3_variant_slots(int variant);   // 16-byte cells of one LDS buffer
-int conv3x3_num_variants();
-const char *conv3x3_variant_name(int variant);
+hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s);
+int conv3x3v_pick_variant(int n, int oh, int ow, int oc2);   // -1: rows too wide for every variant
+int conv3x3v_chunk_units(int variant, int ic2);
+int conv3x3v_num_variants();
+const char *conv3x3v_variant_name(int variant);
 
 hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s);
 hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s);
@@ -164,12 +163,44 @@ __device__ __forceinline__ float requant(int acc, float scale, float shift, bool
   return f;
 }
 
+// ---- weight row order ---------------------------------------------------------------------------
+// Inside every group of 32 rows the packed weights are stored in the order in which the 32x32 MFMA
+// hands rows to lanes: packed row 8g + 4h + j holds output channel 16h + 4g + j (g = 0..3, h = 0..1,
+// j = 0..3).  A lane of the result (which owns rows 8g + 4h + j for its own h and all g, j) then
+// holds 16 CONSECUTIVE output channels, i.e. exactly one 16-channel cell of the blocked output.
+__host__ __device__ __forceinline__ int packed_row_of_oc(int oc)
+{
+  const int o = oc & 31;
+  return (oc & ~31) + 8 * ((o >> 2) & 3) + 4 * (o >> 4) + (o & 3);
+}
+__host__ __device__ __forceinline__ int oc_of_packed_row(int r)
+{
+  const int i = r & 31;
+  return (r & ~31) + 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3);
+}
+
 // ---- fused requantization epilogue of the MFMA kernels -----------------------------------------
-// A lane holds, for each of its NP pixels and MO 16-channel blocks, 4 consecutive output
-// channels (one dword of u8/s8, one float4 of f32/s32).  The per-channel scale/shift are loaded
-// once per kernel (hoisted by the caller), the sum operands are all requested before the first
-// one is used, and the output type is a template parameter, so the epilogue is straight-line code
-// whose memory latencies overlap instead of queueing behind each other.
+// A lane holds, for each of its TN pixels and TM 32-row tiles, 16 consecutive output channels: one
+// 16-byte cell of u8/s8 output, four float4 of f32/s32 output.  The per-channel constants of tile
+// mt+1 are requested before tile mt is processed, the sum operands of a tile are all requested
+// before the first is used, and the output type is a template parameter, so the epilogue is
+// straight-line code whose memory latencies overlap.
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct OcConsts {      // of 16 consecutive output channels
+  float4 sc[4], sh[4];
+  v4i comp[4];
+};
+__device__ __forceinline__ void load_consts(OcConsts &k, const Epilogue &ep, long long idx)
+{
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    k.sc[q] = *reinterpret_cast<const float4 *>(ep.scale + idx + 4 * q);
+    k.sh[q] = *reinterpret_cast<const float4 *>(ep.shift + idx + 4 * q);
+    k.comp[q] = *reinterpret_cast<const v4i *>(ep.comp + idx + 4 * q);
+  }
+}
+
 __device__ __forceinline__ float requant1(int acc, float scale, float shift, bool relu, float lo, float hi)
 {
   float f = __builtin_fmaf((float)acc, scale, shift);
@@ -195,99 +226,143 @@ __device__ __forceinline__ unsigned quant1(float f)
   return (unsigned)ssat8(i) & 0xffu;
 }
 
-template <int MO, int NP, int OUT, bool SUM>
-__device__ __forceinline__ void epilogue_tile(const Epilogue &ep, const v4i (&acc)[MO][NP], const float4 (&sc)[MO],
-                                              const float4 (&sh)[MO], const size_t (&pix)[NP],
-                                              const bool (&pvalid)[NP], const int (&oc_of)[MO], int oc_real,
-                                              size_t oc2_stride, void *out)
+// four channels -> one dword of u8/s8 codes
+template <int OUT, bool SUM, bool FAST>
+__device__ __forceinline__ unsigned quant4(const Epilogue &ep, int a0, int a1, int a2, int a3, const float4 &sc,
+                                           const float4 &sh, unsigned old)
 {
-  // oc_of[mo]: the lane's first channel (a multiple of 4) of its quad in block mo
-  const bool relu = ep.with_relu != 0;
-  unsigned old[MO][NP];
+  float f0 = __builtin_fmaf((float)a0, sc.x, sh.x);
+  float f1 = __builtin_fmaf((float)a1, sc.y, sh.y);
+  float f2 = __builtin_fmaf((float)a2, sc.z, sh.z);
+  float f3 = __builtin_fmaf((float)a3, sc.w, sh.w);
   if (SUM) {
-#pragma unroll
-    for (int mo = 0; mo < MO; ++mo)
-#pragma unroll
-      for (int np = 0; np < NP; ++np) {
-        const int oc = oc_of[mo];
-        const bool ok = pvalid[np] && oc < oc_real;
-        const size_t e = ok ? pix[np] + (size_t)(oc >> 4) * oc2_stride + (oc & 15) : 0;
-        old[mo][np] = *reinterpret_cast<const unsigned *>(static_cast<const uint8_t *>(out) + e);
-      }
+    int o0, o1, o2, o3;
+    if (OUT == EHIP_U8) {
+      o0 = old & 0xff; o1 = (old >> 8) & 0xff; o2 = (old >> 16) & 0xff; o3 = old >> 24;
+    } else {
+      o0 = (int)(signed char)(old & 0xff); o1 = (int)(signed char)((old >> 8) & 0xff);
+      o2 = (int)(signed char)((old >> 16) & 0xff); o3 = (int)(signed char)(old >> 24);
+    }
+    f0 = __builtin_fmaf((float)o0, ep.sum_scale, f0);
+    f1 = __builtin_fmaf((float)o1, ep.sum_scale, f1);
+    f2 = __builtin_fmaf((float)o2, ep.sum_scale, f2);
+    f3 = __builtin_fmaf((float)o3, ep.sum_scale, f3);
   }
+  if (FAST) {
+    // ReLU with a lower bound >= 0: every value is in [0, hi], so "round to nearest even, then
+    // saturate" is a clamp to the code range, a round and one pack-with-saturation instruction
+    // per byte (its input is already an integer, so its own rounding is moot)
+    const float hi = OUT == EHIP_S8 ? __builtin_fminf(ep.hi, 127.0f) : ep.hi;
+    f0 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f0, ep.lo), hi));
+    f1 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f1, ep.lo), hi));
+    f2 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f2, ep.lo), hi));
+    f3 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f3, ep.lo), hi));
+    unsigned q = __builtin_amdgcn_cvt_pk_u8_f32(f0, 0, 0);
+    q = __builtin_amdgcn_cvt_pk_u8_f32(f1, 1, q);
+    q = __builtin_amdgcn_cvt_pk_u8_f32(f2, 2, q);
+    return __builtin_amdgcn_cvt_pk_u8_f32(f3, 3, q);
+  }
+  if (ep.with_relu) {
+    f0 = __builtin_fminf(__builtin_fmaxf(f0, ep.lo), ep.hi);
+    f1 = __builtin_fminf(__builtin_fmaxf(f1, ep.lo), ep.hi);
+    f2 = __builtin_fminf(__builtin_fmaxf(f2, ep.lo), ep.hi);
+    f3 = __builtin_fminf(__builtin_fmaxf(f3, ep.lo), ep.hi);
+  }
+  return quant1<OUT>(f0) | (quant1<OUT>(f1) << 8) | (quant1<OUT>(f2) << 16) | (quant1<OUT>(f3) << 24);
+}
+
+// acc[mt][nt]: s32 sums WITHOUT the u8->s8 compensation (it is added here).  k0 = constants of the
+// lane's channels in tile 0, cidx = their index in the per-channel arrays (tile mt: + 32 * mt),
+// oc_first = the lane's first channel in tile 0 (a multiple of 16), pix[nt] = element offset of
+// the pixel's cell in 16-channel block 0, block_stride = elements between 16-channel blocks.
+template <int TM, int TN, int OUT, bool SUM, bool FAST>
+__device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
+                                                    long long cidx, int oc_first, const size_t (&pix)[TN],
+                                                    const bool (&pvalid)[TN], int oc_real, size_t block_stride,
+                                                    void *out)
+{
+  const bool relu = ep.with_relu != 0;
+  OcConsts k = k0;
 #pragma unroll
-  for (int mo = 0; mo < MO; ++mo) {
-    const int oc = oc_of[mo];
-    if (oc >= oc_real) continue;
+  for (int mt = 0; mt < TM; ++mt) {
+    OcConsts kn;
+    if (mt + 1 < TM) load_consts(kn, ep, cidx + 32 * (mt + 1));
+    const int oc = oc_first + 32 * mt;
+    const bool oc_ok = oc < oc_real;
+    size_t e[TN];
+    bool ok[TN];
+    v4i old[TN];
 #pragma unroll
-    for (int np = 0; np < NP; ++np) {
-      if (!pvalid[np]) continue;
-      const size_t e = pix[np] + (size_t)(oc >> 4) * oc2_stride + (oc & 15);
-      const v4i a4 = acc[mo][np];
+    for (int nt = 0; nt < TN; ++nt) {
+      ok[nt] = oc_ok && pvalid[nt];
+      e[nt] = ok[nt] ? pix[nt] + (size_t)(oc >> 4) * block_stride : 0;
+      if (SUM) old[nt] = *reinterpret_cast<const v4i *>(static_cast<const uint8_t *>(out) + e[nt]);
+    }
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) {
+      const v16i &a = acc[mt][nt];
+      v4i s[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        s[q] = v4i{a[4 * q] + k.comp[q].x, a[4 * q + 1] + k.comp[q].y, a[4 * q + 2] + k.comp[q].z,
+                   a[4 * q + 3] + k.comp[q].w};
       if (OUT == EHIP_S32) {
-        *reinterpret_cast<v4i *>(static_cast<int *>(out) + e) = a4;
+        if (ok[nt]) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) *reinterpret_cast<v4i *>(static_cast<int *>(out) + e[nt] + 4 * q) = s[q];
+        }
       } else if (OUT == EHIP_F32) {
-        float4 r;
-        r.x = requant1(a4.x, sc[mo].x, sh[mo].x, relu, ep.lo, ep.hi);
-        r.y = requant1(a4.y, sc[mo].y, sh[mo].y, relu, ep.lo, ep.hi);
-        r.z = requant1(a4.z, sc[mo].z, sh[mo].z, relu, ep.lo, ep.hi);
-        r.w = requant1(a4.w, sc[mo].w, sh[mo].w, relu, ep.lo, ep.hi);
-        *reinterpret_cast<float4 *>(static_cast<float *>(out) + e) = r;
+        float4 r[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          r[q].x = requant1(s[q].x, k.sc[q].x, k.sh[q].x, relu, ep.lo, ep.hi);
+          r[q].y = requant1(s[q].y, k.sc[q].y, k.sh[q].y, relu, ep.lo, ep.hi);
+          r[q].z = requant1(s[q].z, k.sc[q].z, k.sh[q].z, relu, ep.lo, ep.hi);
+          r[q].w = requant1(s[q].w, k.sc[q].w, k.sh[q].w, relu, ep.lo, ep.hi);
+        }
+        if (ok[nt]) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) *reinterpret_cast<float4 *>(static_cast<float *>(out) + e[nt] + 4 * q) = r[q];
+        }
       } else {
-        float f0 = __builtin_fmaf((float)a4.x, sc[mo].x, sh[mo].x);
-        float f1 = __builtin_fmaf((float)a4.y, sc[mo].y, sh[mo].y);
-        float f2 = __builtin_fmaf((float)a4.z, sc[mo].z, sh[mo].z);
-        float f3 = __builtin_fmaf((float)a4.w, sc[mo].w, sh[mo].w);
-        if (SUM) {
-          const unsigned o = old[mo][np];
-          int o0, o1, o2, o3;
-          if (OUT == EHIP_U8) {
-            o0 = o & 0xff; o1 = (o >> 8) & 0xff; o2 = (o >> 16) & 0xff; o3 = o >> 24;
-          } else {
-            o0 = (int)(signed char)(o & 0xff); o1 = (int)(signed char)((o >> 8) & 0xff);
-            o2 = (int)(signed char)((o >> 16) & 0xff); o3 = (int)(signed char)(o >> 24);
-          }
-          f0 = __builtin_fmaf((float)o0, ep.sum_scale, f0);
-          f1 = __builtin_fmaf((float)o1, ep.sum_scale, f1);
-          f2 = __builtin_fmaf((float)o2, ep.sum_scale, f2);
-          f3 = __builtin_fmaf((float)o3, ep.sum_scale, f3);
-        }
-        if (relu) {
-          f0 = __builtin_fminf(__builtin_fmaxf(f0, ep.lo), ep.hi);
-          f1 = __builtin_fminf(__builtin_fmaxf(f1, ep.lo), ep.hi);
-          f2 = __builtin_fminf(__builtin_fmaxf(f2, ep.lo), ep.hi);
-          f3 = __builtin_fminf(__builtin_fmaxf(f3, ep.lo), ep.hi);
-        }
-        const unsigned q = quant1<OUT>(f0) | (quant1<OUT>(f1) << 8) | (quant1<OUT>(f2) << 16) | (quant1<OUT>(f3) << 24);
-        *reinterpret_cast<unsigned *>(static_cast<uint8_t *>(out) + e) = q;
+        v4i cell;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          cell[q] = (int)quant4<OUT, SUM, FAST>(ep, s[q].x, s[q].y, s[q].z, s[q].w, k.sc[q], k.sh[q],
+                                               SUM ? (unsigned)old[nt][q] : 0u);
+        if (ok[nt]) *reinterpret_cast<v4i *>(static_cast<uint8_t *>(out) + e[nt]) = cell;
       }
     }
+    if (mt + 1 < TM) k = kn;
   }
 }
 
-// one uniform switch on the output type around the whole tile epilogue
-template <int MO, int NP>
-__device__ __forceinline__ void epilogue_dispatch(const Epilogue &ep, const v4i (&acc)[MO][NP], const float4 (&sc)[MO],
-                                                  const float4 (&sh)[MO], const size_t (&pix)[NP],
-                                                  const bool (&pvalid)[NP], const int (&oc_of)[MO], int oc_real,
-                                                  size_t oc2_stride, void *out)
+// one uniform switch on the output type (and on the cheap ReLU form) around the whole epilogue
+template <int TM, int TN>
+__device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
+                                              long long cidx, int oc_first, const size_t (&pix)[TN],
+                                              const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out)
 {
+#define EHIP_EPI(OUT, SUM, FAST) \
+  epilogue_wave_typed<TM, TN, OUT, SUM, FAST>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out)
+  const bool fast = ep.with_relu && ep.lo >= 0.0f && ep.hi >= ep.lo;
   switch (ep.out_type) {
   case EHIP_U8:
-    if (ep.with_sum) epilogue_tile<MO, NP, EHIP_U8, true>(ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, oc2_stride, out);
-    else epilogue_tile<MO, NP, EHIP_U8, false>(ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, oc2_stride, out);
+    if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_U8, true, true); else EHIP_EPI(EHIP_U8, true, false); }
+    else { if (fast) EHIP_EPI(EHIP_U8, false, true); else EHIP_EPI(EHIP_U8, false, false); }
     break;
   case EHIP_S8:
-    if (ep.with_sum) epilogue_tile<MO, NP, EHIP_S8, true>(ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, oc2_stride, out);
-    else epilogue_tile<MO, NP, EHIP_S8, false>(ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, oc2_stride, out);
+    if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_S8, true, true); else EHIP_EPI(EHIP_S8, true, false); }
+    else { if (fast) EHIP_EPI(EHIP_S8, false, true); else EHIP_EPI(EHIP_S8, false, false); }
     break;
   case EHIP_F32:
-    epilogue_tile<MO, NP, EHIP_F32, false>(ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, oc2_stride, out);
+    EHIP_EPI(EHIP_F32, false, false);
     break;
   default:
-    epilogue_tile<MO, NP, EHIP_S32, false>(ep, acc, sc, sh, pix, pvalid, oc_of, oc_real, oc2_stride, out);
+    EHIP_EPI(EHIP_S32, false, false);
     break;
   }
+#undef EHIP_EPI
 }
 
 }  // namespace ehip

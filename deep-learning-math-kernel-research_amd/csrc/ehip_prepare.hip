@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kBlock) void k_quant_pack_direct(const float *w, co
   if (idx >= total) return;
   const int q = (int)(idx & 3);
   long long rest = idx >> 2;
-  const int oc = (int)(rest % ocpp);
+  const int oc = oc_of_packed_row((int)(rest % ocpp));   // the channel this packed row holds
   rest /= ocpp;
   const int u = (int)(rest % units_pad);
   const int tap = (int)(rest / units_pad);
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void k_fold_direct(const unsigned *wpacked,
   int s = 0;
   if (oc < oc_rows) {
     for (int tu = 0; tu < taps * units_pad; ++tu) {
-      const uint4 c = *reinterpret_cast<const uint4 *>(wpacked + ((size_t)tu * ocpp + oc) * 4);
+      const uint4 c = *reinterpret_cast<const uint4 *>(wpacked + ((size_t)tu * ocpp + packed_row_of_oc(oc)) * 4);
       const unsigned d[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
       for (int j = 0; j < 4; ++j)
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kBlock) void k_wino_quant(const float *U, int ocp, 
   int s = 0;
   for (int ic = 0; ic < icp; ++ic) {
     const int q = quant_w(u[ic], am);
-    wpacked[(((size_t)pos * units_pad + (ic >> 4)) * ocpp + oc) * 16 + (ic & 15)] = (int8_t)q;
+    wpacked[(((size_t)pos * units_pad + (ic >> 4)) * ocpp + packed_row_of_oc(oc)) * 16 + (ic & 15)] = (int8_t)q;
     s += q;
   }
   // Sw = absmax / 127; Sw = Sw * tin_S; Zw = -acc * Sw * tin_z  (trans_weights.cpp:523-533)

@@ -72,10 +72,21 @@ def test_conv3x3_no_padding():
     run_and_compare(Layer(2, 32, 32, 12, k=3, pad=0, out_type=ol.U8, seed=3))
 
 
-@pytest.mark.parametrize("variant", range(6))
-def test_conv3x3_every_kernel_variant(variant, monkeypatch):
-    monkeypatch.setenv("EHIP_CONV3X3_VARIANT", str(variant))
-    run_and_compare(Layer(2, 64, 144, 13, k=3, pad=1, out_type=ol.U8, seed=60 + variant))
+@pytest.mark.parametrize("variant", range(11))
+def test_conv3x3_every_virtual_row_kernel_variant(variant, monkeypatch):
+    monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", str(variant))
+    res = run_and_compare(Layer(2, 64, 144, 13, k=3, pad=1, out_type=ol.U8, seed=80 + variant))
+    assert res["conv"].kernel_name.startswith("k_conv3x3v_u8s8")
+
+
+def test_conv3x3_virtual_rows_many_channels_restage():
+    # 1040 input channels = 65 units: more than one LDS fill of the virtual-row kernel, odd unit count
+    res = run_and_compare(Layer(1, 1040, 48, 9, k=3, pad=1, out_type=ol.S8, seed=91, w_sigma=0.02))
+    assert res["conv"].kernel_name.startswith("k_conv3x3v_u8s8")
+
+
+def test_conv3x3_wide_rows():
+    run_and_compare(Layer(1, 16, 32, 70, k=3, pad=1, out_type=ol.U8, seed=92))
 
 
 # ---- depthwise 3x3 ----------------------------------------------------------------------------------
