@@ -253,7 +253,7 @@ int setup_workspace(ehip_conv *c)
 
   if (c->family == FAM_DEPTHWISE) {
     c->ocpp = c->oc2 * 16;
-    c->wpacked_bytes = (size_t)c->oc2 * 9 * 16;
+    c->wpacked_bytes = (size_t)c->oc2 * 3 * 16 * 4;
   } else {
     c->ocpp = up(c->oc2 * 16, kOcTile);
     c->wpacked_bytes = (size_t)c->nbatch * c->taps * c->units_pad * c->ocpp * 16;
@@ -425,7 +425,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.in = static_cast<const uint8_t *>(input_dev);
     a.w = c->wpacked;
     a.out = output_dev;
-    a.scale = c->scale; a.shift = c->shift;
+    a.scale = c->scale; a.shift = c->shift; a.wsum = c->wsum;
     a.n = d.n; a.g2 = c->oc2; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
     a.pad_t = d.pad_t; a.pad_l = d.pad_l;
     a.T = c->T; a.Tr = c->Tr; a.wt = c->wtb;
@@ -501,7 +501,7 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
       HIP_TRY(hipMemcpy(packed.data(), c->wpacked, c->wpacked_bytes, hipMemcpyDeviceToHost));
       int8_t *dst = static_cast<int8_t *>(host_dst);
       for (int g = 0; g < ocp; ++g)
-        for (int k = 0; k < 9; ++k) dst[(size_t)g * 9 + k] = packed[((size_t)(g >> 4) * 9 + k) * 16 + (g & 15)];
+        for (int k = 0; k < 9; ++k) dst[(size_t)g * 9 + k] = packed[(((size_t)(g >> 4) * 3 + k / 3) * 16 + (g & 15)) * 4 + k % 3];
       return EHIP_OK;
     }
     const int taps = c->taps;

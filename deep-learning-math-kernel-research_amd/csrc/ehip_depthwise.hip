@@ -4,12 +4,17 @@
 // (src/elx_int8_conv_direct_depthwise_xopt.hpp:19-66, src/elx_int8_conv_direct_depthwise.cpp:294-319)
 // and the depthwise micro-kernel (src/kernel/elk_u8s8_depthwise_conv.hxx:219-474).
 //
-// There is no contraction over channels, so the matrix cores have nothing to do: every lane owns
-// one output column of one 16-channel block and walks RB output rows down it, so that each input
-// cell (16 bytes = the 16 channels of a pixel) is loaded once per three columns instead of nine
-// times; neighbouring lanes read neighbouring cells (coalesced 16-byte accesses) and the overlap
-// between columns is served by the vector L1.  Out-of-image taps are skipped exactly as the
-// reference skips them.
+// There is no contraction over channels, so the matrix cores have nothing to do; the work is
+// 1 byte in + 1 byte out per 9 multiply-adds and the kernel has to keep the VALU cost per byte
+// below what HBM can deliver.  A lane owns 4 channels (one dword of a 16-channel cell) x 2 output
+// columns x RB output rows.  Per input row it loads the 4 pixels its two columns touch (4 dwords;
+// the 4 lanes of a cell read 16 contiguous bytes), flips the top bits (u8 -> s8, undone by the
+// 128 * sum(w) the accumulators start from; out-of-image pixels count as u8 0), and byte-transposes
+// the 4 pixels x 4 channels block with 8 v_perm_b32 so that one dword holds the four horizontally
+// adjacent pixels of ONE channel.  The three taps of a kernel row are then a single v_dot4_i32_i8
+// against weights packed [kh][channel][kw0 kw1 kw2 0] -- and the same dword serves the second
+// column against the weights shifted by one byte.  The packed layout is the reference's own
+// ([g/16][kh][16][KW=4], src/elx_int8_conv_direct_depthwise.cpp:224-236).
 //
 // The u8 store reproduces the reference's width-block rule: inside every block of T output columns
 // (Tr for the last block) the columns before 4*floor(Tz/4) are rounded toward -infinity and
@@ -18,125 +23,172 @@
 
 namespace ehip {
 
-template <int RB>
+namespace {
+// v_perm_b32: result byte i = byte sel[i] of the 8-byte pool {hi: 4..7, lo: 0..3}
+__device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel)
+{
+  return __builtin_amdgcn_perm(hi, lo, sel);
+}
+}  // namespace
+
+// MODE 0: any output type / bounds.  MODE 1: u8 output, ReLU with 0 <= lo <= hi <= 255 (floor and
+// round-to-nearest both land in the code range, so the pack-with-saturation instruction, which
+// rounds to nearest even itself, finishes either).  MODE 2: as 1 with lo == 0 and hi == 255, where
+// the clamp is the instruction's own saturation.
+template <int RB, int MODE>
 __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 {
   const int ohb = (a.oh + RB - 1) / RB;
-  const long long total = (long long)a.n * a.g2 * ohb * a.ow;
+  const int wp = (a.ow + 1) >> 1;
+  const long long total = (long long)a.n * a.g2 * ohb * wp * 4;
   const long long idx = (long long)blockIdx.x * kBlock + threadIdx.x;
   if (idx >= total) return;
-  const int ow = (int)(idx % a.ow);
-  long long rest = idx / a.ow;
+  const int q = (int)(idx & 3);
+  long long rest = idx >> 2;
+  const int p = (int)(rest % wp);
+  rest /= wp;
   const int hb = (int)(rest % ohb);
   const long long ng = rest / ohb;  // n * g2 + g2 index
   const int g2 = (int)(ng % a.g2);
   const int oh0 = hb * RB;
+  const int c0 = 2 * p;
+  const int ch0 = g2 * 16 + 4 * q;  // first of the lane's 4 channels
 
-  // weights of this 16-channel block: [9][16] s8
-  uint4 wv[9];
-  const uint4 *wp = reinterpret_cast<const uint4 *>(a.w) + (size_t)g2 * 9;
+  // weights: [g2][kh][16][4] -> per kh one dword per channel (kw0 kw1 kw2 0); second column: << 8
+  unsigned wa[3][4], wb[3][4];
 #pragma unroll
-  for (int k = 0; k < 9; ++k) wv[k] = wp[k];
+  for (int kh = 0; kh < 3; ++kh) {
+    const uint4 w4 = *reinterpret_cast<const uint4 *>(a.w + (((size_t)g2 * 3 + kh) * 16 + 4 * q) * 4);
+    wa[kh][0] = w4.x; wa[kh][1] = w4.y; wa[kh][2] = w4.z; wa[kh][3] = w4.w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wb[kh][j] = wa[kh][j] << 8;
+  }
+  const v4i ws = *reinterpret_cast<const v4i *>(a.wsum + ch0);
 
-  int acc[RB][16];
+  int acc[RB][2][4];
 #pragma unroll
   for (int r = 0; r < RB; ++r)
 #pragma unroll
-    for (int c = 0; c < 16; ++c) acc[r][c] = 0;
+    for (int c = 0; c < 2; ++c) {
+      acc[r][c][0] = 128 * ws.x; acc[r][c][1] = 128 * ws.y; acc[r][c][2] = 128 * ws.z; acc[r][c][3] = 128 * ws.w;
+    }
 
-  const uint4 *plane = reinterpret_cast<const uint4 *>(a.in) + (size_t)ng * a.ih * a.iw;
+  // the 4 input columns of this lane (clamped; invalid ones are replaced after the load)
+  int colv[4];
+  bool colok[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int iw = c0 - a.pad_l + k;
+    colok[k] = iw >= 0 && iw < a.iw;
+    colv[k] = iw < 0 ? 0 : (iw >= a.iw ? a.iw - 1 : iw);
+  }
+  const unsigned *plane = reinterpret_cast<const unsigned *>(a.in) + (size_t)ng * a.ih * a.iw * 4 + q;
+
 #pragma unroll
   for (int hr = 0; hr < RB + 2; ++hr) {
     const int ih = oh0 - a.pad_t + hr;
-    if (ih < 0 || ih >= a.ih) continue;
-    uint4 x[3];
+    const bool rowok = ih >= 0 && ih < a.ih;
+    const int ihc = ih < 0 ? 0 : (ih >= a.ih ? a.ih - 1 : ih);
+    unsigned x[4];
 #pragma unroll
-    for (int kw = 0; kw < 3; ++kw) {
-      const int iw = ow - a.pad_l + kw;
-      x[kw] = (iw >= 0 && iw < a.iw) ? plane[(size_t)ih * a.iw + iw] : make_uint4(0u, 0u, 0u, 0u);
+    for (int k = 0; k < 4; ++k) {
+      const unsigned v = plane[((size_t)ihc * a.iw + colv[k]) * 4];
+      x[k] = (rowok && colok[k]) ? v ^ 0x80808080u : 0x80808080u;
     }
+    // 4 pixels x 4 channels -> 4 channels x 4 pixels
+    const unsigned a0 = perm(x[1], x[0], 0x05010400u), a1 = perm(x[1], x[0], 0x07030602u);
+    const unsigned b0 = perm(x[3], x[2], 0x05010400u), b1 = perm(x[3], x[2], 0x07030602u);
+    unsigned t[4];
+    t[0] = perm(b0, a0, 0x05040100u);
+    t[1] = perm(b0, a0, 0x07060302u);
+    t[2] = perm(b1, a1, 0x05040100u);
+    t[3] = perm(b1, a1, 0x07060302u);
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const int kh = hr - r;  // input row ih feeds output row oh0 + r through tap row kh
+      const int kh = hr - r;  // input row ih feeds output row oh0 + r through kernel row kh
       if (kh < 0 || kh > 2) continue;
 #pragma unroll
-      for (int kw = 0; kw < 3; ++kw) {
-        const unsigned xd[4] = {x[kw].x, x[kw].y, x[kw].z, x[kw].w};
-        const uint4 w4 = wv[kh * 3 + kw];
-        const unsigned wd[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-        for (int d = 0; d < 4; ++d)
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const int xb = (int)((xd[d] >> (8 * k)) & 0xffu);
-            const int wb = (int)(signed char)((wd[d] >> (8 * k)) & 0xffu);
-            acc[r][4 * d + k] += xb * wb;
-          }
+      for (int j = 0; j < 4; ++j) {
+        acc[r][0][j] = __builtin_amdgcn_sdot4((int)t[j], (int)wa[kh][j], acc[r][0][j], false);
+        acc[r][1][j] = __builtin_amdgcn_sdot4((int)t[j], (int)wb[kh][j], acc[r][1][j], false);
       }
     }
   }
 
-  // width-block rule for this column
-  const int blk = ow / a.T;
-  const int tpos = ow - blk * a.T;
-  const int Tz = blk == a.wt - 1 ? a.Tr : a.T;
-  const bool floor_col = a.out_type == EHIP_U8 && tpos < 4 * (Tz / 4);
+  const float4 sc = *reinterpret_cast<const float4 *>(a.scale + ch0);
+  const float4 sh = *reinterpret_cast<const float4 *>(a.shift + ch0);
+  const float scv[4] = {sc.x, sc.y, sc.z, sc.w}, shv[4] = {sh.x, sh.y, sh.z, sh.w};
   const bool relu = a.with_relu != 0;
 
-  float sc[16], sh[16];
 #pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const float4 s4 = reinterpret_cast<const float4 *>(a.scale)[g2 * 4 + d];
-    const float4 z4 = reinterpret_cast<const float4 *>(a.shift)[g2 * 4 + d];
-    sc[4 * d] = s4.x; sc[4 * d + 1] = s4.y; sc[4 * d + 2] = s4.z; sc[4 * d + 3] = s4.w;
-    sh[4 * d] = z4.x; sh[4 * d + 1] = z4.y; sh[4 * d + 2] = z4.z; sh[4 * d + 3] = z4.w;
-  }
-
+  for (int c = 0; c < 2; ++c) {
+    const int ow = c0 + c;
+    if (ow >= a.ow) break;
+    // width-block rule for this column
+    const int blk = ow / a.T;
+    const int tpos = ow - blk * a.T;
+    const int Tz = blk == a.wt - 1 ? a.Tr : a.T;
+    const bool floor_col = a.out_type == EHIP_U8 && tpos < 4 * (Tz / 4);
 #pragma unroll
-  for (int r = 0; r < RB; ++r) {
-    const int oh = oh0 + r;
-    if (oh >= a.oh) break;
-    unsigned o[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-      const float f = requant(acc[r][c], sc[c], sh[c], false, 0, 0.f, relu, a.lo, a.hi);
-      unsigned q;
-      if (a.out_type == EHIP_S32) {
-        q = 0;
-      } else if (floor_col) {
-        const int fl = (!(f >= -2147483648.0f && f < 2147483648.0f)) ? (int)0x80000000 : (int)__builtin_floorf(f);
-        q = (unsigned)fl & 0xffu;
-      } else if (a.out_type == EHIP_U8) {
-        q = usat8((unsigned)cvt_s32_rne(f));
-      } else {
-        q = (unsigned)ssat8(cvt_s32_rne(f)) & 0xffu;
+    for (int r = 0; r < RB; ++r) {
+      const int oh = oh0 + r;
+      if (oh >= a.oh) break;
+      const size_t cell = ((size_t)ng * a.oh + oh) * a.ow + ow;
+      if (MODE == 0 && a.out_type == EHIP_S32) {
+        reinterpret_cast<v4i *>(a.out)[cell * 4 + q] = v4i{acc[r][c][0], acc[r][c][1], acc[r][c][2], acc[r][c][3]};
+        continue;
       }
-      o[c >> 2] |= q << (8 * (c & 3));
-    }
-    const size_t cell = ((size_t)ng * a.oh + oh) * a.ow + ow;
-    if (a.out_type == EHIP_S32) {
-      v4i *dst = reinterpret_cast<v4i *>(a.out) + cell * 4;
+      unsigned o = 0u;
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        v4i v = {acc[r][4 * d], acc[r][4 * d + 1], acc[r][4 * d + 2], acc[r][4 * d + 3]};
-        dst[d] = v;
+      for (int j = 0; j < 4; ++j) {
+        float f = __builtin_fmaf((float)acc[r][c][j], scv[j], shv[j]);
+        if (MODE == 0) {
+          if (relu) f = __builtin_fminf(__builtin_fmaxf(f, a.lo), a.hi);
+          unsigned qv;
+          if (floor_col) {
+            const int fl = (!(f >= -2147483648.0f && f < 2147483648.0f)) ? (int)0x80000000 : (int)__builtin_floorf(f);
+            qv = (unsigned)fl & 0xffu;
+          } else if (a.out_type == EHIP_U8) {
+            qv = usat8((unsigned)cvt_s32_rne(f));
+          } else {
+            qv = (unsigned)ssat8(cvt_s32_rne(f)) & 0xffu;
+          }
+          o |= qv << (8 * j);
+        } else {
+          if (MODE == 1) f = __builtin_fminf(__builtin_fmaxf(f, a.lo), a.hi);
+          const float fl = __builtin_floorf(f);
+          f = floor_col ? fl : f;
+          o = __builtin_amdgcn_cvt_pk_u8_f32(f, j, o);
+        }
       }
-    } else {
-      reinterpret_cast<uint4 *>(a.out)[cell] = make_uint4(o[0], o[1], o[2], o[3]);
+      reinterpret_cast<unsigned *>(a.out)[cell * 4 + q] = o;
     }
   }
 }
+
+namespace {
+template <int RB>
+void launch_rb(const DepthwiseArgs &a, int mode, dim3 grid, hipStream_t s)
+{
+  if (mode == 2) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 2>), grid, dim3(kBlock), 0, s, a);
+  else if (mode == 1) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 1>), grid, dim3(kBlock), 0, s, a);
+  else hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 0>), grid, dim3(kBlock), 0, s, a);
+}
+}  // namespace
 
 hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s)
 {
   // four rows per lane on tall planes, fewer where that would leave lanes idle
   const int rb = a.oh >= 16 ? 4 : (a.oh >= 7 ? 2 : 1);
   const int ohb = (a.oh + rb - 1) / rb;
-  const long long total = (long long)a.n * a.g2 * ohb * a.ow;
+  const long long total = (long long)a.n * a.g2 * ohb * ((a.ow + 1) / 2) * 4;
+  int mode = 0;
+  if (a.out_type == EHIP_U8 && a.with_relu && a.lo >= 0.0f && a.hi <= 255.0f && a.hi >= a.lo)
+    mode = (a.lo == 0.0f && a.hi == 255.0f) ? 2 : 1;
   dim3 grid((unsigned)((total + kBlock - 1) / kBlock));
-  if (rb == 4) hipLaunchKernelGGL(k_depthwise3x3_u8s8<4>, grid, dim3(kBlock), 0, s, a);
-  else if (rb == 2) hipLaunchKernelGGL(k_depthwise3x3_u8s8<2>, grid, dim3(kBlock), 0, s, a);
-  else hipLaunchKernelGGL(k_depthwise3x3_u8s8<1>, grid, dim3(kBlock), 0, s, a);
+  if (rb == 4) launch_rb<4>(a, mode, grid, s);
+  else if (rb == 2) launch_rb<2>(a, mode, grid, s);
+  else launch_rb<1>(a, mode, grid, s);
   return hipGetLastError();
 }
 

@@ -65,9 +65,10 @@ struct Conv3x3Args {
 
 struct DepthwiseArgs {
   const uint8_t *in;    // [n][g2][ih][iw][16]
-  const int8_t *w;      // [g2][9][16]
+  const int8_t *w;      // [g2][kh = 3][16 channels][kw0 kw1 kw2 0]
   void *out;            // [n][g2][oh][ow][16]
   const float *scale, *shift;  // [G]
+  const int *wsum;      // [G] sum of the packed weights per channel
   int n, g2, ih, iw, oh, ow, pad_t, pad_l;
   int T, Tr, wt;        // width blocking of the reference kernel (decides floor vs round per column)
   int out_type, with_relu;
@@ -250,13 +251,13 @@ __device__ __forceinline__ unsigned quant4(const Epilogue &ep, int a0, int a1, i
   }
   if (FAST) {
     // ReLU with a lower bound >= 0: every value is in [0, hi], so "round to nearest even, then
-    // saturate" is a clamp to the code range, a round and one pack-with-saturation instruction
-    // per byte (its input is already an integer, so its own rounding is moot)
+    // saturate" is a clamp to the code range and one v_cvt_pk_u8_f32 per byte, which rounds to
+    // nearest even (the wave's float mode, never changed here) and saturates to 0..255 itself
     const float hi = OUT == EHIP_S8 ? __builtin_fminf(ep.hi, 127.0f) : ep.hi;
-    f0 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f0, ep.lo), hi));
-    f1 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f1, ep.lo), hi));
-    f2 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f2, ep.lo), hi));
-    f3 = __builtin_rintf(__builtin_fminf(__builtin_fmaxf(f3, ep.lo), hi));
+    f0 = __builtin_fminf(__builtin_fmaxf(f0, ep.lo), hi);
+    f1 = __builtin_fminf(__builtin_fmaxf(f1, ep.lo), hi);
+    f2 = __builtin_fminf(__builtin_fmaxf(f2, ep.lo), hi);
+    f3 = __builtin_fminf(__builtin_fmaxf(f3, ep.lo), hi);
     unsigned q = __builtin_amdgcn_cvt_pk_u8_f32(f0, 0, 0);
     q = __builtin_amdgcn_cvt_pk_u8_f32(f1, 1, q);
     q = __builtin_amdgcn_cvt_pk_u8_f32(f2, 2, q);

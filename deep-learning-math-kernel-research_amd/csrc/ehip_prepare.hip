@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kBlock) void k_fold_direct(const unsigned *wpacked,
   shift[oc] = sh;
 }
 
-// depthwise: one thread per channel; w is goihw f32 [g][3][3]; packed [g2][9][16]
+// depthwise: one thread per channel; w is goihw f32 [g][3][3]; packed [g2][kh][16][kw0 kw1 kw2 0]
 __global__ __launch_bounds__(kBlock) void k_prepare_depthwise(const float *w, const float *bias, int g, int G,
                                                               FoldParams p, int8_t *wpacked, float *scale,
                                                               float *shift, int *wsum)
@@ -157,9 +157,10 @@ __global__ __launch_bounds__(kBlock) void k_prepare_depthwise(const float *w, co
   int s = 0;
   for (int k = 0; k < 9; ++k) {
     const int q = c < g ? quant_w(w[(size_t)c * 9 + k], am) : 0;
-    wpacked[((size_t)(c >> 4) * 9 + k) * 16 + (c & 15)] = (int8_t)q;
+    wpacked[(((size_t)(c >> 4) * 3 + k / 3) * 16 + (c & 15)) * 4 + k % 3] = (int8_t)q;
     s += q;
   }
+  for (int kh = 0; kh < 3; ++kh) wpacked[(((size_t)(c >> 4) * 3 + kh) * 16 + (c & 15)) * 4 + 3] = 0;
   wsum[c] = s;
   float sc = 0.0f, sh = 0.0f;
   if (c < g) fold(p, am, (float)s, p.with_bias ? bias[c] : 0.0f, &sc, &sh);

@@ -84,7 +84,13 @@ class Layer:
         p = self.p
         if self.depthwise:
             wq, scale, shift, wsum = ol.depthwise_prepare(p, self.wb, self.bias)
-            out, acc = ol.depthwise_execute(p, self.xb, wq, scale, shift)
+            if p.out_type == ol.S32:
+                q = ol.ConvParams.from_buffer_copy(p)
+                q.out_type = ol.U8
+                _, acc = ol.depthwise_execute(q, self.xb, wq, scale, shift)
+                out = acc
+            else:
+                out, acc = ol.depthwise_execute(p, self.xb, wq, scale, shift)
         else:
             wq, scale, shift, wsum = ol.direct_prepare(p, self.wb, self.bias)
             if p.out_type == ol.S32:

@@ -98,6 +98,18 @@ def test_depthwise(out_type, g, hw, T):
                           T=T))
 
 
+@pytest.mark.parametrize("relu_hi,with_relu", [(200.0, True), (ol.FLT_MAX, True), (255.0, False)])
+def test_depthwise_u8_other_bounds(relu_hi, with_relu):
+    # bounds other than [0, 255] leave the one-instruction narrowing and take the general epilogue
+    run_and_compare(Layer(2, 48, 48, 14, k=3, pad=1, out_type=ol.U8, depthwise=True, seed=17, w_sigma=0.1, T=7,
+                          relu_hi=relu_hi, with_relu=with_relu))
+
+
+def test_depthwise_odd_width_and_raw_sums():
+    run_and_compare(Layer(1, 32, 32, 13, k=3, pad=1, out_type=ol.S32, depthwise=True, seed=23, w_sigma=0.1, T=13))
+    run_and_compare(Layer(2, 16, 16, 11, k=3, pad=0, out_type=ol.U8, depthwise=True, seed=29, w_sigma=0.1, T=3))
+
+
 # ---- input quantizer and reorders ---------------------------------------------------------------------
 def test_quantize_input_u8():
     import torch
