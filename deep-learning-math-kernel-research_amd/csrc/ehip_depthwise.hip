@@ -38,18 +38,16 @@ __device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel)
 template <int RB, int MODE>
 __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 {
-  const int ohb = (a.oh + RB - 1) / RB;
+  // grid: x = blocks over one plane's lanes (q fastest, then column pair, then row block),
+  // y = 16-channel block, z = image
   const int wp = (a.ow + 1) >> 1;
-  const long long total = (long long)a.n * a.g2 * ohb * wp * 4;
-  const long long idx = (long long)blockIdx.x * kBlock + threadIdx.x;
-  if (idx >= total) return;
-  const int q = (int)(idx & 3);
-  long long rest = idx >> 2;
-  const int p = (int)(rest % wp);
-  rest /= wp;
-  const int hb = (int)(rest % ohb);
-  const long long ng = rest / ohb;  // n * g2 + g2 index
-  const int g2 = (int)(ng % a.g2);
+  const int local = blockIdx.x * blockDim.x + threadIdx.x;
+  if (local >= a.lanes_per_plane) return;
+  const int q = local & 3;
+  const int hb = fastdiv(local >> 2, wp, a.wp_magic);
+  const int p = (local >> 2) - hb * wp;
+  const int g2 = blockIdx.y;
+  const unsigned ng = blockIdx.z * a.g2 + g2;
   const int oh0 = hb * RB;
   const int c0 = 2 * p;
   const int ch0 = g2 * 16 + 4 * q;  // first of the lane's 4 channels
@@ -73,26 +71,29 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
       acc[r][c][0] = 128 * ws.x; acc[r][c][1] = 128 * ws.y; acc[r][c][2] = 128 * ws.z; acc[r][c][3] = 128 * ws.w;
     }
 
-  // the 4 input columns of this lane (clamped; invalid ones are replaced after the load)
-  int colv[4];
+  // the 4 input columns of this lane (clamped; invalid ones are replaced after the load); all
+  // addresses are 32-bit byte offsets from the tensor base (the launcher checks the size)
+  unsigned coloff[4];
   bool colok[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int iw = c0 - a.pad_l + k;
     colok[k] = iw >= 0 && iw < a.iw;
-    colv[k] = iw < 0 ? 0 : (iw >= a.iw ? a.iw - 1 : iw);
+    coloff[k] = (unsigned)(iw < 0 ? 0 : (iw >= a.iw ? a.iw - 1 : iw)) * 16u;
   }
-  const unsigned *plane = reinterpret_cast<const unsigned *>(a.in) + (size_t)ng * a.ih * a.iw * 4 + q;
+  const unsigned plane_off = ng * (unsigned)(a.ih * a.iw) * 16u + 4u * q;
+  const char *in_base = reinterpret_cast<const char *>(a.in);
 
 #pragma unroll
   for (int hr = 0; hr < RB + 2; ++hr) {
     const int ih = oh0 - a.pad_t + hr;
     const bool rowok = ih >= 0 && ih < a.ih;
     const int ihc = ih < 0 ? 0 : (ih >= a.ih ? a.ih - 1 : ih);
+    const unsigned row_off = plane_off + (unsigned)(ihc * a.iw) * 16u;
     unsigned x[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const unsigned v = plane[((size_t)ihc * a.iw + colv[k]) * 4];
+      const unsigned v = *reinterpret_cast<const unsigned *>(in_base + (size_t)(row_off + coloff[k]));
       x[k] = (rowok && colok[k]) ? v ^ 0x80808080u : 0x80808080u;
     }
     // 4 pixels x 4 channels -> 4 channels x 4 pixels
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
     const int ow = c0 + c;
     if (ow >= a.ow) break;
     // width-block rule for this column
-    const int blk = ow / a.T;
+    const int blk = fastdiv(ow, a.T, a.T_magic);
     const int tpos = ow - blk * a.T;
     const int Tz = blk == a.wt - 1 ? a.Tr : a.T;
     const bool floor_col = a.out_type == EHIP_U8 && tpos < 4 * (Tz / 4);
@@ -133,9 +134,9 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
     for (int r = 0; r < RB; ++r) {
       const int oh = oh0 + r;
       if (oh >= a.oh) break;
-      const size_t cell = ((size_t)ng * a.oh + oh) * a.ow + ow;
+      const unsigned cell = (ng * (unsigned)a.oh + oh) * (unsigned)a.ow + ow;   // < 2^28, checked by the launcher
       if (MODE == 0 && a.out_type == EHIP_S32) {
-        reinterpret_cast<v4i *>(a.out)[cell * 4 + q] = v4i{acc[r][c][0], acc[r][c][1], acc[r][c][2], acc[r][c][3]};
+        reinterpret_cast<v4i *>(a.out)[(size_t)cell * 4 + q] = v4i{acc[r][c][0], acc[r][c][1], acc[r][c][2], acc[r][c][3]};
         continue;
       }
       unsigned o = 0u;
@@ -161,34 +162,44 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
           o = __builtin_amdgcn_cvt_pk_u8_f32(f, j, o);
         }
       }
-      reinterpret_cast<unsigned *>(a.out)[cell * 4 + q] = o;
+      *reinterpret_cast<unsigned *>(static_cast<char *>(a.out) + (size_t)(cell * 16u + 4u * q)) = o;
     }
   }
 }
 
 namespace {
 template <int RB>
-void launch_rb(const DepthwiseArgs &a, int mode, dim3 grid, hipStream_t s)
+void launch_rb(const DepthwiseArgs &a, int mode, dim3 grid, dim3 block, hipStream_t s)
 {
-  if (mode == 2) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 2>), grid, dim3(kBlock), 0, s, a);
-  else if (mode == 1) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 1>), grid, dim3(kBlock), 0, s, a);
-  else hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 0>), grid, dim3(kBlock), 0, s, a);
+  if (mode == 2) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 2>), grid, block, 0, s, a);
+  else if (mode == 1) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 1>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 0>), grid, block, 0, s, a);
 }
 }  // namespace
 
-hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s)
+hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s)
 {
+  DepthwiseArgs a = a0;
   // four rows per lane on tall planes, fewer where that would leave lanes idle
   const int rb = a.oh >= 16 ? 4 : (a.oh >= 7 ? 2 : 1);
   const int ohb = (a.oh + rb - 1) / rb;
-  const long long total = (long long)a.n * a.g2 * ohb * ((a.ow + 1) / 2) * 4;
+  const int wp = (a.ow + 1) / 2;
+  a.lanes_per_plane = ohb * wp * 4;
+  a.wp_magic = div_magic(wp);
+  a.T_magic = div_magic(a.T);
+  // 32-bit byte offsets inside the kernel
+  if ((long long)a.n * a.g2 * a.ih * a.iw * 16 >= (1ll << 32) || (long long)a.n * a.g2 * a.oh * a.ow * 16 >= (1ll << 32)) {
+    set_error("depthwise: tensors of 4 GiB and more are not supported");
+    return hipErrorInvalidValue;
+  }
   int mode = 0;
   if (a.out_type == EHIP_U8 && a.with_relu && a.lo >= 0.0f && a.hi <= 255.0f && a.hi >= a.lo)
     mode = (a.lo == 0.0f && a.hi == 255.0f) ? 2 : 1;
-  dim3 grid((unsigned)((total + kBlock - 1) / kBlock));
-  if (rb == 4) launch_rb<4>(a, mode, grid, s);
-  else if (rb == 2) launch_rb<2>(a, mode, grid, s);
-  else launch_rb<1>(a, mode, grid, s);
+  const int block = a.lanes_per_plane >= kBlock ? kBlock : up(a.lanes_per_plane, kWave);
+  dim3 grid((a.lanes_per_plane + block - 1) / block, a.g2, a.n);
+  if (rb == 4) launch_rb<4>(a, mode, grid, dim3(block), s);
+  else if (rb == 2) launch_rb<2>(a, mode, grid, dim3(block), s);
+  else launch_rb<1>(a, mode, grid, dim3(block), s);
   return hipGetLastError();
 }
 

@@ -71,6 +71,8 @@ struct DepthwiseArgs {
   const int *wsum;      // [G] sum of the packed weights per channel
   int n, g2, ih, iw, oh, ow, pad_t, pad_l;
   int T, Tr, wt;        // width blocking of the reference kernel (decides floor vs round per column)
+  int lanes_per_plane;  // set by the launcher: row blocks x column pairs x 4
+  unsigned wp_magic, T_magic;  // div_magic of the column pairs per row and of T
   int out_type, with_relu;
   float lo, hi;
 };

@@ -1,0 +1,283 @@
+"""Golden cases for the CPU oracle: seeded inputs of the reference's micro-kernel templates and the
+way the oracle evaluates the same case.  make_golden.py runs the COMPILED reference templates
+(oracle/_ref, built from /root/reference by oracle/Makefile) on these inputs and stores inputs +
+reference outputs as .npz; tests/test_golden.py replays the stored inputs through the oracle and
+compares bit for bit -- without needing the reference tree or its build.
+"""
+import ctypes
+
+import numpy as np
+
+import oracle_lib as ol
+
+AT_RELU, AT_SUM, AT_CLEAR, AT_RESTORE = 1 << 1, 1 << 2, 1 << 3, 1 << 5
+KIND_ID = {ol.F32: 0, ol.U8: 1, ol.S8: 2}
+
+
+def _al(a):
+    b = ol.aligned(a.shape, a.dtype)
+    b[...] = a
+    return b
+
+
+def _epi(kind, acc, scale, shift, with_sum, old, sum_s, relu, lo, hi):
+    f = ctypes.c_float()
+    q = ol.oracle().orc_epilogue(kind, int(acc), float(scale), float(shift), int(with_sum), int(old), float(sum_s),
+                                 int(relu), float(lo), float(hi), ctypes.byref(f))
+    return f.value if kind == ol.F32 else q
+
+
+# ---- u8s8 GEMM micro-kernel + epilogue (src/kernel/elk_u8s8_gemm.hxx) ---------------------------
+def gemm_inputs(kind, O, T, with_sum, seed):
+    rng = np.random.default_rng(seed)
+    I2 = 5
+    np_kind = ol.NP_OF[kind]
+    d = dict(kind=np.int32(kind), O=np.int32(O), T=np.int32(T), I2=np.int32(I2), with_sum=np.int32(with_sum),
+             x=rng.integers(0, 256, (I2, T, 16)).astype(np.uint8),
+             w=rng.integers(-127, 128, (I2, 4, O, 16, 4)).astype(np.int8),
+             scale=rng.uniform(1e-4, 3e-3, (O, 16)).astype(np.float32),
+             shift=rng.normal(0, 20, (O, 16)).astype(np.float32),
+             sum_s=np.float32(0.37109375 if with_sum else 0.0),
+             lo=np.float32(0.0 if kind == ol.U8 else -60.0), hi=np.float32(200.0 if kind == ol.U8 else 90.0))
+    if kind == ol.F32:
+        d["old"] = np.zeros((O, T, 16), np.float32)
+    else:
+        d["old"] = (rng.integers(0, 256, (O, T, 16)) if kind == ol.U8 else rng.integers(-128, 128, (O, T, 16))).astype(np_kind)
+    return d
+
+
+def gemm_reference(d, ref):
+    kind, O, T, I2 = int(d["kind"]), int(d["O"]), int(d["T"]), int(d["I2"])
+    tout = ol.aligned((O, T, 16), np.float32)
+    oout = _al(d["old"])
+    attr = AT_CLEAR | AT_RESTORE | AT_RELU | (AT_SUM if int(d["with_sum"]) else 0)
+    x, w, sc, sh = _al(d["x"]), _al(d["w"]), _al(d["scale"]), _al(d["shift"])   # keep the buffers alive
+    rc = ref.ref_u8s8_gemm(KIND_ID[kind], O, T, I2, attr, float(d["lo"]), float(d["hi"]), float(d["sum_s"]),
+                           ol.ptr(tout), ol.ptr(oout), ol.ptr(x), ol.ptr(w), ol.ptr(sc), ol.ptr(sh))
+    assert rc == 0
+    return np.array(tout if kind == ol.F32 else oout)
+
+
+def gemm_oracle(d):
+    kind, O, T, I2 = int(d["kind"]), int(d["O"]), int(d["T"]), int(d["I2"])
+    acc = np.einsum("itvk,ivock->otc", d["x"].reshape(I2, T, 4, 4).astype(np.int64), d["w"].astype(np.int64))
+    out = np.zeros((O, T, 16), ol.NP_OF[kind])
+    for o in range(O):
+        for t in range(T):
+            for c in range(16):
+                out[o, t, c] = _epi(kind, acc[o, t, c], d["scale"][o, c], d["shift"][o, c], int(d["with_sum"]),
+                                    d["old"][o, t, c] if kind != ol.F32 else 0, d["sum_s"], True, d["lo"], d["hi"])
+    return out
+
+
+# ---- depthwise micro-kernel (src/kernel/elk_u8s8_depthwise_conv.hxx) ------------------------------
+def dw_inputs(T, ow, ih, kind, seed, relu_hi):
+    rng = np.random.default_rng(seed)
+    G2 = 2
+    return dict(T=np.int32(T), ow=np.int32(ow), ih=np.int32(ih), kind=np.int32(kind), relu_hi=np.float32(relu_hi),
+                x=rng.integers(0, 256, (1, G2, ih, ow, 16)).astype(np.uint8),
+                w=rng.normal(0, 0.1, (32, 3, 3)).astype(np.float32),
+                bias=rng.normal(0, 0.5, 32).astype(np.float32))
+
+
+def _dw_params(d):
+    return ol.make_params(1, 32, 32, int(d["ih"]), int(d["ow"]), 3, 3, pad=1, g=32, out_type=int(d["kind"]),
+                          T=int(d["T"]), out_scale=6.0 / 255.0, relu_hi=float(d["relu_hi"]))
+
+
+def dw_oracle(d):
+    p = _dw_params(d)
+    wq, scale, shift, _ = ol.depthwise_prepare(p, d["w"], d["bias"])
+    out, _ = ol.depthwise_execute(p, d["x"], wq, scale, shift)
+    return out.reshape(2, int(d["ih"]) * int(d["ow"]), 16)
+
+
+def dw_reference(d, ref):
+    """The reference micro-kernel gets the ORACLE's quantized weights / folded scale and shift (the
+    weight side is pinned separately by closed forms): this pins contraction, borders and the
+    floor-vs-round store rule."""
+    p = _dw_params(d)
+    G2, ih, iw, oh, ow, T, kind = 2, int(d["ih"]), int(d["ow"]), int(d["ih"]), int(d["ow"]), int(d["T"]), int(d["kind"])
+    wq, scale, shift, _ = ol.depthwise_prepare(p, d["w"], d["bias"])
+    xb = ol.aligned(d["x"].size + 256, np.uint8)
+    xb[:d["x"].size] = d["x"].ravel()
+    wr = ol.aligned((G2, 3, 16, 4), np.int8)
+    wr[...] = 0
+    wr[:, :, :, :3] = wq.reshape(G2, 16, 3, 3).transpose(0, 2, 1, 3)
+    sc, sh = _al(scale.reshape(G2, 16)), _al(shift.reshape(G2, 16))
+    got = ol.aligned((G2, oh * ow, 16), ol.NP_OF[kind])
+    wt = (ow + T - 1) // T
+    Tr = ow % T or T
+    for ht in range(oh):
+        for _wt in range(wt):
+            Tz = Tr if _wt == wt - 1 else T
+            rc = ref.ref_u8s8_depthwise(KIND_ID[kind], T, Tz, G2, ih, iw, oh, ow, ht, _wt, 1, 1, 1, 1, 0.0,
+                                        float(d["relu_hi"]), ol.ptr(got), ol.ptr(xb), ol.ptr(wr), ol.ptr(sc), ol.ptr(sh))
+            assert rc == 0
+    return np.array(got)
+
+
+# ---- 3x3 micro-kernel (src/kernel/elk_u8s8_conv.hxx) --------------------------------------------
+def conv_inputs(kind, T, ow, seed):
+    rng = np.random.default_rng(seed)
+    I2, ih = 2, 5
+    return dict(kind=np.int32(kind), T=np.int32(T), ow=np.int32(ow),
+                x=rng.integers(0, 256, (1, I2, ih, ow, 16)).astype(np.uint8),
+                w=rng.normal(0, 0.05, (16, 16 * I2, 3, 3)).astype(np.float32),
+                bias=rng.normal(0, 0.3, 16).astype(np.float32))
+
+
+def _conv_params(d):
+    return ol.make_params(1, 32, 16, 5, int(d["ow"]), 3, 3, pad=1, out_type=int(d["kind"]), out_scale=0.02,
+                          relu_hi=ol.FLT_MAX)
+
+
+def conv_oracle(d):
+    p = _conv_params(d)
+    wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(d["w"]), d["bias"])
+    out, _ = ol.direct_execute(p, d["x"], wq, scale, shift)
+    return out.reshape(5 * int(d["ow"]), 16)
+
+
+def conv_reference(d, ref):
+    p = _conv_params(d)
+    kind, T, ow, I2, ih, oh = int(d["kind"]), int(d["T"]), int(d["ow"]), 2, 5, 5
+    wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(d["w"]), d["bias"])
+    xb = ol.aligned(d["x"].size + 256, np.uint8)
+    xb[:d["x"].size] = d["x"].ravel()
+    wr = ol.aligned((3, 3, I2, 4, 16, 4), np.int8)
+    wr[...] = wq.reshape(16, I2, 4, 4, 3, 3).transpose(4, 5, 1, 2, 0, 3)
+    sc = _al(scale[:16])
+    sh = ol.aligned((T, 16), np.float32)
+    sh[...] = shift[None, :16]
+    tout = ol.aligned((oh * ow, 16), np.float32)
+    rout = ol.aligned((oh * ow, 16), ol.NP_OF[kind])
+    for ht in range(oh):
+        for _wt in range(ow // T):
+            rc = ref.ref_u8s8_conv3x3(KIND_ID[kind], T, I2, ih, ow, oh, ow, ht, _wt, 1, 1, 0.0, ol.FLT_MAX, ol.ptr(tout),
+                                      ol.ptr(rout) if kind != ol.F32 else None, ol.ptr(xb), ol.ptr(wr), ol.ptr(sc),
+                                      ol.ptr(sh))
+            assert rc == 0
+    return np.array(tout if kind == ol.F32 else rout)
+
+
+# ---- Winograd F(4x4,3x3) tile transforms (src/kernel/elk_conv_wino_4x4_3x3_*.hxx) ----------------
+def wino_w_inputs(seed):
+    return dict(w=np.random.default_rng(seed).normal(0, 0.05, (3, 3, 16, 16)).astype(np.float32))
+
+
+def wino_w_reference(d, ref):
+    tw = ol.aligned((6, 6, 16, 16), np.float32)
+    w = _al(d["w"])
+    ref.ref_wino_trans_weights(ol.ptr(tw), ol.ptr(w))
+    return np.array(tw)
+
+
+def wino_w_oracle(d):
+    out = np.zeros((6, 6, 16, 16), np.float32)
+    u = np.zeros(36, np.float32)
+    for i in range(16):
+        for o in range(16):
+            g = np.ascontiguousarray(d["w"][:, :, i, o].ravel())
+            ol.oracle().orc_wino_tile_weights(ol.ptr(g), ol.ptr(u))
+            out[:, :, i, o] = u.reshape(6, 6)
+    return out
+
+
+def wino_in_inputs(h0, w0, seed):
+    return dict(h0=np.int32(h0), w0=np.int32(w0),
+                plane=np.random.default_rng(seed).uniform(0, 1, (12, 12, 16)).astype(np.float32))
+
+
+def _wino_in_range(d):
+    ih = iw = 12
+    h0, w0 = int(d["h0"]), int(d["w0"])
+    hs, he = max(0, -h0), min(5, ih - 1 - h0)
+    ws, we = max(0, -w0), min(5, iw - 1 - w0)
+    return h0, w0, hs, he, ws, we, not (hs == 0 and ws == 0 and he == 5 and we == 5)
+
+
+def wino_in_reference(d, ref):
+    h0, w0, hs, he, ws, we, border = _wino_in_range(d)
+    plane = _al(d["plane"])
+    tin = ol.aligned((6, 6, 16), np.float32)
+    tile_ptr = ctypes.c_void_p(plane.ctypes.data + (h0 * 12 + w0) * 16 * 4)
+    ref.ref_wino_trans_input(int(border), 12, 12, ol.ptr(tin), tile_ptr, hs, he, ws, we)
+    return np.array(tin)
+
+
+def wino_in_oracle(d):
+    h0, w0, hs, he, ws, we, border = _wino_in_range(d)
+    out = np.zeros((6, 6, 16), np.float32)
+    v = np.zeros(36, np.float32)
+    for c in range(16):
+        t = np.zeros((6, 6), np.float32)
+        for i in range(6):
+            for j in range(6):
+                h, w = h0 + i, w0 + j
+                if 0 <= h < 12 and 0 <= w < 12:
+                    t[i, j] = d["plane"][h, w, c]
+        fn = ol.oracle().orc_wino_tile_input_border if border else ol.oracle().orc_wino_tile_input
+        fn(ol.ptr(t), ol.ptr(v))
+        out[:, :, c] = v.reshape(6, 6)
+    return out
+
+
+def wino_out_inputs(with_bias, with_relu, h_end, w_end, seed):
+    rng = np.random.default_rng(seed)
+    return dict(with_bias=np.int32(with_bias), with_relu=np.int32(with_relu), h_end=np.int32(h_end), w_end=np.int32(w_end),
+                m=rng.normal(0, 3, (6, 6, 16)).astype(np.float32), bias=rng.normal(0, 1, 16).astype(np.float32))
+
+
+def wino_out_reference(d, ref):
+    out = ol.aligned((8, 8, 16), np.float32, -777.0)
+    h_end, w_end = int(d["h_end"]), int(d["w_end"])
+    border = not (h_end == 3 and w_end == 3)
+    m, bias = _al(d["m"]), _al(d["bias"])
+    ref.ref_wino_trans_output(int(border), int(d["with_bias"]), int(d["with_relu"]), 8, 8, ol.ptr(out), ol.ptr(m),
+                              ol.ptr(bias), h_end, w_end)
+    return np.array(out[:4, :4, :])
+
+
+def wino_out_oracle(d):
+    out = np.full((4, 4, 16), -777.0, np.float32)
+    y = np.zeros(16, np.float32)
+    for c in range(16):
+        mm = np.ascontiguousarray(d["m"][:, :, c].ravel())
+        ol.oracle().orc_wino_tile_output(ol.ptr(mm), ol.ptr(y))
+        for i in range(4):
+            for j in range(4):
+                if i > int(d["h_end"]) or j > int(d["w_end"]):
+                    continue
+                r = y[4 * i + j]
+                if int(d["with_bias"]):
+                    r = np.float32(r + d["bias"][c])
+                if int(d["with_relu"]):
+                    r = r if r > 0 else np.float32(0)
+                out[i, j, c] = r
+    return out
+
+
+# name -> (inputs, reference runner, oracle runner)
+CASES = {}
+for _k, _kn in ((ol.F32, "f32"), (ol.U8, "u8"), (ol.S8, "s8")):
+    for _sum in (0, 1):
+        if _k == ol.F32 and _sum:
+            continue  # the reference has no sum fusion for f32 output (elk_u8s8_gemm.hxx:234-236)
+        CASES["gemm_%s_sum%d" % (_kn, _sum)] = (lambda k=_k, s=_sum: gemm_inputs(k, 2, 6, s, 7 + k + 10 * s),
+                                                gemm_reference, gemm_oracle)
+for _T, _ow, _ih in ((14, 56, 5), (7, 7, 7), (11, 28, 3), (7, 21, 3)):
+    CASES["depthwise_u8_T%d_w%d" % (_T, _ow)] = (lambda T=_T, ow=_ow, ih=_ih: dw_inputs(T, ow, ih, ol.U8, 100 + T + ow, 255.0),
+                                                 dw_reference, dw_oracle)
+CASES["depthwise_s8_T14_w28"] = (lambda: dw_inputs(14, 28, 4, ol.S8, 5, 127.0), dw_reference, dw_oracle)
+for _k, _kn, _T, _ow in ((ol.U8, "u8", 14, 28), (ol.S8, "s8", 7, 14), (ol.F32, "f32", 7, 7)):
+    CASES["conv3x3_%s_T%d_w%d" % (_kn, _T, _ow)] = (lambda k=_k, T=_T, ow=_ow: conv_inputs(k, T, ow, 3 * T + ow + k),
+                                                    conv_reference, conv_oracle)
+CASES["wino_weights"] = (lambda: wino_w_inputs(21), wino_w_reference, wino_w_oracle)
+for _h0, _w0 in ((2, 3), (-1, -1), (-1, 4), (3, -1), (7, 7), (7, 2), (-1, 7)):
+    CASES["wino_input_h%d_w%d" % (_h0, _w0)] = (lambda h=_h0, w=_w0: wino_in_inputs(h, w, h * 13 + w + 50),
+                                                wino_in_reference, wino_in_oracle)
+for _b, _r, _he, _we in ((1, 1, 3, 3), (1, 0, 1, 3), (0, 0, 3, 0), (1, 1, 2, 2)):
+    CASES["wino_output_b%d_r%d_h%d_w%d" % (_b, _r, _he, _we)] = (
+        lambda b=_b, r=_r, he=_he, we=_we: wino_out_inputs(b, r, he, we, 77 + he * 4 + we), wino_out_reference,
+        wino_out_oracle)
