@@ -47,6 +47,7 @@ struct ehip_conv {
   int T = 1, Tr = 1, wtb = 1;
   // Winograd
   int ht = 0, wt = 0, nt = 0, t = 0;
+  int chunk_n = 0;   // images per pass of the three-stage pipeline (intermediates sized for it)
   uint8_t *tin = nullptr;
   float *tout = nullptr;
   size_t tin_bytes = 0, tout_bytes = 0;
@@ -237,7 +238,19 @@ int setup_workspace(ehip_conv *c)
     c->ht = (d.oh + 3) / 4;
     c->wt = (d.ow + 3) / 4;
     c->nt = c->ht * c->wt;
-    c->t = c->nt * d.n;
+    // The three stages can run over a few images at a time (EHIP_WINO_CHUNK) with the intermediates
+    // sized for one pass; measured on MI355X this only costs (the 256 MB memory-side cache does not
+    // keep the f32 GEMM result away from HBM), so one pass over the whole batch is the default.
+    {
+      long long cn = d.n;
+      const char *env = getenv("EHIP_WINO_CHUNK");
+      if (env && env[0]) cn = atoi(env);
+      if (cn < 1) cn = 1;
+      if (cn > d.n) cn = d.n;
+      c->chunk_n = (int)cn;
+    }
+    c->t = c->nt * c->chunk_n;   // tiles per pass
+    if ((long long)c->t >= (1ll << 31) / 64) return fail(EHIP_UNIMPLEMENTED, "winograd: too many tiles");
     c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, 36);
     c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
     c->kernel_name = std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output_f32";
@@ -435,34 +448,38 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     break;
   }
   case FAM_WINOGRAD: {
-    WinoArgs w = make_wino_args(d, c->ic2, c->oc2);
-    w.in = static_cast<const float *>(input_dev);
-    w.tin = c->tin;
-    w.tout = c->tout;
-    w.out = static_cast<float *>(output_dev);
-    w.bias = static_cast<const float *>(bias_dev);
     if (d.with_bias && !bias_dev) return fail(EHIP_GENERAL_ERROR, "Parameter error. Invalid input data!");
-    // mrepS = input_S * (1 / tinput_S), z = ceil(tinput_z)
-    // (src/elx_conv_wino_trans_input.cpp:617-618, src/elx_int8_conv_wino.cpp:270-276)
-    const float tin_repS = 1.0f / d.tinput_scale;
-    w.mrepS = d.input_scale * tin_repS;
-    w.mz = ceilf(d.tinput_z);
-    HIP_TRY(launch_wino_trans_input(w, s));
-    GemmArgs a;
-    memset(&a, 0, sizeof(a));
-    a.in = c->tin;
-    a.w = c->wpacked;
-    a.out = c->tout;
-    a.ep = make_epilogue(c, EHIP_F32, false, false);
-    a.p_total = c->t;
-    a.ohw = c->t; a.ow = c->t; a.ihw = c->t; a.iw = c->t;
-    a.ohw_magic = div_magic(a.ohw); a.ow_magic = div_magic(a.ow);
-    a.stride_h = 1; a.stride_w = 1;
-    a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
-    a.in_batch_stride = (long long)c->ic2 * c->t * 16;
-    a.out_batch_stride = (long long)c->oc2 * c->t * 16;
-    HIP_TRY(launch_gemm(a, 36, c->variant, s));
-    HIP_TRY(launch_wino_trans_output(w, s));
+    for (int n0 = 0; n0 < d.n; n0 += c->chunk_n) {
+      ehip_conv_desc_t dc = d;
+      dc.n = d.n - n0 < c->chunk_n ? d.n - n0 : c->chunk_n;
+      WinoArgs w = make_wino_args(dc, c->ic2, c->oc2);
+      w.in = static_cast<const float *>(input_dev) + (size_t)n0 * c->ic2 * d.ih * d.iw * 16;
+      w.tin = c->tin;
+      w.tout = c->tout;
+      w.out = static_cast<float *>(output_dev) + (size_t)n0 * c->oc2 * d.oh * d.ow * 16;
+      w.bias = static_cast<const float *>(bias_dev);
+      // mrepS = input_S * (1 / tinput_S), z = ceil(tinput_z)
+      // (src/elx_conv_wino_trans_input.cpp:617-618, src/elx_int8_conv_wino.cpp:270-276)
+      const float tin_repS = 1.0f / d.tinput_scale;
+      w.mrepS = d.input_scale * tin_repS;
+      w.mz = ceilf(d.tinput_z);
+      HIP_TRY(launch_wino_trans_input(w, s));
+      GemmArgs a;
+      memset(&a, 0, sizeof(a));
+      a.in = c->tin;
+      a.w = c->wpacked;
+      a.out = c->tout;
+      a.ep = make_epilogue(c, EHIP_F32, false, false);
+      a.p_total = w.t;
+      a.ohw = w.t; a.ow = w.t; a.ihw = w.t; a.iw = w.t;
+      a.ohw_magic = div_magic(a.ohw); a.ow_magic = div_magic(a.ow);
+      a.stride_h = 1; a.stride_w = 1;
+      a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
+      a.in_batch_stride = (long long)c->ic2 * w.t * 16;
+      a.out_batch_stride = (long long)c->oc2 * w.t * 16;
+      HIP_TRY(launch_gemm(a, 36, c->variant, s));
+      HIP_TRY(launch_wino_trans_output(w, s));
+    }
     break;
   }
   default:
@@ -532,11 +549,13 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
   }
   case EHIP_Q_TINPUT_U8:
     if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "not a Winograd handle");
+    if (c->chunk_n < d.n) return fail(EHIP_UNIMPLEMENTED, "the intermediates of a multi-pass layer hold its last pass only");
     if (!want(c->tin_bytes)) return EHIP_OK;
     HIP_TRY(hipMemcpy(host_dst, c->tin, c->tin_bytes, hipMemcpyDeviceToHost));
     return EHIP_OK;
   case EHIP_Q_TOUTPUT_F32:
     if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "not a Winograd handle");
+    if (c->chunk_n < d.n) return fail(EHIP_UNIMPLEMENTED, "the intermediates of a multi-pass layer hold its last pass only");
     if (!want(c->tout_bytes)) return EHIP_OK;
     HIP_TRY(hipMemcpy(host_dst, c->tout, c->tout_bytes, hipMemcpyDeviceToHost));
     return EHIP_OK;

@@ -193,7 +193,10 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
     pix[nt] = ((size_t)n * a.oc2 * ohw + (pvalid[nt] ? r * a.ow + c : 0)) * 16;
   }
   TRACE_POINT(14);
-  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, (int)cidx, pix, pvalid, oc_real, (size_t)ohw * 16, a.out);
+  const size_t pixT[TN][2] = {};
+  const bool validT[TN][2] = {};
+  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, (int)cidx, pix, pvalid, oc_real, (size_t)ohw * 16, a.out, nullptr, pixT,
+                        validT);
   TRACE_POINT(15);
 }
 

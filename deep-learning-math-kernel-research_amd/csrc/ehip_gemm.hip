@@ -30,7 +30,7 @@
 namespace ehip {
 
 template <int WM, int WN, int TM, int TN, int KC>
-__global__ __launch_bounds__(kBlock, (TM * TN >= 8 ? 1 : 2)) void k_gemm_u8s8(GemmArgs a)
+__global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 {
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
@@ -44,9 +44,11 @@ __global__ __launch_bounds__(kBlock, (TM * TN >= 8 ? 1 : 2)) void k_gemm_u8s8(Ge
   static_assert(KC % 2 == 0, "a k-step is two units");
   static_assert(A_CELLS % kBlock == 0 && B_CELLS % kBlock == 0, "whole passes of the workgroup");
   static_assert(kBlock % P_T == 0 && OC_T <= kOcTile, "tile limits");
+  static_assert(2 * (A_CELLS + B_CELLS) >= 4 * 256, "the epilogue borrows 256 LDS cells per wave");
 
-  __shared__ v4i lds_a[2][A_CELLS];      // [unit][row]
-  __shared__ v4i lds_b[2][B_CELLS];      // [unit][pixel]
+  __shared__ v4i lds[2 * (A_CELLS + B_CELLS)];
+  v4i(*lds_a)[A_CELLS] = reinterpret_cast<v4i(*)[A_CELLS]>(lds);                  // [buf][unit][row]
+  v4i(*lds_b)[B_CELLS] = reinterpret_cast<v4i(*)[B_CELLS]>(lds + 2 * A_CELLS);    // [buf][unit][pixel]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -158,23 +160,37 @@ __global__ __launch_bounds__(kBlock, (TM * TN >= 8 ? 1 : 2)) void k_gemm_u8s8(Ge
   store_stage(buf);
   __syncthreads();
   const long long cidx = (long long)b * a.ocpp + oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
+  // the epilogue's per-channel constants travel while the last fill is multiplied -- unless the
+  // accumulators leave no registers for them (the co-resident workgroup covers the wait then)
   OcConsts k0;
-  load_consts(k0, a.ep, cidx);
+  if (TM * TN < 8) load_consts(k0, a.ep, cidx);
   multiply(buf);
+  if (TM * TN >= 8) load_consts(k0, a.ep, cidx);
 
   // ---- epilogue ------------------------------------------------------------------------------
-  size_t pix[TN];
-  bool pvalid[TN];
-#pragma unroll
-  for (int nt = 0; nt < TN; ++nt) {
-    const int gp = pix0 + pw0 + nt * 32 + l32;
-    pvalid[nt] = gp < a.p_total;
-    const int gpc = pvalid[nt] ? gp : 0;
+  auto pixel_offset = [&](int gp, bool &valid) -> size_t {
+    valid = gp < a.p_total;
+    const int gpc = valid ? gp : 0;
     const int n = a.ohw == a.p_total ? 0 : fastdiv(gpc, a.ohw, a.ohw_magic);
     const int r = gpc - n * a.ohw;
-    pix[nt] = (size_t)b * a.out_batch_stride + ((size_t)n * a.oc2 * a.ohw + r) * 16;
+    return (size_t)b * a.out_batch_stride + ((size_t)n * a.oc2 * a.ohw + r) * 16;
+  };
+  size_t pix[TN], pixT[TN][2];
+  bool pvalid[TN], validT[TN][2];
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) {
+    pix[nt] = pixel_offset(pix0 + pw0 + nt * 32 + l32, pvalid[nt]);
+    pixT[nt][0] = pixel_offset(pix0 + pw0 + nt * 32 + (lane >> 2), validT[nt][0]);
+    pixT[nt][1] = pixel_offset(pix0 + pw0 + nt * 32 + (lane >> 2) + 16, validT[nt][1]);
   }
-  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real, (size_t)a.ohw * 16, a.out);
+  // 4-byte outputs are exchanged through a wave-private 4 KB patch of the (now idle) operand LDS
+  v4i *xlds = nullptr;
+  if (a.ep.out_type == EHIP_F32 || a.ep.out_type == EHIP_S32) {
+    __syncthreads();   // every wave has read its last operands
+    xlds = lds + wave * 256;
+  }
+  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real, (size_t)a.ohw * 16, a.out, xlds,
+                        pixT, validT);
 }
 
 namespace {
@@ -194,8 +210,6 @@ const Variant kVariants[] = {
     V(4, 1, 2, 1, 8),  // 4: 256 oc x  32 px
     V(2, 2, 1, 2, 8),  // 5:  64 oc x 128 px
     V(2, 2, 1, 1, 4),  // 6:  64 oc x  64 px, short K
-    V(2, 2, 2, 4, 4),  // 7: 128 oc x 256 px
-    V(4, 1, 2, 4, 4),  // 8: 256 oc x 128 px
 };
 #undef V
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);

@@ -184,10 +184,10 @@ __host__ __device__ __forceinline__ int oc_of_packed_row(int r)
 
 // ---- fused requantization epilogue of the MFMA kernels -----------------------------------------
 // A lane holds, for each of its TN pixels and TM 32-row tiles, 16 consecutive output channels: one
-// 16-byte cell of u8/s8 output, four float4 of f32/s32 output.  The per-channel constants of tile
-// mt+1 are requested before tile mt is processed, the sum operands of a tile are all requested
-// before the first is used, and the output type is a template parameter, so the epilogue is
-// straight-line code whose memory latencies overlap.
+// 16-byte cell of u8/s8 output, four float4 of f32/s32 output.  The per-channel constants of the
+// first tile are requested while the last k-steps run, the sum operands of a tile are all
+// requested before the first is used, and the output type is a template parameter, so the
+// epilogue is straight-line code whose memory latencies overlap.
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct OcConsts {      // of 16 consecutive output channels
@@ -278,18 +278,28 @@ __device__ __forceinline__ unsigned quant4(const Epilogue &ep, int a0, int a1, i
 // lane's channels in tile 0, cidx = their index in the per-channel arrays (tile mt: + 32 * mt),
 // oc_first = the lane's first channel in tile 0 (a multiple of 16), pix[nt] = element offset of
 // the pixel's cell in 16-channel block 0, block_stride = elements between 16-channel blocks.
-template <int TM, int TN, int OUT, bool SUM, bool FAST>
+//
+// 4-byte outputs (f32, s32) can go through a wave-private 4 KB LDS patch `xlds` (XPOSE): a lane's
+// 16 results are 64 bytes of ONE pixel, so a direct store instruction would scatter 64 pieces of
+// 16 bytes; after the exchange four neighbouring lanes hold the four quarters of one pixel and an
+// instruction writes 1 KB of consecutive memory.  pixT/validT[nt][k] describe pixel
+// (lane / 4) + 16 * k of pixel tile nt, which is the pixel the lane stores after the exchange.
+// The patch is laid out [16-channel block][pixel][quarter ^ ((pixel / 4) & 3)] in 16-byte cells,
+// which keeps both the writes (fixed quarter, 16 pixels) and the reads (4 pixels x 4 quarters)
+// spread over all banks.
+template <int TM, int TN, int OUT, bool SUM, bool FAST, bool XPOSE>
 __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
                                                     long long cidx, int oc_first, const size_t (&pix)[TN],
                                                     const bool (&pvalid)[TN], int oc_real, size_t block_stride,
-                                                    void *out)
+                                                    void *out, v4i *xlds, const size_t (&pixT)[TN][2],
+                                                    const bool (&validT)[TN][2])
 {
   const bool relu = ep.with_relu != 0;
+  const int lane = threadIdx.x & 63;
   OcConsts k = k0;
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt) {
-    OcConsts kn;
-    if (mt + 1 < TM) load_consts(kn, ep, cidx + 32 * (mt + 1));
+    if (mt > 0) load_consts(k, ep, cidx + 32 * mt);   // tile 0's came with the last k-steps
     const int oc = oc_first + 32 * mt;
     const bool oc_ok = oc < oc_real;
     size_t e[TN];
@@ -309,23 +319,39 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
       for (int q = 0; q < 4; ++q)
         s[q] = v4i{a[4 * q] + k.comp[q].x, a[4 * q + 1] + k.comp[q].y, a[4 * q + 2] + k.comp[q].z,
                    a[4 * q + 3] + k.comp[q].w};
-      if (OUT == EHIP_S32) {
-        if (ok[nt]) {
+      if (OUT == EHIP_S32 || OUT == EHIP_F32) {
+        if (OUT == EHIP_F32) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float4 r;
+            r.x = requant1(s[q].x, k.sc[q].x, k.sh[q].x, relu, ep.lo, ep.hi);
+            r.y = requant1(s[q].y, k.sc[q].y, k.sh[q].y, relu, ep.lo, ep.hi);
+            r.z = requant1(s[q].z, k.sc[q].z, k.sh[q].z, relu, ep.lo, ep.hi);
+            r.w = requant1(s[q].w, k.sc[q].w, k.sh[q].w, relu, ep.lo, ep.hi);
+            s[q] = v4i{__float_as_int(r.x), __float_as_int(r.y), __float_as_int(r.z), __float_as_int(r.w)};
+          }
+        }
+        if (XPOSE) {
+          const int l32 = lane & 31, lh = lane >> 5;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) xlds[lh * 128 + l32 * 4 + (q ^ ((l32 >> 2) & 3))] = s[q];
+          __builtin_amdgcn_wave_barrier();
+          // the wave's two 16-channel blocks: oc_first - 16 * lh + 32 * mt + 16 * h
+          const int ocw = oc - 16 * lh;
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+              const int P = (lane >> 2) + 16 * kk, bq = lane & 3;
+              const v4i v = xlds[h * 128 + P * 4 + (bq ^ ((P >> 2) & 3))];
+              if (validT[nt][kk] && ocw + 16 * h < oc_real)
+                *reinterpret_cast<v4i *>(static_cast<int *>(out) + pixT[nt][kk] +
+                                         (size_t)((ocw + 16 * h) >> 4) * block_stride + 4 * bq) = v;
+            }
+          __builtin_amdgcn_wave_barrier();
+        } else if (ok[nt]) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) *reinterpret_cast<v4i *>(static_cast<int *>(out) + e[nt] + 4 * q) = s[q];
-        }
-      } else if (OUT == EHIP_F32) {
-        float4 r[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          r[q].x = requant1(s[q].x, k.sc[q].x, k.sh[q].x, relu, ep.lo, ep.hi);
-          r[q].y = requant1(s[q].y, k.sc[q].y, k.sh[q].y, relu, ep.lo, ep.hi);
-          r[q].z = requant1(s[q].z, k.sc[q].z, k.sh[q].z, relu, ep.lo, ep.hi);
-          r[q].w = requant1(s[q].w, k.sc[q].w, k.sh[q].w, relu, ep.lo, ep.hi);
-        }
-        if (ok[nt]) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) *reinterpret_cast<float4 *>(static_cast<float *>(out) + e[nt] + 4 * q) = r[q];
         }
       } else {
         v4i cell;
@@ -336,33 +362,35 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
         if (ok[nt]) *reinterpret_cast<v4i *>(static_cast<uint8_t *>(out) + e[nt]) = cell;
       }
     }
-    if (mt + 1 < TM) k = kn;
   }
 }
 
-// one uniform switch on the output type (and on the cheap ReLU form) around the whole epilogue
+// one uniform switch on the output type (and on the cheap ReLU form) around the whole epilogue;
+// xlds == nullptr: 4-byte outputs are stored directly
 template <int TM, int TN>
 __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
                                               long long cidx, int oc_first, const size_t (&pix)[TN],
-                                              const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out)
+                                              const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out,
+                                              v4i *xlds, const size_t (&pixT)[TN][2], const bool (&validT)[TN][2])
 {
-#define EHIP_EPI(OUT, SUM, FAST) \
-  epilogue_wave_typed<TM, TN, OUT, SUM, FAST>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out)
+#define EHIP_EPI(OUT, SUM, FAST, XP)                                                                              \
+  epilogue_wave_typed<TM, TN, OUT, SUM, FAST, XP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, \
+                                                  out, xlds, pixT, validT)
   const bool fast = ep.with_relu && ep.lo >= 0.0f && ep.hi >= ep.lo;
   switch (ep.out_type) {
   case EHIP_U8:
-    if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_U8, true, true); else EHIP_EPI(EHIP_U8, true, false); }
-    else { if (fast) EHIP_EPI(EHIP_U8, false, true); else EHIP_EPI(EHIP_U8, false, false); }
+    if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_U8, true, true, false); else EHIP_EPI(EHIP_U8, true, false, false); }
+    else { if (fast) EHIP_EPI(EHIP_U8, false, true, false); else EHIP_EPI(EHIP_U8, false, false, false); }
     break;
   case EHIP_S8:
-    if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_S8, true, true); else EHIP_EPI(EHIP_S8, true, false); }
-    else { if (fast) EHIP_EPI(EHIP_S8, false, true); else EHIP_EPI(EHIP_S8, false, false); }
+    if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_S8, true, true, false); else EHIP_EPI(EHIP_S8, true, false, false); }
+    else { if (fast) EHIP_EPI(EHIP_S8, false, true, false); else EHIP_EPI(EHIP_S8, false, false, false); }
     break;
   case EHIP_F32:
-    EHIP_EPI(EHIP_F32, false, false);
+    if (xlds) EHIP_EPI(EHIP_F32, false, false, true); else EHIP_EPI(EHIP_F32, false, false, false);
     break;
   default:
-    EHIP_EPI(EHIP_S32, false, false);
+    if (xlds) EHIP_EPI(EHIP_S32, false, false, true); else EHIP_EPI(EHIP_S32, false, false, false);
     break;
   }
 #undef EHIP_EPI
