@@ -121,6 +121,11 @@ def main():
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--layers", default="all", help="other layers to report: all, none or a comma list")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size N (scaling studies; "
+                                                         "the headline figure uses the configured N)")
+    ap.add_argument("--hbm-probe", action="store_true",
+                    help="instead of a layer, time plain device copy / fill / read of 1 GiB (the HBM rates a "
+                         "trivial kernel reaches on this box)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="instead of a layer, run 20 plain device copies of MIB MiB (known traffic, used to "
                          "scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -153,7 +158,32 @@ def main():
         print(json.dumps({"calibrate_copy_bytes": n, "launches": 20}))
         return
 
+    if args.hbm_probe:
+        n = 1 << 30
+        a = torch.empty(n, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        af = a.view(torch.float32)
+
+        def rate(fn, nbytes, reps=20):
+            fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return round(nbytes / (e0.elapsed_time(e1) * 1e-3 / reps) / 1e9, 1)
+        print(json.dumps({"hbm_probe_bytes": n, "copy_read_plus_write_GBs": rate(lambda: b.copy_(a), 2 * n),
+                          "fill_write_GBs": rate(lambda: a.zero_(), n), "sum_read_GBs": rate(lambda: af.sum(), n)}))
+        return
+
     wl = W.WORKLOADS[args.workload]
+    if args.batch:
+        import copy
+        wl = copy.copy(wl)
+        wl.n = args.batch
+        wl.key = "%s@N=%d" % (wl.key, wl.n)
     layer = W.DeviceLayer(wl)
     wall, ev = measure(layer, args.steps, args.warmup)
     lat = single_launch_latency(layer)

@@ -412,6 +412,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ihw = d.ih * d.iw; a.iw = d.iw;
     a.stride_h = d.stride_h; a.stride_w = d.stride_w;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
     HIP_TRY(launch_gemm(a, 1, c->variant, s));
     break;
   }

@@ -27,9 +27,21 @@
 // share a CU, so one can multiply while the other waits at its barrier.
 #include "ehip_internal.hpp"
 
+// Development aid (compile with -DEHIP_TRACE): lane 0 of every wave records the shader clock at
+// phase boundaries into GemmArgs::trace.
+#ifdef EHIP_TRACE
+#define TRACE_POINT(i)                                                                             \
+  do {                                                                                             \
+    if (a.trace && lane == 0)                                                                      \
+      a.trace[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
+  } while (0)
+#else
+#define TRACE_POINT(i) do { } while (0)
+#endif
+
 namespace ehip {
 
-template <int WM, int WN, int TM, int TN, int KC>
+template <int WM, int WN, int TM, int TN, int KC, int D>
 __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 {
   constexpr int OC_T = WM * TM * 32;
@@ -62,6 +74,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const int pw0 = (wave / WM) * TN * 32;
   const int oc_real = a.oc2 * 16;
   const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  TRACE_POINT(0);
 
   // ---- staging plan ---------------------------------------------------------------------------
   // B: a thread always copies the same pixel (tid % P_T), units tid / P_T + j * BU of a fill.
@@ -87,28 +100,28 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const int8_t *wb = a.w + (long long)b * a.units_pad * a.ocpp * 16 + (long long)oc0 * 16;
   const long long w_unit = (long long)a.ocpp * 16;
 
-  v4i sta[NA], stb[NB];
+  v4i sta[D][NA], stb[D][NB];   // D fills in flight (global -> registers), see the main loop
   // All global loads of the main loop are unconditional (indices clamped): without branches
   // between a load and its use the compiler counts outstanding loads exactly.
-  auto load_stage = [&](int chunk) {
+  auto load_stage = [&](int chunk, int d) {
 #pragma unroll
     for (int j = 0; j < NA; ++j) {
       const int id = tid + j * kBlock;
-      sta[j] = *reinterpret_cast<const v4i *>(wb + (long long)(chunk * KC + id / OC_T) * w_unit + (id % OC_T) * 16);
+      sta[d][j] = *reinterpret_cast<const v4i *>(wb + (long long)(chunk * KC + id / OC_T) * w_unit + (id % OC_T) * 16);
     }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
       int u = chunk * KC + bu0 + j * BU;
       u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
-      stb[j] = *reinterpret_cast<const v4i *>(inb + (long long)u * unit_stride);
+      stb[d][j] = *reinterpret_cast<const v4i *>(inb + (long long)u * unit_stride);
     }
   };
-  auto store_stage = [&](int buf) {
+  auto store_stage = [&](int buf, int d) {
 #pragma unroll
-    for (int j = 0; j < NA; ++j) lds_a[buf][tid + j * kBlock] = sta[j];
+    for (int j = 0; j < NA; ++j) lds_a[buf][tid + j * kBlock] = sta[d][j];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      lds_b[buf][tid + j * kBlock] = stb[j] ^ (int)0x80808080;
+      lds_b[buf][tid + j * kBlock] = stb[d][j] ^ (int)0x80808080;
     }
   };
 
@@ -147,25 +160,41 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   };
 
   const int nchunks = a.units_pad / KC;
-  load_stage(0);
+  // The layers this kernel serves are small: what a workgroup waits for is the latency of its
+  // global loads, not their bandwidth.  So D fills are kept in flight in registers: the loads of
+  // fill c + D are issued when fill c moves to LDS.  The launcher picks D so that it divides the
+  // number of fills; the last D fills are peeled and prefetch nothing.
+  const int ngroups = nchunks / D;
+#pragma unroll
+  for (int d = 0; d < D; ++d) load_stage(d, d);
+  TRACE_POINT(1);
   int buf = 0;
-  for (int c = 0; c + 1 < nchunks; ++c) {
-    store_stage(buf);
+  for (int g = 0; g + 1 < ngroups; ++g) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      store_stage(buf, d);
+      if (g == 0 && d == 0) TRACE_POINT(2);
+      __syncthreads();
+      if (g == 0 && d == 0) TRACE_POINT(3);
+      load_stage((g + 1) * D + d, d);
+      multiply(buf);
+      if (g == 0 && d == 0) TRACE_POINT(4);
+      buf ^= 1;
+    }
+  }
+  TRACE_POINT(5);
+  const long long cidx = (long long)b * a.ocpp + oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
+  OcConsts k0;
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    store_stage(buf, d);
     __syncthreads();
-    load_stage(c + 1);
+    // the epilogue's per-channel constants travel while the last fill is multiplied
+    if (d == D - 1) load_consts(k0, a.ep, cidx);
     multiply(buf);
     buf ^= 1;
   }
-  // last fill: nothing left to prefetch but the epilogue's per-channel constants
-  store_stage(buf);
-  __syncthreads();
-  const long long cidx = (long long)b * a.ocpp + oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
-  // the epilogue's per-channel constants travel while the last fill is multiplied -- unless the
-  // accumulators leave no registers for them (the co-resident workgroup covers the wait then)
-  OcConsts k0;
-  if (TM * TN < 8) load_consts(k0, a.ep, cidx);
-  multiply(buf);
-  if (TM * TN >= 8) load_consts(k0, a.ep, cidx);
+  TRACE_POINT(6);
 
   // ---- epilogue ------------------------------------------------------------------------------
   auto pixel_offset = [&](int gp, bool &valid) -> size_t {
@@ -189,19 +218,28 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     __syncthreads();   // every wave has read its last operands
     xlds = lds + wave * 256;
   }
+  TRACE_POINT(14);
   epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real, (size_t)a.ohw * 16, a.out, xlds,
                         pixT, validT);
+  TRACE_POINT(15);
 }
 
 namespace {
 struct Variant {
   const char *name;
   int oc_t, p_t, kc;
-  void (*kernel)(GemmArgs);
+  void (*kernel[3])(GemmArgs);   // prefetch depth 1, 2, 4 (null: too many staging registers)
 };
+// depth 4 only where four fills of staging fit in 96 registers
+template <int WM, int WN, int TM, int TN, int KC>
+constexpr void (*deep_or_null())(GemmArgs)
+{
+  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4>;
+  else return nullptr;
+}
 #define V(WM, WN, TM, TN, KC)                                                                    \
   { "k_gemm_u8s8<" #WM "," #WN "," #TM "," #TN "," #KC ">", WM * TM * 32, WN * TN * 32, KC,       \
-    k_gemm_u8s8<WM, WN, TM, TN, KC> }
+    { k_gemm_u8s8<WM, WN, TM, TN, KC, 1>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2>, deep_or_null<WM, WN, TM, TN, KC>() } }
 const Variant kVariants[] = {
     V(2, 2, 2, 2, 8),  // 0: 128 oc x 128 px
     V(2, 2, 2, 1, 8),  // 1: 128 oc x  64 px
@@ -250,7 +288,14 @@ hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s
 {
   const Variant &k = kVariants[variant];
   dim3 grid((a.p_total + k.p_t - 1) / k.p_t, (a.oc2 * 16 + k.oc_t - 1) / k.oc_t, nbatch);
-  hipLaunchKernelGGL(k.kernel, grid, dim3(kBlock), 0, s, a);
+  // prefetch depth: must divide the number of fills.  Measured on the configured layers depth 2 is
+  // as good as it gets (depth 4 costs registers and gains nothing); EHIP_GEMM_DEPTH overrides.
+  const int nchunks = a.units_pad / k.kc;
+  int dl = 1;
+  const char *env = getenv("EHIP_GEMM_DEPTH");
+  if (env && env[0]) dl = atoi(env) >= 4 ? 2 : (atoi(env) >= 2 ? 1 : 0);
+  while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[dl])) --dl;
+  hipLaunchKernelGGL(k.kernel[dl], grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
 

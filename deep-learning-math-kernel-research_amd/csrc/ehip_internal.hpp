@@ -47,6 +47,7 @@ struct GemmArgs {
   int ocpp;             // padded rows in the packed weights
   long long in_batch_stride;   // bytes
   long long out_batch_stride;  // elements
+  long long *trace;            // development aid, normally null (see EHIP_TRACE)
 };
 
 struct Conv3x3Args {
@@ -84,6 +85,7 @@ struct WinoArgs {
   float *out;           // [n][oc2][oh][ow][16]
   const float *bias;
   int n, ic2, oc2, ih, iw, oh, ow, ht, wt, nt, t, pad_t, pad_l;
+  int blocks_interior;  // set by the input-transform launcher: blocks over tiles off the rim
   float mrepS, mz;      // input_S / tinput_S, ceil(tinput_z)
   int with_bias, with_relu;
 };

@@ -131,32 +131,84 @@ __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &
 
 }  // namespace
 
-// grid: (ceil(t / 64), ic2); block: 64 tiles x 4 channel quads
+// Tiles that touch the zero frame take the "border" arithmetic, all others the plain one; a wave
+// that holds both kinds would execute both.  So the grid is split: the first a.blocks_interior
+// blocks enumerate only tiles away from the rim of the tile grid (never border), the remaining
+// blocks enumerate the rim.  Returns false past the end of the group.
+__device__ __forceinline__ bool grouped_tile(const WinoArgs &a, int block, int slot, TileCoord &c, int &t)
+{
+  const int wi = a.wt - 2, hi = a.ht - 2;
+  const int ni = (wi > 0 && hi > 0) ? wi * hi : 0;   // interior tiles per image
+  int n, th, tw;
+  if (block < a.blocks_interior) {
+    const int idx = block * 64 + slot;
+    if (idx >= a.n * ni) return false;
+    n = idx / ni;
+    const int r = idx - n * ni;
+    th = 1 + r / wi;
+    tw = 1 + (r - (th - 1) * wi);
+  } else {
+    const int idx = (block - a.blocks_interior) * 64 + slot;
+    const int nr = a.nt - ni;                        // rim tiles per image
+    if (idx >= a.n * nr) return false;
+    n = idx / nr;
+    const int r = idx - n * nr;
+    if (ni == 0) {                                   // fewer than 3 tile rows or columns: all rim
+      th = r / a.wt;
+      tw = r - th * a.wt;
+    } else if (r < a.wt) {
+      th = 0; tw = r;
+    } else if (r < 2 * a.wt) {
+      th = a.ht - 1; tw = r - a.wt;
+    } else {
+      const int rr = r - 2 * a.wt;
+      th = 1 + (rr >> 1);
+      tw = (rr & 1) ? a.wt - 1 : 0;
+    }
+  }
+  t = n * a.nt + th * a.wt + tw;
+  c.n = n; c.th = th; c.tw = tw;
+  c.h0 = 4 * th - a.pad_t;
+  c.w0 = 4 * tw - a.pad_l;
+  c.border = c.h0 < 0 || c.w0 < 0 || c.h0 + 5 >= a.ih || c.w0 + 5 >= a.iw;
+  return true;
+}
+
+// grid: (interior blocks + rim blocks, ic2); block: 64 tiles x 4 channel quads
 __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
 {
   const int q = threadIdx.x & 3;
-  const int t = blockIdx.x * 64 + (threadIdx.x >> 2);
   const int c2 = blockIdx.y;
-  if (t >= a.t) return;
-  const TileCoord c = tile_coord(a, t);
+  TileCoord c;
+  int t;
+  if (!grouped_tile(a, blockIdx.x, threadIdx.x >> 2, c, t)) return;
   float4 d[36];
   gather_tile(a, c, c2, q, d);
   unsigned packed[36];
 #pragma unroll
   for (int k = 0; k < 36; ++k) packed[k] = 0u;
+  auto channels = [&](bool border) {
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    float f[36], v[36];
+    for (int k = 0; k < 4; ++k) {
+      float f[36], v[36];
 #pragma unroll
-    for (int e = 0; e < 36; ++e) f[e] = comp_of(d[e], k);
-    if (c.border) tile_input(f, v, true);
-    else tile_input(f, v, false);
+      for (int e = 0; e < 36; ++e) f[e] = comp_of(d[e], k);
+      tile_input(f, v, border);
 #pragma unroll
-    for (int e = 0; e < 36; ++e) {
-      // sat_u8(rne(V * (in_S / tin_S) + tin_z)), one rounding in the multiply-add
-      const unsigned u = usat8(cvt_u32_rne(__builtin_fmaf(v[e], a.mrepS, a.mz)));
-      packed[e] |= u << (8 * k);
+      for (int e = 0; e < 36; ++e) {
+        // sat_u8(rne_to_u32(V * (in_S / tin_S) + tin_z)), one rounding in the multiply-add.  The
+        // reference's float -> u32 conversion turns everything below -0.5 (and NaN) into 0xffffffff,
+        // which then saturates to 255; v_cvt_pk_u8_f32 rounds to nearest even and saturates the rest.
+        const float y = __builtin_fmaf(v[e], a.mrepS, a.mz);
+        packed[e] = __builtin_amdgcn_cvt_pk_u8_f32(y >= -0.5f ? y : 300.0f, k, packed[e]);
+      }
     }
+  };
+  if (blockIdx.x < a.blocks_interior) {
+    channels(false);
+  } else {
+    if (c.border) channels(true);
+    else channels(false);
   }
   unsigned *dst = reinterpret_cast<unsigned *>(a.tin) + ((size_t)c2 * a.t + t) * 4 + q;
   const size_t pos_stride = (size_t)a.ic2 * a.t * 4;
@@ -264,9 +316,13 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output_f32(WinoArgs a)
   }
 }
 
-hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s)
+hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s)
 {
-  dim3 grid((a.t + 63) / 64, a.ic2);
+  WinoArgs a = a0;
+  const int ni = (a.wt > 2 && a.ht > 2) ? (a.wt - 2) * (a.ht - 2) : 0;
+  a.blocks_interior = (a.n * ni + 63) / 64;
+  const int blocks_rim = (a.n * (a.nt - ni) + 63) / 64;
+  dim3 grid(a.blocks_interior + blocks_rim, a.ic2);
   hipLaunchKernelGGL(k_wino_trans_input_u8, grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
