@@ -248,19 +248,29 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
     if (v >= 0 && v < kNumVariants && conv3x3v_fits(v, ow)) return v;
     return -1;
   }
+  // Measured on MI355X (3x3 128 -> 128 @28x28, N = 32 .. 512): a workgroup's time is the time to
+  // pull its weights through the CU's vector-memory path, so tiles whose four waves own disjoint
+  // channels (no weight row loaded twice: variants 8-10) win; among those the 64-pixel tile while
+  // the grid is small (more workgroups to spread over the chip), the 128-pixel tile once it is not.
   const int oc = oc2 * 16, vpx = oh * (ow + 2);
+  static const double pref[] = {0.80, 0.78, 0.92, 0.90, 1.0, 0.95, 1.0, 0.95, 0.85, 0.97, 1.0};
   int best = -1;
   double best_score = -1;
+  for (int pass = 0; pass < 2 && best < 0; ++pass)   // second pass: any channel tile that fits the rows
   for (int v = 0; v < kNumVariants; ++v) {
     if (!conv3x3v_fits(v, ow)) continue;
     const Variant &k = kVariants[v];
+    if (pass == 0) {
+      if (oc > 64 && k.oc_t < 128) continue;
+      if (oc <= 64 && oc > 32 && k.oc_t != 64) continue;
+      if (oc <= 32 && k.oc_t != 32) continue;
+    }
     const int gx = (vpx + k.p_t - 1) / k.p_t, gy = (oc + k.oc_t - 1) / k.oc_t;
     const long long wgs = (long long)gx * gy * n;
-    const double util = ((double)oc / ((double)gy * k.oc_t)) * ((double)(oh * ow) / ((double)gx * k.p_t));
-    const long long rounds = (wgs + 511) / 512;
-    const double fill = (double)wgs / (double)(rounds * 512);
-    const double lean = (double)(k.p_t + 2 * (ow + 2) + 2) / (double)k.cells;  // unused LDS costs occupancy
-    const double score = util * (0.5 + 0.5 * fill) * (0.75 + 0.25 * lean) * (k.oc_t >= 64 ? 1.0 : 0.8);
+    const double util = (double)(oh * ow) / ((double)gx * k.p_t);
+    const double fill = wgs >= 256 ? 1.0 : (double)wgs / 256.0;
+    const double big = (k.p_t >= 128 && wgs >= 1024) ? 1.15 : 1.0;   // enough work: amortise the weights
+    const double score = util * fill * big * pref[v];
     if (score > best_score) { best_score = score; best = v; }
   }
   return best;
