@@ -204,7 +204,7 @@ int setup_workspace(ehip_conv *c)
       return fail(EHIP_UNIMPLEMENTED, "1x1: n*oh*ow*oh*ow must stay below 2^32");
     c->taps = 1;
     c->nbatch = 1;
-    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2, 1);
+    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2, 1, d.stride_w);
     c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
     c->kernel_name = gemm_variant_name(c->variant);
     break;
@@ -251,7 +251,7 @@ int setup_workspace(ehip_conv *c)
     }
     c->t = c->nt * c->chunk_n;   // tiles per pass
     if ((long long)c->t >= (1ll << 31) / 64) return fail(EHIP_UNIMPLEMENTED, "winograd: too many tiles");
-    c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, 36);
+    c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, 36, 1);
     c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
     c->kernel_name = std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output_f32";
     c->tin_bytes = (size_t)36 * c->ic2 * c->t * 16;

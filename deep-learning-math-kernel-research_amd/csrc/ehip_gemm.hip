@@ -259,7 +259,7 @@ int gemm_num_variants() { return kNumVariants; }
 
 // Score = useful fraction of the padded tile grid x how well the grid fills the chip (two
 // workgroups per CU) x operand reuse of the tile.
-int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch)
+int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride)
 {
   const char *env = getenv("EHIP_GEMM_VARIANT");
   if (env && env[0]) {
@@ -277,7 +277,9 @@ int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch)
                         ((double)ic2 / (double)up(ic2, k.kc));
     const long long rounds = (wgs + 511) / 512;
     const double fill = (double)wgs / (double)(rounds * 512);
-    const double reuse = (double)k.oc_t * k.p_t / (double)(k.oc_t + k.p_t) / 64.0;  // 1.0 for 128 x 128
+    double reuse = (double)k.oc_t * k.p_t / (double)(k.oc_t + k.p_t) / 64.0;  // 1.0 for 128 x 128
+    // a strided 1x1 gathers its pixels in 16-byte pieces: the more channels share one gather the better
+    if (stride > 1) reuse *= (double)k.oc_t / 128.0;
     const double score = util * fill * (0.25 + reuse);
     if (score > best_score) { best_score = score; best = v; }
   }

@@ -92,7 +92,7 @@ struct WinoArgs {
 
 // ---- launchers (implemented next to their kernels) ------------------------------------------
 hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s);
-int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch);
+int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride);
 int gemm_variant_chunk(int variant);
 int gemm_num_variants();
 const char *gemm_variant_name(int variant);
