@@ -48,6 +48,7 @@ struct ehip_conv {
   // Winograd
   int ht = 0, wt = 0, nt = 0, t = 0;
   int chunk_n = 0;   // images per pass of the three-stage pipeline (intermediates sized for it)
+  bool fused = true; // GEMM and output transform in one kernel (no f32 GEMM result in memory)
   uint8_t *tin = nullptr;
   float *tout = nullptr;
   size_t tin_bytes = 0, tout_bytes = 0;
@@ -253,10 +254,15 @@ int setup_workspace(ehip_conv *c)
     if ((long long)c->t >= (1ll << 31) / 64) return fail(EHIP_UNIMPLEMENTED, "winograd: too many tiles");
     c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, 36, 1);
     c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
-    c->kernel_name = std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output_f32";
-    c->tin_bytes = (size_t)36 * c->ic2 * c->t * 16;
-    c->tout_bytes = (size_t)36 * c->oc2 * c->t * 16 * sizeof(float);
-    if ((rc = dev_alloc(&c->tin, c->tin_bytes, false)) != EHIP_OK) return rc;
+    {
+      const char *env = getenv("EHIP_WINO_FUSED");
+      c->fused = !(env && env[0] == '0');
+    }
+    c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
+                              : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output_f32";
+    c->tin_bytes = (size_t)36 * c->ic2 * c->t * 16;   // allocated with one pad unit behind it
+    c->tout_bytes = c->fused ? 16 : (size_t)36 * c->oc2 * c->t * 16 * sizeof(float);
+    if ((rc = dev_alloc(&c->tin, c->tin_bytes + (size_t)c->t * 16, true)) != EHIP_OK) return rc;
     if ((rc = dev_alloc(reinterpret_cast<uint8_t **>(&c->tout), c->tout_bytes, false)) != EHIP_OK) return rc;
     break;
   }
@@ -465,6 +471,18 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       w.mrepS = d.input_scale * tin_repS;
       w.mz = ceilf(d.tinput_z);
       HIP_TRY(launch_wino_trans_input(w, s));
+      if (c->fused) {
+        WinoFusedArgs f;
+        memset(&f, 0, sizeof(f));
+        f.tin = c->tin; f.w = c->wpacked; f.out = w.out; f.bias = w.bias;
+        f.scale = c->scale; f.shift = c->shift; f.comp = c->comp;
+        f.n = w.n; f.ic2 = c->ic2; f.units_pad = c->units_pad; f.oc2 = c->oc2; f.ocpp = c->ocpp;
+        f.oh = d.oh; f.ow = d.ow; f.ht = w.ht; f.wt = w.wt; f.nt = w.nt; f.t = w.t;
+        f.with_bias = d.with_bias; f.with_relu = d.with_relu;
+        f.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
+        HIP_TRY(launch_wino_gemm_output(f, s));
+        continue;
+      }
       GemmArgs a;
       memset(&a, 0, sizeof(a));
       a.in = c->tin;
@@ -557,6 +575,7 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
   case EHIP_Q_TOUTPUT_F32:
     if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "not a Winograd handle");
     if (c->chunk_n < d.n) return fail(EHIP_UNIMPLEMENTED, "the intermediates of a multi-pass layer hold its last pass only");
+    if (c->fused) return fail(EHIP_UNIMPLEMENTED, "the fused schedule keeps the GEMM result on chip (set EHIP_WINO_FUSED=0)");
     if (!want(c->tout_bytes)) return EHIP_OK;
     HIP_TRY(hipMemcpy(host_dst, c->tout, c->tout_bytes, hipMemcpyDeviceToHost));
     return EHIP_OK;

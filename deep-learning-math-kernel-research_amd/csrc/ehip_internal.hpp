@@ -90,6 +90,19 @@ struct WinoArgs {
   int with_bias, with_relu;
 };
 
+struct WinoFusedArgs {
+  const uint8_t *tin;   // [36][ic2][t][16] u8
+  const int8_t *w;      // [36][units_pad][OCpp][16] s8
+  float *out;           // [n][oc2][oh][ow][16]
+  const float *bias;
+  const float *scale, *shift;  // [36][OCpp]
+  const int *comp;
+  int n, ic2, units_pad, oc2, ocpp, oh, ow, ht, wt, nt, t;
+  int with_bias, with_relu;
+  int nx, ny;           // set by the launcher: blocks of 32 tiles, of 64 channels
+  long long *trace;     // development aid, normally null (see EHIP_TRACE)
+};
+
 // ---- launchers (implemented next to their kernels) ------------------------------------------
 hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s);
 int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride);
@@ -106,6 +119,7 @@ const char *conv3x3v_variant_name(int variant);
 hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s);
 hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s);
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s);
+hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s);
 hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_dev, hipStream_t s);
 
 // weight preparation

@@ -23,6 +23,15 @@
 // product of the last row pass) separately.
 #include "ehip_internal.hpp"
 
+#ifdef EHIP_TRACE
+#define TRACE_POINT(i)                                                                             \
+  do {                                                                                             \
+    if (a.trace && lane == 0) a.trace[((size_t)blockIdx.x * 4 + wave) * 16 + (i)] = clock64();     \
+  } while (0)
+#else
+#define TRACE_POINT(i) do { } while (0)
+#endif
+
 namespace ehip {
 
 namespace {
@@ -254,27 +263,12 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
   }
 }
 
-// grid: (ceil(t / 64), oc2); block: 64 tiles x 4 channel quads
-__global__ __launch_bounds__(kBlock) void k_wino_trans_output_f32(WinoArgs a)
+// Y = At M A (+ bias)(ReLU) of one tile x four channels (the four components of the float4s) and
+// its store; dst points at the tile's image plane, channel quad already applied.  Border tiles
+// write their valid rows and columns only.
+__device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 &bias, bool with_bias, bool with_relu,
+                                            float4 *dst, int th, int tw, int oh_n, int ow_n)
 {
-  const int q = threadIdx.x & 3;
-  const int t = blockIdx.x * 64 + (threadIdx.x >> 2);
-  const int o2 = blockIdx.y;
-  if (t >= a.t) return;
-  const int n = t / a.nt;
-  const int rem = t - n * a.nt;
-  const int th = rem / a.wt;
-  const int tw = rem - th * a.wt;
-
-  const float4 *src = reinterpret_cast<const float4 *>(a.tout) + ((size_t)o2 * a.t + t) * 4 + q;
-  const size_t pos_stride = (size_t)a.oc2 * a.t * 4;
-  float4 m[36];
-#pragma unroll
-  for (int e = 0; e < 36; ++e) m[e] = src[e * pos_stride];
-
-  float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (a.with_bias) bias = reinterpret_cast<const float4 *>(a.bias)[o2 * 4 + q];
-
   float y[4][16];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -296,23 +290,217 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output_f32(WinoArgs a)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float r = o[j];
-        if (a.with_bias) r = r + b;
-        if (a.with_relu) r = r > 0.0f ? r : 0.0f;
+        if (with_bias) r = r + b;
+        if (with_relu) r = r > 0.0f ? r : 0.0f;
         y[k][4 * i + j] = r;
       }
     }
   }
-  float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 4 + q;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int oh = 4 * th + i;
-    if (oh >= a.oh) break;
+    if (oh >= oh_n) break;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int ow = 4 * tw + j;
-      if (ow >= a.ow) break;
-      dst[((size_t)oh * a.ow + ow) * 4] = make_float4(y[0][4 * i + j], y[1][4 * i + j], y[2][4 * i + j], y[3][4 * i + j]);
+      if (ow >= ow_n) break;
+      dst[((size_t)oh * ow_n + ow) * 4] = make_float4(y[0][4 * i + j], y[1][4 * i + j], y[2][4 * i + j], y[3][4 * i + j]);
     }
+  }
+}
+
+// grid: (ceil(t / 64), oc2); block: 64 tiles x 4 channel quads
+__global__ __launch_bounds__(kBlock) void k_wino_trans_output_f32(WinoArgs a)
+{
+  const int q = threadIdx.x & 3;
+  const int t = blockIdx.x * 64 + (threadIdx.x >> 2);
+  const int o2 = blockIdx.y;
+  if (t >= a.t) return;
+  const int n = t / a.nt;
+  const int rem = t - n * a.nt;
+  const int th = rem / a.wt;
+  const int tw = rem - th * a.wt;
+
+  const float4 *src = reinterpret_cast<const float4 *>(a.tout) + ((size_t)o2 * a.t + t) * 4 + q;
+  const size_t pos_stride = (size_t)a.oc2 * a.t * 4;
+  float4 m[36];
+#pragma unroll
+  for (int e = 0; e < 36; ++e) m[e] = src[e * pos_stride];
+
+  float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (a.with_bias) bias = reinterpret_cast<const float4 *>(a.bias)[o2 * 4 + q];
+  float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 4 + q;
+  output_tile(m, bias, a.with_bias != 0, a.with_relu != 0, dst, th, tw, a.oh, a.ow);
+}
+
+// ---- the 36 GEMMs and the output transform in one kernel ----------------------------------------
+// Replaces elx_int8_conv_wino_gemm_t::execute + trans_output as the reference's fused schedule does
+// per thread (a161, src/elx_int8_conv_wino_xopt.hpp:21-179): the f32 GEMM result of a block of
+// tiles never leaves the chip.  Written out it is 36/16 x 4 bytes per output value each way --
+// more than twice the traffic of everything else in the layer together.
+//
+// A workgroup owns 64 output channels x 32 tiles at ALL 36 positions.  Each of its four waves
+// takes nine positions and runs their GEMMs on v_mfma_i32_32x32x32_i8 with both operands loaded
+// straight from memory into a register ring of KS k-steps (nothing is shared between waves, so
+// there is no LDS traffic and no barrier in the main loop; a slot is refilled with the operand
+// KS steps ahead as soon as its MFMAs are issued).  Then, for each half of the channels, the waves
+// requantize their accumulators to f32 (the GEMM's own epilogue: fma(float(acc), scale, shift) per
+// position and channel), exchange them through LDS -- 36 x 32 x 32 floats = 144 KB -- and every
+// thread gathers the 36 values of one tile x four channels, applies Y = At M A + bias, ReLU, and
+// stores its 4 x 4 pixels exactly like the stand-alone output transform.
+//
+// Workgroups are numbered so that the channel blocks of one tile block run next to each other on
+// the same XCD (blockIdx.x % 8), where the second and later ones find the tiles in that XCD's L2.
+template <int KS>
+__global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
+{
+  extern __shared__ float4 xl[];   // [36][32 tiles][8 cells of 4 channels], cell ^ ((tile / 2) & 7)
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int by = seq % a.ny;
+  const int bx = (seq / a.ny) * 8 + xcd;
+  if (bx >= a.nx) return;          // whole workgroup
+  const int t0 = bx * 32, oc0 = by * 64;
+  const int oc_real = a.oc2 * 16;
+  const int p0 = 9 * wave;
+  const int nks = a.units_pad >> 1;   // k-steps (32 channels) per position
+  const int nkc = nks / KS;
+
+  // operand addresses = wave-uniform pointer (scalar arithmetic) + a per-lane 32-bit offset that
+  // never changes: lane = packed row / tile l32 of unit 2 * ks + lh
+  const unsigned a_lane = (unsigned)(lh * a.ocpp + l32) * 16u;
+  const int tile = t0 + l32 < a.t ? t0 + l32 : a.t - 1;
+  const unsigned b_lane = (unsigned)(lh * a.t + tile) * 16u;
+  const int ks_last = ((a.ic2 + 1) >> 1) - 1;   // last k-step that holds real channels
+
+  TRACE_POINT(0);
+  v4i ra[KS][2], rb[KS];
+  auto issue = [&](int slot, int p, int ks) {
+    const int8_t *pa = a.w + (((long long)p * a.units_pad + 2 * ks) * a.ocpp + oc0) * 16;
+    ra[slot][0] = *reinterpret_cast<const v4i *>(pa + a_lane);
+    ra[slot][1] = *reinterpret_cast<const v4i *>(pa + 512 + a_lane);
+    // padded k-steps multiply zero weights: any valid cell will do (an odd unit count reads one
+    // unit past the position, which is the next position or the pad unit behind the buffer)
+    const int ksc = ks < ks_last ? ks : ks_last;
+    const uint8_t *pb = a.tin + ((long long)p * a.ic2 + 2 * ksc) * a.t * 16;
+    rb[slot] = *reinterpret_cast<const v4i *>(pb + b_lane);
+  };
+
+  // Per-(position, channel) scale / shift / compensation of the wave's nine positions, one half of
+  // the channels at a time: 27 rows of 32 dwords, staged in the 16 KB of LDS the exchange buffer
+  // leaves free.  Read from there every lane pays one LDS broadcast per constant instead of a
+  // global load instruction (which costs the address path as much as a full 1 KB load).
+  float4 *cl = xl + 36 * 32 * 8 + wave * 216;
+  float4 cst[4];
+  auto load_consts_half = [&](int h) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int idx = lane + 64 * j;
+      idx = idx < 216 ? idx : 215;
+      const int row = idx >> 3, cell = idx & 7;
+      const int i = row / 3, arr = row - 3 * i;
+      const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
+      cst[j] = *reinterpret_cast<const float4 *>(src + (long long)(p0 + i) * a.ocpp + oc0 + 32 * h + 4 * cell);
+    }
+  };
+  auto store_consts_half = [&]() {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int idx = lane + 64 * j;
+      cl[idx < 216 ? idx : 215] = cst[j];
+    }
+  };
+  load_consts_half(0);
+  store_consts_half();
+
+  v16i acc[9][2];
+#pragma unroll
+  for (int i = 0; i < 9; ++i)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][h][v] = 0;
+
+#pragma unroll
+  for (int k = 0; k < KS; ++k) issue(k, p0, k);
+#pragma unroll
+  for (int i = 0; i < 9; ++i) {
+    for (int c = 0; c < nkc; ++c) {
+#pragma unroll
+      for (int k = 0; k < KS; ++k) {
+        const v4i b = rb[k] ^ (int)0x80808080;
+        acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][0], b, acc[i][0], 0, 0, 0);
+        acc[i][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][1], b, acc[i][1], 0, 0, 0);
+        // refill the slot with the operands KS steps ahead (the very last block re-reads itself)
+        int pn = p0 + i, ksn = (c + 1) * KS + k;
+        if (ksn >= nks) { ksn -= nks; pn += 1; }
+        if (pn > p0 + 8) { pn = p0 + 8; ksn = nks - KS + k; }
+        issue(k, pn, ksn);
+      }
+    }
+  }
+
+  load_consts_half(1);   // second half's constants travel while the first half is processed
+  TRACE_POINT(1);
+  // ---- requantize, exchange, output transform ----------------------------------------------------
+  const int tile_l = tid >> 3, q8 = tid & 7;
+  const int t = t0 + tile_l;
+  const int tc = t < a.t ? t : a.t - 1;
+  const int n = tc / a.nt;
+  const int rem = tc - n * a.nt;
+  const int th = rem / a.wt;
+  const int tw = rem - th * a.wt;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (h) __syncthreads();        // everyone has gathered the first half
+    __builtin_amdgcn_wave_barrier();
+    // constants of position i + 1 are read from LDS while position i is requantized
+    float4 kq[2][12];
+    auto read_consts = [&](int i, int slot) {
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) kq[slot][4 * r + q] = cl[(3 * i + r) * 8 + 4 * lh + q];
+    };
+    read_consts(0, 0);
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+      const int p = p0 + i;
+      if (i + 1 < 9) read_consts(i + 1, (i + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 sc = kq[i & 1][q], sh = kq[i & 1][4 + q], cf = kq[i & 1][8 + q];
+        float4 r;
+        r.x = __builtin_fmaf((float)(acc[i][h][4 * q + 0] + __float_as_int(cf.x)), sc.x, sh.x);
+        r.y = __builtin_fmaf((float)(acc[i][h][4 * q + 1] + __float_as_int(cf.y)), sc.y, sh.y);
+        r.z = __builtin_fmaf((float)(acc[i][h][4 * q + 2] + __float_as_int(cf.z)), sc.z, sh.z);
+        r.w = __builtin_fmaf((float)(acc[i][h][4 * q + 3] + __float_as_int(cf.w)), sc.w, sh.w);
+        xl[(p * 32 + l32) * 8 + ((4 * lh + q) ^ ((l32 >> 1) & 7))] = r;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (h == 0) store_consts_half();   // the wave is done with the first half's constants
+    TRACE_POINT(2 + 4 * h);
+    __syncthreads();
+    TRACE_POINT(3 + 4 * h);
+    const int oc = oc0 + 32 * h + 4 * q8;
+    if (t < a.t && oc < oc_real) {
+      float4 m[36];
+#pragma unroll
+      for (int e = 0; e < 36; ++e) m[e] = xl[(e * 32 + tile_l) * 8 + (q8 ^ ((tile_l >> 1) & 7))];
+      float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
+      float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 4 + ((oc >> 2) & 3);
+      TRACE_POINT(4 + 4 * h);
+      output_tile(m, bias, a.with_bias != 0, a.with_relu != 0, dst, th, tw, a.oh, a.ow);
+    }
+    TRACE_POINT(5 + 4 * h);
   }
 }
 
@@ -331,6 +519,26 @@ hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s)
 {
   dim3 grid((a.t + 63) / 64, a.oc2);
   hipLaunchKernelGGL(k_wino_trans_output_f32, grid, dim3(kBlock), 0, s, a);
+  return hipGetLastError();
+}
+
+// k-steps per ring block: the largest of 8, 4, 2 that divides the k-steps of a position
+hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s)
+{
+  WinoFusedArgs a = a0;
+  a.nx = (a.t + 31) / 32;
+  a.ny = (a.oc2 * 16 + 63) / 64;
+  const int nks = a.units_pad / 2;
+  const size_t lds = (size_t)36 * 32 * 32 * sizeof(float) + 4 * 216 * sizeof(float4);   // exchange + constants
+  dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
+  int ks_max = 8;
+  if (const char *env = getenv("EHIP_WINO_KS")) ks_max = atoi(env);
+  void (*kernel)(WinoFusedArgs) = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8>
+      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4> : k_wino_gemm_output<2>);
+  if (nks % 2 != 0) return hipErrorInvalidValue;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, grid, dim3(kBlock), lds, s, a);
   return hipGetLastError();
 }
 

@@ -28,8 +28,9 @@ def make_wino(n, ic, oc, hw, seed, with_bias=True, with_relu=True):
 
 
 @pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 10), (1, 64, 48, 12), (3, 16, 80, 7), (1, 32, 32, 28)])
-def test_wino_pipeline(n, ic, oc, hw):
+def test_wino_pipeline(n, ic, oc, hw, monkeypatch):
     import torch
+    monkeypatch.setenv("EHIP_WINO_FUSED", "0")   # three kernels: every stage can be inspected
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 100 + hw)
     d_x = dev(xb)
     # calibration of wino_tinput_quant from the fp32 transformed input
@@ -61,6 +62,31 @@ def test_wino_pipeline(n, ic, oc, hw):
     assert np.array_equal(bits(g_tout), bits(tout)), "GEMM result differs"
     got = host(d_out)
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d" % int((got != exp).sum())
+
+
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 10), (1, 64, 48, 12), (3, 16, 80, 7), (1, 32, 144, 28),
+                                        (2, 256, 64, 9), (1, 272, 32, 6)])
+def test_wino_fused_gemm_and_output_transform(n, ic, oc, hw):
+    """Default schedule: GEMM + output transform in one kernel; final output bit for bit."""
+    import torch
+    E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
+    s_t, z_t = 22.0 / 255.0, 104.0
+    p.tin_scale, p.tin_z = s_t, z_t
+    d.tinput_scale, d.tinput_z = s_t, z_t
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tin = ol.wino_trans_input(p, xb)
+    tout, _ = ol.wino_gemm(p, tin, twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias)
+    conv = E.Conv(d)
+    assert conv.kernel_name.endswith("k_wino_gemm_output")
+    d_b = dev(bias)
+    d_out = torch.full(exp.shape, -7.0, dtype=torch.float32, device="cuda")
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, dev(xb), None, d_b)
+    torch.cuda.synchronize()
+    assert np.array_equal(conv.query(E.Q_TINPUT_U8).reshape(tin.shape), tin)
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
 def test_wino_no_bias_no_relu():
