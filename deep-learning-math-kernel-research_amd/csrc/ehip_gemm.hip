@@ -33,7 +33,7 @@
 #define TRACE_POINT(i)                                                                             \
   do {                                                                                             \
     if (a.trace && lane == 0)                                                                      \
-      a.trace[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
+      a.trace[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
   } while (0)
 #else
 #define TRACE_POINT(i) do { } while (0)
@@ -67,9 +67,16 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
-  const int b = blockIdx.z;
-  const int pix0 = blockIdx.x * P_T;
-  const int oc0 = blockIdx.y * OC_T;
+  // Workgroups go to the 8 XCDs round-robin by their linear index.  The channel blocks of one pixel
+  // block are numbered so that they follow each other on ONE XCD: the first one pulls the pixels
+  // into that XCD's L2, the others find them there.
+  const int b = blockIdx.y;
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int by = seq % a.ny;
+  const int bx = (seq / a.ny) * 8 + xcd;
+  if (bx >= a.nx) return;   // whole workgroup (grid padded to a multiple of 8 pixel blocks)
+  const int pix0 = bx * P_T;
+  const int oc0 = by * OC_T;
   const int mw0 = (wave % WM) * TM * 32;   // wave's first row / pixel inside the workgroup tile
   const int pw0 = (wave / WM) * TN * 32;
   const int oc_real = a.oc2 * 16;
@@ -286,10 +293,13 @@ int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride)
   return best;
 }
 
-hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s)
+hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s)
 {
   const Variant &k = kVariants[variant];
-  dim3 grid((a.p_total + k.p_t - 1) / k.p_t, (a.oc2 * 16 + k.oc_t - 1) / k.oc_t, nbatch);
+  GemmArgs a = a0;
+  a.nx = (a.p_total + k.p_t - 1) / k.p_t;
+  a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
+  dim3 grid(8 * a.ny * ((a.nx + 7) / 8), nbatch);
   // prefetch depth: must divide the number of fills.  Measured on the configured layers depth 2 is
   // as good as it gets (depth 4 costs registers and gains nothing); EHIP_GEMM_DEPTH overrides.
   const int nchunks = a.units_pad / k.kc;

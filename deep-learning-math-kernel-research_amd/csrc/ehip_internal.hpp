@@ -47,6 +47,7 @@ struct GemmArgs {
   int ocpp;             // padded rows in the packed weights
   long long in_batch_stride;   // bytes
   long long out_batch_stride;  // elements
+  int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
 };
 
