@@ -132,7 +132,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU: every layer is a single-device kernel and nothing here "
-              "shards across devices (batch-parallel sharding is described in DESIGN.md); use --gpus 1",
+              "shards across devices (the layers would shard by batch: every image is independent); use --gpus 1",
               file=sys.stderr)
         sys.exit(2)
 

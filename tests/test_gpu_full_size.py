@@ -1,4 +1,4 @@
-"""The configured layers at their full sizes (BASELINE configs C1..C5) through the C-ABI.
+"""The configured layers at their full sizes (workloads C1..C5b of workloads.py) through the C-ABI.
 
 Direct 1x1 / 3x3 / depthwise layers are compared bit for bit with the CPU oracle over the whole
 batch.  The Winograd layers run at full batch on the GPU; every image is an independent problem, so
