@@ -95,13 +95,14 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   // `first`: the weight operands of pair 0 are requested right behind the first batch of pixel
   // loads -- loads return in order, and the pixels are needed first (LDS store, barrier).
   const int nk = a.chunk_units / G;    // units per thread and pass
+  constexpr int SB = 8;                // loads in flight per thread: one round trip for up to 8 units
   auto stage = [&](int chunk, bool first) {
 #pragma unroll
     for (int p = 0; p < NPASS; ++p) {
-      for (int k0 = 0; k0 < nk; k0 += 4) {
-        v4i t[4];
+      for (int k0 = 0; k0 < nk; k0 += SB) {
+        v4i t[SB];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < SB; ++j) {
           const int k = k0 + j < nk ? k0 + j : nk - 1;
           int u = chunk * a.chunk_units + ug + G * k;
           u = u < a.ic2 ? u : a.ic2 - 1;   // padded units multiply zero weights
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
           for (int tap = 0; tap < 9; ++tap) load_a(tap, 0);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < SB; ++j) {
           if (k0 + j < nk) {
             const v4i x = t[j] ^ (int)0x80808080;
             const v4i z = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
