@@ -54,6 +54,14 @@ def build(verbose=True, jobs=8):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    # a small client of the C++ API (include/euler.hpp), used by the GPU tests
+    check = os.path.join(objdir, "euler_api_check")
+    cmd = [hipcc, "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cxx", "euler_api_check.cpp"), "-o", check,
+           "-L" + HERE, "-leuler_hip", "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/.."]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
     return LIB
 
 
