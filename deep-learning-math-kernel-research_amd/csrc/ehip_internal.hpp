@@ -273,10 +273,12 @@ __device__ __forceinline__ unsigned quant4(const Epilogue &ep, int a0, int a1, i
     // saturate" is a clamp to the code range and one v_cvt_pk_u8_f32 per byte, which rounds to
     // nearest even (the wave's float mode, never changed here) and saturates to 0..255 itself
     const float hi = OUT == EHIP_S8 ? __builtin_fminf(ep.hi, 127.0f) : ep.hi;
-    f0 = __builtin_fminf(__builtin_fmaxf(f0, ep.lo), hi);
-    f1 = __builtin_fminf(__builtin_fmaxf(f1, ep.lo), hi);
-    f2 = __builtin_fminf(__builtin_fmaxf(f2, ep.lo), hi);
-    f3 = __builtin_fminf(__builtin_fmaxf(f3, ep.lo), hi);
+    // lo <= hi here, so min(max(f, lo), hi) is the median of the three -- also for a NaN f, where
+    // v_med3_f32 falls back to min3 = lo, which is what max(NaN, lo) = lo gives the reference
+    f0 = __builtin_amdgcn_fmed3f(f0, ep.lo, hi);
+    f1 = __builtin_amdgcn_fmed3f(f1, ep.lo, hi);
+    f2 = __builtin_amdgcn_fmed3f(f2, ep.lo, hi);
+    f3 = __builtin_amdgcn_fmed3f(f3, ep.lo, hi);
     unsigned q = __builtin_amdgcn_cvt_pk_u8_f32(f0, 0, 0);
     q = __builtin_amdgcn_cvt_pk_u8_f32(f1, 1, q);
     q = __builtin_amdgcn_cvt_pk_u8_f32(f2, 2, q);
@@ -393,7 +395,8 @@ __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&a
 #define EHIP_EPI(OUT, SUM, FAST, XP)                                                                              \
   epilogue_wave_typed<TM, TN, OUT, SUM, FAST, XP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, \
                                                   out, xlds, pixT, validT)
-  const bool fast = ep.with_relu && ep.lo >= 0.0f && ep.hi >= ep.lo;
+  // cheap narrowing: ReLU bounds 0 <= lo <= hi (and lo inside the s8 code range for s8 output)
+  const bool fast = ep.with_relu && ep.lo >= 0.0f && ep.hi >= ep.lo && (ep.out_type != EHIP_S8 || ep.lo <= 127.0f);
   switch (ep.out_type) {
   case EHIP_U8:
     if (ep.with_sum) { if (fast) EHIP_EPI(EHIP_U8, true, true, false); else EHIP_EPI(EHIP_U8, true, false, false); }
