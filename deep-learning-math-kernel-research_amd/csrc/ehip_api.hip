@@ -107,8 +107,17 @@ int classify(ehip_conv *c)
     if (d.input_scale == kNoCali || d.input_z == kNoCali) return fail(EHIP_GENERAL_ERROR, "input_quant is not set");
     if (out_q && (d.output_scale == kNoCali || d.output_z == kNoCali || d.output_scale == 0.0f))
       return fail(EHIP_GENERAL_ERROR, "output_quant is not set");
-    if (d.input_fmt != EHIP_NCHW16C || d.output_fmt != EHIP_NCHW16C)
-      return fail(EHIP_UNIMPLEMENTED, "only the blocked nChw16c activation format is built");
+    // nhwc activations (src/elx_int8_conv_direct_1x1.cpp:374-396,417-468, src/elx_int8_conv_direct.cpp:596-668)
+    // are built for the 1x1 GEMM family; the reference refuses channel tails there as well
+    // ("Or not support", src/elx_int8_conv_direct_1x1.cpp:88-91)
+    const bool in_ok = d.input_fmt == EHIP_NCHW16C || d.input_fmt == EHIP_NHWC;
+    const bool out_ok = d.output_fmt == EHIP_NCHW16C || d.output_fmt == EHIP_NHWC;
+    if (!in_ok || !out_ok) return fail(EHIP_UNIMPLEMENTED, "activation formats: nChw16c or nhwc");
+    const bool any_nhwc = d.input_fmt == EHIP_NHWC || d.output_fmt == EHIP_NHWC;
+    if (any_nhwc && !(d.kh == 1 && d.kw == 1 && !depthwise))
+      return fail(EHIP_UNIMPLEMENTED, "nhwc activations are only built for 1x1 convolutions");
+    if ((d.input_fmt == EHIP_NHWC && d.ic % 16) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
+      return fail(EHIP_UNIMPLEMENTED, "nhwc: channel counts must be multiples of 16");
   }
 
   if (d.algorithm == EHIP_CONV_DIRECT_1X1) {
@@ -418,6 +427,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ihw = d.ih * d.iw; a.iw = d.iw;
     a.stride_h = d.stride_h; a.stride_w = d.stride_w;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    a.in_nhwc = d.input_fmt == EHIP_NHWC; a.out_nhwc = d.output_fmt == EHIP_NHWC;
     a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
     HIP_TRY(launch_gemm(a, 1, c->variant, s));
     break;

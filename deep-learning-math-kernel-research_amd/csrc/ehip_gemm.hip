@@ -41,7 +41,7 @@
 
 namespace ehip {
 
-template <int WM, int WN, int TM, int TN, int KC, int D>
+template <int WM, int WN, int TM, int TN, int KC, int D, bool NHWC>
 __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 {
   constexpr int OC_T = WM * TM * 32;
@@ -84,25 +84,31 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   TRACE_POINT(0);
 
   // ---- staging plan ---------------------------------------------------------------------------
-  // B: a thread always copies the same pixel (tid % P_T), units tid / P_T + j * BU of a fill.
-  const uint8_t *inb = a.in + (long long)b * a.in_batch_stride;
-  {
-    int gp = pix0 + tid % P_T;
+  // Byte offset of output pixel gp's first input cell (unit 0); nhwc: the pixel's channel vector.
+  auto input_pixel = [&](int gp) -> long long {
     gp = gp < a.p_total ? gp : a.p_total - 1;
     const int n = a.ohw == a.p_total ? 0 : fastdiv(gp, a.ohw, a.ohw_magic);
     const int r = gp - n * a.ohw;
-    long long off;
+    long long sp;   // pixel index inside the image
     if (dense) {
-      off = (long long)n * a.ic2 * a.ihw + r;
+      sp = r;
     } else {
       const int oh = fastdiv(r, a.ow, a.ow_magic);
       const int ow = r - oh * a.ow;
-      off = (long long)n * a.ic2 * a.ihw + (long long)(oh * a.stride_h) * a.iw + ow * a.stride_w;
+      sp = (long long)(oh * a.stride_h) * a.iw + ow * a.stride_w;
     }
-    inb += off * 16;
-  }
-  const int bu0 = tid / P_T;
-  const long long unit_stride = (long long)a.ihw * 16;
+    return NHWC ? ((long long)n * a.ihw + sp) * a.ic2 * 16 : ((long long)n * a.ic2 * a.ihw + sp) * 16;
+  };
+  // B, blocked input: a thread always copies the same pixel (tid % P_T), units tid / P_T + j * BU of
+  // a fill (a unit's pixels are contiguous).  B, nhwc input: cell id = tid + j * 256 -> pixel
+  // id / KC, unit id % KC (a pixel's units are contiguous: KC lanes read 16 * KC consecutive bytes).
+  constexpr int NPIX = NHWC ? NB : 1;
+  const uint8_t *inb[NPIX];
+#pragma unroll
+  for (int j = 0; j < NPIX; ++j)
+    inb[j] = a.in + (long long)b * a.in_batch_stride + input_pixel(pix0 + (NHWC ? (tid + j * kBlock) / KC : tid % P_T));
+  const int bu0 = NHWC ? tid % KC : tid / P_T;
+  const long long unit_stride = NHWC ? 16 : (long long)a.ihw * 16;
   // A: cell id = tid + j * 256 -> unit id / OC_T, row id % OC_T; rows of a unit are contiguous.
   const int8_t *wb = a.w + (long long)b * a.units_pad * a.ocpp * 16 + (long long)oc0 * 16;
   const long long w_unit = (long long)a.ocpp * 16;
@@ -118,17 +124,23 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      int u = chunk * KC + bu0 + j * BU;
+      int u = chunk * KC + bu0 + (NHWC ? 0 : j * BU);
       u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
-      stb[d][j] = *reinterpret_cast<const v4i *>(inb + (long long)u * unit_stride);
+      stb[d][j] = *reinterpret_cast<const v4i *>(inb[NHWC ? j : 0] + (long long)u * unit_stride);
     }
   };
+  // LDS keeps B as [unit][pixel].  The nhwc plan writes one pixel's KC units from neighbouring
+  // lanes, which would all land in the same banks: there pixel p of unit u sits at p ^ (2u & 15),
+  // a permutation inside every aligned group of 16 pixels that spreads those writes over all banks
+  // and leaves the reads (32 consecutive pixels of one unit) conflict free.
   auto store_stage = [&](int buf, int d) {
 #pragma unroll
     for (int j = 0; j < NA; ++j) lds_a[buf][tid + j * kBlock] = sta[d][j];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      lds_b[buf][tid + j * kBlock] = stb[d][j] ^ (int)0x80808080;
+      const int id = tid + j * kBlock;
+      const int cell = NHWC ? (id % KC) * P_T + ((id / KC) ^ ((2 * (id % KC)) & 15)) : id;
+      lds_b[buf][cell] = stb[d][j] ^ (int)0x80808080;
     }
   };
 
@@ -144,7 +156,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   v4i opa[2][TM], opb[2][TN];
   auto read_ops = [&](int buf, int ks, int slot) {
     const v4i *pa = &lds_a[buf][(2 * ks + lh) * OC_T + mw0 + l32];
-    const v4i *pb = &lds_b[buf][(2 * ks + lh) * P_T + pw0 + l32];
+    const v4i *pb = &lds_b[buf][(2 * ks + lh) * P_T + pw0 + (NHWC ? l32 ^ ((4 * ks + 2 * lh) & 15) : l32)];
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) opa[slot][mt] = pa[mt * 32];
 #pragma unroll
@@ -204,9 +216,11 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   TRACE_POINT(6);
 
   // ---- epilogue ------------------------------------------------------------------------------
+  // element offset of output pixel gp's cell in 16-channel block 0 (nhwc: its channel vector)
   auto pixel_offset = [&](int gp, bool &valid) -> size_t {
     valid = gp < a.p_total;
     const int gpc = valid ? gp : 0;
+    if (a.out_nhwc) return (size_t)gpc * oc_real;
     const int n = a.ohw == a.p_total ? 0 : fastdiv(gpc, a.ohw, a.ohw_magic);
     const int r = gpc - n * a.ohw;
     return (size_t)b * a.out_batch_stride + ((size_t)n * a.oc2 * a.ohw + r) * 16;
@@ -221,13 +235,13 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   }
   // 4-byte outputs are exchanged through a wave-private 4 KB patch of the (now idle) operand LDS
   v4i *xlds = nullptr;
-  if (a.ep.out_type == EHIP_F32 || a.ep.out_type == EHIP_S32) {
+  if ((a.ep.out_type == EHIP_F32 || a.ep.out_type == EHIP_S32) && !a.out_nhwc) {
     __syncthreads();   // every wave has read its last operands
     xlds = lds + wave * 256;
   }
   TRACE_POINT(14);
-  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real, (size_t)a.ohw * 16, a.out, xlds,
-                        pixT, validT);
+  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real,
+                        a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT);
   TRACE_POINT(15);
 }
 
@@ -235,18 +249,21 @@ namespace {
 struct Variant {
   const char *name;
   int oc_t, p_t, kc;
-  void (*kernel[3])(GemmArgs);   // prefetch depth 1, 2, 4 (null: too many staging registers)
+  void (*kernel[2][3])(GemmArgs);   // [nhwc input][prefetch depth 1, 2, 4] (null: too many staging registers)
 };
 // depth 4 only where four fills of staging fit in 96 registers
-template <int WM, int WN, int TM, int TN, int KC>
+template <int WM, int WN, int TM, int TN, int KC, bool NHWC>
 constexpr void (*deep_or_null())(GemmArgs)
 {
-  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4>;
+  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4, NHWC>;
   else return nullptr;
 }
 #define V(WM, WN, TM, TN, KC)                                                                    \
   { "k_gemm_u8s8<" #WM "," #WN "," #TM "," #TN "," #KC ">", WM * TM * 32, WN * TN * 32, KC,       \
-    { k_gemm_u8s8<WM, WN, TM, TN, KC, 1>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2>, deep_or_null<WM, WN, TM, TN, KC>() } }
+    { { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false>,                       \
+        deep_or_null<WM, WN, TM, TN, KC, false>() },                                                              \
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true>,                         \
+        deep_or_null<WM, WN, TM, TN, KC, true>() } } }
 const Variant kVariants[] = {
     V(2, 2, 2, 2, 8),  // 0: 128 oc x 128 px
     V(2, 2, 2, 1, 8),  // 1: 128 oc x  64 px
@@ -306,8 +323,9 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   int dl = 1;
   const char *env = getenv("EHIP_GEMM_DEPTH");
   if (env && env[0]) dl = atoi(env) >= 4 ? 2 : (atoi(env) >= 2 ? 1 : 0);
-  while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[dl])) --dl;
-  hipLaunchKernelGGL(k.kernel[dl], grid, dim3(kBlock), 0, s, a);
+  const int fmt = a.in_nhwc ? 1 : 0;
+  while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[fmt][dl])) --dl;
+  hipLaunchKernelGGL(k.kernel[fmt][dl], grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
 

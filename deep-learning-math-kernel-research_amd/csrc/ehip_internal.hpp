@@ -47,6 +47,7 @@ struct GemmArgs {
   int ocpp;             // padded rows in the packed weights
   long long in_batch_stride;   // bytes
   long long out_batch_stride;  // elements
+  int in_nhwc, out_nhwc;       // activations as [n][h][w][c] instead of [n][c/16][h][w][16] (c % 16 == 0)
   int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
 };

@@ -9,8 +9,8 @@ algorithmic.
 """
 import math
 
-from . import (CONV_DIRECT, CONV_DIRECT_1X1, CONV_WINOGRAD, EL_NO_CALI, F32, FLT_MAX, S8, U8, Conv, make_desc,
-               up16, wino_tinput_range)
+from . import (CONV_DIRECT, CONV_DIRECT_1X1, CONV_WINOGRAD, EL_NO_CALI, F32, FLT_MAX, NHWC, S8, U8, Conv,
+               make_desc, up16, wino_tinput_range)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
@@ -18,11 +18,12 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 class Workload:
     def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
-                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False):
+                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False):
         self.key, self.title = key, title
         self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
         self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
         self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
+        self.nhwc = nhwc   # activations [n][h][w][c] on both sides instead of nChw16c
         self.oh = (hw + 2 * pad - k) // stride + 1
 
     # 2 * MACs, padded taps excluded
@@ -73,14 +74,17 @@ class Workload:
         if self.out_type == S8:
             relu = (0.0, 127.0)
         g = self.ic if self.depthwise else 1
-        return make_desc(self.n, self.ic, self.oc, self.hw, self.hw, self.k, self.k, self.pad, self.stride, g=g,
-                         algorithm=self.algorithm, input_type=self.in_type, output_type=self.out_type,
-                         with_bias=True, with_relu=True, with_ip_sum=self.with_sum,
-                         input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, 0.0),
-                         output_quant=(out_scale, 0.0), sum_quant=(0.7, 0.0) if self.with_sum else (0.0, 0.0),
-                         wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
-                         tile_size=6 if self.algorithm == CONV_WINOGRAD else 0,
-                         execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
+        d = make_desc(self.n, self.ic, self.oc, self.hw, self.hw, self.k, self.k, self.pad, self.stride, g=g,
+                      algorithm=self.algorithm, input_type=self.in_type, output_type=self.out_type,
+                      with_bias=True, with_relu=True, with_ip_sum=self.with_sum,
+                      input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, 0.0),
+                      output_quant=(out_scale, 0.0), sum_quant=(0.7, 0.0) if self.with_sum else (0.0, 0.0),
+                      wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
+                      tile_size=6 if self.algorithm == CONV_WINOGRAD else 0,
+                      execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
+        if self.nhwc:
+            d.input_fmt = d.output_fmt = NHWC
+        return d
 
 
 WORKLOADS = {w.key: w for w in [
@@ -91,6 +95,12 @@ WORKLOADS = {w.key: w for w in [
              algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True),
     Workload("C3b", "1x1 s2 512->1024 28x28->14x14 N=64, sum+ReLU, s8 out (ResNet-50 res4 projection)", 64, 512, 1024,
              28, stride=2, algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True),
+    # the same two layers with nhwc activations, as the reference's tuned ResNet-v1.5 run feeds them
+    # (scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh:62 "--input-format=nhwc --output-format=nhwc")
+    Workload("C3a_nhwc", "1x1 1024->256 @14x14 N=64, sum+ReLU, s8 out, nhwc activations", 64, 1024, 256, 14,
+             algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True, nhwc=True),
+    Workload("C3b_nhwc", "1x1 s2 512->1024 28x28->14x14 N=64, sum+ReLU, s8 out, nhwc activations", 64, 512, 1024,
+             28, stride=2, algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True, nhwc=True),
     Workload("C4a", "Winograd F(4,3) 256->256 @56x56 N=64, fp32 in/out (VGG-16 conv3)", 64, 256, 256, 56, k=3, pad=1,
              algorithm=CONV_WINOGRAD, in_type=F32, out_type=F32, w_sigma=0.02),
     Workload("C4b", "Winograd F(4,3) 512->512 @28x28 N=64, fp32 in/out (VGG-16 conv4)", 64, 512, 512, 28, k=3, pad=1,
@@ -114,6 +124,7 @@ class DeviceLayer:
         ic2, oc2 = up16(wl.ic) // 16, up16(wl.oc) // 16
         if wl.in_type == U8:
             # fp32 U[0,1) activations quantized with scale 1/255 are uniform codes 0..255
+            # (random codes: the nhwc tensor has the same number of bytes, only their meaning differs)
             self.x = torch.randint(0, 256, (wl.n, ic2, wl.hw, wl.hw, 16), dtype=torch.uint8, device="cuda",
                                    generator=gen)
         else:

@@ -33,12 +33,14 @@ class Layer:
     parameters and the product's descriptor side by side."""
 
     def __init__(self, n, ic, oc, hw, k=1, pad=0, stride=1, out_type=ol.U8, algorithm=None, with_sum=False,
-                 depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None):
+                 depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None,
+                 in_nhwc=False, out_nhwc=False):
         E = pkg()
         rng = np.random.default_rng(seed)
         self.E = E
         self.n, self.ic, self.oc, self.hw, self.k = n, ic, oc, hw, k
         self.depthwise = depthwise
+        self.in_nhwc, self.out_nhwc = in_nhwc, out_nhwc
         g = ic if depthwise else 1
         x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
         self.x_u8 = ol.quantize_input_u8(x, 1.0 / 255.0, 0.0)
@@ -78,6 +80,10 @@ class Layer:
                                 output_type=out_type, with_bias=with_bias, with_relu=with_relu, with_ip_sum=with_sum,
                                 output_quant=(out_scale, 0.0), sum_quant=(sum_scale, 0.0),
                                 relu_bound=(0.0, relu_hi), flatting_t=T)
+        if in_nhwc:
+            self.desc.input_fmt = E.NHWC
+        if out_nhwc:
+            self.desc.output_fmt = E.NHWC
 
     # ---- oracle -----------------------------------------------------------------------------
     def oracle(self):
@@ -100,6 +106,8 @@ class Layer:
                 out = acc
             else:
                 out, acc = ol.direct_execute(p, self.xb, wq, scale, shift, out_init=self.old)
+        if self.out_nhwc:   # the arithmetic does not depend on the layout: only the index map changes
+            out = ol.blocked_to_nhwc(out, self.oc)
         return dict(wq=wq, scale=scale, shift=shift, wsum=wsum, out=out, acc=acc)
 
     # ---- product ----------------------------------------------------------------------------
@@ -107,12 +115,12 @@ class Layer:
         import torch
         E = self.E
         conv = E.Conv(self.desc)
-        d_x, d_w, d_b = dev(self.xb), dev(self.wb), dev(self.bias)
+        d_x, d_w, d_b = dev(ol.blocked_to_nhwc(self.xb, self.ic) if self.in_nhwc else self.xb), dev(self.wb), dev(self.bias)
         oc2 = ol.up16(self.oc) // 16
-        shape = (self.n, oc2, self.desc.oh, self.desc.ow, 16)
+        shape = (self.n, self.desc.oh, self.desc.ow, self.oc) if self.out_nhwc else (self.n, oc2, self.desc.oh, self.desc.ow, 16)
         tdt = {ol.U8: torch.uint8, ol.S8: torch.int8, ol.F32: torch.float32, ol.S32: torch.int32}[self.p.out_type]
         if self.old is not None:
-            d_out = dev(self.old)
+            d_out = dev(ol.blocked_to_nhwc(self.old, self.oc) if self.out_nhwc else self.old)
         else:
             d_out = torch.full(shape, 77, dtype=tdt, device="cuda")
         if lazy_prepare:

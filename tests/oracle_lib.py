@@ -130,6 +130,13 @@ def from_blocked(xb, c):
     return np.ascontiguousarray(xb.transpose(0, 1, 4, 2, 3).reshape(n, c2 * 16, h, w)[:, :c])
 
 
+def blocked_to_nhwc(xb, c):
+    """nChw16c -> nhwc = [n][h][w][c] (the reference indexes it as [n*h*w][c],
+    src/elx_int8_conv_direct_1x1.cpp:417-425)"""
+    n, c2, h, w, _ = xb.shape
+    return np.ascontiguousarray(xb.transpose(0, 2, 3, 1, 4).reshape(n, h, w, c2 * 16)[..., :c])
+
+
 def weights_to_blocked(wt):
     """oihw -> OIhw16i16o"""
     o, i, kh, kw = wt.shape

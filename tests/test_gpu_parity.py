@@ -61,6 +61,38 @@ def test_conv1x1_every_kernel_variant(variant, monkeypatch):
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
+# nhwc activations on either side (src/elx_int8_conv_direct_1x1.cpp:374-396,417-468); the expected
+# values are the oracle's, moved through the closed-form index map [n][c/16][h][w][16] -> [n][h][w][c]
+@pytest.mark.parametrize("in_nhwc,out_nhwc", [(True, True), (True, False), (False, True)])
+@pytest.mark.parametrize("out_type", [ol.S32, ol.U8, ol.S8, ol.F32])
+def test_conv1x1_nhwc(in_nhwc, out_nhwc, out_type):
+    run_and_compare(Layer(3, 128, 272 if not out_nhwc else 176, 5, out_type=out_type, seed=70 + out_type,
+                          in_nhwc=in_nhwc, out_nhwc=out_nhwc))
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_conv1x1_nhwc_sum_relu(stride):
+    run_and_compare(Layer(2, 96, 64, 14, stride=stride, out_type=ol.S8, with_sum=True, seed=75, in_nhwc=True, out_nhwc=True))
+
+
+@pytest.mark.parametrize("variant", range(7))
+def test_conv1x1_nhwc_every_kernel_variant(variant, monkeypatch):
+    monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
+    run_and_compare(Layer(2, 144, 80, 11, out_type=ol.U8, with_sum=True, seed=80 + variant, in_nhwc=True, out_nhwc=True))
+
+
+def test_nhwc_is_refused_where_it_is_not_built():
+    E = pkg()
+    d = E.make_desc(1, 40, 64, 8, 8, algorithm=E.CONV_DIRECT_1X1)
+    d.input_fmt = E.NHWC   # channel tail
+    with pytest.raises(E.EulerHipError):
+        E.Conv(d)
+    d = E.make_desc(1, 64, 64, 8, 8, 3, 3, 1, algorithm=E.CONV_DIRECT)
+    d.output_fmt = E.NHWC  # 3x3
+    with pytest.raises(E.EulerHipError):
+        E.Conv(d)
+
+
 # ---- 3x3 direct (c160) ------------------------------------------------------------------------------
 @pytest.mark.parametrize("out_type", [ol.S32, ol.U8, ol.S8, ol.F32])
 @pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 14), (1, 128, 128, 28), (2, 48, 80, 10), (1, 64, 16, 7)])
