@@ -163,12 +163,24 @@ int classify(ehip_conv *c)
       c->family = FAM_GEMM_1X1;
       return EHIP_OK;
     }
-    if (d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.pad_l <= 1 && d.pad_t <= 1) {
-      if (d.input_z != 0.0f && (d.pad_l || d.pad_t))
+    // c160 shapes (src/elx_int8_conv_direct.cpp:66-77): 3/5/7 kernels, stride 1 or 2, every pad
+    // k/2 - 1 or k/2.  Right and bottom pads follow from the output size, as the reference
+    // recomputes them (src/elx_conv.cpp:36-37).
+    const bool k_ok = (d.kh == 3 || d.kh == 5 || d.kh == 7) && (d.kw == 3 || d.kw == 5 || d.kw == 7);
+    const bool s_ok = (d.stride_w == 1 || d.stride_w == 2) && (d.stride_h == 1 || d.stride_h == 2);
+    const int rp = (d.ow - 1) * d.stride_w + d.kw - d.iw - d.pad_l, bp = (d.oh - 1) * d.stride_h + d.kh - d.ih - d.pad_t;
+    auto pad_ok = [](int p, int k) { return p == k / 2 - 1 || p == k / 2; };
+    if (k_ok && s_ok && pad_ok(d.pad_l, d.kw) && pad_ok(d.pad_t, d.kh) && pad_ok(rp < 0 ? d.kw / 2 - 1 : rp, d.kw) &&
+        pad_ok(bp < 0 ? d.kh / 2 - 1 : bp, d.kh)) {
+      const bool padded = d.pad_l || d.pad_t || rp > 0 || bp > 0;
+      if (d.input_z != 0.0f && padded)
         return fail(EHIP_UNIMPLEMENTED, "direct: input zero point with padding is not built");
-      if (d.flatting_t > 0 && d.ow % (d.flatting_t > d.ow ? d.ow : d.flatting_t))
+      const int T = d.flatting_t > d.ow ? d.ow : d.flatting_t;
+      if (T > 0 && d.ow % T)
         return fail(EHIP_UNIMPLEMENTED, "direct: c160: ow must be a multiple of T (the reference mis-indexes shift for Tr != T)");
-      c->family = FAM_CONV_3X3;
+      const bool s1_3x3 = d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 &&
+          d.ow == d.iw + d.pad_l + d.pad_r - 2 && d.oh == d.ih + d.pad_t + d.pad_b - 2;
+      c->family = s1_3x3 ? FAM_CONV_3X3 : FAM_GEMM_1X1;   // the GEMM family walks [tap][unit] for kh x kw
       return EHIP_OK;
     }
     return fail(EHIP_UNIMPLEMENTED, "direct: c160: shape not supported");
@@ -209,28 +221,31 @@ int setup_workspace(ehip_conv *c)
   c->oc2 = up(d.oc, 16) / 16;
   int rc;
   switch (c->family) {
-  case FAM_GEMM_1X1: {
-    if ((long long)d.n * d.oh * d.ow * d.oh * d.ow >= (1ll << 32))
-      return fail(EHIP_UNIMPLEMENTED, "1x1: n*oh*ow*oh*ow must stay below 2^32");
-    c->taps = 1;
-    c->nbatch = 1;
-    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2, 1, d.stride_w);
-    c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
-    c->kernel_name = gemm_variant_name(c->variant);
-    break;
-  }
   case FAM_CONV_3X3: {
     c->taps = 9;
     c->nbatch = 1;
-    if (d.ow != d.iw + d.pad_l + d.pad_r - 2 || d.oh != d.ih + d.pad_t + d.pad_b - 2)
-      return fail(EHIP_GENERAL_ERROR, "direct 3x3: output size does not match input size and padding");
     if ((long long)(d.oh + 2) * (d.ow + 2) * (d.ow + 2) >= (1ll << 31))
       return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too large");
     c->variant = conv3x3v_pick_variant(d.n, d.oh, d.ow, c->oc2);
-    if (c->variant < 0) return fail(EHIP_UNIMPLEMENTED, "direct 3x3: rows too wide for the staged tile");
-    c->chunk_units = conv3x3v_chunk_units(c->variant, c->ic2);
-    c->units_pad = up(c->ic2, c->chunk_units);
-    c->kernel_name = conv3x3v_variant_name(c->variant);
+    if (c->variant >= 0) {
+      c->chunk_units = conv3x3v_chunk_units(c->variant, c->ic2);
+      c->units_pad = up(c->ic2, c->chunk_units);
+      c->kernel_name = conv3x3v_variant_name(c->variant);
+      break;
+    }
+    c->family = FAM_GEMM_1X1;   // rows too wide for the staged tile: the GEMM form has no such limit
+  }
+  // fall through
+  case FAM_GEMM_1X1: {
+    if ((long long)d.n * d.oh * d.ow * d.oh * d.ow >= (1ll << 32))
+      return fail(EHIP_UNIMPLEMENTED, "direct: n*oh*ow*oh*ow must stay below 2^32");
+    c->taps = d.kh * d.kw;
+    c->nbatch = 1;
+    if (c->taps > 1 && (long long)d.n * c->ic2 * d.ih * d.iw * 16 >= (1ll << 40))
+      return fail(EHIP_UNIMPLEMENTED, "direct: input too large");
+    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2 * c->taps, 1, c->taps > 1 ? 1 : d.stride_w);
+    c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
+    c->kernel_name = gemm_variant_name(c->variant);
     break;
   }
   case FAM_DEPTHWISE: {
@@ -428,6 +443,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.stride_h = d.stride_h; a.stride_w = d.stride_w;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
     a.in_nhwc = d.input_fmt == EHIP_NHWC; a.out_nhwc = d.output_fmt == EHIP_NHWC;
+    a.kh = d.kh; a.kw = d.kw; a.pad_t = d.pad_t; a.pad_l = d.pad_l; a.ih = d.ih;
     a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
     HIP_TRY(launch_gemm(a, 1, c->variant, s));
     break;

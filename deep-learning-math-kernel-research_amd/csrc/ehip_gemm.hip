@@ -41,9 +41,10 @@
 
 namespace ehip {
 
-template <int WM, int WN, int TM, int TN, int KC, int D, bool NHWC>
+template <int WM, int WN, int TM, int TN, int KC, int D, bool NHWC, bool CONV>
 __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 {
+  static_assert(!(NHWC && CONV), "the kh x kw form is built for blocked input only");
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
   constexpr int KS = KC / 2;               // MFMA k-steps per fill
@@ -80,11 +81,15 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const int mw0 = (wave % WM) * TM * 32;   // wave's first row / pixel inside the workgroup tile
   const int pw0 = (wave / WM) * TN * 32;
   const int oc_real = a.oc2 * 16;
-  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  const bool dense = !CONV && a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
   TRACE_POINT(0);
 
   // ---- staging plan ---------------------------------------------------------------------------
   // Byte offset of output pixel gp's first input cell (unit 0); nhwc: the pixel's channel vector.
+  // kh x kw form (CONV): the cell under tap (0, 0), which may lie outside the image, and the set of
+  // taps that fall inside it.
+  unsigned long long tapmask = 0;
+  long long safe_off = 0;   // a cell of the same image that every unit offset keeps in bounds
   auto input_pixel = [&](int gp) -> long long {
     gp = gp < a.p_total ? gp : a.p_total - 1;
     const int n = a.ohw == a.p_total ? 0 : fastdiv(gp, a.ohw, a.ohw_magic);
@@ -95,7 +100,14 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     } else {
       const int oh = fastdiv(r, a.ow, a.ow_magic);
       const int ow = r - oh * a.ow;
-      sp = (long long)(oh * a.stride_h) * a.iw + ow * a.stride_w;
+      const int ih0 = oh * a.stride_h - (CONV ? a.pad_t : 0), iw0 = ow * a.stride_w - (CONV ? a.pad_l : 0);
+      sp = (long long)ih0 * a.iw + iw0;
+      if (CONV) {
+        for (int kh = 0; kh < a.kh; ++kh)
+          for (int kw = 0; kw < a.kw; ++kw)
+            if (ih0 + kh >= 0 && ih0 + kh < a.ih && iw0 + kw >= 0 && iw0 + kw < a.iw) tapmask |= 1ull << (kh * a.kw + kw);
+        safe_off = (long long)n * a.ic2 * a.ihw * 16;
+      }
     }
     return NHWC ? ((long long)n * a.ihw + sp) * a.ic2 * 16 : ((long long)n * a.ic2 * a.ihw + sp) * 16;
   };
@@ -107,6 +119,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 #pragma unroll
   for (int j = 0; j < NPIX; ++j)
     inb[j] = a.in + (long long)b * a.in_batch_stride + input_pixel(pix0 + (NHWC ? (tid + j * kBlock) / KC : tid % P_T));
+  const uint8_t *safe = a.in + safe_off;
   const int bu0 = NHWC ? tid % KC : tid / P_T;
   const long long unit_stride = NHWC ? 16 : (long long)a.ihw * 16;
   // A: cell id = tid + j * 256 -> unit id / OC_T, row id % OC_T; rows of a unit are contiguous.
@@ -114,19 +127,33 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const long long w_unit = (long long)a.ocpp * 16;
 
   v4i sta[D][NA], stb[D][NB];   // D fills in flight (global -> registers), see the main loop
+  bool stv[D];                  // CONV: the fill's tap lies inside the image for this thread's pixel
   // All global loads of the main loop are unconditional (indices clamped): without branches
   // between a load and its use the compiler counts outstanding loads exactly.
+  // CONV: the K axis is [tap][unit]; a fill never straddles two taps (KC divides the padded units),
+  // the packed weights are contiguous in that order, and the input cell of tap (kh, kw) sits
+  // (kh * iw + kw) cells behind the one of tap (0, 0).  Taps outside the image read a safe cell and
+  // are replaced by u8 0 on the way to LDS, which contributes nothing -- the reference skips them.
   auto load_stage = [&](int chunk, int d) {
 #pragma unroll
     for (int j = 0; j < NA; ++j) {
       const int id = tid + j * kBlock;
       sta[d][j] = *reinterpret_cast<const v4i *>(wb + (long long)(chunk * KC + id / OC_T) * w_unit + (id % OC_T) * 16);
     }
+    int ub = chunk * KC;
+    const uint8_t *src0 = inb[0];
+    if (CONV) {
+      const int tap = fastdiv(chunk, a.chunks_per_tap, a.cpt_magic);
+      ub = (chunk - tap * a.chunks_per_tap) * KC;
+      const int kh = fastdiv(tap, a.kw, a.kw_magic);
+      stv[d] = (tapmask >> tap) & 1;
+      src0 = stv[d] ? inb[0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * 16 : safe;
+    }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      int u = chunk * KC + bu0 + (NHWC ? 0 : j * BU);
+      int u = ub + bu0 + (NHWC ? 0 : j * BU);
       u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
-      stb[d][j] = *reinterpret_cast<const v4i *>(inb[NHWC ? j : 0] + (long long)u * unit_stride);
+      stb[d][j] = *reinterpret_cast<const v4i *>((CONV ? src0 : inb[NHWC ? j : 0]) + (long long)u * unit_stride);
     }
   };
   // LDS keeps B as [unit][pixel].  The nhwc plan writes one pixel's KC units from neighbouring
@@ -140,7 +167,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     for (int j = 0; j < NB; ++j) {
       const int id = tid + j * kBlock;
       const int cell = NHWC ? (id % KC) * P_T + ((id / KC) ^ ((2 * (id % KC)) & 15)) : id;
-      lds_b[buf][cell] = stb[d][j] ^ (int)0x80808080;
+      const v4i x = (CONV && !stv[d]) ? v4i{0, 0, 0, 0} : stb[d][j];
+      lds_b[buf][cell] = x ^ (int)0x80808080;
     }
   };
 
@@ -178,7 +206,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     }
   };
 
-  const int nchunks = a.units_pad / KC;
+  const int nchunks = a.k_units / KC;
   // The layers this kernel serves are small: what a workgroup waits for is the latency of its
   // global loads, not their bandwidth.  So D fills are kept in flight in registers: the loads of
   // fill c + D are issued when fill c moves to LDS.  The launcher picks D so that it divides the
@@ -249,21 +277,22 @@ namespace {
 struct Variant {
   const char *name;
   int oc_t, p_t, kc;
-  void (*kernel[2][3])(GemmArgs);   // [nhwc input][prefetch depth 1, 2, 4] (null: too many staging registers)
+  void (*kernel[3][3])(GemmArgs);   // [blocked | nhwc | blocked kh x kw][prefetch depth 1, 2, 4] (null: not built)
 };
 // depth 4 only where four fills of staging fit in 96 registers
 template <int WM, int WN, int TM, int TN, int KC, bool NHWC>
 constexpr void (*deep_or_null())(GemmArgs)
 {
-  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4, NHWC>;
+  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4, NHWC, false>;
   else return nullptr;
 }
 #define V(WM, WN, TM, TN, KC)                                                                    \
   { "k_gemm_u8s8<" #WM "," #WN "," #TM "," #TN "," #KC ">", WM * TM * 32, WN * TN * 32, KC,       \
-    { { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false>,                       \
+    { { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, false>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, false>,         \
         deep_or_null<WM, WN, TM, TN, KC, false>() },                                                              \
-      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true>,                         \
-        deep_or_null<WM, WN, TM, TN, KC, true>() } } }
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true, false>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true, false>,           \
+        deep_or_null<WM, WN, TM, TN, KC, true>() },                                                               \
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, true>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, true>, nullptr } } }
 const Variant kVariants[] = {
     V(2, 2, 2, 2, 8),  // 0: 128 oc x 128 px
     V(2, 2, 2, 1, 8),  // 1: 128 oc x  64 px
@@ -319,11 +348,17 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8), nbatch);
   // prefetch depth: must divide the number of fills.  Measured on the configured layers depth 2 is
   // as good as it gets (depth 4 costs registers and gains nothing); EHIP_GEMM_DEPTH overrides.
-  const int nchunks = a.units_pad / k.kc;
+  const int taps = a.kh * a.kw > 1 ? a.kh * a.kw : 1;
+  a.k_units = taps * a.units_pad;
+  a.chunks_per_tap = a.units_pad / k.kc;
+  a.cpt_magic = div_magic(a.chunks_per_tap);
+  a.kw_magic = div_magic(a.kw > 0 ? a.kw : 1);
+  const int nchunks = a.k_units / k.kc;
   int dl = 1;
   const char *env = getenv("EHIP_GEMM_DEPTH");
   if (env && env[0]) dl = atoi(env) >= 4 ? 2 : (atoi(env) >= 2 ? 1 : 0);
-  const int fmt = a.in_nhwc ? 1 : 0;
+  if (taps > 1 && (a.in_nhwc || taps > 64 || nbatch != 1)) return hipErrorInvalidValue;
+  const int fmt = taps > 1 ? 2 : (a.in_nhwc ? 1 : 0);
   while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[fmt][dl])) --dl;
   hipLaunchKernelGGL(k.kernel[fmt][dl], grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();

@@ -48,6 +48,9 @@ struct GemmArgs {
   long long in_batch_stride;   // bytes
   long long out_batch_stride;  // elements
   int in_nhwc, out_nhwc;       // activations as [n][h][w][c] instead of [n][c/16][h][w][16] (c % 16 == 0)
+  int kh, kw, pad_t, pad_l, ih;   // kh * kw > 1: direct convolution as a GEMM over [tap][unit] (blocked input)
+  int k_units, chunks_per_tap;    // set by the launcher: taps * units_pad, units_pad / KC
+  unsigned cpt_magic, kw_magic;
   int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
 };

@@ -34,7 +34,7 @@ class Layer:
 
     def __init__(self, n, ic, oc, hw, k=1, pad=0, stride=1, out_type=ol.U8, algorithm=None, with_sum=False,
                  depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None,
-                 in_nhwc=False, out_nhwc=False):
+                 in_nhwc=False, out_nhwc=False, out_hw=None):
         E = pkg()
         rng = np.random.default_rng(seed)
         self.E = E
@@ -80,6 +80,12 @@ class Layer:
                                 output_type=out_type, with_bias=with_bias, with_relu=with_relu, with_ip_sum=with_sum,
                                 output_quant=(out_scale, 0.0), sum_quant=(sum_scale, 0.0),
                                 relu_bound=(0.0, relu_hi), flatting_t=T)
+        if out_hw is not None:
+            # output size given by the caller: right / bottom pads follow from it, as the reference
+            # recomputes them (src/elx_conv.cpp:36-37)
+            assert not with_sum
+            self.p.oh = self.p.ow = self.desc.oh = self.desc.ow = out_hw
+            self.desc.pad_r = self.desc.pad_b = max(0, (out_hw - 1) * stride + k - hw - pad)
         if in_nhwc:
             self.desc.input_fmt = E.NHWC
         if out_nhwc:

@@ -121,6 +121,33 @@ def test_conv3x3_wide_rows():
     run_and_compare(Layer(1, 16, 32, 70, k=3, pad=1, out_type=ol.U8, seed=92))
 
 
+# ---- k x k direct as a GEMM over [tap][unit]: stride 2, 5x5 / 7x7, one-sided pads (c160 shapes,
+# src/elx_int8_conv_direct.cpp:66-77) ----------------------------------------------------------------
+@pytest.mark.parametrize("out_type", [ol.S32, ol.U8, ol.S8, ol.F32])
+@pytest.mark.parametrize("n,ic,oc,hw,k,pad,stride,out_hw", [
+    (2, 32, 32, 15, 3, 0, 2, None),     # pre-padded input, as the tuned ResNet-v1.5 run feeds it
+    (2, 64, 48, 14, 3, 1, 2, None),     # pad 1 on every side
+    (1, 48, 80, 14, 3, 0, 2, 7),        # pads only right / bottom (output size fixes them)
+    (1, 32, 32, 12, 5, 2, 1, None),
+    (1, 16, 32, 17, 7, 3, 2, None),
+    (2, 128, 64, 9, 5, 1, 2, None),
+])
+def test_direct_kxk_strided(out_type, n, ic, oc, hw, k, pad, stride, out_hw):
+    res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=90 + k + stride,
+                                out_hw=out_hw))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
+@pytest.mark.parametrize("variant", range(7))
+def test_direct_3x3_stride2_every_kernel_variant(variant, monkeypatch):
+    monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
+    run_and_compare(Layer(2, 80, 96, 13, k=3, pad=1, stride=2, out_type=ol.U8, seed=120 + variant))
+
+
+def test_direct_3x3_very_wide_rows():
+    run_and_compare(Layer(1, 16, 16, 240, k=3, pad=1, out_type=ol.U8, seed=130))
+
+
 # ---- depthwise 3x3 ----------------------------------------------------------------------------------
 @pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
 @pytest.mark.parametrize("g,hw,T", [(32, 14, 7), (144, 56, 14), (64, 7, 7), (16, 28, 11), (32, 9, 4), (32, 5, 0)])
