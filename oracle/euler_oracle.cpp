@@ -497,7 +497,9 @@ int orc_depthwise_execute(const orc_conv_params *p, const uint8_t *input, const 
                           const float *scale, const float *shift, void *output, int32_t *acc_out)
 {
   const int G2 = up16(p->g) / 16, IH = p->ih, IW = p->iw, OH = p->oh, OW = p->ow;
-  if (p->kh != 3 || p->kw != 3 || p->stride_h != 1 || p->stride_w != 1) return -1;
+  // stride 1 and 2 share everything but the input index (the kernel's S template parameter,
+  // src/kernel/elk_u8s8_depthwise_conv.hxx:153,176-178,371-403)
+  if (p->kh != 3 || p->kw != 3 || p->stride_h < 1 || p->stride_h > 2 || p->stride_w != p->stride_h) return -1;
   if (p->out_type != ORC_U8 && p->out_type != ORC_S8) return -1;
   const int T = p->T > 0 ? std::min(p->T, OW) : 1;
   const int wt = (OW + T - 1) / T;
@@ -517,10 +519,10 @@ int orc_depthwise_execute(const orc_conv_params *p, const uint8_t *input, const 
               const int g = g2 * 16 + v;
               int32_t a = 0;
               for (int kh = 0; kh < 3; ++kh) {
-                int ih = oh + kh - p->pad_t;
+                int ih = oh * p->stride_h + kh - p->pad_t;
                 if (ih < 0 || ih >= IH) continue;
                 for (int kw = 0; kw < 3; ++kw) {
-                  int iw = ow + kw - p->pad_l;
+                  int iw = ow * p->stride_w + kw - p->pad_l;
                   if (iw < 0 || iw >= IW) continue;
                   a += (int32_t)in[((size_t)ih * IW + iw) * 16 + v] * (int32_t)wq[(size_t)g * 9 + kh * 3 + kw];
                 }

@@ -75,23 +75,23 @@ void run_gemm_ccc(elx_param_t &ep, float *toutput, void *ooutput, uint8_t *input
       nullptr, nullptr, wscale, wshift);
 }
 
-template <typename OT, int T>
+template <typename OT, int T, int S = 1>
 void run_dw(elx_param_t &ep, void *routput, uint8_t *input, int8_t *weights,
     float *wscale, float *wshift, int khs, int khe, int pad_l, int pad_r, int attr)
 {
   using ker = u8s8_depthwise_conv_kernel<conv_impl::INT8_F32, OT, 16, 4, ISA_AVX512,
-      estl::integer_sequence<1, GKF_DCD, 1, T, 3>>;
+      estl::integer_sequence<S, GKF_DCD, 1, T, 3>>;
   ker::conv(ep, nullptr, (OT *)routput, input, weights, nullptr, nullptr, nullptr,
       wscale, wshift, khs, khe, 0, 3, pad_l, pad_r, attr);
 }
 
-template <typename OT, int T>
+template <typename OT, int T, int S = 1>
 void run_conv3(elx_param_t &ep, float *toutput, void *routput, uint8_t *input,
     int8_t *weights, float *wscale, float *wshift, int khs, int khe, int kws,
     int kwe, int pad_l, int pad_r, int attr)
 {
   using ker = u8s8_conv_kernel<conv_impl::INT8_F32, OT, 16, 4, ISA_AVX512,
-      estl::integer_sequence<1, GKF_DCD, 1, T, 3>>;
+      estl::integer_sequence<S, GKF_DCD, 1, T, 3>>;
   ker::conv(ep, toutput, (OT *)routput, input, weights, nullptr, nullptr, nullptr,
       wscale, wshift, khs, khe, kws, kwe, pad_l, pad_r, attr);
 }
@@ -208,6 +208,89 @@ int ref_u8s8_conv3x3(int out_kind, int T, int I2, int ih, int iw, int oh, int ow
   CV_CASE(1, uint8_t, 7) CV_CASE(1, uint8_t, 14)
   CV_CASE(2, int8_t, 7) CV_CASE(2, int8_t, 14)
 #undef CV_CASE
+  return -1;
+}
+
+// The same 3x3 micro-kernel at stride 2 with independent left / right / top pads (0 or 1), set up
+// as conv_c160 does (src/elx_int8_conv_direct.cpp:502-571) and bound as the executor binds it:
+// the "lean left padding" instantiation S2_LLP when lp > rp, plain 2 otherwise
+// (src/elx_int8_conv_direct_bind.hpp:108-117).  T = 7.
+// Note for rp = 1: this 3x3-specialised template applies the kw = 2 tap to all T positions at
+// stride 2 (unroll_for(_T, T - 1 + S - 1), src/kernel/elk_u8s8_conv.hxx:829-884), i.e. it reads the
+// pixel behind the row's end for the last output column, where the template for other kernel
+// sizes (:341-347) skips that position.  The golden cases therefore keep rp = 0.
+int ref_u8s8_conv3x3_s2(int out_kind, int T, int I2, int ih, int iw, int oh, int ow,
+    int _ht, int _wt, int tp, int lp, int rp, int with_relu, float relu_lo, float relu_hi,
+    float *toutput, void *routput, uint8_t *input, int8_t *weights, float *wscale,
+    float *wshift)
+{
+  elx_param_t ep;
+  fill_common(ep, relu_lo, relu_hi, 0.f);
+  ep.kh = ep.kw = 3; ep.I2 = I2; ep.ic2 = I2; ep.IC = ep.ic = 16 * I2;
+  ep.OC = ep.oc = 16; ep.oc2 = 1;
+  ep.ih = ih; ep.iw = iw; ep.oh = oh; ep.ow = ow; ep.T = T;
+  ep.hs = ep.ws = 2;
+  ep.tp = tp; ep.lp = lp; ep.rp = rp; ep.bp = 0;
+  const int wt = (ow + T - 1) / T;
+  int khs = tp - 2 * _ht > 0 ? tp - 2 * _ht : 0;
+  int khe = 3 < ih + tp - 2 * _ht ? 3 : ih + tp - 2 * _ht;
+  int kws = _wt == 0 ? lp : 0;
+  int kwe = _wt == wt - 1 ? 3 - rp : 3;
+  int pad_l = _wt == 0 ? lp : 0;
+  int pad_r = _wt == wt - 1 ? rp : 0;
+  int cih = 2 * _ht + 1 - tp, ciw = 2 * _wt * T + 1 - lp;
+  uint8_t *in = input + ((long)cih * iw + ciw) * 16;
+  size_t ooff = ((size_t)_ht * ow + _wt * T) * 16;
+  int attr = AT_CLEAR_OUTPUT_MASK | AT_RESTORE_OUTPUT_MASK
+      | (with_relu ? (int)AT_RELU_MASK : 0);
+#define CV_CASE(k, OT, t)                                                       \
+  if (out_kind == k && T == t) {                                                \
+    if (lp > rp)                                                                \
+      run_conv3<OT, t, S2_LLP>(ep, toutput ? toutput + ooff : nullptr,          \
+          routput ? (char *)routput + ooff * sizeof(OT) : nullptr, in, weights, \
+          wscale, wshift, khs, khe, kws, kwe, pad_l, pad_r, attr);              \
+    else                                                                        \
+      run_conv3<OT, t, 2>(ep, toutput ? toutput + ooff : nullptr,               \
+          routput ? (char *)routput + ooff * sizeof(OT) : nullptr, in, weights, \
+          wscale, wshift, khs, khe, kws, kwe, pad_l, pad_r, attr);              \
+    return 0;                                                                   \
+  }
+  CV_CASE(0, float, 7) CV_CASE(1, uint8_t, 7) CV_CASE(2, int8_t, 7)
+#undef CV_CASE
+  return -1;
+}
+
+// The depthwise micro-kernel at stride 2 (its S != 1 branch,
+// src/kernel/elk_u8s8_depthwise_conv.hxx:371-403), set up as conv_c160 of the depthwise executor
+// does (src/elx_int8_conv_direct_depthwise.cpp:294-319).  Tz in {4, 7}.
+int ref_u8s8_depthwise_s2(int out_kind, int T, int Tz, int G2, int ih, int iw, int oh, int ow,
+    int _ht, int _wt, int tp, int lp, int rp, int with_relu, float relu_lo,
+    float relu_hi, void *routput, uint8_t *input, int8_t *weights, float *wscale,
+    float *wshift)
+{
+  elx_param_t ep;
+  fill_common(ep, relu_lo, relu_hi, 0.f);
+  ep.kh = ep.kw = 3; ep.G2 = G2; ep.ic2 = G2; ep.oc2 = G2; ep.I2 = G2;
+  ep.ih = ih; ep.iw = iw; ep.oh = oh; ep.ow = ow; ep.T = T;
+  ep.hs = ep.ws = 2;
+  ep.tp = tp; ep.lp = lp; ep.rp = rp;
+  const int wt = (ow + T - 1) / T;
+  int khs = tp - 2 * _ht > 0 ? tp - 2 * _ht : 0;
+  int khe = 3 < ih + tp - 2 * _ht ? 3 : ih + tp - 2 * _ht;
+  int pad_l = (_wt == 0) && lp > 0;
+  int pad_r = (_wt == wt - 1) && rp > 0;
+  int cih = 2 * _ht + 1 - tp, ciw = 2 * _wt * T + 1 - lp;
+  uint8_t *in = input + ((long)cih * iw + ciw) * 16;
+  char *out = (char *)routput + ((size_t)_ht * ow + _wt * T) * 16;
+  int attr = with_relu ? (int)AT_RELU_MASK : 0;
+#define DW_CASE(k, OT, t)                                                       \
+  if (out_kind == k && Tz == t) {                                                \
+    run_dw<OT, t, 2>(ep, out, in, weights, wscale, wshift, khs, khe, pad_l,     \
+        pad_r, attr);                                                           \
+    return 0;                                                                   \
+  }
+  DW_CASE(1, uint8_t, 4) DW_CASE(1, uint8_t, 7) DW_CASE(2, int8_t, 7)
+#undef DW_CASE
   return -1;
 }
 

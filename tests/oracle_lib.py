@@ -33,12 +33,16 @@ FLT_MAX = float(np.finfo(np.float32).max)
 def make_params(n, ic, oc, ih, iw, kh=1, kw=1, pad=0, stride=1, g=1, out_type=U8, with_bias=True,
                 with_relu=True, with_sum=False, T=0, in_scale=1.0 / 255.0, in_z=0.0, out_scale=1.0,
                 out_z=0.0, sum_scale=0.0, sum_z=0.0, tin_scale=1.0, tin_z=0.0, relu_lo=0.0,
-                relu_hi=FLT_MAX):
+                relu_hi=FLT_MAX, pad_tl=None, out_hw=None):
+    """pad: on every side; pad_tl / out_hw: top-left pad and output size given separately (the right and
+    bottom pads are then whatever the output size implies, src/elx_conv.cpp:36-37)"""
     oh = (ih + 2 * pad - kh) // stride + 1
     ow = (iw + 2 * pad - kw) // stride + 1
+    if out_hw is not None:
+        oh, ow = out_hw
     p = ConvParams()
     p.n, p.g, p.ic, p.oc, p.ih, p.iw, p.oh, p.ow, p.kh, p.kw = n, g, ic, oc, ih, iw, oh, ow, kh, kw
-    p.pad_t = p.pad_l = pad
+    p.pad_t = p.pad_l = pad if pad_tl is None else pad_tl
     p.stride_h = p.stride_w = stride
     p.out_type, p.with_bias, p.with_relu, p.with_sum, p.T = out_type, int(with_bias), int(with_relu), int(with_sum), T
     p.in_scale, p.in_z, p.out_scale, p.out_z = in_scale, in_z, out_scale, out_z
@@ -102,6 +106,9 @@ def ref_kernels():
         lib.ref_u8s8_gemm.argtypes = [ci, ci, ci, ci, ci, fl, fl, fl, vp, vp, vp, vp, vp, vp]
         lib.ref_u8s8_depthwise.argtypes = [ci] * 14 + [fl, fl, vp, vp, vp, vp, vp]
         lib.ref_u8s8_conv3x3.argtypes = [ci] * 11 + [fl, fl, vp, vp, vp, vp, vp, vp]
+        if hasattr(lib, "ref_u8s8_conv3x3_s2"):
+            lib.ref_u8s8_conv3x3_s2.argtypes = [ci] * 13 + [fl, fl, vp, vp, vp, vp, vp, vp]
+            lib.ref_u8s8_depthwise_s2.argtypes = [ci] * 14 + [fl, fl, vp, vp, vp, vp, vp]
         lib.ref_wino_trans_input.argtypes = [ci, ci, ci, vp, vp, ci, ci, ci, ci]
         lib.ref_wino_trans_weights.argtypes = [vp, vp]
         lib.ref_wino_trans_output.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ci, ci]
