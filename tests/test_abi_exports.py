@@ -55,7 +55,7 @@ def test_library_loads_and_binding_matches_header():
 def test_create_rejects_bad_descriptors_without_a_gpu():
     """Descriptor validation is host logic and runs before any device call."""
     pkg = importlib.import_module("deep-learning-math-kernel-research_amd")
-    d = pkg.make_desc(1, 64, 64, 8, 8, 5, 5, pad=2, algorithm=pkg.CONV_DIRECT)
+    d = pkg.make_desc(1, 64, 64, 9, 9, 3, 3, pad=1, stride=3, algorithm=pkg.CONV_DIRECT)
     h = ctypes.c_void_p()
     rc = pkg.lib.ehip_conv_create(ctypes.byref(d), ctypes.byref(h))
     assert rc == pkg.EHIP_UNIMPLEMENTED and not h.value

@@ -216,7 +216,8 @@ def test_setup_rejects_what_the_reference_rejects():
     bad = [
         E.make_desc(1, 64, 64, 8, 8, 1, 1, pad=1, algorithm=E.CONV_DIRECT_1X1),            # padding in 1x1
         E.make_desc(1, 64, 64, 8, 8, 3, 3, pad=1, algorithm=E.CONV_DIRECT_1X1),            # not a 1x1
-        E.make_desc(1, 64, 64, 8, 8, 5, 5, pad=2, algorithm=E.CONV_DIRECT),                # 5x5 not built
+        E.make_desc(1, 64, 64, 9, 9, 3, 3, pad=1, stride=3, algorithm=E.CONV_DIRECT),      # stride 3
+        E.make_desc(1, 64, 64, 8, 8, 5, 5, pad=0, algorithm=E.CONV_DIRECT),                # pad below k/2 - 1
         E.make_desc(1, 64, 64, 8, 8, 3, 3, pad=1, algorithm=E.CONV_DIRECT, sampling_kind=E.FINE),
         E.make_desc(1, 24, 24, 8, 8, 3, 3, pad=1, g=24, algorithm=E.CONV_DIRECT),          # g % 16
         E.make_desc(1, 64, 64, 8, 8, 1, 1, algorithm=E.CONV_DIRECT_1X1, output_type=E.F32),
