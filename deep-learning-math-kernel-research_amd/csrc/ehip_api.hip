@@ -141,7 +141,8 @@ int classify(ehip_conv *c)
       if (!(out_q || d.output_type == EHIP_S32)) return fail(EHIP_UNIMPLEMENTED, "depthwise: only u8/s8 output");
       if (d.kh != 3 || d.kw != 3 || d.pad_l > 1 || d.pad_t > 1)
         return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: int8: shape not supported");
-      if (d.stride_h != 1 || d.stride_w != 1) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: stride 2 is not built");
+      if (d.stride_h != d.stride_w || d.stride_h < 1 || d.stride_h > 2)
+        return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: stride must be 1 or 2");
       if (d.g % 16) return fail(EHIP_UNIMPLEMENTED, "conv: g blocking error for depthwise conv");
       if (d.weights_fmt != EHIP_GOIHW) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: format not supported");
       if (d.with_ip_sum) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: no sum fusion");
@@ -473,6 +474,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.out = output_dev;
     a.scale = c->scale; a.shift = c->shift; a.wsum = c->wsum;
     a.n = d.n; a.g2 = c->oc2; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
+    a.stride = d.stride_h;
     a.pad_t = d.pad_t; a.pad_l = d.pad_l;
     a.T = c->T; a.Tr = c->Tr; a.wt = c->wtb;
     a.out_type = d.output_type; a.with_relu = d.with_relu;

@@ -1,4 +1,4 @@
-// Depthwise 3x3 stride-1 u8 x s8 convolution with fused requantization: a bandwidth kernel.
+// Depthwise 3x3 u8 x s8 convolution (stride 1 and 2) with fused requantization: a bandwidth kernel.
 //
 // Replaces elx_int8_conv_direct_depthwise_t::__execute_c160 + conv_c160
 // (src/elx_int8_conv_direct_depthwise_xopt.hpp:19-66, src/elx_int8_conv_direct_depthwise.cpp:294-319)
@@ -15,6 +15,11 @@
 // against weights packed [kh][channel][kw0 kw1 kw2 0] -- and the same dword serves the second
 // column against the weights shifted by one byte.  The packed layout is the reference's own
 // ([g/16][kh][16][KW=4], src/elx_int8_conv_direct_depthwise.cpp:224-236).
+//
+// Stride 2 (the micro-kernel's S template parameter, src/kernel/elk_u8s8_depthwise_conv.hxx:371-403):
+// the lane's two output columns sit two input pixels apart, so a fifth pixel is loaded and one more
+// v_perm_b32 per channel splices it behind pixels 2 and 3 of the transposed dword; an output row
+// reads input rows 2r .. 2r + 2.
 //
 // The u8 store reproduces the reference's width-block rule: inside every block of T output columns
 // (Tr for the last block) the columns before 4*floor(Tz/4) are rounded toward -infinity and
@@ -35,9 +40,11 @@ __device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel)
 // round-to-nearest both land in the code range, so the pack-with-saturation instruction, which
 // rounds to nearest even itself, finishes either).  MODE 2: as 1 with lo == 0 and hi == 255, where
 // the clamp is the instruction's own saturation.
-template <int RB, int MODE>
+template <int RB, int MODE, int S>
 __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 {
+  constexpr int NPX = S == 1 ? 4 : 5;          // input pixels per row a lane touches
+  constexpr int NROWS = S * (RB - 1) + 3;      // input rows
   // grid: x = blocks over one plane's lanes (q fastest, then column pair, then row block),
   // y = 16-channel block, z = image
   const int wp = (a.ow + 1) >> 1;
@@ -73,11 +80,11 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 
   // the 4 input columns of this lane (clamped; invalid ones are replaced after the load); all
   // addresses are 32-bit byte offsets from the tensor base (the launcher checks the size)
-  unsigned coloff[4];
-  bool colok[4];
+  unsigned coloff[NPX];
+  bool colok[NPX];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int iw = c0 - a.pad_l + k;
+  for (int k = 0; k < NPX; ++k) {
+    const int iw = S * c0 - a.pad_l + k;
     colok[k] = iw >= 0 && iw < a.iw;
     coloff[k] = (unsigned)(iw < 0 ? 0 : (iw >= a.iw ? a.iw - 1 : iw)) * 16u;
   }
@@ -85,14 +92,14 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
   const char *in_base = reinterpret_cast<const char *>(a.in);
 
 #pragma unroll
-  for (int hr = 0; hr < RB + 2; ++hr) {
-    const int ih = oh0 - a.pad_t + hr;
+  for (int hr = 0; hr < NROWS; ++hr) {
+    const int ih = S * oh0 - a.pad_t + hr;
     const bool rowok = ih >= 0 && ih < a.ih;
     const int ihc = ih < 0 ? 0 : (ih >= a.ih ? a.ih - 1 : ih);
     const unsigned row_off = plane_off + (unsigned)(ihc * a.iw) * 16u;
-    unsigned x[4];
+    unsigned x[NPX];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < NPX; ++k) {
       const unsigned v = *reinterpret_cast<const unsigned *>(in_base + (size_t)(row_off + coloff[k]));
       x[k] = (rowok && colok[k]) ? v ^ 0x80808080u : 0x80808080u;
     }
@@ -104,14 +111,21 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
     t[1] = perm(b0, a0, 0x07060302u);
     t[2] = perm(b1, a1, 0x05040100u);
     t[3] = perm(b1, a1, 0x07060302u);
+    // second column, stride 2: pixels 2, 3, 4 of channel j = bytes 2, 3 of t[j] and byte j of x[4]
+    unsigned t2[4];
+    if (S == 2) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t2[j] = perm(x[NPX - 1], t[j], 0x00040302u + ((unsigned)j << 16));
+    }
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const int kh = hr - r;  // input row ih feeds output row oh0 + r through kernel row kh
+      const int kh = hr - S * r;  // input row ih feeds output row oh0 + r through kernel row kh
       if (kh < 0 || kh > 2) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         acc[r][0][j] = __builtin_amdgcn_sdot4((int)t[j], (int)wa[kh][j], acc[r][0][j], false);
-        acc[r][1][j] = __builtin_amdgcn_sdot4((int)t[j], (int)wb[kh][j], acc[r][1][j], false);
+        if (S == 1) acc[r][1][j] = __builtin_amdgcn_sdot4((int)t[j], (int)wb[kh][j], acc[r][1][j], false);
+        else acc[r][1][j] = __builtin_amdgcn_sdot4((int)t2[j], (int)wa[kh][j], acc[r][1][j], false);
       }
     }
   }
@@ -168,18 +182,28 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 }
 
 namespace {
+template <int RB, int S>
+void launch_rbs(const DepthwiseArgs &a, int mode, dim3 grid, dim3 block, hipStream_t s)
+{
+  if (mode == 2) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 2, S>), grid, block, 0, s, a);
+  else if (mode == 1) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 1, S>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 0, S>), grid, block, 0, s, a);
+}
 template <int RB>
 void launch_rb(const DepthwiseArgs &a, int mode, dim3 grid, dim3 block, hipStream_t s)
 {
-  if (mode == 2) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 2>), grid, block, 0, s, a);
-  else if (mode == 1) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 1>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 0>), grid, block, 0, s, a);
+  if (a.stride == 2) launch_rbs<RB, 2>(a, mode, grid, block, s);
+  else launch_rbs<RB, 1>(a, mode, grid, block, s);
 }
 }  // namespace
 
 hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s)
 {
   DepthwiseArgs a = a0;
+  if (a.stride != 1 && a.stride != 2) {
+    set_error("depthwise: stride must be 1 or 2");
+    return hipErrorInvalidValue;
+  }
   // four rows per lane on tall planes, fewer where that would leave lanes idle
   const int rb = a.oh >= 16 ? 4 : (a.oh >= 7 ? 2 : 1);
   const int ohb = (a.oh + rb - 1) / rb;

@@ -76,6 +76,7 @@ struct DepthwiseArgs {
   const float *scale, *shift;  // [G]
   const int *wsum;      // [G] sum of the packed weights per channel
   int n, g2, ih, iw, oh, ow, pad_t, pad_l;
+  int stride;           // 1 or 2, both directions
   int T, Tr, wt;        // width blocking of the reference kernel (decides floor vs round per column)
   int lanes_per_plane;  // set by the launcher: row blocks x column pairs x 4
   unsigned wp_magic, T_magic;  // div_magic of the column pairs per row and of T

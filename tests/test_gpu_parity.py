@@ -164,6 +164,20 @@ def test_depthwise_u8_other_bounds(relu_hi, with_relu):
                           relu_hi=relu_hi, with_relu=with_relu))
 
 
+# stride 2 (MobileNet's down-sampling layers, scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh:48:
+# pad 0 with the output size asking for one pad row / column at the bottom / right)
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
+@pytest.mark.parametrize("g,hw,pad,out_hw,T", [(32, 14, 0, 7, 7), (64, 28, 1, None, 14), (16, 15, 0, None, 7), (48, 13, 1, None, 4),
+                                               (32, 56, 0, 28, 28), (32, 6, 1, None, 0)])
+def test_depthwise_stride2(out_type, g, hw, pad, out_hw, T):
+    run_and_compare(Layer(2, g, g, hw, k=3, pad=pad, stride=2, out_type=out_type, depthwise=True, seed=g + hw + T + 3,
+                          w_sigma=0.1, T=T, out_hw=out_hw))
+
+
+def test_depthwise_stride2_raw_sums():
+    run_and_compare(Layer(1, 32, 32, 11, k=3, pad=1, stride=2, out_type=ol.S32, depthwise=True, seed=78, w_sigma=0.1, T=3))
+
+
 def test_depthwise_odd_width_and_raw_sums():
     run_and_compare(Layer(1, 32, 32, 13, k=3, pad=1, out_type=ol.S32, depthwise=True, seed=23, w_sigma=0.1, T=13))
     run_and_compare(Layer(2, 16, 16, 11, k=3, pad=0, out_type=ol.U8, depthwise=True, seed=29, w_sigma=0.1, T=3))
