@@ -18,13 +18,14 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 class Workload:
     def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
-                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False):
+                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None):
         self.key, self.title = key, title
         self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
         self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
         self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
         self.nhwc = nhwc   # activations [n][h][w][c] on both sides instead of nChw16c
-        self.oh = (hw + 2 * pad - k) // stride + 1
+        # oh given: the right / bottom pads are whatever that output size needs (src/elx_conv.cpp:36-37)
+        self.oh = oh if oh is not None else (hw + 2 * pad - k) // stride + 1
 
     # 2 * MACs, padded taps excluded
     def ops(self):
@@ -84,6 +85,9 @@ class Workload:
                       execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
         if self.nhwc:
             d.input_fmt = d.output_fmt = NHWC
+        if d.oh != self.oh:
+            d.oh = d.ow = self.oh
+            d.pad_r = d.pad_b = max(0, (self.oh - 1) * self.stride + self.k - self.hw - self.pad)
         return d
 
 
@@ -101,6 +105,13 @@ WORKLOADS = {w.key: w for w in [
              algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True, nhwc=True),
     Workload("C3b_nhwc", "1x1 s2 512->1024 28x28->14x14 N=64, sum+ReLU, s8 out, nhwc activations", 64, 512, 1024,
              28, stride=2, algorithm=CONV_DIRECT_1X1, out_type=S8, with_sum=True, nhwc=True),
+    # stride-2 layers of the reference's tuned int8 runs
+    # (scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh conv2d_13: pre-padded 58x58 input;
+    #  scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh Conv2d_4_depthwise: pad only right / bottom)
+    Workload("R13", "3x3 s2 128->128 58x58->28x28 N=64 pad 0, bias+ReLU, s8 out (ResNet-50 v1.5 conv2d_13)", 64, 128, 128,
+             58, k=3, pad=0, stride=2, out_type=S8, T=14),
+    Workload("M4", "depthwise 3x3 s2 C=128 56x56->28x28 N=64, bias+ReLU6, u8 out (MobileNet-v1 Conv2d_4)", 64, 128, 128,
+             56, k=3, pad=0, stride=2, depthwise=True, w_sigma=0.1, T=28, relu6=True, oh=28),
     Workload("C4a", "Winograd F(4,3) 256->256 @56x56 N=64, fp32 in/out (VGG-16 conv3)", 64, 256, 256, 56, k=3, pad=1,
              algorithm=CONV_WINOGRAD, in_type=F32, out_type=F32, w_sigma=0.02),
     Workload("C4b", "Winograd F(4,3) 512->512 @28x28 N=64, fp32 in/out (VGG-16 conv4)", 64, 512, 512, 28, k=3, pad=1,
