@@ -34,7 +34,7 @@ class Layer:
 
     def __init__(self, n, ic, oc, hw, k=1, pad=0, stride=1, out_type=ol.U8, algorithm=None, with_sum=False,
                  depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None,
-                 in_nhwc=False, out_nhwc=False, out_hw=None):
+                 in_nhwc=False, out_nhwc=False, out_hw=None, x_blocked=None):
         E = pkg()
         rng = np.random.default_rng(seed)
         self.E = E
@@ -45,6 +45,9 @@ class Layer:
         x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
         self.x_u8 = ol.quantize_input_u8(x, 1.0 / 255.0, 0.0)
         self.xb = ol.to_blocked(self.x_u8)
+        if x_blocked is not None:   # u8 activations handed over by a previous layer
+            assert x_blocked.shape == self.xb.shape and x_blocked.dtype == np.uint8
+            self.xb = x_blocked
         if depthwise:
             self.w = rng.normal(0, w_sigma, (ic, k, k)).astype(f32)
             self.wb = self.w

@@ -224,6 +224,35 @@ def test_device_reorders():
     assert np.array_equal(host(dw), ol.weights_to_blocked(w))
 
 
+# ---- layers chained on the device (the reference's --output-as-input, tests/elt_conv.cpp:407-410):
+# the u8 output of one layer is the next layer's input without leaving the GPU; requantization to
+# the next layer's input scale is the producing layer's own epilogue ------------------------------------
+def test_three_layers_chained_on_the_device():
+    import torch
+    E = pkg()
+    l1 = Layer(2, 64, 96, 14, k=3, pad=1, out_type=ol.U8, seed=301, T=14)
+    o1 = l1.oracle()["out"]
+    l2 = Layer(2, 96, 96, 14, k=3, pad=1, out_type=ol.U8, depthwise=True, seed=302, w_sigma=0.1, T=14, x_blocked=o1)
+    o2 = l2.oracle()["out"]
+    l3 = Layer(2, 96, 48, 14, stride=2, out_type=ol.S8, seed=303, x_blocked=o2)
+    o3 = l3.oracle()["out"]
+    convs, bufs = [], []
+    for l in (l1, l2, l3):
+        c = E.Conv(l.desc)
+        c.prepare(dev(l.wb), dev(l.bias))
+        convs.append(c)
+        bufs.append(torch.zeros(tuple(l.oracle()["out"].shape), dtype=torch.int8 if l.p.out_type == ol.S8 else torch.uint8,
+                                device="cuda"))
+    x = dev(l1.xb)
+    convs[0].execute(bufs[0], x)
+    convs[1].execute(bufs[1], bufs[0])
+    convs[2].execute(bufs[2], bufs[1])
+    torch.cuda.synchronize()
+    assert np.array_equal(host(bufs[0]), o1)
+    assert np.array_equal(host(bufs[1]), o2)
+    assert np.array_equal(host(bufs[2]), o3)
+
+
 # ---- error behaviour of setup ---------------------------------------------------------------------------
 def test_setup_rejects_what_the_reference_rejects():
     E = pkg()
