@@ -722,7 +722,26 @@ int orc_wino_gemm(const orc_conv_params *p, const uint8_t *tinput, const int8_t 
   return 0;
 }
 
-int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const float *bias, float *output)
+// One output value after the tile transform: bias, [u8 / s8 output: * (1 / out_S) + ceil(out_z),
+// one rounding], ReLU as max(., 0) only, then round-to-nearest-even and saturate
+// (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:94-111,159-195; src/elx_int8_conv_wino.cpp:272-276).
+// The u8 conversion goes through an UNSIGNED 32-bit integer: anything below -0.5 becomes 0xffffffff
+// and saturates to 255.  Returns the code for u8 / s8, the float through *f32_out.
+int orc_wino_output_value(float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
+                          int with_relu, float *f32_out)
+{
+  float r = y;
+  if (with_bias) r += bias;
+  if (out_type == ORC_U8 || out_type == ORC_S8) r = fmaf(r, 1.0f / out_scale, std::ceil(out_z));
+  if (with_relu) r = r > 0.0f ? r : 0.0f;  // vmaxps(p, 0): no upper bound here
+  if (f32_out) *f32_out = r;
+  if (out_type == ORC_U8) return usat8(cvt_u32_rne(r));
+  if (out_type == ORC_S8) return ssat8(cvt_s32_rne(r));
+  return 0;
+}
+
+// output: f32, u8 or s8 nChw16c according to p->out_type
+int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const float *bias, void *output)
 {
   const WinoGeom g = wino_geom(p);
 #pragma omp parallel for collapse(2)
@@ -739,10 +758,13 @@ int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const 
               for (int j = 0; j < 4; ++j) {
                 int oh = 4 * th + i, ow = 4 * tw + j;
                 if (oh >= p->oh || ow >= p->ow) continue;
-                float r = y[4 * i + j];
-                if (p->with_bias) r += bias[o2 * 16 + v];
-                if (p->with_relu) r = r > 0.0f ? r : 0.0f;  // vmaxps(p, 0): no upper bound here
-                output[((((size_t)n * g.OC2 + o2) * p->oh + oh) * p->ow + ow) * 16 + v] = r;
+                float r;
+                const int q = orc_wino_output_value(y[4 * i + j], p->with_bias, p->with_bias ? bias[o2 * 16 + v] : 0.0f,
+                                                    p->out_type, p->out_scale, p->out_z, p->with_relu, &r);
+                const size_t oi = ((((size_t)n * g.OC2 + o2) * p->oh + oh) * p->ow + ow) * 16 + v;
+                if (p->out_type == ORC_U8) ((uint8_t *)output)[oi] = (uint8_t)q;
+                else if (p->out_type == ORC_S8) ((int8_t *)output)[oi] = (int8_t)q;
+                else ((float *)output)[oi] = r;
               }
           }
         }

@@ -84,7 +84,10 @@ int orc_depthwise_prepare(const orc_conv_params *p, const float *w_goihw, const 
 int orc_depthwise_execute(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
                           const float *scale, const float *shift, void *output, int32_t *acc);
 
-/* ---- Winograd F(4x4,3x3), int8 GEMM, fp32 user tensors ----
+/* ---- Winograd F(4x4,3x3), int8 GEMM ----
+ * User input fp32, or u8 codes handed over as floats (the reference converts the codes to float
+ * and transforms them as they are, src/kernel/elk_conv_wino_4x4_3x3_input.hxx:40-47; the input scale
+ * only enters the quantization factor in_S / tin_S).  User output fp32, u8 or s8 (p->out_type).
  * tiles: t = n*ht*wt + th*wt + tw (src/elx_conv_wino_trans_input.cpp:10-24).
  * twq [36][OCp][ICp] s8; tscale/tshift [36][OCp];
  * tinput [36][ICp/16][t][16] u8; toutput [36][OCp/16][t][16] f32. */
@@ -102,7 +105,11 @@ int orc_wino_gemm(const orc_conv_params *p, const uint8_t *tinput, const int8_t 
                   const float *tscale, const float *tshift, float *toutput, int32_t *acc);
 /* src/kernel/elk_conv_wino_4x4_3x3_output.hxx:19-201 + src/elx_conv_wino_trans_output.cpp:212-277 */
 int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const float *bias,
-                          float *output);
+                          void *output);
+/* what the output transform does to one value after Y = At M A (bias, output quantization, ReLU,
+ * rounding, saturation; src/kernel/elk_conv_wino_4x4_3x3_output.hxx:94-111,159-195) */
+int orc_wino_output_value(float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
+                          int with_relu, float *f32_out);
 
 /* single 6x6 / 3x3 / 4x4 tile transforms, exposed so they can be compared one-to-one with the
  * reference's compiled kernel templates */

@@ -345,4 +345,29 @@ void ref_wino_trans_output(int border, int with_bias, int with_relu, int oh, int
 #undef WO_CASE
 }
 
+// The same output transform storing u8 (out_kind 1) or s8 (2): * output_quant_repS + output_quant_z
+// before the ReLU, round-to-nearest and saturate in the store
+// (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:94-111,165-171).  `out` is an [oh][ow][16] byte plane.
+void ref_wino_trans_output_q(int out_kind, int border, int with_bias, int with_relu, int oh, int ow,
+    void *out, float *toutput, float *bias, int h_end, int w_end, float repS, float z)
+{
+  elx_param_t ep;
+  fill_common(ep, 0.f, FLT_MAX, 0.f);
+  ep.oh = oh; ep.ow = ow;
+  ep.output_quant_repS = repS;
+  ep.output_quant_z = z;
+#define WQ_CASE(k, OT, b, wb, wr)                                               \
+  if (out_kind == k && !!border == b && !!with_bias == wb && !!with_relu == wr) { \
+    elk_conv_wino_trans_output<float, OT, float, TKF_BLOCKED, b, wb, wr,        \
+        false, ISA_AVX512, 6, 3, 16>::execute(ep, (OT *)out, toutput, bias,     \
+        h_end, w_end);                                                          \
+    return;                                                                     \
+  }
+  WQ_CASE(1, uint8_t, false, true, true) WQ_CASE(1, uint8_t, false, true, false)
+  WQ_CASE(1, uint8_t, true, true, true) WQ_CASE(1, uint8_t, true, false, false)
+  WQ_CASE(2, int8_t, false, true, true) WQ_CASE(2, int8_t, false, false, false)
+  WQ_CASE(2, int8_t, true, true, false) WQ_CASE(2, int8_t, true, true, true)
+#undef WQ_CASE
+}
+
 } // extern "C"

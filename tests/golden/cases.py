@@ -356,6 +356,47 @@ def wino_out_oracle(d):
     return out
 
 
+# quantized store of the output transform (u8 / s8 user output)
+def wino_outq_inputs(kind, with_bias, with_relu, h_end, w_end, seed):
+    d = wino_out_inputs(with_bias, with_relu, h_end, w_end, seed)
+    d["kind"] = np.int32(kind)
+    d["out_scale"] = np.float32(0.0437)   # values of a few units land all over (and outside) the code range
+    d["out_z"] = np.float32(0.0 if kind == ol.S8 else 3.0)
+    return d
+
+
+def wino_outq_reference(d, ref):
+    kind = int(d["kind"])
+    out = ol.aligned((8, 8, 16), ol.NP_OF[kind], 99)
+    h_end, w_end = int(d["h_end"]), int(d["w_end"])
+    border = not (h_end == 3 and w_end == 3)
+    m, bias = _al(d["m"]), _al(d["bias"])
+    rep = np.float32(1.0) / d["out_scale"]
+    ref.ref_wino_trans_output_q(KIND_ID[kind], int(border), int(d["with_bias"]), int(d["with_relu"]), 8, 8, ol.ptr(out),
+                                ol.ptr(m), ol.ptr(bias), h_end, w_end, float(rep), float(np.ceil(d["out_z"])))
+    return np.array(out[:4, :4, :])
+
+
+def wino_outq_oracle(d):
+    kind = int(d["kind"])
+    out = np.full((4, 4, 16), 99, ol.NP_OF[kind])
+    y = np.zeros(16, np.float32)
+    fn = ol.oracle().orc_wino_output_value
+    fn.argtypes = [ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int,
+                   ctypes.c_void_p]
+    for c in range(16):
+        mm = np.ascontiguousarray(d["m"][:, :, c].ravel())
+        ol.oracle().orc_wino_tile_output(ol.ptr(mm), ol.ptr(y))
+        for i in range(4):
+            for j in range(4):
+                if i > int(d["h_end"]) or j > int(d["w_end"]):
+                    continue
+                q = fn(float(y[4 * i + j]), int(d["with_bias"]), float(d["bias"][c]), kind, float(d["out_scale"]),
+                       float(d["out_z"]), int(d["with_relu"]), None)
+                out[i, j, c] = np.array(q).astype(ol.NP_OF[kind])
+    return out
+
+
 # name -> (inputs, reference runner, oracle runner)
 CASES = {}
 for _k, _kn in ((ol.F32, "f32"), (ol.U8, "u8"), (ol.S8, "s8")):
@@ -384,6 +425,12 @@ for _k, _kn, _iw, _lp, _rp, _T in ((ol.U8, "u8", 15, 0, 0, 7), (ol.U8, "u8", 14,
     CASES["depthwise_s2_%s_w%d_l%d_r%d" % (_kn, _iw, _lp, _rp)] = (
         lambda k=_k, iw=_iw, lp=_lp, rp=_rp, T=_T: dw_s2_inputs(k, iw, lp, rp, T, 400 + iw + 2 * lp + rp + k), dw_s2_reference,
         dw_s2_oracle)
+for _k, _kn, _b, _r, _he, _we in ((ol.U8, "u8", 1, 1, 3, 3), (ol.U8, "u8", 1, 0, 3, 3), (ol.U8, "u8", 1, 1, 2, 1),
+                                  (ol.U8, "u8", 0, 0, 1, 3), (ol.S8, "s8", 1, 1, 3, 3), (ol.S8, "s8", 0, 0, 3, 3),
+                                  (ol.S8, "s8", 1, 0, 3, 2), (ol.S8, "s8", 1, 1, 0, 0)):
+    CASES["wino_output_%s_b%d_r%d_h%d_w%d" % (_kn, _b, _r, _he, _we)] = (
+        lambda k=_k, b=_b, r=_r, he=_he, we=_we: wino_outq_inputs(k, b, r, he, we, 500 + 16 * k + 8 * b + 4 * r + he + we),
+        wino_outq_reference, wino_outq_oracle)
 CASES["wino_weights"] = (lambda: wino_w_inputs(21), wino_w_reference, wino_w_oracle)
 for _h0, _w0 in ((2, 3), (-1, -1), (-1, 4), (3, -1), (7, 7), (7, 2), (-1, 7)):
     CASES["wino_input_h%d_w%d" % (_h0, _w0)] = (lambda h=_h0, w=_w0: wino_in_inputs(h, w, h * 13 + w + 50),

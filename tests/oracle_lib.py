@@ -112,6 +112,8 @@ def ref_kernels():
         lib.ref_wino_trans_input.argtypes = [ci, ci, ci, vp, vp, ci, ci, ci, ci]
         lib.ref_wino_trans_weights.argtypes = [vp, vp]
         lib.ref_wino_trans_output.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ci, ci]
+        if hasattr(lib, "ref_wino_trans_output_q"):
+            lib.ref_wino_trans_output_q.argtypes = [ci, ci, ci, ci, ci, ci, vp, vp, vp, ci, ci, fl, fl]
         _ref = lib
     return _ref
 
@@ -236,7 +238,7 @@ def wino_gemm(p, tin, twq, tscale, tshift):
 
 
 def wino_trans_output(p, tout, bias):
-    out = np.zeros((p.n, up16(p.oc) // 16, p.oh, p.ow, 16), np.float32)
+    out = np.zeros((p.n, up16(p.oc) // 16, p.oh, p.ow, 16), NP_OF[p.out_type])
     assert oracle().orc_wino_trans_output(ctypes.byref(p), ptr(tout), ptr(bias), ptr(out)) == 0
     return out
 
