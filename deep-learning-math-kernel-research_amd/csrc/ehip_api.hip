@@ -191,9 +191,14 @@ int classify(ehip_conv *c)
     if (d.stride_h != 1 || d.stride_w != 1 || d.kh != 3 || d.kw != 3)
       return fail(EHIP_UNIMPLEMENTED, "Algorithm CONV_WINOGRAD: data shape not supported");
     if (d.g != 1) return fail(EHIP_UNIMPLEMENTED, "winograd: groups are not supported");
-    if (!all_f32) return fail(EHIP_UNIMPLEMENTED, "winograd: only fp32 user tensors are built");
-    if ((d.execution_mode & 0xF00) != 0x100)
+    // user types (src/eld_conv.cpp:275-305): u8 input with f32 / u8 / s8 output always takes the int8
+    // implementation; all-f32 tensors take it when execution_mode says so
+    const bool u8_user = in_u8 && (out_q || d.output_type == EHIP_F32);
+    if (!all_f32 && !u8_user) return fail(EHIP_UNIMPLEMENTED, "winograd: user types must be f32 or u8 input with f32/u8/s8 output");
+    if (all_f32 && (d.execution_mode & 0xF00) != 0x100)
       return fail(EHIP_UNIMPLEMENTED, "winograd: only the int8 implementation (execution_mode 0xa1xx) is built");
+    if (out_q && (d.output_scale == kNoCali || d.output_z == kNoCali || d.output_scale == 0.0f))
+      return fail(EHIP_GENERAL_ERROR, "output_quant is not set");
     if (d.tile_size == 0) {
       const int t = d.n * ((d.oh + 3) / 4) * ((d.ow + 3) / 4);
       const int ocp = up(d.oc, 16);
@@ -284,7 +289,7 @@ int setup_workspace(ehip_conv *c)
       c->fused = !(env && env[0] == '0');
     }
     c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
-                              : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output_f32";
+                              : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output";
     c->tin_bytes = (size_t)36 * c->ic2 * c->t * 16;   // allocated with one pad unit behind it
     c->tout_bytes = c->fused ? 16 : (size_t)36 * c->oc2 * c->t * 16 * sizeof(float);
     if ((rc = dev_alloc(&c->tin, c->tin_bytes + (size_t)c->t * 16, true)) != EHIP_OK) return rc;
@@ -337,6 +342,13 @@ WinoArgs make_wino_args(const ehip_conv_desc_t &d, int ic2, int oc2)
   w.nt = w.ht * w.wt; w.t = w.nt * d.n;
   w.pad_t = d.pad_t; w.pad_l = d.pad_l;
   w.with_bias = d.with_bias; w.with_relu = d.with_relu;
+  w.in_u8 = d.input_type == EHIP_U8;
+  w.out_type = d.output_type;
+  if (d.output_type == EHIP_U8 || d.output_type == EHIP_S8) {
+    // src/elx_int8_conv_wino.cpp:272-276
+    w.out_repS = 1.0f / d.output_scale;
+    w.out_z = ceilf(d.output_z);
+  }
   return w;
 }
 
@@ -488,10 +500,11 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       ehip_conv_desc_t dc = d;
       dc.n = d.n - n0 < c->chunk_n ? d.n - n0 : c->chunk_n;
       WinoArgs w = make_wino_args(dc, c->ic2, c->oc2);
-      w.in = static_cast<const float *>(input_dev) + (size_t)n0 * c->ic2 * d.ih * d.iw * 16;
+      const size_t in_esz = d.input_type == EHIP_U8 ? 1 : 4, out_esz = d.output_type == EHIP_F32 ? 4 : 1;
+      w.in = static_cast<const uint8_t *>(input_dev) + (size_t)n0 * c->ic2 * d.ih * d.iw * 16 * in_esz;
       w.tin = c->tin;
       w.tout = c->tout;
-      w.out = static_cast<float *>(output_dev) + (size_t)n0 * c->oc2 * d.oh * d.ow * 16;
+      w.out = static_cast<uint8_t *>(output_dev) + (size_t)n0 * c->oc2 * d.oh * d.ow * 16 * out_esz;
       w.bias = static_cast<const float *>(bias_dev);
       // mrepS = input_S * (1 / tinput_S), z = ceil(tinput_z)
       // (src/elx_conv_wino_trans_input.cpp:617-618, src/elx_int8_conv_wino.cpp:270-276)
@@ -507,6 +520,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.n = w.n; f.ic2 = c->ic2; f.units_pad = c->units_pad; f.oc2 = c->oc2; f.ocpp = c->ocpp;
         f.oh = d.oh; f.ow = d.ow; f.ht = w.ht; f.wt = w.wt; f.nt = w.nt; f.t = w.t;
         f.with_bias = d.with_bias; f.with_relu = d.with_relu;
+        f.out_type = w.out_type; f.out_repS = w.out_repS; f.out_z = w.out_z;
         f.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
         HIP_TRY(launch_wino_gemm_output(f, s));
         continue;
@@ -628,11 +642,11 @@ EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *in
 {
   if (!desc || !input_dev || !min_out || !max_out) return fail(EHIP_GENERAL_ERROR, "null argument");
   const ehip_conv_desc_t &d = *desc;
-  if (d.kh != 3 || d.kw != 3 || d.stride_h != 1 || d.stride_w != 1 || d.input_type != EHIP_F32 ||
-      d.input_fmt != EHIP_NCHW16C)
-    return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 blocked 3x3 stride-1 layers only");
+  if (d.kh != 3 || d.kw != 3 || d.stride_h != 1 || d.stride_w != 1 ||
+      (d.input_type != EHIP_F32 && d.input_type != EHIP_U8) || d.input_fmt != EHIP_NCHW16C)
+    return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 or u8 blocked 3x3 stride-1 layers only");
   WinoArgs w = make_wino_args(d, up(d.ic, 16) / 16, up(d.oc, 16) / 16);
-  w.in = static_cast<const float *>(input_dev);
+  w.in = input_dev;
   unsigned *mm = nullptr;
   HIP_TRY(hipMalloc(reinterpret_cast<void **>(&mm), 2 * sizeof(unsigned)));
   const unsigned init[2] = {0xffffffffu, 0u};

@@ -85,11 +85,13 @@ struct DepthwiseArgs {
 };
 
 struct WinoArgs {
-  const float *in;      // [n][ic2][ih][iw][16] f32
+  const void *in;       // [n][ic2][ih][iw][16] f32, or u8 codes (in_u8)
   uint8_t *tin;         // [36][ic2][t][16]
   const float *tout;    // [36][oc2][t][16]
-  float *out;           // [n][oc2][oh][ow][16]
+  void *out;            // [n][oc2][oh][ow][16] f32 / u8 / s8 (out_type)
   const float *bias;
+  int in_u8, out_type;
+  float out_repS, out_z;   // u8 / s8 output: 1 / output_S, ceil(output_z)
   int n, ic2, oc2, ih, iw, oh, ow, ht, wt, nt, t, pad_t, pad_l;
   int blocks_interior;  // set by the input-transform launcher: blocks over tiles off the rim
   float mrepS, mz;      // input_S / tinput_S, ceil(tinput_z)
@@ -99,10 +101,12 @@ struct WinoArgs {
 struct WinoFusedArgs {
   const uint8_t *tin;   // [36][ic2][t][16] u8
   const int8_t *w;      // [36][units_pad][OCpp][16] s8
-  float *out;           // [n][oc2][oh][ow][16]
+  void *out;            // [n][oc2][oh][ow][16] f32 / u8 / s8 (out_type)
   const float *bias;
   const float *scale, *shift;  // [36][OCpp]
   const int *comp;
+  int out_type;
+  float out_repS, out_z;   // u8 / s8 output: 1 / output_S, ceil(output_z)
   int n, ic2, units_pad, oc2, ocpp, oh, ow, ht, wt, nt, t;
   int with_bias, with_relu;
   int nx, ny;           // set by the launcher: blocks of 32 tiles, of 64 channels

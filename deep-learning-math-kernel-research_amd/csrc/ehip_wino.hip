@@ -100,6 +100,13 @@ __device__ __forceinline__ float comp_of(const float4 &v, int k)
   return k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w));
 }
 
+// four u8 codes in a dword: the reference turns the codes into floats as they are
+// (src/kernel/elk_conv_wino_4x4_3x3_input.hxx:40-47)
+__device__ __forceinline__ float comp_of(const unsigned &v, int k)
+{
+  return (float)((v >> (8 * k)) & 0xffu);
+}
+
 // order-preserving map float -> unsigned, for atomicMin/atomicMax
 __device__ __forceinline__ unsigned f2ord(float f)
 {
@@ -124,6 +131,7 @@ __device__ __forceinline__ TileCoord tile_coord(const WinoArgs &a, int t)
   return c;
 }
 
+// the lane's four channels of the 36 pixels of a tile: float4 (f32 input) or 4 packed codes (u8)
 __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, float4 d[36])
 {
   const float4 *plane = reinterpret_cast<const float4 *>(a.in) +
@@ -135,6 +143,18 @@ __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &
       const int h = c.h0 + i, w = c.w0 + j;
       d[6 * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4]
                                                                    : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+__device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, unsigned d[36])
+{
+  const unsigned *plane = reinterpret_cast<const unsigned *>(a.in) +
+      ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4 + q;
+#pragma unroll
+  for (int i = 0; i < 6; ++i)
+#pragma unroll
+    for (int j = 0; j < 6; ++j) {
+      const int h = c.h0 + i, w = c.w0 + j;
+      d[6 * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4] : 0u;   // the frame is 0.0f
     }
 }
 
@@ -194,7 +214,9 @@ __device__ __forceinline__ bool grouped_tile(const WinoArgs &a, int block, int s
   return true;
 }
 
-// grid: (interior blocks + rim blocks, ic2); block: 64 tiles x 4 channel quads
+// grid: (interior blocks + rim blocks, ic2); block: 64 tiles x 4 channel quads.
+// Cell = float4 (f32 user input) or unsigned (u8 user input: four codes per lane and pixel).
+template <typename Cell>
 __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
 {
   const int q = threadIdx.x & 3;
@@ -202,7 +224,7 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   TileCoord c;
   int t;
   if (!grouped_tile(a, blockIdx.x, threadIdx.x >> 2, c, t)) return;
-  float4 d[36];
+  Cell d[36];
   gather_tile(a, c, c2, q, d);
   unsigned packed[36];
 #pragma unroll
@@ -237,6 +259,7 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
 }
 
 // minmax_dev[0] = ordered-min, [1] = ordered-max (see f2ord); real channels only
+template <typename Cell>
 __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic_real, unsigned *minmax_dev)
 {
   const int q = threadIdx.x & 3;
@@ -245,7 +268,7 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
   float mn = 3.4e38f, mx = -3.4e38f;
   if (t < a.t) {
     const TileCoord c = tile_coord(a, t);
-    float4 d[36];
+    Cell d[36];
     gather_tile(a, c, c2, q, d);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -274,11 +297,15 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
   }
 }
 
-// Y = At M A (+ bias)(ReLU) of one tile x four channels (the four components of the float4s) and
-// its store; dst points at the tile's image plane, channel quad already applied.  Border tiles
-// write their valid rows and columns only.
+// Y = At M A (+ bias)(output quantization)(ReLU) of one tile x four channels (the four components
+// of the float4s) and its store.  `plane` is the tile's image plane ([oh][ow][16] of OUT's type), q the
+// lane's channel quad.  u8 / s8 output (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:94-111,165-171):
+// value * (1 / out_S) + out_z in one rounding BEFORE the ReLU, then round to nearest even and
+// saturate; the u8 store converts through an unsigned integer, so anything below -0.5 (and NaN)
+// ends as 255.  Border tiles write their valid rows and columns only.
+template <int OUT>
 __device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 &bias, bool with_bias, bool with_relu,
-                                            float4 *dst, int th, int tw, int oh_n, int ow_n)
+                                            float repS, float z, void *plane, int q, int th, int tw, int oh_n, int ow_n)
 {
   float y[4][16];
 #pragma unroll
@@ -302,6 +329,7 @@ __device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 
       for (int j = 0; j < 4; ++j) {
         float r = o[j];
         if (with_bias) r = r + b;
+        if (OUT != EHIP_F32) r = __builtin_fmaf(r, repS, z);
         if (with_relu) r = r > 0.0f ? r : 0.0f;
         y[k][4 * i + j] = r;
       }
@@ -315,13 +343,27 @@ __device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 
     for (int j = 0; j < 4; ++j) {
       const int ow = 4 * tw + j;
       if (ow >= ow_n) break;
-      dst[((size_t)oh * ow_n + ow) * 4] = make_float4(y[0][4 * i + j], y[1][4 * i + j], y[2][4 * i + j], y[3][4 * i + j]);
+      const int e = 4 * i + j;
+      const size_t cell = ((size_t)oh * ow_n + ow) * 16 + 4 * q;   // element index inside the plane
+      if (OUT == EHIP_F32) {
+        *reinterpret_cast<float4 *>(static_cast<float *>(plane) + cell) = make_float4(y[0][e], y[1][e], y[2][e], y[3][e]);
+      } else {
+        unsigned o = 0u;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float r = y[k][e];
+          if (OUT == EHIP_U8) o = __builtin_amdgcn_cvt_pk_u8_f32(r >= -0.5f ? r : 300.0f, k, o);
+          else o |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
+        }
+        *reinterpret_cast<unsigned *>(static_cast<uint8_t *>(plane) + cell) = o;
+      }
     }
   }
 }
 
 // grid: (ceil(t / 64), oc2); block: 64 tiles x 4 channel quads
-__global__ __launch_bounds__(kBlock) void k_wino_trans_output_f32(WinoArgs a)
+template <int OUT>
+__global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 {
   const int q = threadIdx.x & 3;
   const int t = blockIdx.x * 64 + (threadIdx.x >> 2);
@@ -340,8 +382,10 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output_f32(WinoArgs a)
 
   float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
   if (a.with_bias) bias = reinterpret_cast<const float4 *>(a.bias)[o2 * 4 + q];
-  float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 4 + q;
-  output_tile(m, bias, a.with_bias != 0, a.with_relu != 0, dst, th, tw, a.oh, a.ow);
+  const size_t plane = ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 16;
+  void *dst = OUT == EHIP_F32 ? static_cast<void *>(static_cast<float *>(a.out) + plane)
+                              : static_cast<void *>(static_cast<uint8_t *>(a.out) + plane);
+  output_tile<OUT>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z, dst, q, th, tw, a.oh, a.ow);
 }
 
 // ---- the 36 GEMMs and the output transform in one kernel ----------------------------------------
@@ -507,9 +551,18 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
       for (int e = 0; e < 36; ++e) m[e] = xl[(e * 32 + tile_l) * 8 + (q8 ^ ((tile_l >> 1) & 7))];
       float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
       if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
-      float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 4 + ((oc >> 2) & 3);
+      const size_t plane = ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 16;
+      const int q = (oc >> 2) & 3;
       TRACE_POINT(4 + 4 * h);
-      output_tile(m, bias, a.with_bias != 0, a.with_relu != 0, dst, th, tw, a.oh, a.ow);
+      if (a.out_type == EHIP_U8)
+        output_tile<EHIP_U8>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
+                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow);
+      else if (a.out_type == EHIP_S8)
+        output_tile<EHIP_S8>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
+                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow);
+      else
+        output_tile<EHIP_F32>(m, bias, a.with_bias != 0, a.with_relu != 0, 0.f, 0.f, static_cast<float *>(a.out) + plane, q,
+                              th, tw, a.oh, a.ow);
     }
     TRACE_POINT(5 + 4 * h);
   }
@@ -526,14 +579,17 @@ hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s)
     blocks_rim = (a.t + 63) / 64;
   }
   dim3 grid(a.blocks_interior + blocks_rim, a.ic2);
-  hipLaunchKernelGGL(k_wino_trans_input_u8, grid, dim3(kBlock), 0, s, a);
+  if (a.in_u8) hipLaunchKernelGGL(k_wino_trans_input_u8<unsigned>, grid, dim3(kBlock), 0, s, a);
+  else hipLaunchKernelGGL(k_wino_trans_input_u8<float4>, grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
 
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s)
 {
   dim3 grid((a.t + 63) / 64, a.oc2);
-  hipLaunchKernelGGL(k_wino_trans_output_f32, grid, dim3(kBlock), 0, s, a);
+  if (a.out_type == EHIP_U8) hipLaunchKernelGGL(k_wino_trans_output<EHIP_U8>, grid, dim3(kBlock), 0, s, a);
+  else if (a.out_type == EHIP_S8) hipLaunchKernelGGL(k_wino_trans_output<EHIP_S8>, grid, dim3(kBlock), 0, s, a);
+  else hipLaunchKernelGGL(k_wino_trans_output<EHIP_F32>, grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
 
@@ -560,7 +616,8 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s)
 hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_dev, hipStream_t s)
 {
   dim3 grid((a.t + 63) / 64, a.ic2);
-  hipLaunchKernelGGL(k_wino_tinput_range, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
+  if (a.in_u8) hipLaunchKernelGGL(k_wino_tinput_range<unsigned>, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
+  else hipLaunchKernelGGL(k_wino_tinput_range<float4>, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
   return hipGetLastError();
 }
 

@@ -116,6 +116,12 @@ WORKLOADS = {w.key: w for w in [
              algorithm=CONV_WINOGRAD, in_type=F32, out_type=F32, w_sigma=0.02),
     Workload("C4b", "Winograd F(4,3) 512->512 @28x28 N=64, fp32 in/out (VGG-16 conv4)", 64, 512, 512, 28, k=3, pad=1,
              algorithm=CONV_WINOGRAD, in_type=F32, out_type=F32, w_sigma=0.02),
+    # the same two layers as the reference's tuned VGG int8 run feeds them: u8 in, s8 out
+    # (scripts/best_configs/vgg-n64-8180-1s-int8.sh:9,28,36 "--data-type-cfg=U8F32S8F32")
+    Workload("C4a_i8", "Winograd F(4,3) 256->256 @56x56 N=64, u8 in / s8 out (VGG-16 conv3, U8F32S8F32)", 64, 256, 256, 56,
+             k=3, pad=1, algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02),
+    Workload("C4b_i8", "Winograd F(4,3) 512->512 @28x28 N=64, u8 in / s8 out (VGG-16 conv4, U8F32S8F32)", 64, 512, 512, 28,
+             k=3, pad=1, algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02),
     Workload("C5a", "depthwise 3x3 C=144 @56x56 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 144, 144, 56, k=3, pad=1,
              depthwise=True, w_sigma=0.1, T=14, relu6=True),
     Workload("C5b", "depthwise 3x3 C=960 @7x7 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 960, 960, 7, k=3, pad=1,
@@ -155,6 +161,8 @@ class DeviceLayer:
         tq = (EL_NO_CALI, EL_NO_CALI)
         if wl.algorithm == CONV_WINOGRAD:
             mn, mx = wino_tinput_range(wl.descriptor(tinput_quant=(1.0, 0.0)), self.x)
+            in_s = 1.0 / 255.0 if wl.in_type == U8 else 1.0   # u8 input: the range comes back in code units
+            mn, mx = mn * in_s, mx * in_s
             diff = mx - mn + 1e-6
             tq = (diff / 255.0, -mn * 255.0 / diff)
         self.desc = wl.descriptor(tinput_quant=tq)

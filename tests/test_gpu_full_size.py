@@ -11,7 +11,7 @@ import pytest
 
 import oracle_lib as ol
 from gpu_common import Layer, bits, dev, host, pkg
-from test_gpu_wino import make_wino
+from test_gpu_wino import make_wino, make_wino_u8
 
 pytestmark = pytest.mark.gpu
 W = importlib.import_module("deep-learning-math-kernel-research_amd.workloads")
@@ -72,3 +72,31 @@ def test_configured_winograd_layer(key, check_images):
     # images beyond the checked ones were written too, and the layer is not degenerate
     assert not (got == -7.0).any()
     assert float(got.max()) > 0.0
+
+
+@pytest.mark.parametrize("key,check_images", [("C4a_i8", 2), ("C4b_i8", 4)])
+def test_configured_winograd_layer_u8_in_s8_out(key, check_images):
+    """The VGG layers as the reference's tuned int8 run feeds them (u8 input, s8 output)."""
+    import torch
+    wl = W.WORKLOADS[key]
+    E, p, d, xq, wb, bias = make_wino_u8(wl.n, wl.ic, wl.oc, wl.hw, seed=91 + wl.hw, out_type=ol.S8)
+    s_t, z_t = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = s_t, z_t
+    conv = E.Conv(d)
+    d_out = torch.full((wl.n, ol.up16(wl.oc) // 16, wl.hw, wl.hw, 16), -7, dtype=torch.int8, device="cuda")
+    d_b = dev(bias)
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, dev(xq), None, d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    k = check_images
+    pk = ol.make_params(k, wl.ic, wl.oc, wl.hw, wl.hw, 3, 3, 1, out_type=ol.S8, in_scale=1.0 / 255.0, with_bias=True,
+                        with_relu=True, out_scale=p.out_scale, out_z=p.out_z)
+    pk.tin_scale, pk.tin_z = s_t, z_t
+    twq, tscale, tshift = ol.wino_prepare(pk, wb)
+    tin = ol.wino_trans_input(pk, np.ascontiguousarray(xq[:k]).astype(np.float32))
+    tout, _ = ol.wino_gemm(pk, tin, twq, tscale, tshift)
+    exp = ol.wino_trans_output(pk, tout, bias)
+    assert np.array_equal(got[:k], exp), "%d values differ" % int((got[:k] != exp).sum())
+    assert not (got == -7).any()          # ReLU output: every cell was written
+    assert len(np.unique(got)) > 60       # and the s8 codes use their range

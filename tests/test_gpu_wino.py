@@ -89,6 +89,87 @@ def test_wino_fused_gemm_and_output_transform(n, ic, oc, hw):
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
+def make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=True, with_relu=True, out_scale=None, out_z=0.0):
+    """u8 user input (codes of U[0,1) at scale 1/255), f32 / u8 / s8 user output: the data-type
+    configurations U8F32F32F32, U8F32U8F32, U8F32S8F32 of the reference (src/eld_conv.cpp:275-281)."""
+    E = pkg()
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
+    w = rng.normal(0, 0.02, (oc, ic, 3, 3)).astype(f32)
+    bias = np.zeros(ol.up16(oc), f32)
+    bias[:oc] = rng.normal(0, 0.01, oc)
+    xq = ol.to_blocked(ol.quantize_input_u8(x, 1.0 / 255.0, 0.0))
+    wb = ol.weights_to_blocked(w)
+    if out_scale is None:
+        out_scale = 4.0 * 0.02 * np.sqrt(9 * ic / 3.0) / (127.0 if out_type == ol.S8 else 255.0)
+    p = ol.make_params(n, ic, oc, hw, hw, 3, 3, 1, out_type=out_type, in_scale=1.0 / 255.0, with_bias=with_bias,
+                       with_relu=with_relu, out_scale=out_scale, out_z=out_z)
+    d = E.make_desc(n, ic, oc, hw, hw, 3, 3, 1, algorithm=E.CONV_WINOGRAD, input_type=E.U8, output_type=out_type,
+                    with_bias=with_bias, with_relu=with_relu, input_quant=(1.0 / 255.0, 0.0), tile_size=6,
+                    execution_mode=0xa161, wino_tinput_quant=(1.0, 0.0), output_quant=(out_scale, out_z))
+    return E, p, d, xq, wb, bias
+
+
+def _oracle_u8(p, xq, wb, bias):
+    # the reference transforms the u8 codes as floats (src/kernel/elk_conv_wino_4x4_3x3_input.hxx:40-47)
+    xf = xq.astype(f32)
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tin = ol.wino_trans_input(p, xf)
+    tout, _ = ol.wino_gemm(p, tin, twq, tscale, tshift)
+    return tin, ol.wino_trans_output(p, tout, bias)
+
+
+@pytest.mark.parametrize("fused", ["1", "0"])
+@pytest.mark.parametrize("out_type", [ol.F32, ol.U8, ol.S8])
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 10), (1, 64, 80, 12), (1, 48, 32, 7)])
+def test_wino_u8_input_quantized_output(fused, out_type, n, ic, oc, hw, monkeypatch):
+    import torch
+    monkeypatch.setenv("EHIP_WINO_FUSED", fused)
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=7 * n + hw + ic + out_type, out_type=out_type)
+    d_x = dev(xq)
+    # calibration on the codes: the transformed-input range in code units, times the input scale
+    mn, mx = E.wino_tinput_range(d, d_x)
+    omn, omx = ol.wino_tinput_range(p, xq.astype(f32))
+    assert (f32(mn), f32(mx)) == (f32(omn), f32(omx))
+    diff = (f32(mx) - f32(mn)) * f32(1.0 / 255.0) + f32(0.000001)
+    s_t, z_t = float(diff / f32(255.0)), float(-f32(mn) * f32(1.0 / 255.0) * f32(255.0) / diff)
+    p.tin_scale, p.tin_z = s_t, z_t
+    d.tinput_scale, d.tinput_z = s_t, z_t
+    tin, exp = _oracle_u8(p, xq, wb, bias)
+    conv = E.Conv(d)
+    d_b = dev(bias)
+    tdt = {ol.F32: torch.float32, ol.U8: torch.uint8, ol.S8: torch.int8}[out_type]
+    d_out = torch.full(exp.shape, 5, dtype=tdt, device="cuda")
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, d_x, None, d_b)
+    torch.cuda.synchronize()
+    g_tin = conv.query(E.Q_TINPUT_U8).reshape(tin.shape)
+    assert np.array_equal(g_tin, tin), "u8 transformed input differs at %d cells" % int((g_tin != tin).sum())
+    got = host(d_out)
+    assert got.dtype == exp.dtype
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+    if out_type != ol.F32:   # the codes really use the range
+        assert len(np.unique(got)) > 40
+
+
+def test_wino_u8_output_without_relu_wraps_negatives_to_255():
+    """No ReLU and u8 output: the reference's store converts through an unsigned integer, so negative
+    values saturate to 255 (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:97-101)."""
+    import torch
+    E, p, d, xq, wb, bias = make_wino_u8(1, 32, 32, 9, seed=11, out_type=ol.U8, with_relu=False, out_z=2.4)
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    _, exp = _oracle_u8(p, xq, wb, bias)
+    conv = E.Conv(d)
+    d_out = torch.zeros(exp.shape, dtype=torch.uint8, device="cuda")
+    d_b = dev(bias)
+    conv.execute(d_out, dev(xq), dev(wb), d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    assert np.array_equal(got, exp)
+    assert (exp == 255).sum() > exp.size // 10
+
+
 def test_wino_no_bias_no_relu():
     import torch
     E, p, d, xb, wb, bias = make_wino(1, 32, 32, 9, seed=4, with_bias=False, with_relu=False)
