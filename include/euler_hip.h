@@ -80,7 +80,18 @@ EHIP_API const char *ehip_last_error(void);
 /* Replaces eld_conv_t::setup(): validates the descriptor, picks the executor
  * (src/eld_conv.cpp:166-313: direct 1x1 / direct KxK / depthwise / Winograd F(4,3) int8) and
  * allocates the device workspace.  Unsupported shapes return EHIP_UNIMPLEMENTED where the
- * reference calls el_error()/abort(). */
+ * reference calls el_error()/abort().  What is accepted:
+ *  - CONV_DIRECT_1X1 (src/elx_int8_conv_direct_1x1.cpp): u8 input, u8/s8/s32 output, stride 1 or 2,
+ *    no padding, sum fusion; activations nChw16c or nhwc on either side (nhwc: channels % 16 == 0);
+ *  - CONV_DIRECT with a 1x1 kernel (a160, src/elx_int8_conv_direct.cpp:574-718): also f32 output;
+ *  - CONV_DIRECT with a 3/5/7 kernel (c160, src/elx_int8_conv_direct.cpp:66-77): stride 1 or 2, every
+ *    pad k/2 or k/2 - 1 (right/bottom pads follow from oh/ow), nChw16c, ow % flatting_t == 0;
+ *  - depthwise 3x3 (g == ic == oc, src/elx_int8_conv_direct_depthwise.cpp): stride 1 or 2, pads 0/1,
+ *    u8/s8 output, weights goihw;
+ *  - CONV_WINOGRAD tile_size 6 (src/elx_int8_conv_wino.cpp): f32 tensors with execution_mode 0xa1xx, or
+ *    u8 input with f32/u8/s8 output (U8F32F32F32 / U8F32U8F32 / U8F32S8F32, src/eld_conv.cpp:275-281);
+ *    wino_tinput_quant must be set (calibrated sampling).
+ * A non-zero input zero point is accepted only where no tap falls on padding. */
 EHIP_API int ehip_conv_create(const ehip_conv_desc_t *desc, ehip_conv_t **out);
 EHIP_API int ehip_conv_destroy(ehip_conv_t *conv);
 
@@ -122,7 +133,8 @@ EHIP_API int ehip_quantize_input_u8(void *dst_dev, const void *src_dev, size_t c
                                     float z, void *hip_stream);
 
 /* Replaces the harness-side calibration of wino_tinput_quant (tests/elt_conv_utils.cpp:222-262):
- * min and max over the fp32 Winograd-transformed input.  Synchronous. */
+ * min and max over the fp32 Winograd-transformed input.  u8 input: over the transformed CODES
+ * (multiply by the input scale for real units).  Synchronous. */
 EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev,
                                     float *min_out, float *max_out);
 
