@@ -2,7 +2,7 @@
 // fill eld_conv_t, setup(), elx_conv() on HOST buffers in the blocked formats made with reorder<>),
 // so that the pytest side can compare the result with the CPU oracle.
 //
-//   euler_api_check <in.bin> <out.bin> n ic oc hw k pad stride out_type algorithm with_sum T out_scale sum_scale g
+//   euler_api_check <in.bin> <out.bin> n ic oc hw k pad stride out_type algorithm with_sum T out_scale sum_scale g [nhwc]
 //
 // in.bin : u8 input nchw | f32 weights oihw (goihw for g > 1) | f32 bias[oc] | [old output nchw, output type]
 // out.bin: output nchw in the output type
@@ -20,7 +20,7 @@ static size_t up16(size_t x) { return (x + 15) / 16 * 16; }
 
 int main(int argc, char **argv)
 {
-  if (argc != 17) {
+  if (argc != 17 && argc != 18) {
     fprintf(stderr, "usage: see source\n");
     return 2;
   }
@@ -30,6 +30,7 @@ int main(int argc, char **argv)
   const int with_sum = atoi(argv[12]), T = atoi(argv[13]);
   const float out_scale = (float)atof(argv[14]), sum_scale = (float)atof(argv[15]);
   const int g = atoi(argv[16]);
+  const bool use_nhwc = argc == 18 && atoi(argv[17]) != 0;   // activations [n][h][w][c] on both sides
   const int oh = (hw + 2 * pad - k) / stride + 1;
   const size_t osz = out_type == f32 ? 4 : 1;
 
@@ -50,7 +51,7 @@ int main(int argc, char **argv)
   desc.strides = {stride, stride};
   desc.dilations = {1, 1};
   desc.data_type.input = u8; desc.data_type.weights = f32; desc.data_type.output = (uint8_t)out_type; desc.data_type.bias = f32;
-  desc.formats = {nChw16c, g > 1 ? goihw : OIhw16i16o, nChw16c};
+  desc.formats = {use_nhwc ? nhwc : nChw16c, g > 1 ? goihw : OIhw16i16o, use_nhwc ? nhwc : nChw16c};
   desc.algorithm = algorithm;
   desc.with_relu = true; desc.with_bias = true; desc.with_ip_sum = with_sum != 0;
   desc.relu_bound.lower = 0.0f;
@@ -68,11 +69,14 @@ int main(int argc, char **argv)
 
   std::vector<uint8_t> xb(desc.byte_sizes.input), ob(desc.byte_sizes.output, 0x5a);
   std::vector<float> wb(desc.sizes.weights, 0.0f);
-  reorder<uint8_t, nChw16c, nchw>(xb.data(), x.data(), n, ic, hw, hw);
+  if (use_nhwc) reorder<uint8_t, nhwc, nchw>(xb.data(), x.data(), n, ic, hw, hw);
+  else reorder<uint8_t, nChw16c, nchw>(xb.data(), x.data(), n, ic, hw, hw);
   if (g > 1) memcpy(wb.data(), w.data(), w.size() * 4);   // depthwise weights stay goihw
   else reorder<float, OIhw16i16o, oihw>(wb.data(), w.data(), oc, ic, k, k);
   if (with_sum) {
-    if (osz == 1) reorder<uint8_t, nChw16c, nchw>(ob.data(), old.data(), n, oc, oh, oh);
+    if (use_nhwc && osz == 1) reorder<uint8_t, nhwc, nchw>(ob.data(), old.data(), n, oc, oh, oh);
+    else if (use_nhwc) reorder<float, nhwc, nchw>((float *)ob.data(), (float *)old.data(), n, oc, oh, oh);
+    else if (osz == 1) reorder<uint8_t, nChw16c, nchw>(ob.data(), old.data(), n, oc, oh, oh);
     else reorder<float, nChw16c, nchw>((float *)ob.data(), (float *)old.data(), n, oc, oh, oh);
   }
   // first call prepares the weights; the second is the steady state (the sum operand is re-staged)
@@ -82,7 +86,9 @@ int main(int argc, char **argv)
   if (elx_conv(desc, ob.data(), xb.data(), wb.data(), bias.data()) != ELX_OK) return 5;
 
   std::vector<uint8_t> out((size_t)n * oc * oh * oh * osz);
-  if (osz == 1) reorder<uint8_t, nchw, nChw16c>(out.data(), ob.data(), n, oc, oh, oh);
+  if (use_nhwc && osz == 1) reorder<uint8_t, nchw, nhwc>(out.data(), ob.data(), n, oc, oh, oh);
+  else if (use_nhwc) reorder<float, nchw, nhwc>((float *)out.data(), (float *)ob.data(), n, oc, oh, oh);
+  else if (osz == 1) reorder<uint8_t, nchw, nChw16c>(out.data(), ob.data(), n, oc, oh, oh);
   else reorder<float, nchw, nChw16c>((float *)out.data(), (float *)ob.data(), n, oc, oh, oh);
   f = fopen(out_path, "wb");
   if (!f || fwrite(out.data(), 1, out.size(), f) != out.size()) return 6;

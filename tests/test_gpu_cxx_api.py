@@ -26,10 +26,13 @@ def from_blocked(b, c):
     dict(n=2, ic=96, oc=64, hw=7, k=1, pad=0, out_type=ol.S8, with_sum=True),
     dict(n=1, ic=32, oc=80, hw=9, k=1, pad=0, out_type=ol.F32),
     dict(n=2, ic=32, oc=32, hw=14, k=3, pad=1, out_type=ol.U8, depthwise=True, T=7),
-], ids=["3x3_u8", "1x1_s8_sum", "1x1_f32", "depthwise_u8"])
+    dict(n=2, ic=64, oc=64, hw=14, k=3, pad=1, stride=2, out_type=ol.S8, T=7),
+    dict(n=2, ic=32, oc=32, hw=14, k=3, pad=1, stride=2, out_type=ol.U8, depthwise=True, T=7),
+    dict(n=2, ic=96, oc=64, hw=7, k=1, pad=0, out_type=ol.S8, with_sum=True, nhwc=True),
+], ids=["3x3_u8", "1x1_s8_sum", "1x1_f32", "depthwise_u8", "3x3_s2_s8", "depthwise_s2_u8", "1x1_s8_sum_nhwc"])
 def test_elx_conv_on_host_buffers(case, tmp_path):
     assert os.path.exists(CHECK), "euler_api_check is not built (python -c 'import __graft_entry__ as g; g.build()')"
-    c = dict(stride=1, with_sum=False, depthwise=False, T=0)
+    c = dict(stride=1, with_sum=False, depthwise=False, T=0, nhwc=False)
     c.update(case)
     layer = Layer(c["n"], c["ic"], c["oc"], c["hw"], k=c["k"], pad=c["pad"], stride=c["stride"], out_type=c["out_type"],
                   with_sum=c["with_sum"], depthwise=c["depthwise"], seed=321 + c["ic"], T=c["T"],
@@ -46,7 +49,7 @@ def test_elx_conv_on_host_buffers(case, tmp_path):
     g = c["ic"] if c["depthwise"] else 1
     args = [CHECK, str(fin), str(fout)] + [str(v) for v in (
         c["n"], c["ic"], c["oc"], c["hw"], c["k"], c["pad"], c["stride"], c["out_type"], d.algorithm,
-        int(c["with_sum"]), c["T"], repr(float(d.output_scale)), repr(float(d.sum_scale)), g)]
+        int(c["with_sum"]), c["T"], repr(float(d.output_scale)), repr(float(d.sum_scale)), g, int(c["nhwc"]))]
     r = subprocess.run(args, capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, "rc=%d stdout=%s stderr=%s" % (r.returncode, r.stdout, r.stderr)
     got = np.fromfile(fout, dtype=exp.dtype).reshape(exp.shape)
