@@ -1,0 +1,98 @@
+"""Seeded random shapes for every executor family through the C-ABI against the CPU oracle, bit for
+bit: ragged channel counts, odd image sizes, one-sided pads, every output type, both layouts."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_common import Layer
+from test_gpu_parity import run_and_compare
+
+pytestmark = pytest.mark.gpu
+OUT_TYPES = [ol.S32, ol.U8, ol.S8, ol.F32]
+
+
+def _rng(seed):
+    return np.random.default_rng(1000 + seed)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_1x1(seed):
+    r = _rng(seed)
+    stride = int(r.choice([1, 1, 2]))
+    nhwc_in, nhwc_out = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+    ic = int(r.integers(1, 20)) * (16 if nhwc_in else int(r.choice([3, 8, 16])))
+    oc = int(r.integers(1, 20)) * (16 if nhwc_out else int(r.choice([5, 8, 16])))
+    hw = int(r.integers(2, 19))
+    if stride == 2:
+        hw = max(3, hw | 1)   # (hw - 1) divisible by the stride: the reference has no tail there
+    out_type = OUT_TYPES[int(r.integers(0, 4))]
+    with_sum = bool(r.integers(0, 2)) and out_type in (ol.U8, ol.S8)
+    run_and_compare(Layer(int(r.integers(1, 4)), ic, oc, hw, stride=stride, out_type=out_type, with_sum=with_sum,
+                          seed=seed, in_nhwc=nhwc_in, out_nhwc=nhwc_out, with_bias=bool(r.integers(0, 2))))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_kxk(seed):
+    r = _rng(100 + seed)
+    k = int(r.choice([3, 3, 3, 5, 7]))
+    stride = int(r.choice([1, 2]))
+    pad = int(r.choice([k // 2 - 1, k // 2]))
+    hw = int(r.integers(k + 1, 26))
+    ic = int(r.integers(1, 9)) * int(r.choice([4, 16, 24]))
+    oc = int(r.integers(1, 9)) * int(r.choice([6, 16]))
+    out_hw = None
+    natural = (hw + 2 * pad - k) // stride + 1
+    if stride == 2 and pad == k // 2 - 1 and (natural) * stride + k - hw - pad <= k // 2:
+        # ask for one more output row / column: pads only at the right / bottom
+        if r.integers(0, 2):
+            out_hw = natural + 1
+    out_type = OUT_TYPES[int(r.integers(0, 4))]
+    run_and_compare(Layer(int(r.integers(1, 3)), ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=seed,
+                          out_hw=out_hw))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_depthwise(seed):
+    r = _rng(200 + seed)
+    stride = int(r.choice([1, 2]))
+    pad = int(r.integers(0, 2))
+    hw = int(r.integers(4, 40))
+    g = 16 * int(r.integers(1, 8))
+    oh = (hw + 2 * pad - 3) // stride + 1
+    divs = [t for t in range(1, oh + 1) if oh % t == 0]
+    T = int(r.choice(divs + [0, oh]))
+    out_type = [ol.U8, ol.S8, ol.S32][int(r.integers(0, 3))]
+    run_and_compare(Layer(int(r.integers(1, 4)), g, g, hw, k=3, pad=pad, stride=stride, out_type=out_type, depthwise=True,
+                          seed=seed, w_sigma=0.1, T=T))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_winograd(seed):
+    import torch
+    from gpu_common import bits, dev, host
+    from test_gpu_wino import make_wino, make_wino_u8
+    r = _rng(300 + seed)
+    n, hw = int(r.integers(1, 4)), int(r.integers(4, 23))
+    ic, oc = int(r.integers(1, 20)) * int(r.choice([8, 16])), int(r.integers(1, 12)) * int(r.choice([8, 16]))
+    u8_in = bool(r.integers(0, 2))
+    out_type = [ol.F32, ol.U8, ol.S8][int(r.integers(0, 3))] if u8_in else ol.F32
+    bias_on, relu_on = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+    if u8_in:
+        E, p, d, x, wb, bias = make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=bias_on, with_relu=relu_on)
+        xf = x.astype(np.float32)
+    else:
+        E, p, d, x, wb, bias = make_wino(n, ic, oc, hw, seed, with_bias=bias_on, with_relu=relu_on)
+        xf = x
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xf), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias)
+    conv = E.Conv(d)
+    tdt = {ol.F32: torch.float32, ol.U8: torch.uint8, ol.S8: torch.int8}[out_type]
+    d_out = torch.full(exp.shape, 3, dtype=tdt, device="cuda")
+    d_b = dev(bias) if bias_on else None
+    conv.execute(d_out, dev(x), dev(wb), d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "%d of %d values differ" % (int((got != exp).sum()), got.size)
