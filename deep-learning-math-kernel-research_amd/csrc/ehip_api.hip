@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <utility>
 #include <vector>
 
 #include "ehip_internal.hpp"
@@ -41,6 +42,11 @@ struct ehip_conv {
   int *wsum = nullptr, *comp = nullptr;
   size_t per_oc = 0;  // elements in scale/shift/wsum/comp
 
+  // k x k direct with a non-zero input zero point and padding: classes of output pixels by their
+  // set of valid taps (a rectangle of kernel rows x columns) and one shift row per class
+  int nclass = 0, ncls_w = 0;
+  int *cls_h = nullptr, *cls_w = nullptr, *rects = nullptr;
+  float *shift_tab = nullptr;
   // 3x3
   int chunk_units = 2;
   // depthwise
@@ -66,7 +72,8 @@ int fail(int code, const std::string &msg)
 
 void free_all(ehip_conv *c)
 {
-  void *ptrs[] = {c->wpacked, c->scale, c->shift, c->absmax, c->wsum, c->comp, c->tin, c->tout};
+  void *ptrs[] = {c->wpacked, c->scale, c->shift, c->absmax, c->wsum, c->comp, c->tin, c->tout,
+                  c->cls_h, c->cls_w, c->rects, c->shift_tab};
   for (void *p : ptrs)
     if (p) (void)hipFree(p);
 }
@@ -174,14 +181,18 @@ int classify(ehip_conv *c)
     if (k_ok && s_ok && pad_ok(d.pad_l, d.kw) && pad_ok(d.pad_t, d.kh) && pad_ok(rp < 0 ? d.kw / 2 - 1 : rp, d.kw) &&
         pad_ok(bp < 0 ? d.kh / 2 - 1 : bp, d.kh)) {
       const bool padded = d.pad_l || d.pad_t || rp > 0 || bp > 0;
-      if (d.input_z != 0.0f && padded)
-        return fail(EHIP_UNIMPLEMENTED, "direct: input zero point with padding is not built");
+      // zero point with padding (src/elx_int8_conv_direct.cpp:247-255): every pad must be coverable
+      if (d.input_z != 0.0f && padded &&
+          (d.pad_l + d.ow < d.kw || (rp > 0 ? rp : 0) + d.ow < d.kw || d.pad_t + d.oh < d.kh || (bp > 0 ? bp : 0) + d.oh < d.kh))
+        return fail(EHIP_UNIMPLEMENTED, "Shape not support for U8 input with zero-point");
       const int T = d.flatting_t > d.ow ? d.ow : d.flatting_t;
       if (T > 0 && d.ow % T)
         return fail(EHIP_UNIMPLEMENTED, "direct: c160: ow must be a multiple of T (the reference mis-indexes shift for Tr != T)");
       const bool s1_3x3 = d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 &&
           d.ow == d.iw + d.pad_l + d.pad_r - 2 && d.oh == d.ih + d.pad_t + d.pad_b - 2;
-      c->family = s1_3x3 ? FAM_CONV_3X3 : FAM_GEMM_1X1;   // the GEMM family walks [tap][unit] for kh x kw
+      // the GEMM family walks [tap][unit] for kh x kw; it also owns the per-pixel shift that a zero
+      // point with padding needs
+      c->family = (s1_3x3 && !(d.input_z != 0.0f && padded)) ? FAM_CONV_3X3 : FAM_GEMM_1X1;
       return EHIP_OK;
     }
     return fail(EHIP_UNIMPLEMENTED, "direct: c160: shape not supported");
@@ -243,15 +254,51 @@ int setup_workspace(ehip_conv *c)
   }
   // fall through
   case FAM_GEMM_1X1: {
-    if ((long long)d.n * d.oh * d.ow * d.oh * d.ow >= (1ll << 32))
-      return fail(EHIP_UNIMPLEMENTED, "direct: n*oh*ow*oh*ow must stay below 2^32");
+    if ((long long)d.n * d.oh * d.ow >= (1ll << 30) || (long long)d.oh * d.ow * d.ow >= (1ll << 32))
+      return fail(EHIP_UNIMPLEMENTED, "direct: more than 2^30 output pixels");
     c->taps = d.kh * d.kw;
     c->nbatch = 1;
     if (c->taps > 1 && (long long)d.n * c->ic2 * d.ih * d.iw * 16 >= (1ll << 40))
       return fail(EHIP_UNIMPLEMENTED, "direct: input too large");
     c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2 * c->taps, 1, c->taps > 1 ? 1 : d.stride_w);
-    c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
+    // kh x kw: the K axis is [tap][ic2 real units]; only its end is padded to the kernel's chunk
+    c->units_pad = c->taps > 1 ? c->ic2 : up(c->ic2, gemm_variant_chunk(c->variant));
     c->kernel_name = gemm_variant_name(c->variant);
+    if (c->taps > 1 && d.input_z != 0.0f) {
+      // classes of output rows / columns by their range of valid kernel rows / columns
+      auto classes = [](int on, int in, int k, int stride, int pad, std::vector<int> &cls, std::vector<std::pair<int, int>> &rng) {
+        cls.resize(on);
+        for (int o = 0; o < on; ++o) {
+          int lo = pad - o * stride; lo = lo < 0 ? 0 : lo;
+          int hi = in - 1 + pad - o * stride; hi = hi > k - 1 ? k - 1 : hi;
+          const std::pair<int, int> r(lo, hi);
+          size_t i = 0;
+          while (i < rng.size() && rng[i] != r) ++i;
+          if (i == rng.size()) rng.push_back(r);
+          cls[o] = (int)i;
+        }
+      };
+      std::vector<int> ch, cw;
+      std::vector<std::pair<int, int>> rh, rw;
+      classes(d.oh, d.ih, d.kh, d.stride_h, d.pad_t, ch, rh);
+      classes(d.ow, d.iw, d.kw, d.stride_w, d.pad_l, cw, rw);
+      if (rh.size() * rw.size() > 1) {
+        c->ncls_w = (int)rw.size();
+        c->nclass = (int)(rh.size() * rw.size());
+        std::vector<int> rects((size_t)c->nclass * 4);
+        for (size_t i = 0; i < rh.size(); ++i)
+          for (size_t j = 0; j < rw.size(); ++j) {
+            int *r = &rects[(i * rw.size() + j) * 4];
+            r[0] = rh[i].first; r[1] = rh[i].second; r[2] = rw[j].first; r[3] = rw[j].second;
+          }
+        if ((rc = dev_alloc(&c->cls_h, ch.size(), false)) != EHIP_OK) return rc;
+        if ((rc = dev_alloc(&c->cls_w, cw.size(), false)) != EHIP_OK) return rc;
+        if ((rc = dev_alloc(&c->rects, rects.size(), false)) != EHIP_OK) return rc;
+        HIP_TRY(hipMemcpy(c->cls_h, ch.data(), ch.size() * sizeof(int), hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(c->cls_w, cw.data(), cw.size() * sizeof(int), hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(c->rects, rects.data(), rects.size() * sizeof(int), hipMemcpyHostToDevice));
+      }
+    }
     break;
   }
   case FAM_DEPTHWISE: {
@@ -305,7 +352,8 @@ int setup_workspace(ehip_conv *c)
     c->wpacked_bytes = (size_t)c->oc2 * 3 * 16 * 4;
   } else {
     c->ocpp = up(c->oc2 * 16, kOcTile);
-    c->wpacked_bytes = (size_t)c->nbatch * c->taps * c->units_pad * c->ocpp * 16;
+    // (the K loop may run up to one chunk of 8 units past the last real one: zero rows)
+    c->wpacked_bytes = (size_t)c->nbatch * up(c->taps * c->units_pad, 8) * c->ocpp * 16;
   }
   c->per_oc = (size_t)c->nbatch * c->ocpp;
   if ((rc = dev_alloc(&c->wpacked, c->wpacked_bytes, true)) != EHIP_OK) return rc;
@@ -314,6 +362,7 @@ int setup_workspace(ehip_conv *c)
   if ((rc = dev_alloc(&c->absmax, c->per_oc, true)) != EHIP_OK) return rc;
   if ((rc = dev_alloc(&c->wsum, c->per_oc, true)) != EHIP_OK) return rc;
   if ((rc = dev_alloc(&c->comp, c->per_oc, true)) != EHIP_OK) return rc;
+  if (c->nclass > 1 && (rc = dev_alloc(&c->shift_tab, (size_t)c->nclass * c->ocpp, true)) != EHIP_OK) return rc;
   return EHIP_OK;
 }
 
@@ -329,6 +378,8 @@ Epilogue make_epilogue(const ehip_conv *c, int out_type, bool sum, bool relu)
   e.out_type = out_type;
   e.with_sum = sum ? 1 : 0;
   e.with_relu = relu ? 1 : 0;
+  e.shift_tab = nullptr;
+  e.tab_stride = 0;
   return e;
 }
 
@@ -408,6 +459,9 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const vo
   case FAM_CONV_3X3:
     HIP_TRY(launch_prepare_direct(w, b, d.oc, d.ic, d.kh, d.kw, c->units_pad, c->ocpp, d, c->absmax, c->wpacked,
                                   c->scale, c->shift, c->wsum, c->comp, s));
+    if (c->nclass > 1)
+      HIP_TRY(launch_fold_direct_border(c->wpacked, c->absmax, b, d.oc, d.kw, c->units_pad, c->ocpp, d, c->rects,
+                                        c->nclass, c->shift_tab, s));
     break;
   case FAM_DEPTHWISE:
     HIP_TRY(launch_prepare_depthwise(w, b, d.g, d, c->wpacked, c->scale, c->shift, c->wsum, s));
@@ -457,6 +511,10 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
     a.in_nhwc = d.input_fmt == EHIP_NHWC; a.out_nhwc = d.output_fmt == EHIP_NHWC;
     a.kh = d.kh; a.kw = d.kw; a.pad_t = d.pad_t; a.pad_l = d.pad_l; a.ih = d.ih;
+    if (c->nclass > 1) {
+      a.ep.shift_tab = c->shift_tab; a.ep.tab_stride = c->ocpp;
+      a.cls_h = c->cls_h; a.cls_w = c->cls_w; a.ncls_w = c->ncls_w;
+    }
     a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
     HIP_TRY(launch_gemm(a, 1, c->variant, s));
     break;

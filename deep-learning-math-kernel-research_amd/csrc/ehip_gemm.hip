@@ -41,7 +41,7 @@
 
 namespace ehip {
 
-template <int WM, int WN, int TM, int TN, int KC, int D, bool NHWC, bool CONV>
+template <int WM, int WN, int TM, int TN, int KC, int D, bool NHWC, int CONV>
 __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 {
   static_assert(!(NHWC && CONV), "the kh x kw form is built for blocked input only");
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   long long safe_off = 0;   // a cell of the same image that every unit offset keeps in bounds
   auto input_pixel = [&](int gp) -> long long {
     gp = gp < a.p_total ? gp : a.p_total - 1;
-    const int n = a.ohw == a.p_total ? 0 : fastdiv(gp, a.ohw, a.ohw_magic);
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic);
     const int r = gp - n * a.ohw;
     long long sp;   // pixel index inside the image
     if (dense) {
@@ -127,33 +127,51 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const long long w_unit = (long long)a.ocpp * 16;
 
   v4i sta[D][NA], stb[D][NB];   // D fills in flight (global -> registers), see the main loop
-  bool stv[D];                  // CONV: the fill's tap lies inside the image for this thread's pixel
+  unsigned stz[D];              // CONV: bit j = cell j of the fill belongs to a tap outside the image
   // All global loads of the main loop are unconditional (indices clamped): without branches
   // between a load and its use the compiler counts outstanding loads exactly.
-  // CONV: the K axis is [tap][unit]; a fill never straddles two taps (KC divides the padded units),
-  // the packed weights are contiguous in that order, and the input cell of tap (kh, kw) sits
-  // (kh * iw + kw) cells behind the one of tap (0, 0).  Taps outside the image read a safe cell and
-  // are replaced by u8 0 on the way to LDS, which contributes nothing -- the reference skips them.
+  // CONV: the K axis is [tap][unit] with the ic2 real units per tap and nothing in between (a layer
+  // with few input channels would otherwise multiply mostly padding); the packed weights are
+  // contiguous in that order, zero behind the last real unit, and the input cell of tap (kh, kw)
+  // sits (kh * iw + kw) cells behind the one of tap (0, 0).  Cells of taps outside the image read a
+  // safe cell and are replaced by u8 0 on the way to LDS, which contributes nothing -- the
+  // reference skips such taps.
   auto load_stage = [&](int chunk, int d) {
 #pragma unroll
     for (int j = 0; j < NA; ++j) {
       const int id = tid + j * kBlock;
       sta[d][j] = *reinterpret_cast<const v4i *>(wb + (long long)(chunk * KC + id / OC_T) * w_unit + (id % OC_T) * 16);
     }
-    int ub = chunk * KC;
-    const uint8_t *src0 = inb[0];
-    if (CONV) {
-      const int tap = fastdiv(chunk, a.chunks_per_tap, a.cpt_magic);
-      ub = (chunk - tap * a.chunks_per_tap) * KC;
+    if (CONV == 1) {
+      // ic2 is a multiple of KC: the whole fill belongs to one tap (scalar arithmetic)
+      const int tap = fastdiv(chunk * KC, a.ic2, a.ic2_magic);
+      const int ub = chunk * KC - tap * a.ic2;
       const int kh = fastdiv(tap, a.kw, a.kw_magic);
-      stv[d] = (tapmask >> tap) & 1;
-      src0 = stv[d] ? inb[0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * 16 : safe;
+      const bool inside = (tapmask >> tap) & 1;
+      stz[d] = inside ? 0u : ~0u;
+      const uint8_t *src = inside ? inb[0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * 16 : safe;
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        stb[d][j] = *reinterpret_cast<const v4i *>(src + (long long)(ub + bu0 + j * BU) * unit_stride);
+      return;
     }
+    if (CONV) stz[d] = 0u;
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      int u = ub + bu0 + (NHWC ? 0 : j * BU);
-      u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
-      stb[d][j] = *reinterpret_cast<const v4i *>((CONV ? src0 : inb[NHWC ? j : 0]) + (long long)u * unit_stride);
+      int u = chunk * KC + bu0 + (NHWC ? 0 : j * BU);
+      const uint8_t *src = inb[NHWC ? j : 0];
+      if (CONV) {   // any ic2: the tap is worked out per cell
+        u = u < a.k_real ? u : a.k_real - 1;   // behind the last real unit the weights are zero
+        const int tap = fastdiv(u, a.ic2, a.ic2_magic);
+        u -= tap * a.ic2;
+        const int kh = fastdiv(tap, a.kw, a.kw_magic);
+        const bool inside = (tapmask >> tap) & 1;
+        stz[d] |= inside ? 0u : 1u << j;
+        src = inside ? inb[0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * 16 : safe;
+      } else {
+        u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
+      }
+      stb[d][j] = *reinterpret_cast<const v4i *>(src + (long long)u * unit_stride);
     }
   };
   // LDS keeps B as [unit][pixel].  The nhwc plan writes one pixel's KC units from neighbouring
@@ -167,7 +185,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     for (int j = 0; j < NB; ++j) {
       const int id = tid + j * kBlock;
       const int cell = NHWC ? (id % KC) * P_T + ((id / KC) ^ ((2 * (id % KC)) & 15)) : id;
-      const v4i x = (CONV && !stv[d]) ? v4i{0, 0, 0, 0} : stb[d][j];
+      const v4i x = (CONV && ((stz[d] >> j) & 1u)) ? v4i{0, 0, 0, 0} : stb[d][j];
       lds_b[buf][cell] = x ^ (int)0x80808080;
     }
   };
@@ -249,14 +267,23 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     valid = gp < a.p_total;
     const int gpc = valid ? gp : 0;
     if (a.out_nhwc) return (size_t)gpc * oc_real;
-    const int n = a.ohw == a.p_total ? 0 : fastdiv(gpc, a.ohw, a.ohw_magic);
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
     const int r = gpc - n * a.ohw;
     return (size_t)b * a.out_batch_stride + ((size_t)n * a.oc2 * a.ohw + r) * 16;
   };
   size_t pix[TN], pixT[TN][2];
   bool pvalid[TN], validT[TN][2];
+  int cls[TN];
 #pragma unroll
   for (int nt = 0; nt < TN; ++nt) {
+    cls[nt] = 0;
+    if (CONV && a.ep.shift_tab) {   // border class of the lane's pixel
+      int gp = pix0 + pw0 + nt * 32 + l32;
+      gp = gp < a.p_total ? gp : a.p_total - 1;
+      const int r = gp - (a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic)) * a.ohw;
+      const int oh = fastdiv(r, a.ow, a.ow_magic);
+      cls[nt] = a.cls_h[oh] * a.ncls_w + a.cls_w[r - oh * a.ow];
+    }
     pix[nt] = pixel_offset(pix0 + pw0 + nt * 32 + l32, pvalid[nt]);
     pixT[nt][0] = pixel_offset(pix0 + pw0 + nt * 32 + (lane >> 2), validT[nt][0]);
     pixT[nt][1] = pixel_offset(pix0 + pw0 + nt * 32 + (lane >> 2) + 16, validT[nt][1]);
@@ -268,8 +295,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     xlds = lds + wave * 256;
   }
   TRACE_POINT(14);
-  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real,
-                        a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT);
+  epilogue_wave<TM, TN, CONV != 0>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real,
+                        a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT, cls);
   TRACE_POINT(15);
 }
 
@@ -277,22 +304,24 @@ namespace {
 struct Variant {
   const char *name;
   int oc_t, p_t, kc;
-  void (*kernel[3][3])(GemmArgs);   // [blocked | nhwc | blocked kh x kw][prefetch depth 1, 2, 4] (null: not built)
+  // [blocked | nhwc | blocked kh x kw, ic2 % KC == 0 | blocked kh x kw, any ic2][prefetch depth 1, 2, 4] (null: not built)
+  void (*kernel[4][3])(GemmArgs);
 };
 // depth 4 only where four fills of staging fit in 96 registers
 template <int WM, int WN, int TM, int TN, int KC, bool NHWC>
 constexpr void (*deep_or_null())(GemmArgs)
 {
-  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4, NHWC, false>;
+  if constexpr (4 * ((WM * TM + WN * TN) * 32 * KC / kBlock) * 4 <= 96) return k_gemm_u8s8<WM, WN, TM, TN, KC, 4, NHWC, 0>;
   else return nullptr;
 }
 #define V(WM, WN, TM, TN, KC)                                                                    \
   { "k_gemm_u8s8<" #WM "," #WN "," #TM "," #TN "," #KC ">", WM * TM * 32, WN * TN * 32, KC,       \
-    { { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, false>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, false>,         \
+    { { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, 0>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, 0>,                 \
         deep_or_null<WM, WN, TM, TN, KC, false>() },                                                              \
-      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true, false>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true, false>,           \
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true, 0>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true, 0>,                   \
         deep_or_null<WM, WN, TM, TN, KC, true>() },                                                               \
-      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, true>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, true>, nullptr } } }
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, 1>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, 1>, nullptr },      \
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, 2>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, 2>, nullptr } } }
 const Variant kVariants[] = {
     V(2, 2, 2, 2, 8),  // 0: 128 oc x 128 px
     V(2, 2, 2, 1, 8),  // 1: 128 oc x  64 px
@@ -349,16 +378,16 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   // prefetch depth: must divide the number of fills.  Measured on the configured layers depth 2 is
   // as good as it gets (depth 4 costs registers and gains nothing); EHIP_GEMM_DEPTH overrides.
   const int taps = a.kh * a.kw > 1 ? a.kh * a.kw : 1;
-  a.k_units = taps * a.units_pad;
-  a.chunks_per_tap = a.units_pad / k.kc;
-  a.cpt_magic = div_magic(a.chunks_per_tap);
+  a.k_real = taps * a.units_pad;   // kh x kw: units_pad is the ic2 real units of a tap
+  a.k_units = up(a.k_real, k.kc);
+  a.ic2_magic = div_magic(a.ic2);
   a.kw_magic = div_magic(a.kw > 0 ? a.kw : 1);
   const int nchunks = a.k_units / k.kc;
   int dl = 1;
   const char *env = getenv("EHIP_GEMM_DEPTH");
   if (env && env[0]) dl = atoi(env) >= 4 ? 2 : (atoi(env) >= 2 ? 1 : 0);
   if (taps > 1 && (a.in_nhwc || taps > 64 || nbatch != 1)) return hipErrorInvalidValue;
-  const int fmt = taps > 1 ? 2 : (a.in_nhwc ? 1 : 0);
+  const int fmt = taps > 1 ? (a.ic2 % k.kc == 0 ? 2 : 3) : (a.in_nhwc ? 1 : 0);
   while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[fmt][dl])) --dl;
   hipLaunchKernelGGL(k.kernel[fmt][dl], grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();

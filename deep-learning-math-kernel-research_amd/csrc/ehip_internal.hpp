@@ -28,6 +28,11 @@ struct Epilogue {
   float sum_scale, lo, hi;
   int out_type;         // EHIP_F32 / U8 / S8 / S32
   int with_sum, with_relu;
+  // Non-zero input zero point with padding: the shift depends on which taps fall inside the image
+  // for the output pixel.  shift_tab holds one shift row per class of pixels ([class][tab_stride]);
+  // null = the shift depends on the channel only.
+  const float *shift_tab;
+  int tab_stride;
 };
 
 // D[oc][pixel] = W[oc][k] * X[k][pixel] on MFMA; one "unit" is 16 input channels of one tap.
@@ -49,8 +54,10 @@ struct GemmArgs {
   long long out_batch_stride;  // elements
   int in_nhwc, out_nhwc;       // activations as [n][h][w][c] instead of [n][c/16][h][w][16] (c % 16 == 0)
   int kh, kw, pad_t, pad_l, ih;   // kh * kw > 1: direct convolution as a GEMM over [tap][unit] (blocked input)
-  int k_units, chunks_per_tap;    // set by the launcher: taps * units_pad, units_pad / KC
-  unsigned cpt_magic, kw_magic;
+  const int *cls_h, *cls_w;       // with ep.shift_tab: class of an output row / column; class = cls_h * ncls_w + cls_w
+  int ncls_w;
+  int k_units, k_real;            // set by the launcher: units the K loop walks (a multiple of KC), real ones
+  unsigned ic2_magic, kw_magic;
   int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
 };
@@ -136,6 +143,9 @@ hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_de
 hipError_t launch_prepare_direct(const float *w_blocked, const float *bias, int oc, int ic, int kh, int kw,
                                  int units_pad, int ocpp, const ehip_conv_desc_t &d, float *absmax_scratch,
                                  int8_t *wpacked, float *scale, float *shift, int *wsum, int *comp, hipStream_t s);
+hipError_t launch_fold_direct_border(const int8_t *wpacked, const float *absmax, const float *bias, int oc, int kw,
+                                     int units_pad, int ocpp, const ehip_conv_desc_t &d, const int *rects, int nclass,
+                                     float *shift_tab, hipStream_t s);
 hipError_t launch_prepare_depthwise(const float *w_goihw, const float *bias, int g, const ehip_conv_desc_t &d,
                                     int8_t *wpacked, float *scale, float *shift, int *wsum, hipStream_t s);
 hipError_t launch_prepare_wino(const float *w_blocked, int oc, int ic, int units_pad, int ocpp,
@@ -175,6 +185,14 @@ __device__ __forceinline__ unsigned cvt_u32_rne(float f)
 __device__ __forceinline__ int fastdiv(int n, int d, unsigned magic)
 {
   return d == 1 ? n : (int)__umulhi((unsigned)n, magic);
+}
+// n / d for any 0 <= n < 2^31: the estimate above is never too small and at most one too large
+__device__ __forceinline__ int fastdiv_any(int n, int d, unsigned magic)
+{
+  if (d == 1) return n;
+  unsigned q = __umulhi((unsigned)n, magic);
+  if (q * (unsigned)d > (unsigned)n) --q;
+  return (int)q;
 }
 __device__ __forceinline__ unsigned usat8(unsigned v) { return v > 255u ? 255u : v; }
 __device__ __forceinline__ int ssat8(int v) { return v < -128 ? -128 : (v > 127 ? 127 : v); }
@@ -315,12 +333,12 @@ __device__ __forceinline__ unsigned quant4(const Epilogue &ep, int a0, int a1, i
 // The patch is laid out [16-channel block][pixel][quarter ^ ((pixel / 4) & 3)] in 16-byte cells,
 // which keeps both the writes (fixed quarter, 16 pixels) and the reads (4 pixels x 4 quarters)
 // spread over all banks.
-template <int TM, int TN, int OUT, bool SUM, bool FAST, bool XPOSE>
+template <int TM, int TN, int OUT, bool SUM, bool FAST, bool XPOSE, bool TAB>
 __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
                                                     long long cidx, int oc_first, const size_t (&pix)[TN],
                                                     const bool (&pvalid)[TN], int oc_real, size_t block_stride,
                                                     void *out, v4i *xlds, const size_t (&pixT)[TN][2],
-                                                    const bool (&validT)[TN][2])
+                                                    const bool (&validT)[TN][2], const int *cls)
 {
   const bool relu = ep.with_relu != 0;
   const int lane = threadIdx.x & 63;
@@ -342,6 +360,12 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt) {
       const v16i &a = acc[mt][nt];
+      float4 shq[4] = {k.sh[0], k.sh[1], k.sh[2], k.sh[3]};
+      if (TAB) {   // the shift row of the pixel's border class
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          shq[q] = *reinterpret_cast<const float4 *>(ep.shift_tab + (size_t)cls[nt] * ep.tab_stride + cidx + 32 * mt + 4 * q);
+      }
       v4i s[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q)
@@ -352,10 +376,10 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             float4 r;
-            r.x = requant1(s[q].x, k.sc[q].x, k.sh[q].x, relu, ep.lo, ep.hi);
-            r.y = requant1(s[q].y, k.sc[q].y, k.sh[q].y, relu, ep.lo, ep.hi);
-            r.z = requant1(s[q].z, k.sc[q].z, k.sh[q].z, relu, ep.lo, ep.hi);
-            r.w = requant1(s[q].w, k.sc[q].w, k.sh[q].w, relu, ep.lo, ep.hi);
+            r.x = requant1(s[q].x, k.sc[q].x, shq[q].x, relu, ep.lo, ep.hi);
+            r.y = requant1(s[q].y, k.sc[q].y, shq[q].y, relu, ep.lo, ep.hi);
+            r.z = requant1(s[q].z, k.sc[q].z, shq[q].z, relu, ep.lo, ep.hi);
+            r.w = requant1(s[q].w, k.sc[q].w, shq[q].w, relu, ep.lo, ep.hi);
             s[q] = v4i{__float_as_int(r.x), __float_as_int(r.y), __float_as_int(r.z), __float_as_int(r.w)};
           }
         }
@@ -385,7 +409,7 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
         v4i cell;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          cell[q] = (int)quant4<OUT, SUM, FAST>(ep, s[q].x, s[q].y, s[q].z, s[q].w, k.sc[q], k.sh[q],
+          cell[q] = (int)quant4<OUT, SUM, FAST>(ep, s[q].x, s[q].y, s[q].z, s[q].w, k.sc[q], shq[q],
                                                SUM ? (unsigned)old[nt][q] : 0u);
         if (ok[nt]) *reinterpret_cast<v4i *>(static_cast<uint8_t *>(out) + e[nt]) = cell;
       }
@@ -394,16 +418,17 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
 }
 
 // one uniform switch on the output type (and on the cheap ReLU form) around the whole epilogue;
-// xlds == nullptr: 4-byte outputs are stored directly
-template <int TM, int TN>
-__device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
-                                              long long cidx, int oc_first, const size_t (&pix)[TN],
-                                              const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out,
-                                              v4i *xlds, const size_t (&pixT)[TN][2], const bool (&validT)[TN][2])
+// xlds == nullptr: 4-byte outputs are stored directly.  TAB: per-pixel shift rows (ep.shift_tab, cls).
+template <int TM, int TN, bool TAB>
+__device__ __forceinline__ void epilogue_wave_tab(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
+                                                  long long cidx, int oc_first, const size_t (&pix)[TN],
+                                                  const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out,
+                                                  v4i *xlds, const size_t (&pixT)[TN][2], const bool (&validT)[TN][2],
+                                                  const int *cls)
 {
-#define EHIP_EPI(OUT, SUM, FAST, XP)                                                                              \
-  epilogue_wave_typed<TM, TN, OUT, SUM, FAST, XP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, \
-                                                  out, xlds, pixT, validT)
+#define EHIP_EPI(OUT, SUM, FAST, XP)                                                                                   \
+  epilogue_wave_typed<TM, TN, OUT, SUM, FAST, XP, TAB>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, \
+                                                       out, xlds, pixT, validT, cls)
   // cheap narrowing: ReLU bounds 0 <= lo <= hi (and lo inside the s8 code range for s8 output)
   const bool fast = ep.with_relu && ep.lo >= 0.0f && ep.hi >= ep.lo && (ep.out_type != EHIP_S8 || ep.lo <= 127.0f);
   switch (ep.out_type) {
@@ -424,6 +449,22 @@ __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&a
   }
 #undef EHIP_EPI
 }
+
+// BORDER: the kernel can be asked for per-pixel shift rows (the k x k GEMM form); other kernels do
+// not carry that code at all
+template <int TM, int TN, bool BORDER = false>
+__device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
+                                              long long cidx, int oc_first, const size_t (&pix)[TN],
+                                              const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out,
+                                              v4i *xlds, const size_t (&pixT)[TN][2], const bool (&validT)[TN][2],
+                                              const int *cls = nullptr)
+{
+  if (BORDER && ep.shift_tab)
+    epilogue_wave_tab<TM, TN, true>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
+  else
+    epilogue_wave_tab<TM, TN, false>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
+}
+
 
 }  // namespace ehip
 #endif

@@ -141,6 +141,39 @@ __global__ __launch_bounds__(kBlock) void k_fold_direct(const unsigned *wpacked,
   shift[oc] = sh;
 }
 
+// Shift rows for a non-zero input zero point with padding (src/elx_int8_conv_direct.cpp:311-423):
+// class c covers the output pixels whose valid taps are the rectangle rects[c] = {kh_lo, kh_hi,
+// kw_lo, kw_hi} (inclusive); its shift folds the sum of the weights of those taps only.
+// One thread per (class, channel).
+__global__ __launch_bounds__(kBlock) void k_fold_direct_border(const unsigned *wpacked, const float *absmax,
+                                                               const float *bias, int oc_rows, int kw, int units_pad,
+                                                               int ocpp, FoldParams p, const int4 *rects, int nclass,
+                                                               float *shift_tab)
+{
+  const int idx = blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= nclass * ocpp) return;
+  const int c = idx / ocpp, oc = idx - c * ocpp;
+  float sh = 0.0f;
+  if (oc < oc_rows) {
+    const int4 r = rects[c];
+    int s = 0;
+    for (int kh = r.x; kh <= r.y; ++kh)
+      for (int kwi = r.z; kwi <= r.w; ++kwi)
+        for (int u = 0; u < units_pad; ++u) {
+          const size_t tu = (size_t)(kh * kw + kwi) * units_pad + u;
+          const uint4 cell = *reinterpret_cast<const uint4 *>(wpacked + (tu * ocpp + packed_row_of_oc(oc)) * 4);
+          const unsigned d[4] = {cell.x, cell.y, cell.z, cell.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) s += (int)(signed char)((d[j] >> (8 * k)) & 0xffu);
+        }
+    float sc;
+    fold(p, absmax[oc], (float)s, p.with_bias ? bias[oc] : 0.0f, &sc, &sh);
+  }
+  shift_tab[idx] = sh;
+}
+
 // depthwise: one thread per channel; w is goihw f32 [g][3][3]; packed [g2][kh][16][kw0 kw1 kw2 0]
 __global__ __launch_bounds__(kBlock) void k_prepare_depthwise(const float *w, const float *bias, int g, int G,
                                                               FoldParams p, int8_t *wpacked, float *scale,
@@ -340,6 +373,17 @@ hipError_t launch_prepare_direct(const float *w, const float *bias, int oc, int 
   const FoldParams fp = make_fold(d, d.algorithm == EHIP_CONV_DIRECT_1X1);
   hipLaunchKernelGGL(k_fold_direct, grid_for(ocpp), dim3(kBlock), 0, s, reinterpret_cast<const unsigned *>(wpacked),
                      absmax, bias, oc2 * 16, taps, units_pad, ocpp, fp, scale, shift, wsum, comp);
+  return hipGetLastError();
+}
+
+hipError_t launch_fold_direct_border(const int8_t *wpacked, const float *absmax, const float *bias, int oc, int kw,
+                                     int units_pad, int ocpp, const ehip_conv_desc_t &d, const int *rects, int nclass,
+                                     float *shift_tab, hipStream_t s)
+{
+  const FoldParams fp = make_fold(d, d.with_ip_sum != 0 && d.algorithm == EHIP_CONV_DIRECT_1X1);
+  hipLaunchKernelGGL(k_fold_direct_border, grid_for((size_t)nclass * ocpp), dim3(kBlock), 0, s,
+                     reinterpret_cast<const unsigned *>(wpacked), absmax, bias, up(oc, 16), kw, units_pad, ocpp, fp,
+                     reinterpret_cast<const int4 *>(rects), nclass, shift_tab);
   return hipGetLastError();
 }
 

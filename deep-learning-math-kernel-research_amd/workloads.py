@@ -18,11 +18,12 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 class Workload:
     def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
-                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None):
+                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None, in_z=0.0):
         self.key, self.title = key, title
         self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
         self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
         self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
+        self.in_z = in_z   # input zero point (the reference's "...z" data-type configurations)
         self.nhwc = nhwc   # activations [n][h][w][c] on both sides instead of nChw16c
         # oh given: the right / bottom pads are whatever that output size needs (src/elx_conv.cpp:36-37)
         self.oh = oh if oh is not None else (hw + 2 * pad - k) // stride + 1
@@ -78,7 +79,7 @@ class Workload:
         d = make_desc(self.n, self.ic, self.oc, self.hw, self.hw, self.k, self.k, self.pad, self.stride, g=g,
                       algorithm=self.algorithm, input_type=self.in_type, output_type=self.out_type,
                       with_bias=True, with_relu=True, with_ip_sum=self.with_sum,
-                      input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, 0.0),
+                      input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, self.in_z),
                       output_quant=(out_scale, 0.0), sum_quant=(0.7, 0.0) if self.with_sum else (0.0, 0.0),
                       wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
                       tile_size=6 if self.algorithm == CONV_WINOGRAD else 0,
@@ -110,6 +111,11 @@ WORKLOADS = {w.key: w for w in [
     #  scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh Conv2d_4_depthwise: pad only right / bottom)
     Workload("R13", "3x3 s2 128->128 58x58->28x28 N=64 pad 0, bias+ReLU, s8 out (ResNet-50 v1.5 conv2d_13)", 64, 128, 128,
              58, k=3, pad=0, stride=2, out_type=S8, T=14),
+    # ResNet-50's first layer with the zero-point input configuration of the tuned run
+    # (scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh:12 "U8F32S8F32z"), here on nChw16c input:
+    # the three channels occupy one 16-channel unit per tap
+    Workload("R1", "7x7 s2 3->64 224x224->112x112 N=64 pad 3, input zero point 128, bias+ReLU, s8 out (ResNet-50 conv1)",
+             64, 3, 64, 224, k=7, pad=3, stride=2, out_type=S8, T=14, in_z=128.0),
     Workload("M4", "depthwise 3x3 s2 C=128 56x56->28x28 N=64, bias+ReLU6, u8 out (MobileNet-v1 Conv2d_4)", 64, 128, 128,
              56, k=3, pad=0, stride=2, depthwise=True, w_sigma=0.1, T=28, relu6=True, oh=28),
     Workload("C4a", "Winograd F(4,3) 256->256 @56x56 N=64, fp32 in/out (VGG-16 conv3)", 64, 256, 256, 56, k=3, pad=1,

@@ -91,7 +91,9 @@ EHIP_API const char *ehip_last_error(void);
  *  - CONV_WINOGRAD tile_size 6 (src/elx_int8_conv_wino.cpp): f32 tensors with execution_mode 0xa1xx, or
  *    u8 input with f32/u8/s8 output (U8F32F32F32 / U8F32U8F32 / U8F32S8F32, src/eld_conv.cpp:275-281);
  *    wino_tinput_quant must be set (calibrated sampling).
- * A non-zero input zero point is accepted only where no tap falls on padding. */
+ * A non-zero input zero point with padding is accepted by the 3/5/7 direct kernels (the shift then
+ * depends on the output pixel's set of valid taps, src/elx_int8_conv_direct.cpp:227-423); depthwise and
+ * Winograd accept it only where no tap falls on padding. */
 EHIP_API int ehip_conv_create(const ehip_conv_desc_t *desc, ehip_conv_t **out);
 EHIP_API int ehip_conv_destroy(ehip_conv_t *conv);
 

@@ -385,8 +385,10 @@ int orc_direct_prepare(const orc_conv_params *p, const float *w, const float *bi
   return 0;
 }
 
-int orc_direct_execute(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
-                       const float *scale, const float *shift, void *output, int32_t *acc_out)
+// shift_px_stride == 0: shift is [OCp]; otherwise a per-pixel map [oh][ow][OCp] (shift_px_stride = OCp)
+static int direct_execute_impl(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
+                               const float *scale, const float *shift, size_t shift_px_stride, void *output,
+                               int32_t *acc_out)
 {
   const int OCp = up16(p->oc), ICp = up16(p->ic), I2 = ICp / 16, O2 = OCp / 16;
   const int KH = p->kh, KW = p->kw, IH = p->ih, IW = p->iw, OH = p->oh, OW = p->ow;
@@ -452,7 +454,8 @@ int orc_direct_execute(const orc_conv_params *p, const uint8_t *input, const int
                                  : p->out_type == ORC_S8 ? (int)((int8_t *)output)[oi] : 0;
             // the f32-output path of the reference has no sum fusion
             // (src/elx_int8_conv_direct.cpp:656-716, src/kernel/elk_u8s8_gemm.hxx:234-236)
-            float f = epilogue_f32(a, scale[oc], shift[oc], with_sum && p->out_type != ORC_F32, old_q,
+            const float sh = shift[((size_t)oh * OW + ow) * shift_px_stride + oc];
+            float f = epilogue_f32(a, scale[oc], sh, with_sum && p->out_type != ORC_F32, old_q,
                                    p->sum_scale, relu, p->relu_lo, p->relu_hi);
             if (p->out_type == ORC_F32) ((float *)output)[oi] = f;
             else if (p->out_type == ORC_U8) ((uint8_t *)output)[oi] = usat8((uint32_t)cvt_s32_rne(f));
@@ -460,6 +463,62 @@ int orc_direct_execute(const orc_conv_params *p, const uint8_t *input, const int
           }
       }
   return 0;
+}
+
+int orc_direct_execute(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
+                       const float *scale, const float *shift, void *output, int32_t *acc_out)
+{
+  return direct_execute_impl(p, input, wq, scale, shift, 0, output, acc_out);
+}
+
+// Non-zero input zero point with padding (src/elx_int8_conv_direct.cpp:227-423): a padded tap is
+// skipped, so it must not take part in the "- in_z * sum(w) * scale" term either.  The reference
+// keeps one sum of weights per range of valid kernel rows and columns (wacc_h_ranges_ /
+// wacc_w_ranges_) and one shift per (row class, width block, position in the block); what it
+// encodes is: the shift of an output pixel folds the sum of the weights of the taps that fall
+// inside the image for THAT pixel.  shift_map is [oh][ow][OCp].
+int orc_direct_border_shifts(const orc_conv_params *p, const float *w, const float *bias, float *shift_map)
+{
+  const int OCp = up16(p->oc), ICp = up16(p->ic), I2 = ICp / 16, KH = p->kh, KW = p->kw;
+  auto widx = [&](int oc, int ic, int kh, int kw) {
+    return (((((size_t)(oc / 16) * I2 + ic / 16) * KH + kh) * KW + kw) * 16 + ic % 16) * 16 + oc % 16;
+  };
+#pragma omp parallel for
+  for (int oc = 0; oc < OCp; ++oc) {
+    float absmax = 0.0f;
+    for (int ic = 0; ic < p->ic; ++ic)
+      for (int kh = 0; kh < KH; ++kh)
+        for (int kw = 0; kw < KW; ++kw) absmax = std::max(absmax, std::fabs(w[widx(oc, ic, kh, kw)]));
+    std::vector<int32_t> tapsum((size_t)KH * KW, 0);   // sum over input channels per tap
+    for (int kh = 0; kh < KH; ++kh)
+      for (int kw = 0; kw < KW; ++kw)
+        for (int ic = 0; ic < p->ic; ++ic) tapsum[(size_t)kh * KW + kw] += quant_w(w[widx(oc, ic, kh, kw)], absmax);
+    const float w_S = absmax / 127.0f;
+    const float b = p->with_bias ? bias[oc] : 0.0f;
+    for (int oh = 0; oh < p->oh; ++oh)
+      for (int ow = 0; ow < p->ow; ++ow) {
+        int32_t acc = 0;
+        for (int kh = 0; kh < KH; ++kh) {
+          const int ih = oh * p->stride_h + kh - p->pad_t;
+          if (ih < 0 || ih >= p->ih) continue;
+          for (int kw = 0; kw < KW; ++kw) {
+            const int iw = ow * p->stride_w + kw - p->pad_l;
+            if (iw < 0 || iw >= p->iw) continue;
+            acc += tapsum[(size_t)kh * KW + kw];
+          }
+        }
+        float sc, sh;
+        fold_scale_shift(p, w_S, (float)acc, b, &sc, &sh);
+        shift_map[((size_t)oh * p->ow + ow) * OCp + oc] = sh;
+      }
+  }
+  return 0;
+}
+
+int orc_direct_execute_border(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
+                              const float *scale, const float *shift_map, void *output, int32_t *acc_out)
+{
+  return direct_execute_impl(p, input, wq, scale, shift_map, (size_t)up16(p->oc), output, acc_out);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -75,6 +75,12 @@ int orc_direct_prepare(const orc_conv_params *p, const float *w_blocked, const f
  * `acc` (optional) receives the raw s32 accumulators, nChw16c. */
 int orc_direct_execute(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
                        const float *scale, const float *shift, void *output, int32_t *acc);
+/* input_z != 0 with padding (src/elx_int8_conv_direct.cpp:227-423): the shift of an output pixel
+ * folds the weights of the taps that fall inside the image for that pixel.  shift_map [oh][ow][OCp]. */
+int orc_direct_border_shifts(const orc_conv_params *p, const float *w_blocked, const float *bias,
+                             float *shift_map);
+int orc_direct_execute_border(const orc_conv_params *p, const uint8_t *input, const int8_t *wq,
+                              const float *scale, const float *shift_map, void *output, int32_t *acc);
 
 /* ---- depthwise 3x3 ----
  * src/elx_int8_conv_direct_depthwise.cpp:200-292; wq [G][3][3], scale/shift [G], G = g up to 16. */

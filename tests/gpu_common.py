@@ -34,13 +34,14 @@ class Layer:
 
     def __init__(self, n, ic, oc, hw, k=1, pad=0, stride=1, out_type=ol.U8, algorithm=None, with_sum=False,
                  depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None,
-                 in_nhwc=False, out_nhwc=False, out_hw=None, x_blocked=None):
+                 in_nhwc=False, out_nhwc=False, out_hw=None, x_blocked=None, in_z=0.0):
         E = pkg()
         rng = np.random.default_rng(seed)
         self.E = E
         self.n, self.ic, self.oc, self.hw, self.k = n, ic, oc, hw, k
         self.depthwise = depthwise
         self.in_nhwc, self.out_nhwc = in_nhwc, out_nhwc
+        self.in_z = in_z
         g = ic if depthwise else 1
         x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
         self.x_u8 = ol.quantize_input_u8(x, 1.0 / 255.0, 0.0)
@@ -76,13 +77,13 @@ class Layer:
             sum_scale = float(f32(s_r) / f32(out_scale))
         self.p = ol.make_params(n, ic, oc, hw, hw, k, k, pad, stride, g=g, out_type=out_type, with_bias=with_bias,
                                 with_relu=with_relu, with_sum=with_sum, T=T, out_scale=out_scale, sum_scale=sum_scale,
-                                relu_hi=relu_hi)
+                                relu_hi=relu_hi, in_z=in_z)
         if algorithm is None:
             algorithm = E.CONV_DIRECT_1X1 if (k == 1 and out_type in (ol.U8, ol.S8, ol.S32)) else E.CONV_DIRECT
         self.desc = E.make_desc(n, ic, oc, hw, hw, k, k, pad, stride, g=g, algorithm=algorithm,
                                 output_type=out_type, with_bias=with_bias, with_relu=with_relu, with_ip_sum=with_sum,
                                 output_quant=(out_scale, 0.0), sum_quant=(sum_scale, 0.0),
-                                relu_bound=(0.0, relu_hi), flatting_t=T)
+                                relu_bound=(0.0, relu_hi), flatting_t=T, input_quant=(1.0 / 255.0, in_z))
         if out_hw is not None:
             # output size given by the caller: right / bottom pads follow from it, as the reference
             # recomputes them (src/elx_conv.cpp:36-37)
@@ -108,7 +109,10 @@ class Layer:
                 out, acc = ol.depthwise_execute(p, self.xb, wq, scale, shift)
         else:
             wq, scale, shift, wsum = ol.direct_prepare(p, self.wb, self.bias)
-            if p.out_type == ol.S32:
+            if self.in_z != 0.0 and self.k > 1 and p.out_type != ol.S32:
+                # zero point with padding: the shift depends on the pixel's set of valid taps
+                out, acc, _ = ol.direct_execute_border(p, self.xb, self.wb, self.bias, wq, scale)
+            elif p.out_type == ol.S32:
                 q = ol.ConvParams.from_buffer_copy(p)
                 q.out_type = ol.U8
                 _, acc = ol.direct_execute(q, self.xb, wq, scale, shift)

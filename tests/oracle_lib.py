@@ -179,6 +179,18 @@ def direct_execute(p, x_blocked, wq, scale, shift, out_init=None):
     return out, acc
 
 
+def direct_execute_border(p, x_blocked, w_blocked, bias, wq, scale):
+    """non-zero input zero point with padding: per-pixel shift (sum of the weights of the valid taps)"""
+    OCp = up16(p.oc)
+    smap = np.zeros((p.oh, p.ow, OCp), np.float32)
+    assert oracle().orc_direct_border_shifts(ctypes.byref(p), ptr(w_blocked), ptr(bias), ptr(smap)) == 0
+    out = np.zeros((p.n, OCp // 16, p.oh, p.ow, 16), NP_OF[p.out_type])
+    acc = np.zeros((p.n, OCp // 16, p.oh, p.ow, 16), np.int32)
+    assert oracle().orc_direct_execute_border(ctypes.byref(p), ptr(x_blocked), ptr(wq), ptr(scale), ptr(smap), ptr(out),
+                                              ptr(acc)) == 0
+    return out, acc, smap
+
+
 def depthwise_prepare(p, w_goihw, bias):
     G = up16(p.g)
     wq = np.zeros((G, 3, 3), np.int8)

@@ -138,6 +138,23 @@ def test_direct_kxk_strided(out_type, n, ic, oc, hw, k, pad, stride, out_hw):
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
+# non-zero input zero point with padding (the "U8...z" data-type configurations of the reference's
+# first layers, src/elx_int8_conv_direct.cpp:227-423): one shift per class of border pixels
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8, ol.F32])
+@pytest.mark.parametrize("n,ic,oc,hw,k,pad,stride,out_hw", [
+    (2, 3, 64, 30, 7, 3, 2, None),      # ResNet-50 conv1 shape family: 7x7 s2 p3, three input channels
+    (2, 3, 32, 16, 3, 0, 2, 8),         # MobileNet Conv__224 family: 3x3 s2, pads only right / bottom
+    (1, 32, 48, 9, 3, 1, 1, None),      # 3x3 s1 p1 takes the GEMM form when a zero point meets padding
+    (1, 24, 16, 11, 5, 2, 2, None),
+    (2, 16, 16, 8, 3, 0, 1, None),      # no padding: one class, plain shift
+])
+def test_direct_zero_point_with_padding(out_type, n, ic, oc, hw, k, pad, stride, out_hw):
+    res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=140 + k + stride,
+                                out_hw=out_hw, in_z=128.0, with_relu=(out_type != ol.F32)))
+    if pad or out_hw:
+        assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
 @pytest.mark.parametrize("variant", range(7))
 def test_direct_3x3_stride2_every_kernel_variant(variant, monkeypatch):
     monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))

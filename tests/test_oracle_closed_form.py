@@ -216,3 +216,49 @@ def test_winograd_pipeline_matches_float_convolution():
                   [0.119514472455649, 0.179271708683473, 0.26890756302521],
                   [0.119514472455649, -0.179271708683473, 0.26890756302521], [0, 0, 1]])
     assert np.allclose(u.reshape(6, 6), G @ w[3, 5].astype(np.float64) @ G.T, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("k,pad,stride,hw,out_hw", [(3, 1, 1, 9, None), (3, 0, 2, 12, 6), (7, 3, 2, 15, None), (5, 2, 1, 8, None)])
+@pytest.mark.parametrize("out_type", [ol.F32, ol.S8])
+def test_zero_point_with_padding_matches_the_real_valued_convolution(k, pad, stride, hw, out_hw, out_type):
+    """Input zero point with padding: the oracle's per-pixel shift must make the result equal to the
+    real-valued convolution of the DEQUANTIZED input, (u8 - z) * S, with the dequantized weights --
+    where padding contributes exactly zero.  A shift that folded all taps at the border (or none)
+    misses this by far more than the tolerance."""
+    rng = np.random.default_rng(k * 10 + stride + out_type)
+    n, ic, oc = 2, 24, 16
+    z, in_S = 113.0, 0.017
+    x = rng.integers(0, 256, (n, ic, hw, hw)).astype(np.uint8)
+    w = rng.normal(0, 0.05, (oc, ic, k, k)).astype(f32)
+    b = np.zeros(16, f32)
+    b[:oc] = rng.normal(0, 0.3, oc)
+    out_scale = 0.05
+    p = ol.make_params(n, ic, oc, hw, hw, k, k, stride=stride, out_type=out_type, in_scale=in_S, in_z=z,
+                       out_scale=out_scale, with_relu=False, pad_tl=pad,
+                       out_hw=None if out_hw is None else (out_hw, out_hw), pad=pad)
+    wb = ol.weights_to_blocked(w)
+    wq, scale, shift, wsum = ol.direct_prepare(p, wb, b)
+    out, acc, smap = ol.direct_execute_border(p, ol.to_blocked(x), wb, b, wq, scale)
+    # interior pixels use the plain shift
+    ihs = [oh for oh in range(p.oh) if oh * stride - pad >= 0 and oh * stride - pad + k <= hw]
+    assert ihs and np.array_equal(smap[ihs[0], ihs[0]], shift)
+    assert not np.array_equal(smap[0, 0], shift) or pad == 0
+    # float64 model
+    wq_np, absmax = quant_weights_numpy(w)
+    w_deq = wq_np.astype(np.float64) * (absmax.astype(np.float64) / 127.0)[:, None, None, None]
+    xr = (x.astype(np.float64) - z) * in_S
+    exp = np.zeros((n, oc, p.oh, p.ow))
+    for oh in range(p.oh):
+        for ow in range(p.ow):
+            for kh in range(k):
+                for kw in range(k):
+                    ih, iw = oh * stride + kh - pad, ow * stride + kw - pad
+                    if 0 <= ih < hw and 0 <= iw < hw:
+                        exp[:, :, oh, ow] += np.einsum("nc,oc->no", xr[:, :, ih, iw], w_deq[:, :, kh, kw])
+    exp += b[:oc].astype(np.float64)[None, :, None, None]
+    got = ol.from_blocked(out, oc).astype(np.float64)
+    if out_type == ol.S8:
+        got = got * out_scale
+        assert np.abs(got - np.clip(exp, -128 * out_scale, 127 * out_scale)).max() <= 0.5 * out_scale + 1e-4
+    else:
+        assert np.abs(got - exp).max() <= 2e-4 * max(1.0, np.abs(exp).max())
