@@ -123,6 +123,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size N (scaling studies; "
                                                          "the headline figure uses the configured N)")
+    ap.add_argument("--network", default="", help="instead of one layer: every convolution layer of one of the reference's "
+                                                  "tuned int8 model runs (resnet50_v1_5_int8, mobilenet_v1_int8, "
+                                                  "vgg19_int8), each timed on its own synthetic tensors; prints the "
+                                                  "per-layer table and the images/s of the sum")
     ap.add_argument("--hbm-probe", action="store_true",
                     help="instead of a layer, time plain device copy / fill / read of 1 GiB (the HBM rates a "
                          "trivial kernel reaches on this box)")
@@ -176,6 +180,28 @@ def main():
             return round(nbytes / (e0.elapsed_time(e1) * 1e-3 / reps) / 1e9, 1)
         print(json.dumps({"hbm_probe_bytes": n, "copy_read_plus_write_GBs": rate(lambda: b.copy_(a), 2 * n),
                           "fill_write_GBs": rate(lambda: a.zero_(), n), "sum_read_GBs": rate(lambda: af.sum(), n)}))
+        return
+
+    if args.network:
+        net = W.NETWORKS[args.network]
+        rows, total_s, total_ops = [], 0.0, 0.0
+        for count, w2 in net:
+            l2 = W.DeviceLayer(w2)
+            wall2, ev2 = measure(l2, 50 if w2.ops() > 5e10 else 200, 5)
+            rows.append({"layer": w2.key, "title": w2.title, "count": count, "n": w2.n, "us": round(wall2 * 1e6, 2),
+                         "tops": round(w2.ops() / wall2 / 1e12, 1), "kernel": l2.conv.kernel_name})
+            # the FC layers are configured with n = 1 over 8 x 8 "pixels" = one row per image of the batch
+            total_s += count * wall2
+            total_ops += count * w2.ops()
+            del l2
+            torch.cuda.empty_cache()
+        print(json.dumps({"metric": "network_conv_layers_images_per_s", "network": args.network,
+                          "value": round(64 / total_s, 1), "unit": "images/s", "batch": 64,
+                          "layers_total": sum(c for c, _ in net), "ms_per_batch": round(total_s * 1e3, 4),
+                          "effective_tops": round(total_ops / total_s / 1e12, 1), "data": "synthetic",
+                          "note": "sum over the network's convolution layers of count x time of one execute, each "
+                                  "layer timed back to back on its own device-resident tensors; pooling, residual "
+                                  "adds and softmax are not part of the library", "layers": rows}))
         return
 
     wl = W.WORKLOADS[args.workload]

@@ -120,9 +120,11 @@ int classify(ehip_conv *c)
     const bool in_ok = d.input_fmt == EHIP_NCHW16C || d.input_fmt == EHIP_NHWC;
     const bool out_ok = d.output_fmt == EHIP_NCHW16C || d.output_fmt == EHIP_NHWC;
     if (!in_ok || !out_ok) return fail(EHIP_UNIMPLEMENTED, "activation formats: nChw16c or nhwc");
-    const bool any_nhwc = d.input_fmt == EHIP_NHWC || d.output_fmt == EHIP_NHWC;
-    if (any_nhwc && !(d.kh == 1 && d.kw == 1 && !depthwise))
-      return fail(EHIP_UNIMPLEMENTED, "nhwc activations are only built for 1x1 convolutions");
+    // nhwc input: 1x1 only; nhwc output: every layer the GEMM kernel runs (1x1 and kh x kw direct)
+    if (d.input_fmt == EHIP_NHWC && !(d.kh == 1 && d.kw == 1 && !depthwise))
+      return fail(EHIP_UNIMPLEMENTED, "nhwc input is only built for 1x1 convolutions");
+    if (d.output_fmt == EHIP_NHWC && (depthwise || d.algorithm == EHIP_CONV_WINOGRAD))
+      return fail(EHIP_UNIMPLEMENTED, "nhwc output is only built for the direct 1x1 and kh x kw executors");
     if ((d.input_fmt == EHIP_NHWC && d.ic % 16) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
       return fail(EHIP_UNIMPLEMENTED, "nhwc: channel counts must be multiples of 16");
   }
@@ -192,7 +194,7 @@ int classify(ehip_conv *c)
           d.ow == d.iw + d.pad_l + d.pad_r - 2 && d.oh == d.ih + d.pad_t + d.pad_b - 2;
       // the GEMM family walks [tap][unit] for kh x kw; it also owns the per-pixel shift that a zero
       // point with padding needs
-      c->family = (s1_3x3 && !(d.input_z != 0.0f && padded)) ? FAM_CONV_3X3 : FAM_GEMM_1X1;
+      c->family = (s1_3x3 && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC) ? FAM_CONV_3X3 : FAM_GEMM_1X1;
       return EHIP_OK;
     }
     return fail(EHIP_UNIMPLEMENTED, "direct: c160: shape not supported");
@@ -263,7 +265,7 @@ int setup_workspace(ehip_conv *c)
     c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2 * c->taps, 1, c->taps > 1 ? 1 : d.stride_w);
     // kh x kw: the K axis is [tap][ic2 real units]; only its end is padded to the kernel's chunk
     c->units_pad = c->taps > 1 ? c->ic2 : up(c->ic2, gemm_variant_chunk(c->variant));
-    c->kernel_name = gemm_variant_name(c->variant);
+    c->kernel_name = gemm_smallk_applies(c->ic2, c->taps, 1) ? "k_gemm_smallk_u8s8" : gemm_variant_name(c->variant);
     if (c->taps > 1 && d.input_z != 0.0f) {
       // classes of output rows / columns by their range of valid kernel rows / columns
       auto classes = [](int on, int in, int k, int stride, int pad, std::vector<int> &cls, std::vector<std::pair<int, int>> &rng) {

@@ -300,6 +300,117 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   TRACE_POINT(15);
 }
 
+// ---- 1x1 layers with few input channels: weights stay in registers ---------------------------
+// With K <= 128 a workgroup of the kernel above multiplies for a few hundred clocks and spends the
+// rest of its life on start-up, barriers and its epilogue -- and such a layer needs thousands of
+// them.  Here nothing is shared: a wave loads the weights of its 32 output channels ONCE into
+// registers (KS operands of one 32-channel tile), then walks over 32-pixel tiles: the tile's activations go straight
+// from memory into MFMA operands (a lane's operand is one 16-byte cell, blocked or nhwc), the next
+// tile's are in flight while this one is multiplied, and the results leave through the same
+// epilogue.  No LDS (apart from the 4 KB exchange patch of 4-byte outputs), no barrier.
+// The four waves of a workgroup split into a.sk_wo tiles of 32 channels (1, 2 or 4) times
+// 4 / a.sk_wo pixel tiles of TNW x 32 pixels; waves of different channel groups walk the same tiles at the same time,
+// so the activations reach the CU once.  grid: (workgroups over pixel tiles, 4-wave channel blocks).
+template <int TNW, int KS>
+__global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
+{
+  __shared__ v4i xpatch[4 * 256];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int wo = wave % a.sk_wo, wp = wave / a.sk_wo, wpn = 4 / a.sk_wo;
+  const int oc0 = (blockIdx.y * a.sk_wo + wo) * 32;
+  const int oc_real = a.oc2 * 16;
+  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  const long long unit_stride = a.in_nhwc ? 16 : (long long)a.ihw * 16;
+
+  // weights: packed [unit][OCpp rows][16]; lane = row l32 of the wave's tile, unit 2 ks + lh
+  v4i wreg[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    wreg[ks] = *reinterpret_cast<const v4i *>(a.w + ((long long)(2 * ks + lh) * a.ocpp + oc0 + l32) * 16);
+
+  // byte offset of output pixel gp's first input cell (clamped past the end)
+  auto input_pixel = [&](int gp) -> long long {
+    gp = gp < a.p_total ? gp : a.p_total - 1;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic);
+    const int r = gp - n * a.ohw;
+    long long sp;
+    if (dense) {
+      sp = r;
+    } else {
+      const int oh = fastdiv(r, a.ow, a.ow_magic);
+      sp = (long long)(oh * a.stride_h) * a.iw + (r - oh * a.ow) * a.stride_w;
+    }
+    return a.in_nhwc ? ((long long)n * a.ihw + sp) * a.ic2 * 16 : ((long long)n * a.ic2 * a.ihw + sp) * 16;
+  };
+  auto pixel_offset = [&](int gp, bool &valid) -> size_t {
+    valid = gp < a.p_total;
+    const int gpc = valid ? gp : 0;
+    if (a.out_nhwc) return (size_t)gpc * oc_real;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
+    return ((size_t)n * a.oc2 * a.ohw + (gpc - n * a.ohw)) * 16;
+  };
+  // the lane's units: 2 ks + lh, clamped to the real ones (padded units multiply zero weights)
+  int ucl[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ucl[ks] = 2 * ks + lh < a.ic2 ? 2 * ks + lh : a.ic2 - 1;
+
+  // a wave-tile is TNW x 32 consecutive pixels
+  const int ntiles = (a.p_total + 32 * TNW - 1) / (32 * TNW);
+  const int tstep = wpn * gridDim.x;
+  int tile = wpn * blockIdx.x + wp;
+  v4i breg[TNW][KS];
+  auto load_b = [&](int t) {
+#pragma unroll
+    for (int nt = 0; nt < TNW; ++nt) {
+      const uint8_t *src = a.in + input_pixel((t * TNW + nt) * 32 + l32);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) breg[nt][ks] = *reinterpret_cast<const v4i *>(src + (long long)ucl[ks] * unit_stride);
+    }
+  };
+  if (tile < ntiles) load_b(tile);
+  const long long cidx = oc0 + 16 * lh;
+  // the per-channel constants of the wave's tile stay in registers for all its pixel tiles (fetched
+  // per tile they would cost the vector-memory path more than the activations do)
+  OcConsts k0;
+  load_consts(k0, a.ep, cidx);
+  v4i *xlds = ((a.ep.out_type == EHIP_F32 || a.ep.out_type == EHIP_S32) && !a.out_nhwc) ? xpatch + wave * 256 : nullptr;
+  for (; tile < ntiles; tile += tstep) {
+    v16i acc[1][TNW];
+#pragma unroll
+    for (int nt = 0; nt < TNW; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[0][nt][v] = 0;
+    v4i bcur[TNW][KS];
+#pragma unroll
+    for (int nt = 0; nt < TNW; ++nt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) bcur[nt][ks] = breg[nt][ks] ^ (int)0x80808080;
+    // next tile's activations travel during this tile's multiplies and epilogue (the last wave-tile
+    // re-reads its own)
+    load_b(tile + tstep < ntiles ? tile + tstep : tile);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int nt = 0; nt < TNW; ++nt)
+        acc[0][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ks], bcur[nt][ks], acc[0][nt], 0, 0, 0);
+    size_t pix[TNW], pixT[TNW][2];
+    bool pvalid[TNW], validT[TNW][2];
+#pragma unroll
+    for (int nt = 0; nt < TNW; ++nt) {
+      const int p0 = (tile * TNW + nt) * 32;
+      pix[nt] = pixel_offset(p0 + l32, pvalid[nt]);
+      pixT[nt][0] = pixel_offset(p0 + (lane >> 2), validT[nt][0]);
+      pixT[nt][1] = pixel_offset(p0 + (lane >> 2) + 16, validT[nt][1]);
+    }
+    epilogue_wave<1, TNW>(a.ep, acc, k0, cidx, oc0 + 16 * lh, pix, pvalid, oc_real,
+                          a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT);
+  }
+}
+
 namespace {
 struct Variant {
   const char *name;
@@ -368,8 +479,50 @@ int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride)
   return best;
 }
 
+namespace {
+template <int KS>
+void (*smallk_kernel(int tnw))(GemmArgs)
+{
+  return tnw == 2 ? k_gemm_smallk_u8s8<2, KS> : k_gemm_smallk_u8s8<1, KS>;
+}
+}  // namespace
+
+// 1x1 layers with at most 8 input units (128 channels): the weights-in-registers kernel.  The channel
+// rows past the last real block are zero rows of the packed weights (OCpp is a multiple of 256).
+bool gemm_smallk_applies(int ic2, int taps, int nbatch)
+{
+  const char *env = getenv("EHIP_GEMM_SMALLK");
+  if (env && env[0] == '0') return false;
+  return nbatch == 1 && taps <= 1 && ic2 <= 8;
+}
+
+hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s)
+{
+  GemmArgs a = a0;
+  const int ks = a.ic2 <= 2 ? 1 : (a.ic2 <= 4 ? 2 : 4);
+  const int oc_tiles = (a.oc2 * 16 + 31) / 32;
+  // one tile of 32 channels per wave (its constants then stay in registers) x two tiles of 32 pixels
+  const int groups = oc_tiles;
+  a.sk_wo = groups >= 4 ? 4 : (groups >= 2 ? 2 : 1);
+  const int ny = (groups + a.sk_wo - 1) / a.sk_wo;
+  int tnw = 1;   // (two pixel tiles per iteration cost more in occupancy than they gain in overlap)
+  if (const char *env = getenv("EHIP_SMALLK_TNW")) tnw = atoi(env) == 2 ? 2 : 1;
+  const int ntiles = (a.p_total + 32 * tnw - 1) / (32 * tnw);
+  const int wpn = 4 / a.sk_wo;
+  // one resident set of workgroups, so that a wave amortises its weights over many tiles
+  int nx = (ntiles + wpn - 1) / wpn;
+  int wgs = 768;   // three workgroups per CU: what the register budget of the one-tile form admits, and the measured optimum
+  if (const char *env = getenv("EHIP_SMALLK_WGS")) wgs = atoi(env) > 0 ? atoi(env) : wgs;
+  const int cap = (wgs + ny - 1) / ny;
+  if (nx > cap) nx = cap;
+  void (*kernel)(GemmArgs) = ks == 1 ? smallk_kernel<1>(tnw) : (ks == 2 ? smallk_kernel<2>(tnw) : smallk_kernel<4>(tnw));
+  hipLaunchKernelGGL(kernel, dim3(nx, ny), dim3(kBlock), 0, s, a);
+  return hipGetLastError();
+}
+
 hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s)
 {
+  if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s);
   const Variant &k = kVariants[variant];
   GemmArgs a = a0;
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;

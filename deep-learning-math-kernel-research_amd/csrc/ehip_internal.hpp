@@ -56,6 +56,7 @@ struct GemmArgs {
   int kh, kw, pad_t, pad_l, ih;   // kh * kw > 1: direct convolution as a GEMM over [tap][unit] (blocked input)
   const int *cls_h, *cls_w;       // with ep.shift_tab: class of an output row / column; class = cls_h * ncls_w + cls_w
   int ncls_w;
+  int sk_wo;                      // set by the small-K launcher: waves of a workgroup along the channels (1, 2, 4)
   int k_units, k_real;            // set by the launcher: units the K loop walks (a multiple of KC), real ones
   unsigned ic2_magic, kw_magic;
   int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
@@ -122,6 +123,7 @@ struct WinoFusedArgs {
 
 // ---- launchers (implemented next to their kernels) ------------------------------------------
 hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s);
+bool gemm_smallk_applies(int ic2, int taps, int nbatch);
 int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride);
 int gemm_variant_chunk(int variant);
 int gemm_num_variants();

@@ -18,13 +18,14 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 class Workload:
     def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
-                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None, in_z=0.0):
+                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None, in_z=0.0, nhwc_out=False):
         self.key, self.title = key, title
         self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
         self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
         self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
         self.in_z = in_z   # input zero point (the reference's "...z" data-type configurations)
         self.nhwc = nhwc   # activations [n][h][w][c] on both sides instead of nChw16c
+        self.nhwc_in, self.nhwc_out = nhwc, nhwc or nhwc_out
         # oh given: the right / bottom pads are whatever that output size needs (src/elx_conv.cpp:36-37)
         self.oh = oh if oh is not None else (hw + 2 * pad - k) // stride + 1
 
@@ -84,8 +85,10 @@ class Workload:
                       wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
                       tile_size=6 if self.algorithm == CONV_WINOGRAD else 0,
                       execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
-        if self.nhwc:
-            d.input_fmt = d.output_fmt = NHWC
+        if self.nhwc_in:
+            d.input_fmt = NHWC
+        if self.nhwc_out:
+            d.output_fmt = NHWC
         if d.oh != self.oh:
             d.oh = d.ow = self.oh
             d.pad_r = d.pad_b = max(0, (self.oh - 1) * self.stride + self.k - self.hw - self.pad)
@@ -133,6 +136,77 @@ WORKLOADS = {w.key: w for w in [
     Workload("C5b", "depthwise 3x3 C=960 @7x7 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 960, 960, 7, k=3, pad=1,
              depthwise=True, w_sigma=0.1, T=7, relu6=True),
 ]}
+
+
+def _L(count, key, title, n, ic, oc, hw, **kw):
+    """one distinct layer shape of a network and how many of the network's layers have it"""
+    return count, Workload(key, title, n, ic, oc, hw, **kw)
+
+
+def _pw(count, name, ic, oc, hw, stride=1, nhwc_in=False, nhwc_out=False, n=64, out_type=S8, algorithm=CONV_DIRECT_1X1):
+    w = Workload(name, "1x1%s %d->%d @%d" % (" s2" if stride == 2 else "", ic, oc, hw), n, ic, oc, hw, stride=stride,
+                 algorithm=algorithm, out_type=out_type)
+    w.nhwc_in, w.nhwc_out = nhwc_in, nhwc_out
+    return count, w
+
+
+def _wino(count, name, ic, oc, hw):
+    return _L(count, name, "Winograd F(4,3) %d->%d @%d u8->s8" % (ic, oc, hw), 64, ic, oc, hw, k=3, pad=1,
+              algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02)
+
+
+def _dw(count, name, c, hw, stride):
+    if stride == 1:
+        return _L(count, name, "depthwise 3x3 C=%d @%d" % (c, hw), 64, c, c, hw, k=3, pad=1, depthwise=True, w_sigma=0.1,
+                  T=min(hw, 28), relu6=True, out_type=U8)
+    return _L(count, name, "depthwise 3x3 s2 C=%d %d->%d" % (c, hw, hw // 2), 64, c, c, hw, k=3, pad=0, stride=2,
+              depthwise=True, w_sigma=0.1, T=min(hw // 2, 28), relu6=True, oh=hw // 2, out_type=U8)
+
+
+# The convolution layers of the reference's tuned int8 model runs, batch 64, as (count, layer shape):
+# shapes, strides, pads, data types and activation layouts follow the command lines of
+#   scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh   (ResNet-50 v1.5: 53 convolutions + the FC layer)
+#   scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh  (MobileNet-v1: 27 convolutions + the FC layer)
+#   scripts/best_configs/vgg-n64-8180-1s-int8.sh         (VGG-19 without conv1_1: 15 convolutions)
+# and the counts follow the layer names listed above each command there.  Two deviations, both on
+# layers with three input channels or 1001 output channels: the first layers take nChw16c input where
+# the scripts pass three-channel nhwc, and MobileNet's FC writes nChw16c where the script asks for nhwc.
+NETWORKS = {
+    "resnet50_v1_5_int8": [
+        _L(1, "conv2d", "7x7 s2 3->64 224->112 pad 3, zero point 128, nhwc out", 64, 3, 64, 224, k=7, pad=3, stride=2,
+           out_type=S8, T=14, in_z=128.0, nhwc_out=True),
+        _wino(3, "conv2d_3", 64, 64, 56), _wino(3, "conv2d_16", 128, 128, 28), _wino(5, "conv2d_29", 256, 256, 14),
+        _wino(2, "conv2d_48", 512, 512, 7),
+        _L(1, "conv2d_13", "3x3 s2 128->128 58->28", 64, 128, 128, 58, k=3, stride=2, out_type=S8, T=14),
+        _L(1, "conv2d_26", "3x3 s2 256->256 30->14", 64, 256, 256, 30, k=3, stride=2, out_type=S8, T=14),
+        _L(1, "conv2d_45", "3x3 s2 512->512 16->7", 64, 512, 512, 16, k=3, stride=2, out_type=S8, T=7),
+        _pw(1, "conv2d_11", 256, 512, 56, stride=2), _pw(1, "conv2d_24", 512, 1024, 28, stride=2),
+        _pw(1, "conv2d_43", 1024, 2048, 14, stride=2),
+        _pw(1, "conv2d_2", 64, 64, 56), _pw(4, "conv2d_1", 64, 256, 56), _pw(2, "conv2d_5", 256, 64, 56),
+        _pw(1, "conv2d_12", 256, 128, 56),
+        _pw(4, "conv2d_14", 128, 512, 28), _pw(3, "conv2d_15", 512, 128, 28, nhwc_out=True), _pw(1, "conv2d_25", 512, 256, 28),
+        _pw(6, "conv2d_27", 256, 1024, 14, nhwc_out=True), _pw(5, "conv2d_28", 1024, 256, 14, nhwc_in=True, nhwc_out=True),
+        _pw(1, "conv2d_44", 1024, 512, 14, nhwc_in=True, nhwc_out=True),
+        _pw(3, "conv2d_46", 512, 2048, 7, nhwc_out=True), _pw(2, "conv2d_47", 2048, 512, 7, nhwc_in=True, nhwc_out=True),
+        _pw(1, "FC", 2048, 1008, 8, nhwc_in=True, nhwc_out=True, n=1, out_type=F32, algorithm=CONV_DIRECT),
+    ],
+    "mobilenet_v1_int8": [
+        _L(1, "Conv__224", "3x3 s2 3->32 224->112, pads right/bottom, zero point 128", 64, 3, 32, 224, k=3, pad=0, stride=2,
+           out_type=S8, T=14, in_z=128.0, oh=112),
+        _pw(1, "Conv__226", 32, 64, 112), _pw(1, "Conv__228", 64, 128, 56), _pw(1, "Conv__230", 128, 128, 56),
+        _pw(1, "Conv__232", 128, 256, 28), _pw(1, "Conv__234", 256, 256, 28), _pw(1, "Conv__236", 256, 512, 14),
+        _pw(5, "Conv__238", 512, 512, 14), _pw(1, "Conv__248", 512, 1024, 7), _pw(1, "Conv__250", 1024, 1024, 7, nhwc_out=True),
+        _pw(1, "Conv__252", 1024, 1001, 8, nhwc_in=True, n=1, out_type=F32, algorithm=CONV_DIRECT),
+        _dw(1, "Conv2d_1_depthwise", 32, 112, 1), _dw(1, "Conv2d_2_depthwise", 64, 112, 2), _dw(1, "Conv2d_3_depthwise", 128, 56, 1),
+        _dw(1, "Conv2d_4_depthwise", 128, 56, 2), _dw(1, "Conv2d_5_depthwise", 256, 28, 1), _dw(1, "Conv2d_6_depthwise", 256, 28, 2),
+        _dw(5, "Conv2d_7_depthwise", 512, 14, 1), _dw(1, "Conv2d_12_depthwise", 512, 14, 2), _dw(1, "Conv2d_13_depthwise", 1024, 7, 1),
+    ],
+    "vgg19_int8": [
+        _wino(1, "conv1_2", 64, 64, 224), _wino(1, "conv2_1", 64, 128, 112), _wino(1, "conv2_2", 128, 128, 112),
+        _wino(1, "conv3_1", 128, 256, 56), _wino(3, "conv3_2", 256, 256, 56), _wino(1, "conv4_1", 256, 512, 28),
+        _wino(3, "conv4_2", 512, 512, 28), _wino(4, "conv5_1", 512, 512, 14),
+    ],
+}
 
 
 class DeviceLayer:

@@ -57,7 +57,26 @@ def test_conv1x1_lazy_first_run_and_no_bias():
 @pytest.mark.parametrize("variant", range(7))
 def test_conv1x1_every_kernel_variant(variant, monkeypatch):
     monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
-    res = run_and_compare(Layer(2, 128, 80, 11, out_type=ol.S8, with_sum=True, seed=40 + variant))
+    res = run_and_compare(Layer(2, 144, 80, 11, out_type=ol.S8, with_sum=True, seed=40 + variant))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
+# layers with at most 128 input channels take the weights-in-registers kernel
+@pytest.mark.parametrize("out_type", [ol.S32, ol.U8, ol.S8, ol.F32])
+@pytest.mark.parametrize("n,ic,oc,hw,stride,nhwc", [(2, 64, 256, 9, 1, False), (3, 32, 64, 7, 1, False), (1, 128, 512, 6, 1, True),
+                                                    (2, 16, 16, 5, 1, False), (2, 96, 48, 9, 2, False), (1, 8, 40, 33, 1, False),
+                                                    (2, 128, 144, 8, 2, True)])
+def test_conv1x1_few_input_channels(out_type, n, ic, oc, hw, stride, nhwc):
+    if nhwc and oc % 16:
+        pytest.skip("nhwc needs whole channel blocks")
+    res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, seed=170 + ic + oc,
+                                with_sum=out_type in (ol.U8, ol.S8), in_nhwc=nhwc, out_nhwc=nhwc))
+    assert res["conv"].kernel_name == "k_gemm_smallk_u8s8"
+
+
+def test_conv1x1_few_input_channels_can_be_switched_off(monkeypatch):
+    monkeypatch.setenv("EHIP_GEMM_SMALLK", "0")
+    res = run_and_compare(Layer(2, 64, 96, 9, out_type=ol.U8, seed=177))
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
@@ -88,9 +107,15 @@ def test_nhwc_is_refused_where_it_is_not_built():
     with pytest.raises(E.EulerHipError):
         E.Conv(d)
     d = E.make_desc(1, 64, 64, 8, 8, 3, 3, 1, algorithm=E.CONV_DIRECT)
-    d.output_fmt = E.NHWC  # 3x3
+    d.input_fmt = E.NHWC   # nhwc input of a 3x3
     with pytest.raises(E.EulerHipError):
         E.Conv(d)
+
+
+@pytest.mark.parametrize("k,pad,stride", [(3, 1, 1), (3, 1, 2), (7, 3, 2)])
+def test_direct_kxk_nhwc_output(k, pad, stride):
+    res = run_and_compare(Layer(2, 32, 48, 13, k=k, pad=pad, stride=stride, out_type=ol.S8, seed=160 + k + stride, out_nhwc=True))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
 # ---- 3x3 direct (c160) ------------------------------------------------------------------------------
