@@ -127,6 +127,10 @@ def main():
                                                   "tuned int8 model runs (resnet50_v1_5_int8, mobilenet_v1_int8, "
                                                   "vgg19_int8), each timed on its own synthetic tensors; prints the "
                                                   "per-layer table and the images/s of the sum")
+    ap.add_argument("--direct3x3", action="store_true",
+                    help="with --network: run the 3x3 stride-1 layers with CONV_DIRECT instead of the Winograd "
+                         "algorithm the reference's scripts ask for (on this GPU the direct kernel is the faster one; "
+                         "its results are the reference's DIRECT results, not its Winograd results)")
     ap.add_argument("--hbm-probe", action="store_true",
                     help="instead of a layer, time plain device copy / fill / read of 1 GiB (the HBM rates a "
                          "trivial kernel reaches on this box)")
@@ -186,6 +190,9 @@ def main():
         net = W.NETWORKS[args.network]
         rows, total_s, total_ops = [], 0.0, 0.0
         for count, w2 in net:
+            if args.direct3x3 and w2.algorithm == E.CONV_WINOGRAD:
+                w2 = W.Workload(w2.key, "3x3 direct %d->%d @%d u8->s8" % (w2.ic, w2.oc, w2.hw), w2.n, w2.ic, w2.oc, w2.hw, k=3,
+                                pad=1, out_type=w2.out_type, T=14 if w2.hw % 14 == 0 else (7 if w2.hw % 7 == 0 else 0))
             l2 = W.DeviceLayer(w2)
             wall2, ev2 = measure(l2, 50 if w2.ops() > 5e10 else 200, 5)
             rows.append({"layer": w2.key, "title": w2.title, "count": count, "n": w2.n, "us": round(wall2 * 1e6, 2),
@@ -196,6 +203,7 @@ def main():
             del l2
             torch.cuda.empty_cache()
         print(json.dumps({"metric": "network_conv_layers_images_per_s", "network": args.network,
+                          "three_by_three": "direct" if args.direct3x3 else "as configured by the reference's script",
                           "value": round(64 / total_s, 1), "unit": "images/s", "batch": 64,
                           "layers_total": sum(c for c, _ in net), "ms_per_batch": round(total_s * 1e3, 4),
                           "effective_tops": round(total_ops / total_s / 1e12, 1), "data": "synthetic",

@@ -129,7 +129,7 @@ def test_conv3x3_no_padding():
     run_and_compare(Layer(2, 32, 32, 12, k=3, pad=0, out_type=ol.U8, seed=3))
 
 
-@pytest.mark.parametrize("variant", range(11))
+@pytest.mark.parametrize("variant", range(15))
 def test_conv3x3_every_virtual_row_kernel_variant(variant, monkeypatch):
     monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", str(variant))
     res = run_and_compare(Layer(2, 64, 144, 13, k=3, pad=1, out_type=ol.U8, seed=80 + variant))
