@@ -16,6 +16,7 @@ LIB = os.path.join(HERE, "libeuler_hip.so")
 SOURCES = [
     "ehip_gemm.hip",
     "ehip_conv3x3v.hip",
+    "ehip_fewch.hip",
     "ehip_depthwise.hip",
     "ehip_wino.hip",
     "ehip_prepare.hip",

@@ -47,6 +47,9 @@ struct ehip_conv {
   int nclass = 0, ncls_w = 0;
   int *cls_h = nullptr, *cls_w = nullptr, *rects = nullptr;
   float *shift_tab = nullptr;
+  // k x k direct with at most four input channels: ppc = 16 / ic pixels per 16-byte cell, nu cells per
+  // kernel row; gtaps = taps of the K axis of the packed weights (kh * nu there, kh * kw otherwise)
+  int ppc = 0, nu = 0, gtaps = 1;
   // 3x3
   int chunk_units = 2;
   // depthwise
@@ -120,12 +123,14 @@ int classify(ehip_conv *c)
     const bool in_ok = d.input_fmt == EHIP_NCHW16C || d.input_fmt == EHIP_NHWC;
     const bool out_ok = d.output_fmt == EHIP_NCHW16C || d.output_fmt == EHIP_NHWC;
     if (!in_ok || !out_ok) return fail(EHIP_UNIMPLEMENTED, "activation formats: nChw16c or nhwc");
-    // nhwc input: 1x1 only; nhwc output: every layer the GEMM kernel runs (1x1 and kh x kw direct)
-    if (d.input_fmt == EHIP_NHWC && !(d.kh == 1 && d.kw == 1 && !depthwise))
-      return fail(EHIP_UNIMPLEMENTED, "nhwc input is only built for 1x1 convolutions");
+    // nhwc input: 1x1, and kh x kw over at most four channels (the first layer of an image network,
+    // whose nhwc input is compact: ic bytes per pixel); nhwc output: 1x1 and kh x kw direct
+    const bool fewch = d.algorithm == EHIP_CONV_DIRECT && !depthwise && conv_fewch_applies(d.ic, d.kh, d.kw);
+    if (d.input_fmt == EHIP_NHWC && !(d.kh == 1 && d.kw == 1 && !depthwise) && !fewch)
+      return fail(EHIP_UNIMPLEMENTED, "nhwc input is only built for 1x1 convolutions and for kh x kw over at most 4 channels");
     if (d.output_fmt == EHIP_NHWC && (depthwise || d.algorithm == EHIP_CONV_WINOGRAD))
       return fail(EHIP_UNIMPLEMENTED, "nhwc output is only built for the direct 1x1 and kh x kw executors");
-    if ((d.input_fmt == EHIP_NHWC && d.ic % 16) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
+    if ((d.input_fmt == EHIP_NHWC && d.ic % 16 && !fewch) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
       return fail(EHIP_UNIMPLEMENTED, "nhwc: channel counts must be multiples of 16");
   }
 
@@ -195,6 +200,12 @@ int classify(ehip_conv *c)
       // the GEMM family walks [tap][unit] for kh x kw; it also owns the per-pixel shift that a zero
       // point with padding needs
       c->family = (s1_3x3 && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC) ? FAM_CONV_3X3 : FAM_GEMM_1X1;
+      {
+        // at most four input channels: several pixels per operand cell, weights in registers
+        const char *env = getenv("EHIP_FEWCH");
+        if (conv_fewch_applies(d.ic, d.kh, d.kw) && (d.input_fmt == EHIP_NHWC || !(env && env[0] == '0')))
+          c->family = FAM_CONV_FEWCH;
+      }
       return EHIP_OK;
     }
     return fail(EHIP_UNIMPLEMENTED, "direct: c160: shape not supported");
@@ -241,7 +252,7 @@ int setup_workspace(ehip_conv *c)
   int rc;
   switch (c->family) {
   case FAM_CONV_3X3: {
-    c->taps = 9;
+    c->taps = c->gtaps = 9;
     c->nbatch = 1;
     if ((long long)(d.oh + 2) * (d.ow + 2) * (d.ow + 2) >= (1ll << 31))
       return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too large");
@@ -255,6 +266,7 @@ int setup_workspace(ehip_conv *c)
     c->family = FAM_GEMM_1X1;   // rows too wide for the staged tile: the GEMM form has no such limit
   }
   // fall through
+  case FAM_CONV_FEWCH:
   case FAM_GEMM_1X1: {
     if ((long long)d.n * d.oh * d.ow >= (1ll << 30) || (long long)d.oh * d.ow * d.ow >= (1ll << 32))
       return fail(EHIP_UNIMPLEMENTED, "direct: more than 2^30 output pixels");
@@ -262,10 +274,23 @@ int setup_workspace(ehip_conv *c)
     c->nbatch = 1;
     if (c->taps > 1 && (long long)d.n * c->ic2 * d.ih * d.iw * 16 >= (1ll << 40))
       return fail(EHIP_UNIMPLEMENTED, "direct: input too large");
-    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2 * c->taps, 1, c->taps > 1 ? 1 : d.stride_w);
+    c->gtaps = c->taps;
+    if (c->family == FAM_CONV_FEWCH &&
+        (size_t)d.kh * conv_fewch_row_pitch(d.ic, d.kw, d.iw, d.ow, d.stride_w, d.pad_l) > 48 * 1024) {
+      // one strip's input rows do not fit in LDS
+      if (d.input_fmt == EHIP_NHWC) return fail(EHIP_UNIMPLEMENTED, "direct: few-channel nhwc input: rows too wide");
+      c->family = FAM_GEMM_1X1;
+    }
+    if (c->family == FAM_CONV_FEWCH) {
+      c->ppc = 16 / d.ic;
+      c->nu = (d.kw + c->ppc - 1) / c->ppc;
+      c->gtaps = d.kh * c->nu;
+    }
+    c->variant = gemm_pick_variant(d.n * d.oh * d.ow, c->oc2, c->ic2 * c->gtaps, 1, c->taps > 1 ? 1 : d.stride_w);
     // kh x kw: the K axis is [tap][ic2 real units]; only its end is padded to the kernel's chunk
     c->units_pad = c->taps > 1 ? c->ic2 : up(c->ic2, gemm_variant_chunk(c->variant));
     c->kernel_name = gemm_smallk_applies(c->ic2, c->taps, 1) ? "k_gemm_smallk_u8s8" : gemm_variant_name(c->variant);
+    if (c->family == FAM_CONV_FEWCH) c->kernel_name = "k_conv_fewch_u8s8";
     if (c->taps > 1 && d.input_z != 0.0f) {
       // classes of output rows / columns by their range of valid kernel rows / columns
       auto classes = [](int on, int in, int k, int stride, int pad, std::vector<int> &cls, std::vector<std::pair<int, int>> &rng) {
@@ -355,7 +380,7 @@ int setup_workspace(ehip_conv *c)
   } else {
     c->ocpp = up(c->oc2 * 16, kOcTile);
     // (the K loop may run up to one chunk of 8 units past the last real one: zero rows)
-    c->wpacked_bytes = (size_t)c->nbatch * up(c->taps * c->units_pad, 8) * c->ocpp * 16;
+    c->wpacked_bytes = (size_t)c->nbatch * up(c->gtaps * c->units_pad, 8) * c->ocpp * 16;
   }
   c->per_oc = (size_t)c->nbatch * c->ocpp;
   if ((rc = dev_alloc(&c->wpacked, c->wpacked_bytes, true)) != EHIP_OK) return rc;
@@ -457,8 +482,17 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const vo
   const float *w = static_cast<const float *>(weights_dev);
   const float *b = static_cast<const float *>(bias_dev);
   switch (c->family) {
+  case FAM_CONV_FEWCH:
   case FAM_GEMM_1X1:
   case FAM_CONV_3X3:
+    if (c->family == FAM_CONV_FEWCH) {
+      HIP_TRY(launch_prepare_direct_px(w, b, d.oc, d.ic, d.kh, d.kw, c->ppc, c->nu, c->ocpp, d, c->absmax, c->wpacked,
+                                       c->scale, c->shift, c->wsum, c->comp, s));
+      if (c->nclass > 1)
+        HIP_TRY(launch_fold_direct_border_px(c->wpacked, c->absmax, b, d.oc, d.ic, c->ppc, c->nu, c->ocpp, d, c->rects,
+                                             c->nclass, c->shift_tab, s));
+      break;
+    }
     HIP_TRY(launch_prepare_direct(w, b, d.oc, d.ic, d.kh, d.kw, c->units_pad, c->ocpp, d, c->absmax, c->wpacked,
                                   c->scale, c->shift, c->wsum, c->comp, s));
     if (c->nclass > 1)
@@ -519,6 +553,26 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     }
     a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
     HIP_TRY(launch_gemm(a, 1, c->variant, s));
+    break;
+  }
+  case FAM_CONV_FEWCH: {
+    FewChArgs a;
+    memset(&a, 0, sizeof(a));
+    a.in = static_cast<const uint8_t *>(input_dev);
+    a.w = c->wpacked;
+    a.out = output_dev;
+    a.ep = make_epilogue(c, d.output_type, false, d.with_relu);
+    a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow; a.ic = d.ic; a.kh = d.kh; a.kw = d.kw;
+    a.stride_h = d.stride_h; a.stride_w = d.stride_w; a.pad_t = d.pad_t; a.pad_l = d.pad_l;
+    a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    a.in_nhwc = d.input_fmt == EHIP_NHWC; a.out_nhwc = d.output_fmt == EHIP_NHWC;
+    if (c->nclass > 1) {
+      a.ep.shift_tab = c->shift_tab; a.ep.tab_stride = c->ocpp;
+      a.cls_h = c->cls_h; a.cls_w = c->cls_w; a.ncls_w = c->ncls_w;
+    }
+    if (a.in_nhwc && (reinterpret_cast<uintptr_t>(input_dev) & 3))
+      return fail(EHIP_GENERAL_ERROR, "nhwc input of a few-channel layer must be 4-byte aligned");
+    HIP_TRY(launch_conv_fewch(a, s));
     break;
   }
   case FAM_CONV_3X3: {
@@ -646,6 +700,16 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
     if (!want((size_t)c->nbatch * ocp * icp * taps)) return EHIP_OK;
     HIP_TRY(hipMemcpy(packed.data(), c->wpacked, c->wpacked_bytes, hipMemcpyDeviceToHost));
     int8_t *dst = static_cast<int8_t *>(host_dst);
+    if (c->family == FAM_CONV_FEWCH) {
+      for (int oc = 0; oc < ocp; ++oc)
+        for (int ic = 0; ic < icp; ++ic)
+          for (int tap = 0; tap < taps; ++tap) {
+            const int kh = tap / d.kw, kw = tap % d.kw, j = kw / c->ppc, byte = (kw % c->ppc) * d.ic + ic;
+            dst[((size_t)oc * icp + ic) * taps + tap] =
+                ic < d.ic ? packed[((size_t)(kh * c->nu + j) * c->ocpp + packed_row_of_oc(oc)) * 16 + byte] : 0;
+          }
+      return EHIP_OK;
+    }
     for (int b = 0; b < c->nbatch; ++b)
       for (int oc = 0; oc < ocp; ++oc)
         for (int ic = 0; ic < icp; ++ic)

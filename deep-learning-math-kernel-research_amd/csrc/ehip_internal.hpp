@@ -18,7 +18,7 @@ constexpr int kOcTile = 256;     // packed weights are zero-padded to a multiple
 inline int up(int x, int m) { return (x + m - 1) / m * m; }
 inline unsigned div_magic(int d) { return d <= 1 ? 0u : (unsigned)((1ull << 32) / (unsigned)d + 1); }
 
-enum Family { FAM_GEMM_1X1 = 1, FAM_CONV_3X3 = 2, FAM_DEPTHWISE = 3, FAM_WINOGRAD = 4 };
+enum Family { FAM_GEMM_1X1 = 1, FAM_CONV_3X3 = 2, FAM_DEPTHWISE = 3, FAM_WINOGRAD = 4, FAM_CONV_FEWCH = 5 };
 
 // requantization epilogue parameters, by value in kernel arguments
 struct Epilogue {
@@ -145,6 +145,35 @@ hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_de
 hipError_t launch_prepare_direct(const float *w_blocked, const float *bias, int oc, int ic, int kh, int kw,
                                  int units_pad, int ocpp, const ehip_conv_desc_t &d, float *absmax_scratch,
                                  int8_t *wpacked, float *scale, float *shift, int *wsum, int *comp, hipStream_t s);
+// k x k direct convolution of an input with at most four channels (first layers): ppc = 16 / ic
+// pixels per 16-byte operand cell, nu = ceil(kw / ppc) cells per kernel row
+struct FewChArgs {
+  const uint8_t *in;    // nhwc: [n][ih][iw][ic] (compact); blocked: [n][1][ih][iw][16]
+  const int8_t *w;      // [kh * nu cells][OCpp rows][16] s8
+  void *out;            // [n][oc2][oh*ow][16] or nhwc
+  Epilogue ep;
+  int n, ih, iw, oh, ow, ic, kh, kw;
+  int stride_h, stride_w, pad_t, pad_l;
+  int oc2, ocpp;
+  int in_nhwc, out_nhwc;
+  const int *cls_h, *cls_w;   // with ep.shift_tab: class of an output row / column; class = cls_h * ncls_w + cls_w
+  int ncls_w;
+  // set by the launcher
+  int ppc, nu, cells;   // cells = kh * nu
+  int rows, strips;     // output rows per workgroup, workgroups per image
+  int nrows_in, lrow;   // staged input rows and their pitch in bytes (a multiple of 4)
+  int wo;               // waves of a workgroup along the channels (1, 2, 4)
+  unsigned ow_magic, iw_magic, lrow4_magic;
+};
+bool conv_fewch_applies(int ic, int kh, int kw);
+int conv_fewch_row_pitch(int ic, int kw, int iw, int ow, int stride_w, int pad_l);
+hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s);
+hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int kh, int kw, int ppc, int nu,
+                                    int ocpp, const ehip_conv_desc_t &d, float *absmax, int8_t *wpacked, float *scale,
+                                    float *shift, int *wsum, int *comp, hipStream_t s);
+hipError_t launch_fold_direct_border_px(const int8_t *wpacked, const float *absmax, const float *bias, int oc, int ic,
+                                        int ppc, int nu, int ocpp, const ehip_conv_desc_t &d, const int *rects,
+                                        int nclass, float *shift_tab, hipStream_t s);
 hipError_t launch_fold_direct_border(const int8_t *wpacked, const float *absmax, const float *bias, int oc, int kw,
                                      int units_pad, int ocpp, const ehip_conv_desc_t &d, const int *rects, int nclass,
                                      float *shift_tab, hipStream_t s);

@@ -114,6 +114,66 @@ __global__ __launch_bounds__(kBlock) void k_quant_pack_direct(const float *w, co
   wpacked[idx] = packed;
 }
 
+// Layers with at most four input channels (first layers, k_conv_fewch_u8s8): a 16-byte cell
+// holds ppc = 16 / ic horizontally adjacent pixels x ic channels, so one kernel row is
+// nu = ceil(kw / ppc) cells instead of kw.  Packed weights: [kh * nu + j][OCpp rows][16], byte b of
+// unit j = tap kw = j * ppc + b / ic, channel b % ic (zero where kw >= KW or b >= ppc * ic).
+// One thread per packed dword.
+__global__ __launch_bounds__(kBlock) void k_quant_pack_direct_px(const float *w, const float *absmax, int oc2n,
+                                                                 int ic, int KH, int KW, int ppc, int nu, int ocpp,
+                                                                 unsigned *wpacked)
+{
+  const long long total = (long long)KH * nu * ocpp * 4;
+  const long long idx = (long long)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int q = (int)(idx & 3);
+  long long rest = idx >> 2;
+  const int oc = oc_of_packed_row((int)(rest % ocpp));
+  const int t = (int)(rest / ocpp);
+  const int kh = t / nu, j = t - kh * nu;
+  unsigned packed = 0u;
+  if (oc < oc2n * 16) {
+    const float am = absmax[oc];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int b = 4 * q + k;
+      const int jj = b / ic, c = b - jj * ic, kw = j * ppc + jj;
+      int v = 0;
+      if (jj < ppc && kw < KW) v = quant_w(w[((size_t)(oc >> 4) * KH * KW + kh * KW + kw) * 256 + c * 16 + (oc & 15)], am);
+      packed |= ((unsigned)v & 0xffu) << (8 * k);
+    }
+  }
+  wpacked[idx] = packed;
+}
+
+// pixel-packed counterpart of k_fold_direct_border: one thread per (class, channel)
+__global__ __launch_bounds__(kBlock) void k_fold_direct_border_px(const unsigned *wpacked, const float *absmax,
+                                                                  const float *bias, int oc_rows, int ic, int ppc,
+                                                                  int nu, int ocpp, FoldParams p, const int4 *rects,
+                                                                  int nclass, float *shift_tab)
+{
+  const int idx = blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= nclass * ocpp) return;
+  const int c = idx / ocpp, oc = idx - c * ocpp;
+  float sh = 0.0f;
+  if (oc < oc_rows) {
+    const int4 r = rects[c];
+    int s = 0;
+    for (int kh = r.x; kh <= r.y; ++kh)
+      for (int j = 0; j < nu; ++j) {
+        const uint4 cell = *reinterpret_cast<const uint4 *>(wpacked + ((size_t)(kh * nu + j) * ocpp + packed_row_of_oc(oc)) * 4);
+        const unsigned d[4] = {cell.x, cell.y, cell.z, cell.w};
+        for (int b = 0; b < ppc * ic; ++b) {
+          const int kw = j * ppc + b / ic;
+          if (kw >= r.z && kw <= r.w) s += (int)(signed char)((d[b >> 2] >> (8 * (b & 3))) & 0xffu);
+        }
+      }
+    float sc;
+    fold(p, absmax[oc], (float)s, p.with_bias ? bias[oc] : 0.0f, &sc, &sh);
+  }
+  shift_tab[idx] = sh;
+}
+
 // one thread per oc row: sum of the packed weights, compensation, scale/shift
 __global__ __launch_bounds__(kBlock) void k_fold_direct(const unsigned *wpacked, const float *absmax,
                                                         const float *bias, int oc_rows, int taps, int units_pad,
@@ -373,6 +433,33 @@ hipError_t launch_prepare_direct(const float *w, const float *bias, int oc, int 
   const FoldParams fp = make_fold(d, d.algorithm == EHIP_CONV_DIRECT_1X1);
   hipLaunchKernelGGL(k_fold_direct, grid_for(ocpp), dim3(kBlock), 0, s, reinterpret_cast<const unsigned *>(wpacked),
                      absmax, bias, oc2 * 16, taps, units_pad, ocpp, fp, scale, shift, wsum, comp);
+  return hipGetLastError();
+}
+
+// weight side of the pixel-packed form (see k_quant_pack_direct_px): taps = kh * nu units of one cell
+hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int kh, int kw, int ppc, int nu,
+                                    int ocpp, const ehip_conv_desc_t &d, float *absmax, int8_t *wpacked, float *scale,
+                                    float *shift, int *wsum, int *comp, hipStream_t s)
+{
+  const int oc2 = up(oc, 16) / 16;
+  hipLaunchKernelGGL(k_absmax_direct, dim3(oc2), dim3(kBlock), 0, s, w, 1, kh * kw, absmax);
+  const size_t dwords = (size_t)kh * nu * ocpp * 4;
+  hipLaunchKernelGGL(k_quant_pack_direct_px, grid_for(dwords), dim3(kBlock), 0, s, w, absmax, oc2, ic, kh, kw, ppc, nu,
+                     ocpp, reinterpret_cast<unsigned *>(wpacked));
+  const FoldParams fp = make_fold(d, false);
+  hipLaunchKernelGGL(k_fold_direct, grid_for(ocpp), dim3(kBlock), 0, s, reinterpret_cast<const unsigned *>(wpacked),
+                     absmax, bias, oc2 * 16, kh * nu, 1, ocpp, fp, scale, shift, wsum, comp);
+  return hipGetLastError();
+}
+
+hipError_t launch_fold_direct_border_px(const int8_t *wpacked, const float *absmax, const float *bias, int oc, int ic,
+                                        int ppc, int nu, int ocpp, const ehip_conv_desc_t &d, const int *rects,
+                                        int nclass, float *shift_tab, hipStream_t s)
+{
+  const FoldParams fp = make_fold(d, false);
+  hipLaunchKernelGGL(k_fold_direct_border_px, grid_for((size_t)nclass * ocpp), dim3(kBlock), 0, s,
+                     reinterpret_cast<const unsigned *>(wpacked), absmax, bias, up(oc, 16), ic, ppc, nu, ocpp, fp,
+                     reinterpret_cast<const int4 *>(rects), nclass, shift_tab);
   return hipGetLastError();
 }
 

@@ -18,14 +18,15 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 class Workload:
     def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
-                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None, in_z=0.0, nhwc_out=False):
+                 out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None, in_z=0.0, nhwc_out=False,
+                 nhwc_in=False):
         self.key, self.title = key, title
         self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
         self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
         self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
         self.in_z = in_z   # input zero point (the reference's "...z" data-type configurations)
         self.nhwc = nhwc   # activations [n][h][w][c] on both sides instead of nChw16c
-        self.nhwc_in, self.nhwc_out = nhwc, nhwc or nhwc_out
+        self.nhwc_in, self.nhwc_out = nhwc or nhwc_in, nhwc or nhwc_out
         # oh given: the right / bottom pads are whatever that output size needs (src/elx_conv.cpp:36-37)
         self.oh = oh if oh is not None else (hw + 2 * pad - k) // stride + 1
 
@@ -45,7 +46,8 @@ class Workload:
 
     def algorithmic_bytes(self):
         esz = {U8: 1, S8: 1, F32: 4}
-        n_in = self.n * up16(self.ic) * self.hw * self.hw
+        # nhwc input with at most four channels is compact (a first layer's image)
+        n_in = self.n * (self.ic if self.nhwc_in and self.ic <= 4 else up16(self.ic)) * self.hw * self.hw
         if self.stride == 2 and self.k == 1:
             n_in //= 4  # a stride-2 1x1 only samples every other row and column
         n_out = self.n * up16(self.oc) * self.oh * self.oh
@@ -117,8 +119,12 @@ WORKLOADS = {w.key: w for w in [
     # ResNet-50's first layer with the zero-point input configuration of the tuned run
     # (scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh:12 "U8F32S8F32z"), here on nChw16c input:
     # the three channels occupy one 16-channel unit per tap
-    Workload("R1", "7x7 s2 3->64 224x224->112x112 N=64 pad 3, input zero point 128, bias+ReLU, s8 out (ResNet-50 conv1)",
-             64, 3, 64, 224, k=7, pad=3, stride=2, out_type=S8, T=14, in_z=128.0),
+    Workload("R1", "7x7 s2 3->64 224x224->112x112 N=64 pad 3, 3-channel nhwc input with zero point 128, bias+ReLU, "
+             "s8 nhwc out (ResNet-50 conv1)", 64, 3, 64, 224, k=7, pad=3, stride=2, out_type=S8, T=14, in_z=128.0,
+             nhwc_in=True, nhwc_out=True),
+    Workload("M1", "3x3 s2 3->32 224x224->112x112 N=64 pads right/bottom, 3-channel nhwc input with zero point 128, "
+             "bias+ReLU, s8 out (MobileNet-v1 Conv__224)", 64, 3, 32, 224, k=3, pad=0, stride=2, out_type=S8, T=14,
+             in_z=128.0, oh=112, nhwc_in=True),
     Workload("M4", "depthwise 3x3 s2 C=128 56x56->28x28 N=64, bias+ReLU6, u8 out (MobileNet-v1 Conv2d_4)", 64, 128, 128,
              56, k=3, pad=0, stride=2, depthwise=True, w_sigma=0.1, T=28, relu6=True, oh=28),
     Workload("C4a", "Winograd F(4,3) 256->256 @56x56 N=64, fp32 in/out (VGG-16 conv3)", 64, 256, 256, 56, k=3, pad=1,
@@ -168,13 +174,12 @@ def _dw(count, name, c, hw, stride):
 #   scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh   (ResNet-50 v1.5: 53 convolutions + the FC layer)
 #   scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh  (MobileNet-v1: 27 convolutions + the FC layer)
 #   scripts/best_configs/vgg-n64-8180-1s-int8.sh         (VGG-19 without conv1_1: 15 convolutions)
-# and the counts follow the layer names listed above each command there.  Two deviations, both on
-# layers with three input channels or 1001 output channels: the first layers take nChw16c input where
-# the scripts pass three-channel nhwc, and MobileNet's FC writes nChw16c where the script asks for nhwc.
+# and the counts follow the layer names listed above each command there.  One deviation: MobileNet's FC
+# (1001 output channels) writes nChw16c where the script asks for nhwc.
 NETWORKS = {
     "resnet50_v1_5_int8": [
-        _L(1, "conv2d", "7x7 s2 3->64 224->112 pad 3, zero point 128, nhwc out", 64, 3, 64, 224, k=7, pad=3, stride=2,
-           out_type=S8, T=14, in_z=128.0, nhwc_out=True),
+        _L(1, "conv2d", "7x7 s2 3->64 224->112 pad 3, 3-channel nhwc in, zero point 128, nhwc out", 64, 3, 64, 224, k=7,
+           pad=3, stride=2, out_type=S8, T=14, in_z=128.0, nhwc_in=True, nhwc_out=True),
         _wino(3, "conv2d_3", 64, 64, 56), _wino(3, "conv2d_16", 128, 128, 28), _wino(5, "conv2d_29", 256, 256, 14),
         _wino(2, "conv2d_48", 512, 512, 7),
         _L(1, "conv2d_13", "3x3 s2 128->128 58->28", 64, 128, 128, 58, k=3, stride=2, out_type=S8, T=14),
@@ -191,8 +196,8 @@ NETWORKS = {
         _pw(1, "FC", 2048, 1008, 8, nhwc_in=True, nhwc_out=True, n=1, out_type=F32, algorithm=CONV_DIRECT),
     ],
     "mobilenet_v1_int8": [
-        _L(1, "Conv__224", "3x3 s2 3->32 224->112, pads right/bottom, zero point 128", 64, 3, 32, 224, k=3, pad=0, stride=2,
-           out_type=S8, T=14, in_z=128.0, oh=112),
+        _L(1, "Conv__224", "3x3 s2 3->32 224->112, pads right/bottom, 3-channel nhwc in, zero point 128", 64, 3, 32, 224,
+           k=3, pad=0, stride=2, out_type=S8, T=14, in_z=128.0, oh=112, nhwc_in=True),
         _pw(1, "Conv__226", 32, 64, 112), _pw(1, "Conv__228", 64, 128, 56), _pw(1, "Conv__230", 128, 128, 56),
         _pw(1, "Conv__232", 128, 256, 28), _pw(1, "Conv__234", 256, 256, 28), _pw(1, "Conv__236", 256, 512, 14),
         _pw(5, "Conv__238", 512, 512, 14), _pw(1, "Conv__248", 512, 1024, 7), _pw(1, "Conv__250", 1024, 1024, 7, nhwc_out=True),
@@ -221,9 +226,10 @@ class DeviceLayer:
         ic2, oc2 = up16(wl.ic) // 16, up16(wl.oc) // 16
         if wl.in_type == U8:
             # fp32 U[0,1) activations quantized with scale 1/255 are uniform codes 0..255
-            # (random codes: the nhwc tensor has the same number of bytes, only their meaning differs)
-            self.x = torch.randint(0, 256, (wl.n, ic2, wl.hw, wl.hw, 16), dtype=torch.uint8, device="cuda",
-                                   generator=gen)
+            # (random codes: the nhwc tensor has the same number of bytes, only their meaning differs;
+            # nhwc with at most four channels is compact, [n][h][w][ic])
+            shape = (wl.n, wl.hw, wl.hw, wl.ic) if wl.nhwc_in and wl.ic <= 4 else (wl.n, ic2, wl.hw, wl.hw, 16)
+            self.x = torch.randint(0, 256, shape, dtype=torch.uint8, device="cuda", generator=gen)
         else:
             self.x = torch.rand((wl.n, ic2, wl.hw, wl.hw, 16), dtype=torch.float32, device="cuda", generator=gen)
         if wl.depthwise:

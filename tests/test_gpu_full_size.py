@@ -21,11 +21,11 @@ def _layer_of(key, seed):
     wl = W.WORKLOADS[key]
     return Layer(wl.n, wl.ic, wl.oc, wl.hw, k=wl.k, pad=wl.pad, stride=wl.stride, out_type=wl.out_type,
                  algorithm=wl.algorithm, with_sum=wl.with_sum, depthwise=wl.depthwise, seed=seed, w_sigma=wl.w_sigma,
-                 T=wl.T, in_nhwc=wl.nhwc, out_nhwc=wl.nhwc,
+                 T=wl.T, in_nhwc=wl.nhwc_in, out_nhwc=wl.nhwc_out,
                  out_hw=wl.oh if wl.oh != (wl.hw + 2 * wl.pad - wl.k) // wl.stride + 1 else None, in_z=wl.in_z)
 
 
-@pytest.mark.parametrize("key", ["C1", "C2", "C3a", "C3b", "C3a_nhwc", "C3b_nhwc", "R13", "R1", "M4", "C5a", "C5b"])
+@pytest.mark.parametrize("key", ["C1", "C2", "C3a", "C3b", "C3a_nhwc", "C3b_nhwc", "R13", "R1", "M1", "M4", "C5a", "C5b"])
 def test_configured_layer_bit_exact(key):
     layer = _layer_of(key, seed=1000 + sum(map(ord, key)))
     exp = layer.oracle()
@@ -40,7 +40,7 @@ def test_configured_layer_bit_exact(key):
         key, int((got != exp["out"]).sum()), got.size)
     # the layer really is the configured one
     wl = W.WORKLOADS[key]
-    assert got.shape == ((wl.n, wl.oh, wl.oh, wl.oc) if wl.nhwc else (wl.n, ol.up16(wl.oc) // 16, wl.oh, wl.oh, 16))
+    assert got.shape == ((wl.n, wl.oh, wl.oh, wl.oc) if wl.nhwc_out else (wl.n, ol.up16(wl.oc) // 16, wl.oh, wl.oh, 16))
 
 
 @pytest.mark.parametrize("key,check_images", [("C4a", 2), ("C4b", 4)])

@@ -177,7 +177,52 @@ def test_direct_zero_point_with_padding(out_type, n, ic, oc, hw, k, pad, stride,
     res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=140 + k + stride,
                                 out_hw=out_hw, in_z=128.0, with_relu=(out_type != ol.F32)))
     if pad or out_hw:
-        assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+        assert res["conv"].kernel_name.startswith("k_conv_fewch_u8s8" if ic <= 4 else "k_gemm_u8s8")
+
+
+# at most four input channels (first layers; the reference feeds them 3-channel nhwc,
+# scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh:12): 16 / ic pixels per operand cell, a kernel row
+# is ceil(kw / (16 / ic)) cells, input rows staged compactly in LDS
+FEWCH_SHAPES = [
+    (2, 3, 64, 38, 7, 3, 2, None),      # 7x7: two cells of five pixels per kernel row; rows of 114 bytes
+    (2, 3, 32, 24, 3, 0, 2, 12),        # 3x3 s2, pads only right / bottom: one cell per kernel row
+    (1, 4, 16, 13, 5, 2, 1, None),      # four channels: four pixels per cell, two cells per row
+    (2, 1, 32, 17, 3, 1, 1, None),      # one channel: sixteen pixels per cell, rows of 17 bytes
+    (1, 2, 48, 21, 7, 2, 2, None),      # pads k/2 - 1
+    (3, 3, 16, 9, 3, 1, 2, None),       # rows of 27 bytes: every image and row starts at another byte phase
+    (2, 3, 96, 15, 5, 2, 1, None),      # three 32-channel tiles
+    (1, 3, 128, 11, 3, 1, 1, None),     # four channel tiles: one per wave
+]
+
+
+@pytest.mark.parametrize("in_nhwc", [False, True])
+@pytest.mark.parametrize("in_z", [0.0, 128.0])
+@pytest.mark.parametrize("n,ic,oc,hw,k,pad,stride,out_hw", FEWCH_SHAPES)
+def test_direct_few_input_channels(in_z, in_nhwc, n, ic, oc, hw, k, pad, stride, out_hw, monkeypatch):
+    layer = dict(k=k, pad=pad, stride=stride, out_type=ol.U8, seed=170 + k + ic, out_hw=out_hw, in_z=in_z)
+    res = run_and_compare(Layer(n, ic, oc, hw, in_nhwc=in_nhwc, **layer))
+    assert res["conv"].kernel_name == "k_conv_fewch_u8s8"
+    if not in_nhwc:
+        monkeypatch.setenv("EHIP_FEWCH", "0")     # the general kernels give the same bytes
+        res2 = run_and_compare(Layer(n, ic, oc, hw, **layer))
+        assert res2["conv"].kernel_name != "k_conv_fewch_u8s8"
+
+
+@pytest.mark.parametrize("out_type,out_nhwc", [(ol.S32, False), (ol.F32, False), (ol.S8, False), (ol.S8, True),
+                                               (ol.F32, True), (ol.U8, True)])
+def test_direct_few_input_channels_output_types(out_type, out_nhwc):
+    run_and_compare(Layer(2, 3, 64, 19, k=7, pad=3, stride=2, out_type=out_type, seed=181 + out_type, in_z=128.0,
+                          in_nhwc=True, out_nhwc=out_nhwc, with_relu=(out_type != ol.F32)))
+    run_and_compare(Layer(1, 3, 32, 12, k=3, pad=1, stride=1, out_type=out_type, seed=183 + out_type,
+                          in_nhwc=False, out_nhwc=out_nhwc))
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 16])
+def test_direct_few_input_channels_strip_heights(rows, monkeypatch):
+    # output rows per workgroup, including strips that end below the image
+    monkeypatch.setenv("EHIP_FEWCH_ROWS", str(rows))
+    run_and_compare(Layer(2, 3, 64, 27, k=7, pad=3, stride=2, out_type=ol.S8, seed=190 + rows, in_z=128.0, in_nhwc=True))
+    run_and_compare(Layer(2, 3, 32, 13, k=3, pad=1, stride=1, out_type=ol.U8, seed=195 + rows, in_nhwc=True))
 
 
 @pytest.mark.parametrize("variant", range(7))
