@@ -568,7 +568,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.in_nhwc = d.input_fmt == EHIP_NHWC; a.out_nhwc = d.output_fmt == EHIP_NHWC;
     if (c->nclass > 1) {
       a.ep.shift_tab = c->shift_tab; a.ep.tab_stride = c->ocpp;
-      a.cls_h = c->cls_h; a.cls_w = c->cls_w; a.ncls_w = c->ncls_w;
+      a.cls_h = c->cls_h; a.cls_w = c->cls_w; a.ncls_w = c->ncls_w; a.nclass = c->nclass;
     }
     if (a.in_nhwc && (reinterpret_cast<uintptr_t>(input_dev) & 3))
       return fail(EHIP_GENERAL_ERROR, "nhwc input of a few-channel layer must be 4-byte aligned");

@@ -9,8 +9,8 @@
 // A workgroup takes a strip of output rows of one image:
 //   1. the input rows under the strip go to LDS once, as compact rows of ic bytes per pixel with
 //      the left / right padding filled in (u8 0, which contributes nothing), already remapped to s8;
-//      nhwc input is compact in memory as well, so LDS dword d of a row is one aligned global dword
-//      (the row keeps its byte phase), masked at the row's ends;
+//      nhwc input is compact in memory as well: a staged dword is two aligned global dwords shifted
+//      together (rows start at any byte), masked at the row's ends;
 //   2. a wave walks over 32-pixel tiles of the strip: a lane's cell is 16 consecutive LDS bytes at
 //      a byte address of any alignment, read as five dwords and shifted into place;
 //   3. kh * nu / 2 MFMAs per tile against the weights in registers, then the shared epilogue.
@@ -20,16 +20,20 @@
 namespace ehip {
 
 namespace {
-__device__ __forceinline__ unsigned low_bytes(long long k)   // mask of the k lowest bytes, k clamped to 0..4
+__device__ __forceinline__ unsigned low_bytes(int k)   // mask of the k lowest bytes, k clamped to 0..4 (no branches)
 {
-  return k <= 0 ? 0u : k >= 4 ? 0xffffffffu : (1u << (8 * (int)k)) - 1u;
+  k = k < 0 ? 0 : k > 4 ? 4 : k;
+  return (unsigned)((1ull << (8 * k)) - 1ull);
 }
 }  // namespace
 
 template <int KS>
 __global__ __launch_bounds__(kBlock, 2) void k_conv_fewch_u8s8(FewChArgs a)
 {
-  extern __shared__ unsigned rows_lds[];   // [nrows_in][lrow / 4]
+  // [nrows_in][lrow / 4] staged rows; with border classes kept on chip (a.tab_lds): the shift rows of
+  // the workgroup's channels [class][wo * 32], then the class of each of the strip's output rows
+  // (times ncls_w) and of each output column
+  extern __shared__ unsigned rows_lds[];
   __shared__ v4i xpatch[4 * 256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -45,36 +49,91 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv_fewch_u8s8(FewChArgs a)
   const int rowbytes = a.iw * a.ic;
 
   // ---- 1. stage the input rows --------------------------------------------------------------
-  // byte 0 of a staged row = pixel -pad_l of the input row (+ the row's phase for nhwc input)
-  const long long g00 = ((long long)(img * a.ih + ihb) * a.iw - a.pad_l) * a.ic;   // nhwc: global byte of staged (0, 0)
+  // byte 0 of a staged row = pixel -pad_l of the input row.
+  // nhwc: byte offsets inside the image fit an int; the image starts at in + img_off, of which the
+  // 4-byte aligned part goes into the pointer and the rest (e0) into the offsets.  A staged dword is
+  // four consecutive bytes of the row at whatever alignment they have in memory: two aligned dwords
+  // shifted together.
+  const long long img_off = (long long)img * a.ih * a.iw * a.ic;
+  const int e0 = (int)(img_off & 3);
+  const uint8_t *const in_al = a.in + (img_off - e0);
+  const int g00 = (ihb * a.iw - a.pad_l) * a.ic + e0;   // byte of staged (0, 0) relative to in_al
+  const int last_dw = (e0 + a.ih * rowbytes - 1) & ~3;   // the last aligned dword with a byte of this image
+  // Loads are issued kStageDepth at a time, unconditionally (outside the row: a clamped address and
+  // an empty mask), before the first of them is stored: a workgroup waits for memory once per
+  // batch, not once per dword.
+  constexpr int kStageDepth = 8;
+  float *const lds_shift = reinterpret_cast<float *>(rows_lds) + a.tab_lds;   // 16-byte aligned
+  int *const lds_cls_h = reinterpret_cast<int *>(lds_shift + a.nclass * a.wo * 32);
+  int *const lds_cls_w = lds_cls_h + a.rows;
+  if (a.tab_lds) {
+    // a pixel's shift row is looked up per tile: two dependent trips to memory if the tables stay there
+    for (int idx = tid; idx < rows_valid; idx += kBlock) lds_cls_h[idx] = a.cls_h[oh0 + idx] * a.ncls_w;
+    for (int idx = tid; idx < a.ow; idx += kBlock) lds_cls_w[idx] = a.cls_w[idx];
+    const int width = a.wo * 32;
+    for (int idx = tid; idx < a.nclass * width; idx += kBlock) {
+      const int c = idx / width;
+      lds_shift[idx] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - c * width)];
+    }
+  }
   if (a.in_nhwc) {
-    for (int idx = tid; idx < a.nrows_in * lrow4; idx += kBlock) {
-      const int r = fastdiv(idx, lrow4, a.lrow4_magic);
-      const int d = idx - r * lrow4;
-      const int h = ihb + r;
-      unsigned v = 0u;
-      if (h >= 0 && h < a.ih) {
-        const long long g0 = g00 + (long long)r * rowbytes;
-        const long long rs = g0 + a.pad_l * a.ic;           // first byte of the input row
-        const long long ga = g0 - (g0 & 3) + 4 * d;         // the aligned global dword behind LDS dword d
-        const long long lo = rs - ga, hi = rs + rowbytes - ga;   // its bytes lo .. hi - 1 belong to the row
-        if (hi > 0 && lo < 4)
-          v = *reinterpret_cast<const unsigned *>(a.in + ga) & low_bytes(hi) & ~low_bytes(lo);
+    const int total = a.nrows_in * lrow4;
+    for (int base = 0; base < total; base += kBlock * kStageDepth) {
+      unsigned v[kStageDepth], v2[kStageDepth], m[kStageDepth], sft[kStageDepth];
+#pragma unroll
+      for (int u = 0; u < kStageDepth; ++u) {
+        int idx = base + u * kBlock + tid;
+        idx = idx < total ? idx : total - 1;
+        const int r = fastdiv(idx, lrow4, a.lrow4_magic);
+        const int d = idx - r * lrow4;
+        const int h = ihb + r;
+        const int g = g00 + r * rowbytes + 4 * d;   // first byte of the staged dword
+        const int rs = g00 + r * rowbytes + a.pad_l * a.ic;   // first byte of the input row
+        const int lo = rs - g, hi = rs + rowbytes - g;        // bytes lo .. hi - 1 of the dword belong to the row
+        const bool inside = (unsigned)h < (unsigned)a.ih;
+        m[u] = inside ? low_bytes(hi) & ~low_bytes(lo) : 0u;
+        // dwords outside the image hold nothing of the row: any address inside will do for them
+        int ga = g & ~3, gb = ga + 4;
+        ga = ga < 0 ? 0 : ga > last_dw ? last_dw : ga;
+        gb = gb < 0 ? 0 : gb > last_dw ? last_dw : gb;
+        v[u] = *reinterpret_cast<const unsigned *>(in_al + ga);
+        v2[u] = *reinterpret_cast<const unsigned *>(in_al + gb);
+        sft[u] = g & 3;
       }
-      rows_lds[idx] = v ^ 0x80808080u;
+#pragma unroll
+      for (int u = 0; u < kStageDepth; ++u) {
+        const int idx = base + u * kBlock + tid;
+        if (idx < total) rows_lds[idx] = (__builtin_amdgcn_alignbyte(v2[u], v[u], sft[u]) & m[u]) ^ 0x80808080u;
+      }
     }
   } else {
     for (int idx = tid; idx < a.nrows_in * lrow4; idx += kBlock) rows_lds[idx] = 0x80808080u;
     __syncthreads();
     uint8_t *lb = reinterpret_cast<uint8_t *>(rows_lds);
-    for (int idx = tid; idx < a.nrows_in * a.iw; idx += kBlock) {
-      const int r = fastdiv(idx, a.iw, a.iw_magic);
-      const int x = idx - r * a.iw;
-      const int h = ihb + r;
-      if (h >= 0 && h < a.ih) {
-        const unsigned v = *reinterpret_cast<const unsigned *>(a.in + ((long long)(img * a.ih + h) * a.iw + x) * 16) ^ 0x80808080u;
-        for (int c = 0; c < a.ic; ++c) lb[r * a.lrow + (x + a.pad_l) * a.ic + c] = (uint8_t)(v >> (8 * c));
+    const int total = a.nrows_in * a.iw;
+    for (int base = 0; base < total; base += kBlock * kStageDepth) {
+      unsigned v[kStageDepth];
+      int at[kStageDepth];   // LDS byte of the pixel, -1: nothing to store
+#pragma unroll
+      for (int u = 0; u < kStageDepth; ++u) {
+        int idx = base + u * kBlock + tid;
+        const bool in_range = idx < total;
+        idx = in_range ? idx : total - 1;
+        const int r = fastdiv(idx, a.iw, a.iw_magic);
+        const int x = idx - r * a.iw;
+        const int h = ihb + r;
+        const bool inside = in_range && h >= 0 && h < a.ih;
+        at[u] = inside ? r * a.lrow + (x + a.pad_l) * a.ic : -1;
+        v[u] = *reinterpret_cast<const unsigned *>(a.in + (inside ? ((long long)(img * a.ih + h) * a.iw + x) * 16 : 0));
       }
+#pragma unroll
+      for (int u = 0; u < kStageDepth; ++u)
+        if (at[u] >= 0) {
+          const unsigned q = v[u] ^ 0x80808080u;
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            if (c < a.ic) lb[at[u] + c] = (uint8_t)(q >> (8 * c));
+        }
     }
   }
   __syncthreads();
@@ -90,61 +149,73 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv_fewch_u8s8(FewChArgs a)
     wreg[ks] = *reinterpret_cast<const v4i *>(a.w + ((long long)(2 * ks + lh) * a.ocpp + oc0 + l32) * 16);
   // the lane's cells: 2 ks + lh = kernel row * nu + unit, clamped to the real ones (the weights
   // behind them are zero)
-  int cell_row[KS], cell_off[KS];
+  int cell_at[KS];   // LDS byte of the cell relative to the pixel's first cell
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     int tc = 2 * ks + lh;
     tc = tc < a.cells ? tc : a.cells - 1;
-    cell_row[ks] = tc / a.nu;
-    cell_off[ks] = (tc - cell_row[ks] * a.nu) * a.ppc * a.ic;
+    const int kr = tc / a.nu;
+    cell_at[ks] = kr * a.lrow + (tc - kr * a.nu) * a.ppc * a.ic;
   }
-  const int phase0 = a.in_nhwc ? (int)(g00 & 3) : 0;
-  const int phase_step = a.in_nhwc ? rowbytes & 3 : 0;
 
   const long long cidx = oc0 + 16 * lh;
   OcConsts k0;
   load_consts(k0, a.ep, cidx);
+  // the on-chip shift rows get an epilogue of their own: one whose table pointer can only be LDS
+  Epilogue ep_lds = a.ep;
+  ep_lds.shift_tab = lds_shift;
+  ep_lds.tab_stride = a.wo * 32;
   v4i *xlds = ((a.ep.out_type == EHIP_F32 || a.ep.out_type == EHIP_S32) && !a.out_nhwc) ? xpatch + wave * 256 : nullptr;
-  const long long gp0 = (long long)img * ohw + (long long)oh0 * a.ow;   // the strip's first output pixel
-  auto pixel_offset = [&](int p, bool &valid) -> size_t {
-    valid = p < npix;
-    const int pv = valid ? p : 0;
-    if (a.out_nhwc) return (size_t)(gp0 + pv) * oc_real;
-    return ((size_t)img * a.oc2 * ohw + (size_t)oh0 * a.ow + pv) * 16;
-  };
+  // the accumulators start from the u8 -> s8 compensation of the lane's channels
+  v16i comp0;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) comp0[v] = k0.comp[v >> 2][v & 3];
+  // element offset of output pixel p of the strip (cell of 16-channel block 0; nhwc: channel vector): linear in p
+  const size_t px_stride = a.out_nhwc ? (size_t)oc_real : (size_t)16;
+  const size_t out0 = a.out_nhwc ? ((size_t)img * ohw + (size_t)oh0 * a.ow) * oc_real
+                                 : ((size_t)img * a.oc2 * ohw + (size_t)oh0 * a.ow) * 16;
+  const size_t block_stride = a.out_nhwc ? (size_t)16 : (size_t)ohw * 16;
+  const int row_step = a.stride_h * a.lrow, px_step = a.stride_w * a.ic;
   const int ntiles = (npix + 31) >> 5;
   for (int tile = wp; tile < ntiles; tile += wpn) {
     int p = tile * 32 + l32;
     p = p < npix ? p : npix - 1;
     const int ro = fastdiv(p, a.ow, a.ow_magic);
     const int ox = p - ro * a.ow;
-    const int row0 = ro * a.stride_h;
-    const int xbyte = ox * a.stride_w * a.ic;
-    v16i acc[1][1];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[0][0][v] = 0;
+    const int at0 = ro * row_step + ox * px_step;
     v4i b[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int row = row0 + cell_row[ks];
-      const int A = row * a.lrow + ((phase0 + row * phase_step) & 3) + xbyte + cell_off[ks];
+      const int A = at0 + cell_at[ks];
       const unsigned *src = rows_lds + (A >> 2);
       const unsigned sh = A & 3;
       const unsigned d0 = src[0], d1 = src[1], d2 = src[2], d3 = src[3], d4 = src[4];
       b[ks] = v4i{(int)__builtin_amdgcn_alignbyte(d1, d0, sh), (int)__builtin_amdgcn_alignbyte(d2, d1, sh),
                   (int)__builtin_amdgcn_alignbyte(d3, d2, sh), (int)__builtin_amdgcn_alignbyte(d4, d3, sh)};
     }
+    v16i acc[1][1];
+    acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[0], b[0], comp0, 0, 0, 0);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ks], b[ks], acc[0][0], 0, 0, 0);
+    for (int ks = 1; ks < KS; ++ks) acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ks], b[ks], acc[0][0], 0, 0, 0);
     size_t pix[1], pixT[1][2];
     bool pvalid[1], validT[1][2];
     int cls[1] = {0};
-    pix[0] = pixel_offset(tile * 32 + l32, pvalid[0]);
-    pixT[0][0] = pixel_offset(tile * 32 + (lane >> 2), validT[0][0]);
-    pixT[0][1] = pixel_offset(tile * 32 + (lane >> 2) + 16, validT[0][1]);
-    if (a.ep.shift_tab) cls[0] = a.cls_h[oh0 + ro] * a.ncls_w + a.cls_w[ox];
-    epilogue_wave<1, 1, true>(a.ep, acc, k0, cidx, oc0 + 16 * lh, pix, pvalid, oc_real,
-                              a.out_nhwc ? (size_t)16 : (size_t)ohw * 16, a.out, xlds, pixT, validT, cls);
+    const int p0 = tile * 32;
+    pvalid[0] = p0 + l32 < npix;
+    pix[0] = out0 + (size_t)(p0 + l32) * px_stride;
+    validT[0][0] = p0 + (lane >> 2) < npix;
+    validT[0][1] = p0 + (lane >> 2) + 16 < npix;
+    pixT[0][0] = out0 + (size_t)(p0 + (lane >> 2)) * px_stride;
+    pixT[0][1] = pixT[0][0] + 16 * px_stride;
+    if (a.tab_lds) {
+      cls[0] = lds_cls_h[ro] + lds_cls_w[ox];
+      epilogue_wave<1, 1, true, true>(ep_lds, acc, k0, wo * 32 + 16 * lh, oc0 + 16 * lh, pix, pvalid, oc_real,
+                                      block_stride, a.out, xlds, pixT, validT, cls);
+    } else {
+      if (a.ep.shift_tab) cls[0] = a.cls_h[oh0 + ro] * a.ncls_w + a.cls_w[ox];
+      epilogue_wave<1, 1, true, true>(a.ep, acc, k0, cidx, oc0 + 16 * lh, pix, pvalid, oc_real, block_stride, a.out,
+                                      xlds, pixT, validT, cls);
+    }
   }
 }
 
@@ -156,14 +227,14 @@ bool conv_fewch_applies(int ic, int kh, int kw)
 }
 
 // pitch in bytes of a staged input row: pad_l + iw pixels or the last output pixel's last cell
-// (16 bytes), whichever ends later, + 3 bytes of phase + 4 for the fifth dword of a shifted cell
+// (16 bytes), whichever ends later, + 4 for the fifth dword of a shifted cell
 int conv_fewch_row_pitch(int ic, int kw, int iw, int ow, int stride_w, int pad_l)
 {
   const int ppc = 16 / ic, nu = (kw + ppc - 1) / ppc;
   int need = (pad_l + iw) * ic;
   const int last = ((ow - 1) * stride_w + (nu - 1) * ppc) * ic + 16;
   if (last > need) need = last;
-  return up(need + 3 + 4, 4) + 4;
+  return up(need + 4, 4) + 4;
 }
 
 // Fills the derived fields (cells, strip height, LDS row pitch, wave split) and launches.
@@ -179,19 +250,43 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s)
   const int octiles = up(a.oc2 * 16, 32) / 32;   // <= ocpp / 32
   a.wo = octiles % 4 == 0 ? 4 : octiles % 2 == 0 ? 2 : 1;
   const int gy = octiles / a.wo, wpn = 4 / a.wo;
-  // strip height: as many rows as keep about three workgroups per CU in the grid, every wave busy,
-  // and the staged rows inside 48 KB
+  // Strip height (output rows per workgroup).  A taller strip stages fewer overlap rows per output
+  // row; what it must not do is leave waves without tiles, end in a nearly empty strip, or put a
+  // few workgroups more into the grid than the chip runs at once (they would run alone in a second
+  // round).  All of that goes into one relative cost, minimised over the heights whose rows fit in LDS.
   int rows = 1;
   const char *env = getenv("EHIP_FEWCH_ROWS");
   if (env && env[0]) {
     rows = atoi(env);
   } else {
-    for (int r = 1; r <= a.oh && r <= 16; ++r) {
-      if ((size_t)((r - 1) * a.stride_h + a.kh) * a.lrow > 48 * 1024) break;
-      const long long wgs = (long long)a.n * ((a.oh + r - 1) / r) * gy;
-      if (r > 1 && wgs < 768) break;
-      rows = r;
-      if ((r * a.ow + 31) / 32 >= 8 * wpn && (r * a.ow) % 32 == 0) break;
+    static int n_cu = 0;
+    if (!n_cu) {
+      int dev = 0, v = 0;
+      if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+        n_cu = v;
+      else
+        n_cu = 256;
+    }
+    const int ks = (a.cells + 1) / 2;
+    double best = 0.0;
+    for (int r = 1; r <= a.oh && r <= 32; ++r) {
+      const int nrows_in = (r - 1) * a.stride_h + a.kh;
+      const size_t dyn = (size_t)nrows_in * a.lrow + 32;
+      if (dyn > 40 * 1024) break;
+      // workgroups of 4 waves resident per CU: registers (the 14-cell kernel holds 2 waves per SIMD,
+      // the others 3), LDS (16 KB static exchange patch + the rows)
+      int resident = ks > 5 ? 2 : 3;
+      const int by_lds = (int)((160 * 1024) / (16 * 1024 + dyn));
+      if (by_lds < resident) resident = by_lds < 1 ? 1 : by_lds;
+      const double slots = (double)n_cu * resident;
+      const double wgs = (double)a.n * ((a.oh + r - 1) / r) * gy;
+      const double rounds = (double)(long long)((wgs + slots - 1) / slots);
+      const int tiles = (r * a.ow + 31) / 32;
+      const double cost = rounds * slots / wgs                                   // idle slots of the last round
+          * ((tiles + wpn - 1) / wpn * wpn * 32.0 / (r * a.ow))                  // idle waves and lanes of the last tiles
+          * ((double)((a.oh + r - 1) / r) * r / a.oh)                             // rows of the last strip below the image
+          * (1.0 + 0.2 * nrows_in / (r * a.stride_h));                            // staging, relative to the tile work
+      if (best == 0.0 || cost < best) { best = cost; rows = r; }
     }
   }
   if (rows < 1) rows = 1;
@@ -199,8 +294,17 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s)
   a.rows = rows;
   a.strips = (a.oh + rows - 1) / rows;
   a.nrows_in = (rows - 1) * a.stride_h + a.kh;
-  const size_t lds = (size_t)a.nrows_in * a.lrow + 32;
-  if (lds > 48 * 1024 + 64 || (long long)a.nrows_in * a.lrow >= (1ll << 30) || (long long)rows * a.ow * a.ow >= (1ll << 32))
+  size_t lds = (size_t)a.nrows_in * a.lrow + 32;
+  a.tab_lds = 0;
+  if (a.ep.shift_tab) {
+    const size_t tab = (size_t)(rows + a.ow + a.nclass * a.wo * 32) * 4;
+    if (lds + tab <= 48 * 1024) {
+      a.tab_lds = (int)(up((int)lds, 16) / 4);   // dword offset of the tables
+      lds = (size_t)a.tab_lds * 4 + tab;
+    }
+  }
+  if (lds > 48 * 1024 + 64 || (long long)a.nrows_in * a.lrow >= (1ll << 30) ||
+      (long long)(a.ih + 2 * a.kh + 32) * (a.iw + 16) * a.ic >= (1ll << 30) || (long long)rows * a.ow * a.ow >= (1ll << 32))
     return hipErrorInvalidValue;
   a.ow_magic = div_magic(a.ow);
   a.iw_magic = div_magic(a.iw);

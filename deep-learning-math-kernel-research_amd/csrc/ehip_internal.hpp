@@ -157,8 +157,9 @@ struct FewChArgs {
   int oc2, ocpp;
   int in_nhwc, out_nhwc;
   const int *cls_h, *cls_w;   // with ep.shift_tab: class of an output row / column; class = cls_h * ncls_w + cls_w
-  int ncls_w;
+  int ncls_w, nclass;
   // set by the launcher
+  int tab_lds;          // != 0: dword offset in LDS of on-chip copies of the class tables and shift rows
   int ppc, nu, cells;   // cells = kh * nu
   int rows, strips;     // output rows per workgroup, workgroups per image
   int nrows_in, lrow;   // staged input rows and their pitch in bytes (a multiple of 4)
@@ -364,7 +365,8 @@ __device__ __forceinline__ unsigned quant4(const Epilogue &ep, int a0, int a1, i
 // The patch is laid out [16-channel block][pixel][quarter ^ ((pixel / 4) & 3)] in 16-byte cells,
 // which keeps both the writes (fixed quarter, 16 pixels) and the reads (4 pixels x 4 quarters)
 // spread over all banks.
-template <int TM, int TN, int OUT, bool SUM, bool FAST, bool XPOSE, bool TAB>
+// NOCOMP: the accumulators already hold the compensation (they started from it instead of zero).
+template <int TM, int TN, int OUT, bool SUM, bool FAST, bool XPOSE, bool TAB, bool NOCOMP>
 __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
                                                     long long cidx, int oc_first, const size_t (&pix)[TN],
                                                     const bool (&pvalid)[TN], int oc_real, size_t block_stride,
@@ -400,8 +402,9 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
       v4i s[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        s[q] = v4i{a[4 * q] + k.comp[q].x, a[4 * q + 1] + k.comp[q].y, a[4 * q + 2] + k.comp[q].z,
-                   a[4 * q + 3] + k.comp[q].w};
+        s[q] = NOCOMP ? v4i{a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]}
+                      : v4i{a[4 * q] + k.comp[q].x, a[4 * q + 1] + k.comp[q].y, a[4 * q + 2] + k.comp[q].z,
+                            a[4 * q + 3] + k.comp[q].w};
       if (OUT == EHIP_S32 || OUT == EHIP_F32) {
         if (OUT == EHIP_F32) {
 #pragma unroll
@@ -450,7 +453,7 @@ __device__ __forceinline__ void epilogue_wave_typed(const Epilogue &ep, const v1
 
 // one uniform switch on the output type (and on the cheap ReLU form) around the whole epilogue;
 // xlds == nullptr: 4-byte outputs are stored directly.  TAB: per-pixel shift rows (ep.shift_tab, cls).
-template <int TM, int TN, bool TAB>
+template <int TM, int TN, bool TAB, bool NOCOMP = false>
 __device__ __forceinline__ void epilogue_wave_tab(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
                                                   long long cidx, int oc_first, const size_t (&pix)[TN],
                                                   const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out,
@@ -458,7 +461,7 @@ __device__ __forceinline__ void epilogue_wave_tab(const Epilogue &ep, const v16i
                                                   const int *cls)
 {
 #define EHIP_EPI(OUT, SUM, FAST, XP)                                                                                   \
-  epilogue_wave_typed<TM, TN, OUT, SUM, FAST, XP, TAB>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, \
+  epilogue_wave_typed<TM, TN, OUT, SUM, FAST, XP, TAB, NOCOMP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, \
                                                        out, xlds, pixT, validT, cls)
   // cheap narrowing: ReLU bounds 0 <= lo <= hi (and lo inside the s8 code range for s8 output)
   const bool fast = ep.with_relu && ep.lo >= 0.0f && ep.hi >= ep.lo && (ep.out_type != EHIP_S8 || ep.lo <= 127.0f);
@@ -483,7 +486,7 @@ __device__ __forceinline__ void epilogue_wave_tab(const Epilogue &ep, const v16i
 
 // BORDER: the kernel can be asked for per-pixel shift rows (the k x k GEMM form); other kernels do
 // not carry that code at all
-template <int TM, int TN, bool BORDER = false>
+template <int TM, int TN, bool BORDER = false, bool NOCOMP = false>
 __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&acc)[TM][TN], const OcConsts &k0,
                                               long long cidx, int oc_first, const size_t (&pix)[TN],
                                               const bool (&pvalid)[TN], int oc_real, size_t block_stride, void *out,
@@ -491,9 +494,9 @@ __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&a
                                               const int *cls = nullptr)
 {
   if (BORDER && ep.shift_tab)
-    epilogue_wave_tab<TM, TN, true>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
+    epilogue_wave_tab<TM, TN, true, NOCOMP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
   else
-    epilogue_wave_tab<TM, TN, false>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
+    epilogue_wave_tab<TM, TN, false, NOCOMP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
 }
 
 
