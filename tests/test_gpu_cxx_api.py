@@ -29,7 +29,9 @@ def from_blocked(b, c):
     dict(n=2, ic=64, oc=64, hw=14, k=3, pad=1, stride=2, out_type=ol.S8, T=7),
     dict(n=2, ic=32, oc=32, hw=14, k=3, pad=1, stride=2, out_type=ol.U8, depthwise=True, T=7),
     dict(n=2, ic=96, oc=64, hw=7, k=1, pad=0, out_type=ol.S8, with_sum=True, nhwc=True),
-], ids=["3x3_u8", "1x1_s8_sum", "1x1_f32", "depthwise_u8", "3x3_s2_s8", "depthwise_s2_u8", "1x1_s8_sum_nhwc"])
+    dict(n=2, ic=3, oc=64, hw=22, k=7, pad=3, stride=2, out_type=ol.S8, nhwc=True),   # a first layer: 3-channel nhwc image
+], ids=["3x3_u8", "1x1_s8_sum", "1x1_f32", "depthwise_u8", "3x3_s2_s8", "depthwise_s2_u8", "1x1_s8_sum_nhwc",
+        "7x7_s2_3ch_nhwc"])
 def test_elx_conv_on_host_buffers(case, tmp_path):
     assert os.path.exists(CHECK), "euler_api_check is not built (python -c 'import __graft_entry__ as g; g.build()')"
     c = dict(stride=1, with_sum=False, depthwise=False, T=0, nhwc=False)

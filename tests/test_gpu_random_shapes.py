@@ -51,6 +51,36 @@ def test_random_kxk(seed):
                           out_hw=out_hw))
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_first_layer(seed):
+    """k x k over 1..4 input channels: compact nhwc or blocked input, with and without a zero point"""
+    r = _rng(400 + seed)
+    k = int(r.choice([3, 5, 7]))
+    stride = int(r.choice([1, 2]))
+    pad = int(r.choice([k // 2 - 1, k // 2]))
+    hw = int(r.integers(k + 1, 40))
+    ic = int(r.integers(1, 5))
+    oc = int(r.integers(1, 9)) * 16
+    out_hw = None
+    natural = (hw + 2 * pad - k) // stride + 1
+    if stride == 2 and pad == k // 2 - 1 and natural * stride + k - hw - pad <= k // 2 and r.integers(0, 2):
+        out_hw = natural + 1   # pads only at the right / bottom
+    # the right / bottom pad that the output size implies must be k/2 - 1 or k/2 as well (c160 shapes)
+    o = out_hw or natural
+    while (o - 1) * stride + k - hw - pad not in (k // 2 - 1, k // 2) and (o - 1) * stride + k - hw - pad >= 0:
+        hw += 1
+        out_hw = None
+        o = natural = (hw + 2 * pad - k) // stride + 1
+    in_z = float(r.choice([0.0, 128.0, 3.0]))
+    if in_z != 0.0 and (pad or out_hw) and min(natural, out_hw or natural) + (k // 2 - 1) < k:
+        in_z = 0.0   # the reference refuses a zero point where one pad cannot be covered
+    out_type = OUT_TYPES[int(r.integers(0, 4))]
+    res = run_and_compare(Layer(int(r.integers(1, 4)), ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type,
+                                seed=seed, out_hw=out_hw, in_z=in_z, in_nhwc=bool(r.integers(0, 2)),
+                                out_nhwc=bool(r.integers(0, 2)), with_relu=(out_type != ol.F32 or in_z == 0.0)))
+    assert res["conv"].kernel_name == "k_conv_fewch_u8s8"
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_random_depthwise(seed):
     r = _rng(200 + seed)
