@@ -28,7 +28,7 @@ __device__ __forceinline__ unsigned low_bytes(int k)   // mask of the k lowest b
 }  // namespace
 
 template <int KS>
-__global__ __launch_bounds__(kBlock, 2) void k_conv_fewch_u8s8(FewChArgs a)
+__global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
 {
   // [nrows_in][lrow / 4] staged rows; with border classes kept on chip (a.tab_lds): the shift rows of
   // the workgroup's channels [class][wo * 32], then the class of each of the strip's output rows
@@ -267,15 +267,14 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s)
       else
         n_cu = 256;
     }
-    const int ks = (a.cells + 1) / 2;
     double best = 0.0;
     for (int r = 1; r <= a.oh && r <= 32; ++r) {
       const int nrows_in = (r - 1) * a.stride_h + a.kh;
       const size_t dyn = (size_t)nrows_in * a.lrow + 32;
       if (dyn > 40 * 1024) break;
-      // workgroups of 4 waves resident per CU: registers (the 14-cell kernel holds 2 waves per SIMD,
-      // the others 3), LDS (16 KB static exchange patch + the rows)
-      int resident = ks > 5 ? 2 : 3;
+      // workgroups of 4 waves resident per CU: registers (3 waves per SIMD), LDS (16 KB static
+      // exchange patch + the rows)
+      int resident = 3;
       const int by_lds = (int)((160 * 1024) / (16 * 1024 + dyn));
       if (by_lds < resident) resident = by_lds < 1 ? 1 : by_lds;
       const double slots = (double)n_cu * resident;
