@@ -33,6 +33,18 @@ inline uint32_t cvt_u32_rne(float f)
   if (!(r >= 0.0f && r < 4294967296.0f)) return 0xffffffffu;
   return (uint32_t)r;
 }
+// _mm512_cvt_roundps_epi32 / _epu32(x, toward -inf): the store of the F(2x2,3x3) output kernel
+inline int32_t cvt_s32_floor(float f)
+{
+  if (!(f >= -2147483648.0f && f < 2147483648.0f)) return INT32_MIN;
+  return (int32_t)floorf(f);
+}
+inline uint32_t cvt_u32_floor(float f)
+{
+  float r = floorf(f);
+  if (!(r >= 0.0f && r < 4294967296.0f)) return 0xffffffffu;
+  return (uint32_t)r;
+}
 inline uint8_t usat8(uint32_t v) { return v > 255u ? 255 : (uint8_t)v; }         // vpmovusdb
 inline int8_t ssat8(int32_t v) { return (int8_t)std::min(127, std::max(-128, v)); } // vpmovsdb
 
@@ -225,14 +237,142 @@ inline void wino_out_1d(const float f[6], float o[4])
   o[3] = fmaf(t2, z5, t3 * z2) + f[5];
 }
 
+// ---------------------------------------------------------------------------------------
+// F(2x2,3x3), tile size A = 4: additions and exact products only
+// ---------------------------------------------------------------------------------------
+// src/kernel/elk_conv_wino_2x2_3x3_input.hxx:104-150.  d, v: [4][4] row-major (row = h).
+inline void wino4_tile_input(const float d[16], float v[16])
+{
+#define D(i, j) d[4 * (i) + (j)]
+#define V(i, j) v[4 * (i) + (j)]
+  float c1, c2;
+  c1 = D(1, 2) - D(1, 0);
+  c2 = D(2, 0) - D(2, 2);
+  V(0, 0) = (D(0, 0) - D(0, 2)) - c2;
+  V(1, 0) = c1 + c2;
+  V(2, 0) = c2 - c1;
+  V(3, 0) = c1 + (D(3, 0) - D(3, 2));
+  c1 = D(1, 2) - D(1, 1);
+  c2 = D(2, 2) - D(2, 1);
+  V(0, 1) = (D(0, 2) - D(0, 1)) - c2;
+  V(1, 1) = c2 - c1;
+  V(2, 1) = c2 + c1;
+  V(3, 1) = (D(3, 2) - D(3, 1)) - c1;
+  c1 = D(1, 1) + D(1, 2);
+  c2 = D(2, 1) + D(2, 2);
+  V(0, 2) = D(0, 1) + D(0, 2) - c2;
+  V(1, 2) = c2 - c1;
+  V(2, 2) = c2 + c1;
+  V(3, 2) = D(3, 1) + D(3, 2) - c1;
+  c1 = D(1, 1) - D(1, 3);
+  c2 = D(2, 3) - D(2, 1);
+  V(0, 3) = (D(0, 3) - D(0, 1)) - c2;
+  V(1, 3) = c1 + c2;
+  V(2, 3) = c2 - c1;
+  V(3, 3) = (c1 - D(3, 1)) + D(3, 3);
+#undef D
+#undef V
+}
+// src/kernel/elk_conv_wino_2x2_3x3_weights.hxx:72-107.  g: [3][3] (kh, kw), u: [4][4].
+inline void wino4_tile_weights(const float g[9], float u[16])
+{
+#define G(i, j) g[3 * (i) + (j)]
+#define U(i, j) u[4 * (i) + (j)]
+  const float r4 = 0.25f, r2 = 0.5f, z2 = 2.0f;
+  U(0, 0) = G(0, 0);
+  U(1, 0) = r2 * ((G(0, 0) - G(1, 0)) + G(2, 0));
+  U(2, 0) = r2 * ((G(0, 0) + G(1, 0)) + G(2, 0));
+  U(3, 0) = G(2, 0);
+  const float c10 = r4 * ((G(0, 0) - G(0, 1)) + G(0, 2));
+  const float c11 = r4 * ((G(1, 0) - G(1, 1)) + G(1, 2));
+  const float c12 = r4 * ((G(2, 0) - G(2, 1)) + G(2, 2));
+  U(0, 1) = z2 * c10;
+  U(1, 1) = c10 - c11 + c12;
+  U(2, 1) = c10 + c11 + c12;
+  U(3, 1) = z2 * c12;
+  const float c20 = r4 * (G(0, 0) + G(0, 1) + G(0, 2));
+  const float c21 = r4 * (G(1, 0) + G(1, 1) + G(1, 2));
+  const float c22 = r4 * (G(2, 0) + G(2, 1) + G(2, 2));
+  U(0, 2) = z2 * c20;
+  U(1, 2) = c20 - c21 + c22;
+  U(2, 2) = c20 + c21 + c22;
+  U(3, 2) = z2 * c22;
+  U(0, 3) = G(0, 2);
+  U(1, 3) = r2 * (G(0, 2) - G(1, 2) + G(2, 2));
+  U(2, 3) = r2 * (G(0, 2) + G(1, 2) + G(2, 2));
+  U(3, 3) = G(2, 2);
+#undef G
+#undef U
+}
+// src/kernel/elk_conv_wino_2x2_3x3_output.hxx:76-95.  m: [4][4], y: [2][2].
+inline void wino4_tile_output(const float m[16], float y[4])
+{
+#define T(i, j) m[4 * (i) + (j)]
+  const float c0 = T(1, 0) + T(1, 1) + T(1, 2);
+  const float c1 = T(2, 0) + T(2, 1) + T(2, 2);
+  const float c2 = T(1, 2) + T(1, 3) - T(1, 1);
+  const float c3 = T(2, 2) + T(2, 3) - T(2, 1);
+  y[0] = T(0, 0) + T(0, 1) + T(0, 2) + c0 + c1;            // p00
+  y[2] = c1 - c0 + T(3, 0) + T(3, 1) + T(3, 2);            // p10
+  y[1] = T(0, 2) - T(0, 1) + T(0, 3) + c2 + c3;            // p01
+  y[3] = c3 - c2 - T(3, 1) + T(3, 2) + T(3, 3);            // p11
+#undef T
+}
+
+// ---------------------------------------------------------------------------------------
+// F(3x3,3x3), tile size A = 5.  Products with 0.5 and 2 are exact, so only the products with
+// 1.5 (input) and 1/3, 2/3, 4/3 (output) have a fused / unfused question; the compiled
+// reference kernels answer it (tests/test_oracle_ref_kernels.py).
+// ---------------------------------------------------------------------------------------
+// src/kernel/elk_conv_wino_3x3_3x3_input.hxx:91-128.  f2 * 1.5 + f3 is one fused rounding, except in the
+// first (column) pass of the BORDER kernel, whose inputs are zero-or-load selects: there the product is
+// rounded first -- the same behaviour of the compiled reference as in its F(4x4,3x3) border kernel.
+inline void wino5_in_1d(const float f[5], float o[5], bool fuse15)
+{
+  const float z0 = 0.5f, z1 = 1.5f;
+  const float t0 = f[1] * z0;
+  const float t1 = f[2] * z0;
+  const float t2 = f[3] - f[1];
+  o[0] = f[0] * z0 - t1 - t2;
+  o[1] = f[3] - t0 - t1;
+  o[2] = (fuse15 ? fmaf(f[2], z1, f[3]) : f[2] * z1 + f[3]) + t0;
+  o[3] = t2;
+  o[4] = f[3] * z0 + f[4] - f[2] - t0;
+}
+// src/kernel/elk_conv_wino_3x3_3x3_weights.hxx:27-66 (every product exact)
+inline void wino5_w_1d(float f0, float f1, float f2, float o[5])
+{
+  const float t0 = f0 * 2.0f;
+  const float t1 = f0 + f2;
+  o[0] = t0;
+  o[1] = f1 - t1;
+  o[2] = f1 + t1;
+  o[3] = f2 * 0.5f + t0 - f1;
+  o[4] = f2;
+}
+// src/kernel/elk_conv_wino_3x3_3x3_output.hxx:93-131: f2*z0 fuses into both of its uses, every
+// other product into the addition that follows it
+inline void wino5_out_1d(const float f[5], float o[3])
+{
+  const float z0 = 0.3333333333333333f, z1 = 0.6666666666666666f, z2 = 1.3333333333333333f;
+  const float t1 = fmaf(f[2], z0, f[1]);
+  o[0] = fmaf(f[3], z2, f[0]) + t1;
+  o[1] = fmaf(-f[3], z1, fmaf(f[2], z0, -f[1]));
+  o[2] = fmaf(f[3], z0, f[4]) + t1;
+}
+
+inline int wino_tile_A(const orc_conv_params *p) { return (p->wino_tile == 4 || p->wino_tile == 5) ? p->wino_tile : 6; }
+
 struct WinoGeom {
-  int ht, wt, nt, t, IC2, OC2;
+  int A, M, ht, wt, nt, t, IC2, OC2;
 };
 inline WinoGeom wino_geom(const orc_conv_params *p)
 {
   WinoGeom g;
-  g.ht = (p->oh + 3) / 4;  // (oh + A - K) / (A - K + 1), src/elx_int8_conv_wino.cpp:24-27
-  g.wt = (p->ow + 3) / 4;
+  g.A = wino_tile_A(p);
+  g.M = g.A - 2;
+  g.ht = (p->oh + g.M - 1) / g.M;  // (oh + A - K) / (A - K + 1), src/elx_int8_conv_wino.cpp:24-27
+  g.wt = (p->ow + g.M - 1) / g.M;
   g.nt = g.ht * g.wt;
   g.t = g.nt * p->n;
   g.IC2 = up16(p->ic) / 16;
@@ -240,22 +380,24 @@ inline WinoGeom wino_geom(const orc_conv_params *p)
   return g;
 }
 
-// gather one 6x6 tile of one channel (zero outside the image) and transform it
+extern "C" void orc_wino_tile_input_a(int A, int border, const float *d, float *v);
+
+// gather one A x A tile of one channel (zero outside the image) and transform it
 inline void wino_tile_from_input(const orc_conv_params *p, const float *in_plane /*[ih][iw][16]*/,
                                  int th, int tw, int v, float out[36])
 {
   float d[36];
-  const int h0 = 4 * th - p->pad_t, w0 = 4 * tw - p->pad_l;
+  const int A = wino_tile_A(p), M = A - 2;
+  const int h0 = M * th - p->pad_t, w0 = M * tw - p->pad_l;
   bool border = false;  // input_tile_iter::is_border, src/elx_conv_wino_trans_input.hpp:247-249
-  for (int i = 0; i < 6; ++i)
-    for (int j = 0; j < 6; ++j) {
+  for (int i = 0; i < A; ++i)
+    for (int j = 0; j < A; ++j) {
       int h = h0 + i, w = w0 + j;
       bool inside = h >= 0 && h < p->ih && w >= 0 && w < p->iw;
       border |= !inside;
-      d[6 * i + j] = inside ? in_plane[((size_t)h * p->iw + w) * 16 + v] : 0.0f;
+      d[A * i + j] = inside ? in_plane[((size_t)h * p->iw + w) * 16 + v] : 0.0f;
     }
-  if (border) orc_wino_tile_input_border(d, out);
-  else orc_wino_tile_input(d, out);
+  orc_wino_tile_input_a(A, border, d, out);
 }
 
 } // namespace
@@ -660,6 +802,63 @@ void orc_wino_tile_output(const float m[36], float y[16])
   for (int i = 0; i < 4; ++i) wino_out_1d(M[i], &y[4 * i]);
 }
 
+// any tile size: A = 6 as above, A = 4 F(2x2,3x3), A = 5 F(3x3,3x3); arrays are [A][A] row-major
+void orc_wino_tile_input_a(int A, int border, const float *d, float *v)
+{
+  if (A == 4) {
+    wino4_tile_input(d, v);
+  } else if (A == 5) {
+    float m[25];
+    for (int j = 0; j < 5; ++j) {
+      float f[5], o[5];
+      for (int i = 0; i < 5; ++i) f[i] = d[5 * i + j];
+      wino5_in_1d(f, o, !border);
+      for (int i = 0; i < 5; ++i) m[5 * i + j] = o[i];
+    }
+    for (int i = 0; i < 5; ++i) wino5_in_1d(&m[5 * i], &v[5 * i], true);
+  } else if (border) {
+    orc_wino_tile_input_border(d, v);
+  } else {
+    orc_wino_tile_input(d, v);
+  }
+}
+
+void orc_wino_tile_weights_a(int A, const float g[9], float *u)
+{
+  if (A == 4) {
+    wino4_tile_weights(g, u);
+  } else if (A == 5) {
+    float M[5][3];
+    for (int i = 0; i < 3; ++i) {
+      float o[5];
+      wino5_w_1d(g[0 * 3 + i], g[1 * 3 + i], g[2 * 3 + i], o);
+      for (int k = 0; k < 5; ++k) M[k][i] = o[k];
+    }
+    for (int i = 0; i < 5; ++i) wino5_w_1d(M[i][0], M[i][1], M[i][2], &u[5 * i]);
+  } else {
+    orc_wino_tile_weights(g, u);
+  }
+}
+
+// y: [A - 2][A - 2] row-major
+void orc_wino_tile_output_a(int A, const float *m, float *y)
+{
+  if (A == 4) {
+    wino4_tile_output(m, y);
+  } else if (A == 5) {
+    float M[3][5];
+    for (int i = 0; i < 5; ++i) {
+      float f[5], o[3];
+      for (int k = 0; k < 5; ++k) f[k] = m[5 * k + i];
+      wino5_out_1d(f, o);
+      for (int k = 0; k < 3; ++k) M[k][i] = o[k];
+    }
+    for (int i = 0; i < 3; ++i) wino5_out_1d(M[i], &y[3 * i]);
+  } else {
+    orc_wino_tile_output(m, y);
+  }
+}
+
 int orc_wino_tiles(const orc_conv_params *p) { return wino_geom(p).t; }
 
 int orc_wino_tinput_range(const orc_conv_params *p, const float *input, float *min_out, float *max_out)
@@ -676,7 +875,7 @@ int orc_wino_tinput_range(const orc_conv_params *p, const float *input, float *m
             if (c2 * 16 + v >= p->ic) continue;
             float o[36];
             wino_tile_from_input(p, plane, th, tw, v, o);
-            for (int k = 0; k < 36; ++k) { mn = std::min(mn, o[k]); mx = std::max(mx, o[k]); }
+            for (int k = 0; k < g.A * g.A; ++k) { mn = std::min(mn, o[k]); mx = std::max(mx, o[k]); }
           }
     }
   *min_out = mn; *max_out = mx;
@@ -686,20 +885,21 @@ int orc_wino_tinput_range(const orc_conv_params *p, const float *input, float *m
 int orc_wino_prepare(const orc_conv_params *p, const float *w, int8_t *twq, float *tscale, float *tshift)
 {
   const int OCp = up16(p->oc), ICp = up16(p->ic), I2 = ICp / 16;
+  const int A = wino_tile_A(p), AA = A * A;
   const float tin_S = p->tin_scale, tin_z = std::ceil(p->tin_z);  // src/elx_int8_conv_wino.cpp:270-276
-  std::vector<float> U((size_t)36 * OCp * ICp);
+  std::vector<float> U((size_t)AA * OCp * ICp);
 #pragma omp parallel for collapse(2)
   for (int oc = 0; oc < OCp; ++oc)
     for (int ic = 0; ic < ICp; ++ic) {
       float g[9], u[36];
       for (int k = 0; k < 9; ++k)
         g[k] = w[((((size_t)(oc / 16) * I2 + ic / 16) * 9 + k) * 16 + ic % 16) * 16 + oc % 16];
-      orc_wino_tile_weights(g, u);
-      for (int a = 0; a < 36; ++a) U[((size_t)a * OCp + oc) * ICp + ic] = u[a];
+      orc_wino_tile_weights_a(A, g, u);
+      for (int a = 0; a < AA; ++a) U[((size_t)a * OCp + oc) * ICp + ic] = u[a];
     }
   // src/elx_conv_wino_trans_weights.cpp:437-535
 #pragma omp parallel for collapse(2)
-  for (int a = 0; a < 36; ++a)
+  for (int a = 0; a < AA; ++a)
     for (int oc = 0; oc < OCp; ++oc) {
       const float *u = &U[((size_t)a * OCp + oc) * ICp];
       float absmax = 0.0f;
@@ -736,7 +936,7 @@ int orc_wino_trans_input(const orc_conv_params *p, const float *input, uint8_t *
           for (int v = 0; v < 16; ++v) {
             float o[36];
             wino_tile_from_input(p, plane, th, tw, v, o);
-            for (int a = 0; a < 36; ++a) {
+            for (int a = 0; a < g.A * g.A; ++a) {
               float f = fmaf(o[a], mrepS, mz);
               tinput[(((size_t)a * g.IC2 + c2) * g.t + t) * 16 + v] = usat8(cvt_u32_rne(f));
             }
@@ -753,7 +953,7 @@ int orc_wino_gemm(const orc_conv_params *p, const uint8_t *tinput, const int8_t 
   const int OCp = g.OC2 * 16, ICp = g.IC2 * 16;
   const bool vnni = cpu_has_vnni();
 #pragma omp parallel for collapse(2) schedule(static)
-  for (int a = 0; a < 36; ++a)
+  for (int a = 0; a < g.A * g.A; ++a)
     for (int o2 = 0; o2 < g.OC2; ++o2) {
       // [ic/4][16 oc][4 ic]
       std::vector<int8_t> wt((size_t)ICp * 16);
@@ -789,13 +989,22 @@ int orc_wino_gemm(const orc_conv_params *p, const uint8_t *tinput, const int8_t 
 int orc_wino_output_value(float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
                           int with_relu, float *f32_out)
 {
+  return orc_wino_output_value_a(6, y, with_bias, bias, out_type, out_scale, out_z, with_relu, f32_out);
+}
+
+// The same for any tile size.  The F(2x2,3x3) kernel converts toward minus infinity in its u8 / s8
+// store (src/kernel/elk_conv_wino_2x2_3x3_output.hxx:142-151), the others to nearest even
+// (src/kernel/elk_conv_wino_3x3_3x3_output.hxx:74-86).
+int orc_wino_output_value_a(int A, float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
+                            int with_relu, float *f32_out)
+{
   float r = y;
   if (with_bias) r += bias;
   if (out_type == ORC_U8 || out_type == ORC_S8) r = fmaf(r, 1.0f / out_scale, std::ceil(out_z));
   if (with_relu) r = r > 0.0f ? r : 0.0f;  // vmaxps(p, 0): no upper bound here
   if (f32_out) *f32_out = r;
-  if (out_type == ORC_U8) return usat8(cvt_u32_rne(r));
-  if (out_type == ORC_S8) return ssat8(cvt_s32_rne(r));
+  if (out_type == ORC_U8) return usat8(A == 4 ? cvt_u32_floor(r) : cvt_u32_rne(r));
+  if (out_type == ORC_S8) return ssat8(A == 4 ? cvt_s32_floor(r) : cvt_s32_rne(r));
   return 0;
 }
 
@@ -811,15 +1020,16 @@ int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const 
           const size_t t = (size_t)n * g.nt + (size_t)th * g.wt + tw;
           for (int v = 0; v < 16; ++v) {
             float m[36], y[16];
-            for (int a = 0; a < 36; ++a) m[a] = toutput[(((size_t)a * g.OC2 + o2) * g.t + t) * 16 + v];
-            orc_wino_tile_output(m, y);
-            for (int i = 0; i < 4; ++i)
-              for (int j = 0; j < 4; ++j) {
-                int oh = 4 * th + i, ow = 4 * tw + j;
+            for (int a = 0; a < g.A * g.A; ++a) m[a] = toutput[(((size_t)a * g.OC2 + o2) * g.t + t) * 16 + v];
+            orc_wino_tile_output_a(g.A, m, y);
+            for (int i = 0; i < g.M; ++i)
+              for (int j = 0; j < g.M; ++j) {
+                int oh = g.M * th + i, ow = g.M * tw + j;
                 if (oh >= p->oh || ow >= p->ow) continue;
                 float r;
-                const int q = orc_wino_output_value(y[4 * i + j], p->with_bias, p->with_bias ? bias[o2 * 16 + v] : 0.0f,
-                                                    p->out_type, p->out_scale, p->out_z, p->with_relu, &r);
+                const int q = orc_wino_output_value_a(g.A, y[g.M * i + j], p->with_bias,
+                                                      p->with_bias ? bias[o2 * 16 + v] : 0.0f, p->out_type,
+                                                      p->out_scale, p->out_z, p->with_relu, &r);
                 const size_t oi = ((((size_t)n * g.OC2 + o2) * p->oh + oh) * p->ow + ow) * 16 + v;
                 if (p->out_type == ORC_U8) ((uint8_t *)output)[oi] = (uint8_t)q;
                 else if (p->out_type == ORC_S8) ((int8_t *)output)[oi] = (int8_t)q;

@@ -50,6 +50,7 @@ typedef struct orc_conv_params {
   float sum_scale, sum_z;      /* sum_quant    */
   float tin_scale, tin_z;      /* wino_tinput_quant */
   float relu_lo, relu_hi;      /* relu_bound   */
+  int32_t wino_tile;           /* Winograd tile size A: 0 or 6 = F(4x4,3x3), 4 = F(2x2,3x3), 5 = F(3x3,3x3) */
 } orc_conv_params;
 
 /* ---- layout reorders: src/elx_reorder.cpp:35-93 ---- */
@@ -123,6 +124,13 @@ void orc_wino_tile_input(const float d[36], float v[36]);         /* interior ti
 void orc_wino_tile_input_border(const float d[36], float v[36]);  /* tiles that touch the zero border */
 void orc_wino_tile_weights(const float g[9], float u[36]);
 void orc_wino_tile_output(const float m[36], float y[16]);
+/* any tile size A in {4, 5, 6}; arrays are [A][A] (output: [A-2][A-2]) row-major
+ * (src/kernel/elk_conv_wino_2x2_3x3_*.hxx, src/kernel/elk_conv_wino_3x3_3x3_*.hxx) */
+void orc_wino_tile_input_a(int A, int border, const float *d, float *v);
+void orc_wino_tile_weights_a(int A, const float g[9], float *u);
+void orc_wino_tile_output_a(int A, const float *m, float *y);
+int orc_wino_output_value_a(int A, float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
+                            int with_relu, float *f32_out);
 
 /* epilogue on one value, exposed for the same reason (out_kind ORC_*; returns the f32 result
  * for ORC_F32 through *fout, else the quantized byte through the return value) */

@@ -9,7 +9,7 @@
 // the reference's compiled code and not by a reading of it.  Nothing of the reference is
 // copied: the templates are instantiated straight from
 //   src/kernel/elk_u8s8_gemm.hxx, elk_u8s8_conv.hxx, elk_u8s8_depthwise_conv.hxx,
-//   src/kernel/elk_conv_wino_4x4_3x3_{input,weights,output}.hxx.
+//   src/kernel/elk_conv_wino_{4x4,2x2,3x3}_3x3_{input,weights,output}.hxx.
 // The executor classes (src/elx_int8_conv_*.cpp) are NOT built: they bind kernels through
 // tables that the reference's build generates with shell scripts at configure time.
 //
@@ -38,6 +38,12 @@
 #include "elk_conv_wino_4x4_3x3_input.hxx"
 #include "elk_conv_wino_4x4_3x3_weights.hxx"
 #include "elk_conv_wino_4x4_3x3_output.hxx"
+#include "elk_conv_wino_2x2_3x3_input.hxx"
+#include "elk_conv_wino_2x2_3x3_weights.hxx"
+#include "elk_conv_wino_2x2_3x3_output.hxx"
+#include "elk_conv_wino_3x3_3x3_input.hxx"
+#include "elk_conv_wino_3x3_3x3_weights.hxx"
+#include "elk_conv_wino_3x3_3x3_output.hxx"
 
 using namespace euler;
 
@@ -368,6 +374,74 @@ void ref_wino_trans_output_q(int out_kind, int border, int with_bias, int with_r
   WQ_CASE(2, int8_t, false, true, true) WQ_CASE(2, int8_t, false, false, false)
   WQ_CASE(2, int8_t, true, true, false) WQ_CASE(2, int8_t, true, true, true)
 #undef WQ_CASE
+}
+
+// The other tile sizes: A = 4 is F(2x2,3x3) (src/kernel/elk_conv_wino_2x2_3x3_*.hxx), A = 5 is
+// F(3x3,3x3) (src/kernel/elk_conv_wino_3x3_3x3_*.hxx).  Same conventions as the A = 6 drivers above;
+// tinput / toutput are [A][A][16] f32, the f32 or u8 input tile lies in an [ih][iw][16] plane.
+int ref_wino_trans_input_a(int A, int border, int ih, int iw, float *tinput, float *tile,
+    int hs, int he, int ws, int we)
+{
+  elx_param_t ep;
+  fill_common(ep, 0.f, FLT_MAX, 0.f);
+  ep.ih = ih; ep.iw = iw;
+#define WI_CASE(a)                                                              \
+  if (A == a) {                                                                 \
+    if (border)                                                                 \
+      elk_conv_wino_trans_input<float, float, TKF_BLOCKED, true, ISA_AVX512, a, \
+          16>::execute(ep, tinput, tile, hs, he, ws, we);                       \
+    else                                                                        \
+      elk_conv_wino_trans_input<float, float, TKF_BLOCKED, false, ISA_AVX512,   \
+          a, 16>::execute(ep, tinput, tile, 0, a - 1, 0, a - 1);                \
+    return 0;                                                                   \
+  }
+  WI_CASE(4) WI_CASE(5)
+#undef WI_CASE
+  return -1;
+}
+
+// in [3][3][16 ic][16 oc], out [A][A][16 ic][16 oc], f32, 64-byte aligned
+int ref_wino_trans_weights_a(int A, float *tweights, float *weights)
+{
+  if (A == 4) {
+    elk_conv_wino_trans_weights<float, float, ISA_AVX512, 4, 3, 16>::execute(
+        *(float(*)[4][4][16][16])tweights, *(float(*)[3][3][16][16])weights);
+    return 0;
+  }
+  if (A == 5) {
+    elk_conv_wino_trans_weights<float, float, ISA_AVX512, 5, 3, 16>::execute(
+        *(float(*)[5][5][16][16])tweights, *(float(*)[3][3][16][16])weights);
+    return 0;
+  }
+  return -1;
+}
+
+// out_kind 0: f32, 1: u8, 2: s8 output plane [oh][ow][16]; rows > h_end / cols > w_end are not
+// written when border != 0
+int ref_wino_trans_output_a(int A, int out_kind, int border, int with_bias, int with_relu, int oh,
+    int ow, void *out, float *toutput, float *bias, int h_end, int w_end, float repS, float z)
+{
+  elx_param_t ep;
+  fill_common(ep, 0.f, FLT_MAX, 0.f);
+  ep.oh = oh; ep.ow = ow;
+  ep.output_quant_repS = repS;
+  ep.output_quant_z = z;
+#define WA_CASE(a, k, OT, b, wb, wr)                                            \
+  if (A == a && out_kind == k && !!border == b && !!with_bias == wb && !!with_relu == wr) { \
+    elk_conv_wino_trans_output<float, OT, float, TKF_BLOCKED, b, wb, wr,        \
+        false, ISA_AVX512, a, 3, 16>::execute(ep, (OT *)out, toutput, bias,     \
+        h_end, w_end);                                                          \
+    return 0;                                                                   \
+  }
+#define WA_ALL(a, k, OT)                                                        \
+  WA_CASE(a, k, OT, false, false, false) WA_CASE(a, k, OT, false, true, false)  \
+  WA_CASE(a, k, OT, false, true, true) WA_CASE(a, k, OT, true, false, false)    \
+  WA_CASE(a, k, OT, true, true, false) WA_CASE(a, k, OT, true, true, true)
+  WA_ALL(4, 0, float) WA_ALL(4, 1, uint8_t) WA_ALL(4, 2, int8_t)
+  WA_ALL(5, 0, float) WA_ALL(5, 1, uint8_t) WA_ALL(5, 2, int8_t)
+#undef WA_ALL
+#undef WA_CASE
+  return -1;
 }
 
 } // extern "C"

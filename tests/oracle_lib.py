@@ -24,7 +24,7 @@ class ConvParams(ctypes.Structure):
         "pad_t", "pad_l", "stride_h", "stride_w", "out_type",
         "with_bias", "with_relu", "with_sum", "T")] + [(k, ctypes.c_float) for k in (
         "in_scale", "in_z", "out_scale", "out_z", "sum_scale", "sum_z",
-        "tin_scale", "tin_z", "relu_lo", "relu_hi")]
+        "tin_scale", "tin_z", "relu_lo", "relu_hi")] + [("wino_tile", ctypes.c_int32)]
 
 
 FLT_MAX = float(np.finfo(np.float32).max)
@@ -33,7 +33,7 @@ FLT_MAX = float(np.finfo(np.float32).max)
 def make_params(n, ic, oc, ih, iw, kh=1, kw=1, pad=0, stride=1, g=1, out_type=U8, with_bias=True,
                 with_relu=True, with_sum=False, T=0, in_scale=1.0 / 255.0, in_z=0.0, out_scale=1.0,
                 out_z=0.0, sum_scale=0.0, sum_z=0.0, tin_scale=1.0, tin_z=0.0, relu_lo=0.0,
-                relu_hi=FLT_MAX, pad_tl=None, out_hw=None):
+                relu_hi=FLT_MAX, pad_tl=None, out_hw=None, wino_tile=0):
     """pad: on every side; pad_tl / out_hw: top-left pad and output size given separately (the right and
     bottom pads are then whatever the output size implies, src/elx_conv.cpp:36-37)"""
     oh = (ih + 2 * pad - kh) // stride + 1
@@ -48,6 +48,7 @@ def make_params(n, ic, oc, ih, iw, kh=1, kw=1, pad=0, stride=1, g=1, out_type=U8
     p.in_scale, p.in_z, p.out_scale, p.out_z = in_scale, in_z, out_scale, out_z
     p.sum_scale, p.sum_z, p.tin_scale, p.tin_z = sum_scale, sum_z, tin_scale, tin_z
     p.relu_lo, p.relu_hi = relu_lo, relu_hi
+    p.wino_tile = wino_tile   # Winograd tile size A (0 / 6, 4 or 5)
     return p
 
 
@@ -79,6 +80,12 @@ def oracle():
         lib = ctypes.CDLL(ORACLE_SO)
         lib.orc_quantize_input_u8.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                                               ctypes.c_float, ctypes.c_float]
+        lib.orc_wino_tile_input_a.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        lib.orc_wino_tile_weights_a.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        lib.orc_wino_tile_output_a.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        lib.orc_wino_output_value_a.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int,
+                                                ctypes.c_float, ctypes.c_float, ctypes.c_int,
+                                                ctypes.POINTER(ctypes.c_float)]
         lib.orc_epilogue.argtypes = [ctypes.c_int, ctypes.c_int32, ctypes.c_float, ctypes.c_float, ctypes.c_int,
                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_float,
                                      ctypes.POINTER(ctypes.c_float)]
@@ -114,6 +121,10 @@ def ref_kernels():
         lib.ref_wino_trans_output.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ci, ci]
         if hasattr(lib, "ref_wino_trans_output_q"):
             lib.ref_wino_trans_output_q.argtypes = [ci, ci, ci, ci, ci, ci, vp, vp, vp, ci, ci, fl, fl]
+        if hasattr(lib, "ref_wino_trans_input_a"):
+            lib.ref_wino_trans_input_a.argtypes = [ci, ci, ci, ci, vp, vp, ci, ci, ci, ci]
+            lib.ref_wino_trans_weights_a.argtypes = [ci, vp, vp]
+            lib.ref_wino_trans_output_a.argtypes = [ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, ci, ci, fl, fl]
         _ref = lib
     return _ref
 
@@ -223,18 +234,24 @@ def wino_tinput_range(p, x_blocked):
     return mn.value, mx.value
 
 
+def wino_positions(p):
+    """A x A positions of the Winograd tile size the parameters ask for"""
+    a = p.wino_tile if p.wino_tile in (4, 5) else 6
+    return a * a
+
+
 def wino_prepare(p, w_blocked):
     OCp, ICp = up16(p.oc), up16(p.ic)
-    twq = np.zeros((36, OCp, ICp), np.int8)
-    tscale = np.zeros((36, OCp), np.float32)
-    tshift = np.zeros((36, OCp), np.float32)
+    twq = np.zeros((wino_positions(p), OCp, ICp), np.int8)
+    tscale = np.zeros((wino_positions(p), OCp), np.float32)
+    tshift = np.zeros((wino_positions(p), OCp), np.float32)
     assert oracle().orc_wino_prepare(ctypes.byref(p), ptr(w_blocked), ptr(twq), ptr(tscale), ptr(tshift)) == 0
     return twq, tscale, tshift
 
 
 def wino_trans_input(p, x_blocked):
     t = wino_tiles(p)
-    tin = np.zeros((36, up16(p.ic) // 16, t, 16), np.uint8)
+    tin = np.zeros((wino_positions(p), up16(p.ic) // 16, t, 16), np.uint8)
     assert oracle().orc_wino_trans_input(ctypes.byref(p), ptr(x_blocked), ptr(tin)) == 0
     return tin
 
@@ -242,8 +259,8 @@ def wino_trans_input(p, x_blocked):
 def wino_gemm(p, tin, twq, tscale, tshift):
     t = wino_tiles(p)
     OC2 = up16(p.oc) // 16
-    tout = np.zeros((36, OC2, t, 16), np.float32)
-    acc = np.zeros((36, OC2, t, 16), np.int32)
+    tout = np.zeros((wino_positions(p), OC2, t, 16), np.float32)
+    acc = np.zeros((wino_positions(p), OC2, t, 16), np.int32)
     assert oracle().orc_wino_gemm(ctypes.byref(p), ptr(tin), ptr(twq), ptr(tscale), ptr(tshift), ptr(tout),
                                   ptr(acc)) == 0
     return tout, acc

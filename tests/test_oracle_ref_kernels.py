@@ -236,3 +236,85 @@ def test_wino_output_transform_bits(with_bias, with_relu, h_end, w_end):
                 if with_relu:
                     r = r if r > 0 else np.float32(0)
                 assert np.float32(r).view(np.uint32) == out[i, j, c].view(np.uint32), (i, j, c)
+
+
+# ---- the other Winograd tile sizes: A = 4 F(2x2,3x3), A = 5 F(3x3,3x3) ------------------------------
+@pytest.mark.parametrize("A", [4, 5])
+def test_wino_weights_transform_bits_other_tiles(A):
+    rng = np.random.default_rng(21 + A)
+    w = ol.aligned((3, 3, 16, 16), np.float32)
+    w[...] = rng.normal(0, 0.05, w.shape)
+    tw = ol.aligned((A, A, 16, 16), np.float32)
+    assert ref.ref_wino_trans_weights_a(A, ol.ptr(tw), ol.ptr(w)) == 0
+    u = np.zeros(A * A, np.float32)
+    for i in range(16):
+        for o in range(16):
+            g = np.ascontiguousarray(w[:, :, i, o].ravel())
+            ol.oracle().orc_wino_tile_weights_a(A, ol.ptr(g), ol.ptr(u))
+            assert np.array_equal(u.view(np.uint32), tw[:, :, i, o].ravel().view(np.uint32))
+
+
+@pytest.mark.parametrize("A", [4, 5])
+@pytest.mark.parametrize("h0,w0", [(2, 3), (1, 1), (0, 0), (3, 3), (6, 6), (2, 4), (-1, -1), (-1, 4), (3, -1), (8, 8), (9, 2), (-1, 9),
+                                   (-2, 5), (4, 10)])
+def test_wino_input_transform_bits_other_tiles(A, h0, w0):
+    rng = np.random.default_rng(h0 * 13 + w0 + 50 + A)
+    ih = iw = 12
+    plane = ol.aligned((ih, iw, 16), np.float32)
+    plane[...] = rng.uniform(0, 255, plane.shape).round() if (h0 + w0) % 2 else rng.uniform(0, 1, plane.shape)
+    hs, he = max(0, -h0), min(A - 1, ih - 1 - h0)
+    ws, we = max(0, -w0), min(A - 1, iw - 1 - w0)
+    border = not (hs == 0 and ws == 0 and he == A - 1 and we == A - 1)
+    tin = ol.aligned((A, A, 16), np.float32)
+    tile_ptr = ctypes.c_void_p(plane.ctypes.data + (h0 * iw + w0) * 16 * 4)
+    assert ref.ref_wino_trans_input_a(A, int(border), ih, iw, ol.ptr(tin), tile_ptr, hs, he, ws, we) == 0
+    v = np.zeros(A * A, np.float32)
+    for c in range(16):
+        d = np.zeros((A, A), np.float32)
+        for i in range(A):
+            for j in range(A):
+                h, w = h0 + i, w0 + j
+                if 0 <= h < ih and 0 <= w < iw:
+                    d[i, j] = plane[h, w, c]
+        ol.oracle().orc_wino_tile_input_a(A, int(border), ol.ptr(d), ol.ptr(v))
+        assert np.array_equal(v.view(np.uint32), tin[:, :, c].ravel().view(np.uint32)), (c, v, tin[:, :, c].ravel())
+
+
+@pytest.mark.parametrize("A", [4, 5])
+@pytest.mark.parametrize("kind", [ol.F32, ol.U8, ol.S8])
+@pytest.mark.parametrize("with_bias,with_relu", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("ends", ["full", "rows", "cols"])
+def test_wino_output_transform_bits_other_tiles(A, kind, with_bias, with_relu, ends):
+    M = A - 2
+    h_end, w_end = {"full": (M - 1, M - 1), "rows": (0, M - 1), "cols": (M - 1, M - 2)}[ends]
+    rng = np.random.default_rng(77 + h_end * 4 + w_end + A + kind)
+    oh = ow = 8
+    m = ol.aligned((A, A, 16), np.float32)
+    m[...] = rng.normal(0, 3, m.shape)
+    bias = ol.aligned(16, np.float32)
+    bias[...] = rng.normal(0, 1, 16)
+    np_kind = ol.NP_OF[kind]
+    fill = -777.0 if kind == ol.F32 else 93
+    out = ol.aligned((oh, ow, 16), np_kind, fill)
+    border = not (h_end == M - 1 and w_end == M - 1)
+    out_scale, out_z = 0.11, 3.0 if kind == ol.U8 else 0.0
+    rc = ref.ref_wino_trans_output_a(A, {ol.F32: 0, ol.U8: 1, ol.S8: 2}[kind], int(border), int(with_bias),
+                                     int(with_relu), oh, ow, ol.ptr(out), ol.ptr(m), ol.ptr(bias), h_end, w_end,
+                                     np.float32(1.0) / np.float32(out_scale), out_z)
+    assert rc == 0
+    y = np.zeros(M * M, np.float32)
+    for c in range(16):
+        mm = np.ascontiguousarray(m[:, :, c].ravel())
+        ol.oracle().orc_wino_tile_output_a(A, ol.ptr(mm), ol.ptr(y))
+        for i in range(M):
+            for j in range(M):
+                if i > h_end or j > w_end:
+                    assert out[i, j, c] == np_kind(fill)
+                    continue
+                r = ctypes.c_float()
+                q = ol.oracle().orc_wino_output_value_a(A, float(y[M * i + j]), int(with_bias), float(bias[c]), kind,
+                                                        out_scale, out_z, int(with_relu), ctypes.byref(r))
+                if kind == ol.F32:
+                    assert np.float32(r.value).view(np.uint32) == out[i, j, c].view(np.uint32), (i, j, c)
+                else:
+                    assert np_kind(q) == out[i, j, c], (i, j, c, q, out[i, j, c], r.value)
