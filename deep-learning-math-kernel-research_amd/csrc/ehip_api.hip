@@ -55,7 +55,7 @@ struct ehip_conv {
   // depthwise
   int T = 1, Tr = 1, wtb = 1;
   // Winograd
-  int ht = 0, wt = 0, nt = 0, t = 0;
+  int ht = 0, wt = 0, nt = 0, t = 0, wino_tile = 6;
   int chunk_n = 0;   // images per pass of the three-stage pipeline (intermediates sized for it)
   bool fused = true; // GEMM and output transform in one kernel (no f32 GEMM result in memory)
   uint8_t *tin = nullptr;
@@ -87,6 +87,15 @@ int dev_alloc(T **p, size_t count, bool zero)
   HIP_TRY(hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T)));
   if (zero) HIP_TRY(hipMemset(*p, 0, count * sizeof(T)));
   return EHIP_OK;
+}
+
+// tile_size 0: the reference's choice between 6 and 4 (src/eld_conv.cpp:231-236)
+int wino_auto_tile(const ehip_conv_desc_t &d)
+{
+  const int t = d.n * ((d.oh + 3) / 4) * ((d.ow + 3) / 4);
+  const int ocp = up(d.oc, 16);
+  const float mac_per_read = (float)((double)t * ocp) / (float)(t + ocp);
+  return mac_per_read > 25.0f ? 6 : 4;
 }
 
 // mirrors the dispatch of eld_conv_t::setup (src/eld_conv.cpp:148-313) for the int8 executors
@@ -223,13 +232,9 @@ int classify(ehip_conv *c)
       return fail(EHIP_UNIMPLEMENTED, "winograd: only the int8 implementation (execution_mode 0xa1xx) is built");
     if (out_q && (d.output_scale == kNoCali || d.output_z == kNoCali || d.output_scale == 0.0f))
       return fail(EHIP_GENERAL_ERROR, "output_quant is not set");
-    if (d.tile_size == 0) {
-      const int t = d.n * ((d.oh + 3) / 4) * ((d.ow + 3) / 4);
-      const int ocp = up(d.oc, 16);
-      const float mac_per_read = (float)((double)t * ocp) / (float)(t + ocp);
-      d.tile_size = mac_per_read > 25.0f ? 6 : 4;
-    }
-    if (d.tile_size != 6) return fail(EHIP_UNIMPLEMENTED, "winograd: only tile_size 6 (F(4x4,3x3)) is built");
+    if (d.tile_size == 0) d.tile_size = wino_auto_tile(d);
+    // src/eld_conv.cpp:257-270: the int8 executor exists for tile sizes 4, 5 and 6
+    if (d.tile_size < 4 || d.tile_size > 6) return fail(EHIP_UNIMPLEMENTED, "Unimplemented tile size");
     if (d.sampling_kind != 2) return fail(EHIP_UNIMPLEMENTED, "Winograd: to enable sampling from elk_u8s8_gemm");
     if (d.input_scale == kNoCali || d.input_z == kNoCali)
       return fail(EHIP_UNIMPLEMENTED, "winograd: input_quant must be set (FINE sampling is not built)");
@@ -339,9 +344,10 @@ int setup_workspace(ehip_conv *c)
   }
   case FAM_WINOGRAD: {
     c->taps = 1;
-    c->nbatch = 36;
-    c->ht = (d.oh + 3) / 4;
-    c->wt = (d.ow + 3) / 4;
+    c->wino_tile = d.tile_size;
+    c->nbatch = d.tile_size * d.tile_size;
+    c->ht = (d.oh + d.tile_size - 3) / (d.tile_size - 2);
+    c->wt = (d.ow + d.tile_size - 3) / (d.tile_size - 2);
     c->nt = c->ht * c->wt;
     // The three stages can run over a few images at a time (EHIP_WINO_CHUNK) with the intermediates
     // sized for one pass; measured on MI355X this only costs (the 256 MB memory-side cache does not
@@ -356,16 +362,18 @@ int setup_workspace(ehip_conv *c)
     }
     c->t = c->nt * c->chunk_n;   // tiles per pass
     if ((long long)c->t >= (1ll << 31) / 64) return fail(EHIP_UNIMPLEMENTED, "winograd: too many tiles");
-    c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, 36, 1);
+    c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, c->nbatch, 1);
     c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
     {
       const char *env = getenv("EHIP_WINO_FUSED");
-      c->fused = !(env && env[0] == '0');
+      // the fused GEMM + output transform is built for F(4x4,3x3); the other tile sizes run the
+      // three-kernel schedule
+      c->fused = !(env && env[0] == '0') && d.tile_size == 6;
     }
     c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
                               : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output";
-    c->tin_bytes = (size_t)36 * c->ic2 * c->t * 16;   // allocated with one pad unit behind it
-    c->tout_bytes = c->fused ? 16 : (size_t)36 * c->oc2 * c->t * 16 * sizeof(float);
+    c->tin_bytes = (size_t)c->nbatch * c->ic2 * c->t * 16;   // allocated with one pad unit behind it
+    c->tout_bytes = c->fused ? 16 : (size_t)c->nbatch * c->oc2 * c->t * 16 * sizeof(float);
     if ((rc = dev_alloc(&c->tin, c->tin_bytes + (size_t)c->t * 16, true)) != EHIP_OK) return rc;
     if ((rc = dev_alloc(reinterpret_cast<uint8_t **>(&c->tout), c->tout_bytes, false)) != EHIP_OK) return rc;
     break;
@@ -416,7 +424,8 @@ WinoArgs make_wino_args(const ehip_conv_desc_t &d, int ic2, int oc2)
   memset(&w, 0, sizeof(w));
   w.n = d.n; w.ic2 = ic2; w.oc2 = oc2;
   w.ih = d.ih; w.iw = d.iw; w.oh = d.oh; w.ow = d.ow;
-  w.ht = (d.oh + 3) / 4; w.wt = (d.ow + 3) / 4;
+  w.tile = d.tile_size == 0 ? wino_auto_tile(d) : d.tile_size;
+  w.ht = (d.oh + w.tile - 3) / (w.tile - 2); w.wt = (d.ow + w.tile - 3) / (w.tile - 2);
   w.nt = w.ht * w.wt; w.t = w.nt * d.n;
   w.pad_t = d.pad_t; w.pad_l = d.pad_l;
   w.with_bias = d.with_bias; w.with_relu = d.with_relu;
@@ -504,9 +513,9 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const vo
     break;
   case FAM_WINOGRAD: {
     float *u_tmp = nullptr;
-    const size_t n = (size_t)36 * up(d.oc, 16) * up(d.ic, 16);
+    const size_t n = (size_t)c->nbatch * up(d.oc, 16) * up(d.ic, 16);
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&u_tmp), n * sizeof(float)));
-    hipError_t e = launch_prepare_wino(w, d.oc, d.ic, c->units_pad, c->ocpp, d, u_tmp, c->wpacked, c->scale,
+    hipError_t e = launch_prepare_wino(w, d.oc, d.ic, c->wino_tile, c->units_pad, c->ocpp, d, u_tmp, c->wpacked, c->scale,
                                        c->shift, c->wsum, c->comp, s);
     hipError_t e2 = hipStreamSynchronize(s);
     (void)hipFree(u_tmp);
@@ -652,7 +661,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
       a.in_batch_stride = (long long)c->ic2 * w.t * 16;
       a.out_batch_stride = (long long)c->oc2 * w.t * 16;
-      HIP_TRY(launch_gemm(a, 36, c->variant, s));
+      HIP_TRY(launch_gemm(a, c->nbatch, c->variant, s));
       HIP_TRY(launch_wino_trans_output(w, s));
     }
     break;
@@ -769,6 +778,7 @@ EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *in
   if (d.kh != 3 || d.kw != 3 || d.stride_h != 1 || d.stride_w != 1 ||
       (d.input_type != EHIP_F32 && d.input_type != EHIP_U8) || d.input_fmt != EHIP_NCHW16C)
     return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 or u8 blocked 3x3 stride-1 layers only");
+  if (d.tile_size != 0 && (d.tile_size < 4 || d.tile_size > 6)) return fail(EHIP_UNIMPLEMENTED, "Unimplemented tile size");
   WinoArgs w = make_wino_args(d, up(d.ic, 16) / 16, up(d.oc, 16) / 16);
   w.in = input_dev;
   unsigned *mm = nullptr;

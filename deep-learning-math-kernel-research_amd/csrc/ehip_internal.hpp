@@ -101,6 +101,7 @@ struct WinoArgs {
   int in_u8, out_type;
   float out_repS, out_z;   // u8 / s8 output: 1 / output_S, ceil(output_z)
   int n, ic2, oc2, ih, iw, oh, ow, ht, wt, nt, t, pad_t, pad_l;
+  int tile;             // tile size A: 6 (or 0) = F(4x4,3x3), 4 = F(2x2,3x3), 5 = F(3x3,3x3); 36 below reads A * A
   int blocks_interior;  // set by the input-transform launcher: blocks over tiles off the rim
   float mrepS, mz;      // input_S / tinput_S, ceil(tinput_z)
   int with_bias, with_relu;
@@ -180,7 +181,7 @@ hipError_t launch_fold_direct_border(const int8_t *wpacked, const float *absmax,
                                      float *shift_tab, hipStream_t s);
 hipError_t launch_prepare_depthwise(const float *w_goihw, const float *bias, int g, const ehip_conv_desc_t &d,
                                     int8_t *wpacked, float *scale, float *shift, int *wsum, hipStream_t s);
-hipError_t launch_prepare_wino(const float *w_blocked, int oc, int ic, int units_pad, int ocpp,
+hipError_t launch_prepare_wino(const float *w_blocked, int oc, int ic, int tile, int units_pad, int ocpp,
                                const ehip_conv_desc_t &d, float *u_tmp, int8_t *wpacked, float *scale,
                                float *shift, int *wsum, int *comp, hipStream_t s);
 hipError_t launch_quantize_input(uint8_t *dst, const float *src, size_t count, float scale, float z,

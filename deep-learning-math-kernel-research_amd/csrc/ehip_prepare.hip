@@ -14,6 +14,7 @@
 // reference's compiled code.  Packed weights are laid out [tap][unit][oc][16 ic] so that one lane
 // of an MFMA A-operand is 16 contiguous bytes and a wave's operand load is one contiguous KiB.
 #include "ehip_internal.hpp"
+#include "ehip_wino_tiles.hpp"
 
 namespace ehip {
 
@@ -262,25 +263,8 @@ __global__ __launch_bounds__(kBlock) void k_prepare_depthwise(const float *w, co
 }
 
 // ---- Winograd weights --------------------------------------------------------------------------
-// 1-D stage of U = G g Gt as the reference's compiled kernel rounds it: z0*f2 feeds two adds and
-// fuses into both, z1*f0 and z2*f0 are rounded products.
-__device__ __forceinline__ void w_1d(float f0, float f1, float f2, float o[6])
-{
-  const float z0 = 0.26890756302521f, z1 = -0.688403361344538f, z2 = 0.119514472455649f,
-              z3 = 1.13777777777778f, z4 = 0.430252100840336f, z5 = 0.179271708683473f;
-  const float pq = z1 * f0;
-  const float qq = z2 * f0;
-  const float t1 = __builtin_fmaf(-z0, f2, pq);
-  const float t2 = __builtin_fmaf(z0, f2, qq);
-  o[0] = z3 * f0;
-  o[1] = __builtin_fmaf(-z4, f1, t1);
-  o[2] = __builtin_fmaf(z4, f1, t1);
-  o[3] = __builtin_fmaf(z5, f1, t2);
-  o[4] = __builtin_fmaf(-z5, f1, t2);
-  o[5] = f2;
-}
-
-// one thread per (oc, ic): U[pos][oc][ic] f32
+// U = G g Gt (tile arithmetic in ehip_wino_tiles.hpp); one thread per (oc, ic): U[pos][oc][ic] f32
+template <int A>
 __global__ __launch_bounds__(kBlock) void k_wino_weights_u(const float *w, int ocp, int icp, float *U)
 {
   const long long idx = (long long)blockIdx.x * kBlock + threadIdx.x;
@@ -290,30 +274,19 @@ __global__ __launch_bounds__(kBlock) void k_wino_weights_u(const float *w, int o
   float g[9];
 #pragma unroll
   for (int k = 0; k < 9; ++k) g[k] = src[(size_t)k * 256];
-  float M[6][3];
+  float u[A * A];
+  wino::tile_weights<A>(g, u);
 #pragma unroll
-  for (int i = 0; i < 3; ++i) {
-    float o[6];
-    w_1d(g[i], g[3 + i], g[6 + i], o);
-#pragma unroll
-    for (int k = 0; k < 6; ++k) M[k][i] = o[k];
-  }
-#pragma unroll
-  for (int i = 0; i < 6; ++i) {
-    float o[6];
-    w_1d(M[i][0], M[i][1], M[i][2], o);
-#pragma unroll
-    for (int j = 0; j < 6; ++j) U[((size_t)(6 * i + j) * ocp + oc) * icp + ic] = o[j];
-  }
+  for (int e = 0; e < A * A; ++e) U[((size_t)e * ocp + oc) * icp + ic] = u[e];
 }
 
 // one thread per (pos, oc): abs-max over ic, quantize, pack, fold
-__global__ __launch_bounds__(kBlock) void k_wino_quant(const float *U, int ocp, int icp, int units_pad, int ocpp,
+__global__ __launch_bounds__(kBlock) void k_wino_quant(const float *U, int npos, int ocp, int icp, int units_pad, int ocpp,
                                                        float tin_S, float tin_z, int8_t *wpacked, float *scale,
                                                        float *shift, int *wsum, int *comp)
 {
   const int idx = blockIdx.x * kBlock + threadIdx.x;
-  if (idx >= 36 * ocp) return;
+  if (idx >= npos * ocp) return;
   const int pos = idx / ocp, oc = idx - pos * ocp;
   const float *u = U + ((size_t)pos * ocp + oc) * icp;
   float am = 0.0f;
@@ -484,13 +457,16 @@ hipError_t launch_prepare_depthwise(const float *w, const float *bias, int g, co
   return hipGetLastError();
 }
 
-hipError_t launch_prepare_wino(const float *w, int oc, int ic, int units_pad, int ocpp, const ehip_conv_desc_t &d,
+// tile: the Winograd tile size A (4, 5 or 6); u_tmp holds A * A * ocp * icp floats
+hipError_t launch_prepare_wino(const float *w, int oc, int ic, int tile, int units_pad, int ocpp, const ehip_conv_desc_t &d,
                                float *u_tmp, int8_t *wpacked, float *scale, float *shift, int *wsum, int *comp,
                                hipStream_t s)
 {
   const int ocp = up(oc, 16), icp = up(ic, 16);
-  hipLaunchKernelGGL(k_wino_weights_u, grid_for((size_t)ocp * icp), dim3(kBlock), 0, s, w, ocp, icp, u_tmp);
-  hipLaunchKernelGGL(k_wino_quant, grid_for((size_t)36 * ocp), dim3(kBlock), 0, s, u_tmp, ocp, icp, units_pad, ocpp,
+  void (*kern)(const float *, int, int, float *) = tile == 4 ? k_wino_weights_u<4> : (tile == 5 ? k_wino_weights_u<5> : k_wino_weights_u<6>);
+  const int npos = tile == 4 ? 16 : (tile == 5 ? 25 : 36);
+  hipLaunchKernelGGL(kern, grid_for((size_t)ocp * icp), dim3(kBlock), 0, s, w, ocp, icp, u_tmp);
+  hipLaunchKernelGGL(k_wino_quant, grid_for((size_t)npos * ocp), dim3(kBlock), 0, s, u_tmp, npos, ocp, icp, units_pad, ocpp,
                      d.tinput_scale, ceilf(d.tinput_z), wpacked, scale, shift, wsum, comp);
   return hipGetLastError();
 }

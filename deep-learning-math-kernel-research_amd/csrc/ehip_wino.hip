@@ -1,4 +1,6 @@
-// Winograd F(4x4,3x3) transforms around the int8 GEMM: bandwidth kernels.
+// Winograd transforms around the int8 GEMM: bandwidth kernels.  Tile size A = 6 is F(4x4,3x3) (described
+// below), A = 4 F(2x2,3x3) and A = 5 F(3x3,3x3) are the same kernels with an A x A tile and an
+// (A-2) x (A-2) output tile (template parameter; tile arithmetic in ehip_wino_tiles.hpp).
 //
 //   trans_input : fp32 nChw16c -> gather 6x6 tiles (zero frame) -> V = Bt d B -> u8
 //                 replaces elx_conv_wino_trans_input_t<uint8_t,...>::__execute_blocked_nhwc
@@ -22,6 +24,7 @@
 // kernel, whose compiled form rounds the products of raw inputs in the column pass (and one
 // product of the last row pass) separately.
 #include "ehip_internal.hpp"
+#include "ehip_wino_tiles.hpp"
 
 #ifdef EHIP_TRACE
 #define TRACE_POINT(i)                                                                             \
@@ -35,65 +38,6 @@
 namespace ehip {
 
 namespace {
-
-__device__ __forceinline__ void in_1d(const float f[6], float o[6], bool raw_unfused, bool t4_unfused)
-{
-  const float z0 = -2.25f, z1 = -0.390625f, z2 = 0.87890625f, z3 = -2.640625f, z4 = 0.625f, z5 = 1.5f;
-  float t0, t1, t2, t3, t4, t5;
-  if (raw_unfused) {
-    t0 = f[2] * z0 + f[4];
-    t1 = f[1] * z0 + f[3];
-    t2 = f[2] * z1 + f[4];
-    t3 = f[1] * z1 + f[3];
-    t4 = f[0] * z2 + f[4];
-    t5 = f[1] * z2 + f[5];
-    o[0] = f[2] * z3 + t4;
-    o[5] = f[3] * z3 + t5;
-  } else {
-    t0 = __builtin_fmaf(f[2], z0, f[4]);
-    t1 = __builtin_fmaf(f[1], z0, f[3]);
-    t2 = __builtin_fmaf(f[2], z1, f[4]);
-    t3 = __builtin_fmaf(f[1], z1, f[3]);
-    t4 = t4_unfused ? f[0] * z2 + f[4] : __builtin_fmaf(f[0], z2, f[4]);
-    t5 = __builtin_fmaf(f[1], z2, f[5]);
-    o[0] = __builtin_fmaf(f[2], z3, t4);
-    o[5] = __builtin_fmaf(f[3], z3, t5);
-  }
-  o[1] = __builtin_fmaf(t1, z4, t0);
-  o[2] = __builtin_fmaf(-t1, z4, t0);
-  o[3] = __builtin_fmaf(t3, z5, t2);
-  o[4] = __builtin_fmaf(-t3, z5, t2);
-}
-
-// d, v: [6][6] row-major
-__device__ __forceinline__ void tile_input(const float d[36], float v[36], bool border)
-{
-  float m[36];
-#pragma unroll
-  for (int j = 0; j < 6; ++j) {
-    float f[6], o[6];
-#pragma unroll
-    for (int i = 0; i < 6; ++i) f[i] = d[6 * i + j];
-    in_1d(f, o, border, false);
-#pragma unroll
-    for (int i = 0; i < 6; ++i) m[6 * i + j] = o[i];
-  }
-#pragma unroll
-  for (int i = 0; i < 6; ++i) in_1d(&m[6 * i], &v[6 * i], false, border && i == 5);
-}
-
-__device__ __forceinline__ void out_1d(const float f[6], float o[4])
-{
-  const float z0 = 1.5f, z1 = 2.25f, z2 = 3.375f, z3 = 0.625f, z4 = 0.390625f, z5 = 0.244140625f;
-  const float t0 = f[1] + f[2];
-  const float t1 = f[3] + f[4];
-  const float t2 = f[1] - f[2];
-  const float t3 = f[3] - f[4];
-  o[0] = t0 + t1 + f[0];
-  o[1] = __builtin_fmaf(t2, z3, t3 * z0);
-  o[2] = __builtin_fmaf(t0, z4, t1 * z1);
-  o[3] = __builtin_fmaf(t2, z5, t3 * z2) + f[5];
-}
 
 __device__ __forceinline__ float comp_of(const float4 &v, int k)
 {
@@ -118,6 +62,7 @@ struct TileCoord {
   int n, th, tw, h0, w0;
   bool border;
 };
+template <int A>
 __device__ __forceinline__ TileCoord tile_coord(const WinoArgs &a, int t)
 {
   TileCoord c;
@@ -125,36 +70,38 @@ __device__ __forceinline__ TileCoord tile_coord(const WinoArgs &a, int t)
   const int rem = t - c.n * a.nt;
   c.th = rem / a.wt;
   c.tw = rem - c.th * a.wt;
-  c.h0 = 4 * c.th - a.pad_t;
-  c.w0 = 4 * c.tw - a.pad_l;
-  c.border = c.h0 < 0 || c.w0 < 0 || c.h0 + 5 >= a.ih || c.w0 + 5 >= a.iw;
+  c.h0 = (A - 2) * c.th - a.pad_t;
+  c.w0 = (A - 2) * c.tw - a.pad_l;
+  c.border = c.h0 < 0 || c.w0 < 0 || c.h0 + A - 1 >= a.ih || c.w0 + A - 1 >= a.iw;
   return c;
 }
 
-// the lane's four channels of the 36 pixels of a tile: float4 (f32 input) or 4 packed codes (u8)
-__device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, float4 d[36])
+// the lane's four channels of the A x A pixels of a tile: float4 (f32 input) or 4 packed codes (u8)
+template <int A>
+__device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, float4 *d)
 {
   const float4 *plane = reinterpret_cast<const float4 *>(a.in) +
       ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4 + q;
 #pragma unroll
-  for (int i = 0; i < 6; ++i)
+  for (int i = 0; i < A; ++i)
 #pragma unroll
-    for (int j = 0; j < 6; ++j) {
+    for (int j = 0; j < A; ++j) {
       const int h = c.h0 + i, w = c.w0 + j;
-      d[6 * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4]
+      d[A * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4]
                                                                    : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
-__device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, unsigned d[36])
+template <int A>
+__device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, unsigned *d)
 {
   const unsigned *plane = reinterpret_cast<const unsigned *>(a.in) +
       ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4 + q;
 #pragma unroll
-  for (int i = 0; i < 6; ++i)
+  for (int i = 0; i < A; ++i)
 #pragma unroll
-    for (int j = 0; j < 6; ++j) {
+    for (int j = 0; j < A; ++j) {
       const int h = c.h0 + i, w = c.w0 + j;
-      d[6 * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4] : 0u;   // the frame is 0.0f
+      d[A * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4] : 0u;   // the frame is 0.0f
     }
 }
 
@@ -169,12 +116,13 @@ constexpr bool kSplitRim = false;
 // that holds both kinds would execute both.  So the grid is split: the first a.blocks_interior
 // blocks enumerate only tiles away from the rim of the tile grid (never border), the remaining
 // blocks enumerate the rim.  Returns false past the end of the group.
+template <int A>
 __device__ __forceinline__ bool grouped_tile(const WinoArgs &a, int block, int slot, TileCoord &c, int &t)
 {
   if (!kSplitRim) {
     t = block * 64 + slot;
     if (t >= a.t) return false;
-    c = tile_coord(a, t);
+    c = tile_coord<A>(a, t);
     return true;
   }
   const int wi = a.wt - 2, hi = a.ht - 2;
@@ -208,36 +156,37 @@ __device__ __forceinline__ bool grouped_tile(const WinoArgs &a, int block, int s
   }
   t = n * a.nt + th * a.wt + tw;
   c.n = n; c.th = th; c.tw = tw;
-  c.h0 = 4 * th - a.pad_t;
-  c.w0 = 4 * tw - a.pad_l;
-  c.border = c.h0 < 0 || c.w0 < 0 || c.h0 + 5 >= a.ih || c.w0 + 5 >= a.iw;
+  c.h0 = (A - 2) * th - a.pad_t;
+  c.w0 = (A - 2) * tw - a.pad_l;
+  c.border = c.h0 < 0 || c.w0 < 0 || c.h0 + A - 1 >= a.ih || c.w0 + A - 1 >= a.iw;
   return true;
 }
 
 // grid: (interior blocks + rim blocks, ic2); block: 64 tiles x 4 channel quads.
 // Cell = float4 (f32 user input) or unsigned (u8 user input: four codes per lane and pixel).
-template <typename Cell>
+template <typename Cell, int A = 6>
 __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
 {
+  constexpr int AA = A * A;
   const int q = threadIdx.x & 3;
   const int c2 = blockIdx.y;
   TileCoord c;
   int t;
-  if (!grouped_tile(a, blockIdx.x, threadIdx.x >> 2, c, t)) return;
-  Cell d[36];
-  gather_tile(a, c, c2, q, d);
-  unsigned packed[36];
+  if (!grouped_tile<A>(a, blockIdx.x, threadIdx.x >> 2, c, t)) return;
+  Cell d[AA];
+  gather_tile<A>(a, c, c2, q, d);
+  unsigned packed[AA];
 #pragma unroll
-  for (int k = 0; k < 36; ++k) packed[k] = 0u;
+  for (int k = 0; k < AA; ++k) packed[k] = 0u;
   auto channels = [&](bool border) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      float f[36], v[36];
+      float f[AA], v[AA];
 #pragma unroll
-      for (int e = 0; e < 36; ++e) f[e] = comp_of(d[e], k);
-      tile_input(f, v, border);
+      for (int e = 0; e < AA; ++e) f[e] = comp_of(d[e], k);
+      wino::tile_input<A>(f, v, border);
 #pragma unroll
-      for (int e = 0; e < 36; ++e) {
+      for (int e = 0; e < AA; ++e) {
         // sat_u8(rne_to_u32(V * (in_S / tin_S) + tin_z)), one rounding in the multiply-add.  The
         // reference's float -> u32 conversion turns everything below -0.5 (and NaN) into 0xffffffff,
         // which then saturates to 255; v_cvt_pk_u8_f32 rounds to nearest even and saturates the rest.
@@ -255,31 +204,32 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   unsigned *dst = reinterpret_cast<unsigned *>(a.tin) + ((size_t)c2 * a.t + t) * 4 + q;
   const size_t pos_stride = (size_t)a.ic2 * a.t * 4;
 #pragma unroll
-  for (int e = 0; e < 36; ++e) dst[e * pos_stride] = packed[e];
+  for (int e = 0; e < AA; ++e) dst[e * pos_stride] = packed[e];
 }
 
 // minmax_dev[0] = ordered-min, [1] = ordered-max (see f2ord); real channels only
-template <typename Cell>
+template <typename Cell, int A = 6>
 __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic_real, unsigned *minmax_dev)
 {
+  constexpr int AA = A * A;
   const int q = threadIdx.x & 3;
   const int t = blockIdx.x * 64 + (threadIdx.x >> 2);
   const int c2 = blockIdx.y;
   float mn = 3.4e38f, mx = -3.4e38f;
   if (t < a.t) {
-    const TileCoord c = tile_coord(a, t);
-    Cell d[36];
-    gather_tile(a, c, c2, q, d);
+    const TileCoord c = tile_coord<A>(a, t);
+    Cell d[AA];
+    gather_tile<A>(a, c, c2, q, d);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       if (c2 * 16 + 4 * q + k >= ic_real) continue;
-      float f[36], v[36];
+      float f[AA], v[AA];
 #pragma unroll
-      for (int e = 0; e < 36; ++e) f[e] = comp_of(d[e], k);
-      if (c.border) tile_input(f, v, true);
-      else tile_input(f, v, false);
+      for (int e = 0; e < AA; ++e) f[e] = comp_of(d[e], k);
+      if (c.border) wino::tile_input<A>(f, v, true);
+      else wino::tile_input<A>(f, v, false);
 #pragma unroll
-      for (int e = 0; e < 36; ++e) {
+      for (int e = 0; e < AA; ++e) {
         mn = v[e] < mn ? v[e] : mn;
         mx = v[e] > mx ? v[e] : mx;
       }
@@ -303,47 +253,39 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
 // value * (1 / out_S) + out_z in one rounding BEFORE the ReLU, then round to nearest even and
 // saturate; the u8 store converts through an unsigned integer, so anything below -0.5 (and NaN)
 // ends as 255.  Border tiles write their valid rows and columns only.
-template <int OUT>
-__device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 &bias, bool with_bias, bool with_relu,
+// The F(2x2,3x3) kernel converts toward minus infinity in its u8 / s8 store
+// (src/kernel/elk_conv_wino_2x2_3x3_output.hxx:142-151), the others to nearest even.
+template <int OUT, int A = 6>
+__device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias, bool with_bias, bool with_relu,
                                             float repS, float z, void *plane, int q, int th, int tw, int oh_n, int ow_n)
 {
-  float y[4][16];
+  constexpr int AA = A * A, M = A - 2;
+  float y[4][M * M];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    float M[4][6];
+    float f[AA], o[M * M];
 #pragma unroll
-    for (int i = 0; i < 6; ++i) {
-      float f[6], o[4];
-#pragma unroll
-      for (int r = 0; r < 6; ++r) f[r] = comp_of(m[6 * r + i], k);
-      out_1d(f, o);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) M[r][i] = o[r];
-    }
+    for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
+    wino::tile_output<A>(f, o);
     const float b = comp_of(bias, k);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float o[4];
-      out_1d(M[i], o);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float r = o[j];
-        if (with_bias) r = r + b;
-        if (OUT != EHIP_F32) r = __builtin_fmaf(r, repS, z);
-        if (with_relu) r = r > 0.0f ? r : 0.0f;
-        y[k][4 * i + j] = r;
-      }
+    for (int e = 0; e < M * M; ++e) {
+      float r = o[e];
+      if (with_bias) r = r + b;
+      if (OUT != EHIP_F32) r = __builtin_fmaf(r, repS, z);
+      if (with_relu) r = r > 0.0f ? r : 0.0f;
+      y[k][e] = r;
     }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int oh = 4 * th + i;
+  for (int i = 0; i < M; ++i) {
+    const int oh = M * th + i;
     if (oh >= oh_n) break;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int ow = 4 * tw + j;
+    for (int j = 0; j < M; ++j) {
+      const int ow = M * tw + j;
       if (ow >= ow_n) break;
-      const int e = 4 * i + j;
+      const int e = M * i + j;
       const size_t cell = ((size_t)oh * ow_n + ow) * 16 + 4 * q;   // element index inside the plane
       if (OUT == EHIP_F32) {
         *reinterpret_cast<float4 *>(static_cast<float *>(plane) + cell) = make_float4(y[0][e], y[1][e], y[2][e], y[3][e]);
@@ -352,8 +294,15 @@ __device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const float r = y[k][e];
-          if (OUT == EHIP_U8) o = __builtin_amdgcn_cvt_pk_u8_f32(r >= -0.5f ? r : 300.0f, k, o);
-          else o |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
+          if (A == 4) {
+            // floor; u8 through an unsigned integer: negative values and NaN end as 255
+            const float fl = __builtin_floorf(r);
+            if (OUT == EHIP_U8) o = __builtin_amdgcn_cvt_pk_u8_f32(r >= 0.0f ? fl : 300.0f, k, o);
+            else o |= ((unsigned)ssat8(cvt_s32_rne(fl)) & 0xffu) << (8 * k);
+          } else {
+            if (OUT == EHIP_U8) o = __builtin_amdgcn_cvt_pk_u8_f32(r >= -0.5f ? r : 300.0f, k, o);
+            else o |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
+          }
         }
         *reinterpret_cast<unsigned *>(static_cast<uint8_t *>(plane) + cell) = o;
       }
@@ -362,9 +311,10 @@ __device__ __forceinline__ void output_tile(const float4 (&m)[36], const float4 
 }
 
 // grid: (ceil(t / 64), oc2); block: 64 tiles x 4 channel quads
-template <int OUT>
+template <int OUT, int A = 6>
 __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 {
+  constexpr int AA = A * A;
   const int q = threadIdx.x & 3;
   const int t = blockIdx.x * 64 + (threadIdx.x >> 2);
   const int o2 = blockIdx.y;
@@ -376,16 +326,16 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 
   const float4 *src = reinterpret_cast<const float4 *>(a.tout) + ((size_t)o2 * a.t + t) * 4 + q;
   const size_t pos_stride = (size_t)a.oc2 * a.t * 4;
-  float4 m[36];
+  float4 m[AA];
 #pragma unroll
-  for (int e = 0; e < 36; ++e) m[e] = src[e * pos_stride];
+  for (int e = 0; e < AA; ++e) m[e] = src[e * pos_stride];
 
   float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
   if (a.with_bias) bias = reinterpret_cast<const float4 *>(a.bias)[o2 * 4 + q];
   const size_t plane = ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 16;
   void *dst = OUT == EHIP_F32 ? static_cast<void *>(static_cast<float *>(a.out) + plane)
                               : static_cast<void *>(static_cast<uint8_t *>(a.out) + plane);
-  output_tile<OUT>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z, dst, q, th, tw, a.oh, a.ow);
+  output_tile<OUT, A>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z, dst, q, th, tw, a.oh, a.ow);
 }
 
 // ---- the 36 GEMMs and the output transform in one kernel ----------------------------------------
@@ -579,17 +529,26 @@ hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s)
     blocks_rim = (a.t + 63) / 64;
   }
   dim3 grid(a.blocks_interior + blocks_rim, a.ic2);
-  if (a.in_u8) hipLaunchKernelGGL(k_wino_trans_input_u8<unsigned>, grid, dim3(kBlock), 0, s, a);
-  else hipLaunchKernelGGL(k_wino_trans_input_u8<float4>, grid, dim3(kBlock), 0, s, a);
+  void (*kern)(WinoArgs) = nullptr;
+  if (a.tile == 4) kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 4> : k_wino_trans_input_u8<float4, 4>;
+  else if (a.tile == 5) kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 5> : k_wino_trans_input_u8<float4, 5>;
+  else kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 6> : k_wino_trans_input_u8<float4, 6>;
+  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
 
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s)
 {
   dim3 grid((a.t + 63) / 64, a.oc2);
-  if (a.out_type == EHIP_U8) hipLaunchKernelGGL(k_wino_trans_output<EHIP_U8>, grid, dim3(kBlock), 0, s, a);
-  else if (a.out_type == EHIP_S8) hipLaunchKernelGGL(k_wino_trans_output<EHIP_S8>, grid, dim3(kBlock), 0, s, a);
-  else hipLaunchKernelGGL(k_wino_trans_output<EHIP_F32>, grid, dim3(kBlock), 0, s, a);
+  void (*kern)(WinoArgs) = nullptr;
+#define EHIP_WO(A)                                                                                         \
+  kern = a.out_type == EHIP_U8 ? k_wino_trans_output<EHIP_U8, A>                                           \
+      : (a.out_type == EHIP_S8 ? k_wino_trans_output<EHIP_S8, A> : k_wino_trans_output<EHIP_F32, A>)
+  if (a.tile == 4) EHIP_WO(4);
+  else if (a.tile == 5) EHIP_WO(5);
+  else EHIP_WO(6);
+#undef EHIP_WO
+  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();
 }
 
@@ -616,8 +575,11 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s)
 hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_dev, hipStream_t s)
 {
   dim3 grid((a.t + 63) / 64, a.ic2);
-  if (a.in_u8) hipLaunchKernelGGL(k_wino_tinput_range<unsigned>, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
-  else hipLaunchKernelGGL(k_wino_tinput_range<float4>, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
+  void (*kern)(WinoArgs, int, unsigned *) = nullptr;
+  if (a.tile == 4) kern = a.in_u8 ? k_wino_tinput_range<unsigned, 4> : k_wino_tinput_range<float4, 4>;
+  else if (a.tile == 5) kern = a.in_u8 ? k_wino_tinput_range<unsigned, 5> : k_wino_tinput_range<float4, 5>;
+  else kern = a.in_u8 ? k_wino_tinput_range<unsigned, 6> : k_wino_tinput_range<float4, 6>;
+  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
   return hipGetLastError();
 }
 

@@ -180,6 +180,13 @@ int eld_conv_t::setup(bool fully_setup)
   d.sum_scale = sum_quant.scale; d.sum_z = sum_quant.z;
   d.relu_lower = relu_bound.lower; d.relu_upper = relu_bound.upper;
   if (with_op_sum || with_argmax) return ELD_UNIMPLEMENTED;
+  if (algorithm == CONV_WINOGRAD && tile_size == 0) {
+    // the reference's choice between F(4x4,3x3) and F(2x2,3x3), written back like there (src/eld_conv.cpp:231-236)
+    const int t = dims.n * ((dims.oh + 3) / 4) * ((dims.ow + 3) / 4);
+    const int ocp = (dims.oc + 15) / 16 * 16;
+    const float mac_per_read = (float)((double)t * ocp) / (float)(t + ocp);
+    d.tile_size = tile_size = mac_per_read > 25.0f ? 6 : 4;
+  }
 
   ehip_conv_t *h = nullptr;
   const int rc = ehip_conv_create(&d, &h);
@@ -189,7 +196,6 @@ int eld_conv_t::setup(bool fully_setup)
   }
   xc = new elx_conv_t();
   xc->handle = h;
-  if (algorithm == CONV_WINOGRAD && tile_size == 0) tile_size = 6;
   return ELD_OK;
 }
 

@@ -84,7 +84,7 @@ struct EULER_API eld_conv_t {
 
   int prop_kind;
   int algorithm;
-  int tile_size;  // Winograd only: 6 = F(4x4,3x3)
+  int tile_size;  // Winograd only: 4 = F(2x2,3x3), 5 = F(3x3,3x3), 6 = F(4x4,3x3); 0 = chosen by setup()
 
   bool with_relu;
   bool with_bias;

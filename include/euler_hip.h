@@ -90,7 +90,7 @@ EHIP_API const char *ehip_last_error(void);
  *    aligned base address); nChw16c or nhwc output;
  *  - depthwise 3x3 (g == ic == oc, src/elx_int8_conv_direct_depthwise.cpp): stride 1 or 2, pads 0/1,
  *    u8/s8 output, weights goihw;
- *  - CONV_WINOGRAD tile_size 6 (src/elx_int8_conv_wino.cpp): f32 tensors with execution_mode 0xa1xx, or
+ *  - CONV_WINOGRAD tile_size 4, 5 or 6 (0: the reference's automatic choice; src/elx_int8_conv_wino.cpp, src/eld_conv.cpp:231-270): f32 tensors with execution_mode 0xa1xx, or
  *    u8 input with f32/u8/s8 output (U8F32F32F32 / U8F32U8F32 / U8F32S8F32, src/eld_conv.cpp:275-281);
  *    wino_tinput_quant must be set (calibrated sampling).
  * A non-zero input zero point with padding is accepted by the 3/5/7 direct kernels (the shift then

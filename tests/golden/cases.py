@@ -439,3 +439,125 @@ for _b, _r, _he, _we in ((1, 1, 3, 3), (1, 0, 1, 3), (0, 0, 3, 0), (1, 1, 2, 2))
     CASES["wino_output_b%d_r%d_h%d_w%d" % (_b, _r, _he, _we)] = (
         lambda b=_b, r=_r, he=_he, we=_we: wino_out_inputs(b, r, he, we, 77 + he * 4 + we), wino_out_reference,
         wino_out_oracle)
+
+
+# ---- the other Winograd tile sizes: A = 4 F(2x2,3x3) (src/kernel/elk_conv_wino_2x2_3x3_*.hxx) and
+# A = 5 F(3x3,3x3) (src/kernel/elk_conv_wino_3x3_3x3_*.hxx) -------------------------------------------
+def winoa_w_inputs(A, seed):
+    d = wino_w_inputs(seed)
+    d["A"] = np.int32(A)
+    return d
+
+
+def winoa_w_reference(d, ref):
+    A = int(d["A"])
+    tw = ol.aligned((A, A, 16, 16), np.float32)
+    w = _al(d["w"])
+    assert ref.ref_wino_trans_weights_a(A, ol.ptr(tw), ol.ptr(w)) == 0
+    return np.array(tw)
+
+
+def winoa_w_oracle(d):
+    A = int(d["A"])
+    out = np.zeros((A, A, 16, 16), np.float32)
+    u = np.zeros(A * A, np.float32)
+    for i in range(16):
+        for o in range(16):
+            g = np.ascontiguousarray(d["w"][:, :, i, o].ravel())
+            ol.oracle().orc_wino_tile_weights_a(A, ol.ptr(g), ol.ptr(u))
+            out[:, :, i, o] = u.reshape(A, A)
+    return out
+
+
+def winoa_in_inputs(A, h0, w0, seed):
+    d = wino_in_inputs(h0, w0, seed)
+    d["A"] = np.int32(A)
+    return d
+
+
+def _winoa_in_range(d):
+    A = int(d["A"])
+    h0, w0 = int(d["h0"]), int(d["w0"])
+    hs, he = max(0, -h0), min(A - 1, 11 - h0)
+    ws, we = max(0, -w0), min(A - 1, 11 - w0)
+    return A, h0, w0, hs, he, ws, we, not (hs == 0 and ws == 0 and he == A - 1 and we == A - 1)
+
+
+def winoa_in_reference(d, ref):
+    A, h0, w0, hs, he, ws, we, border = _winoa_in_range(d)
+    plane = _al(d["plane"])
+    tin = ol.aligned((A, A, 16), np.float32)
+    tile_ptr = ctypes.c_void_p(plane.ctypes.data + (h0 * 12 + w0) * 16 * 4)
+    assert ref.ref_wino_trans_input_a(A, int(border), 12, 12, ol.ptr(tin), tile_ptr, hs, he, ws, we) == 0
+    return np.array(tin)
+
+
+def winoa_in_oracle(d):
+    A, h0, w0, hs, he, ws, we, border = _winoa_in_range(d)
+    out = np.zeros((A, A, 16), np.float32)
+    v = np.zeros(A * A, np.float32)
+    for c in range(16):
+        t = np.zeros((A, A), np.float32)
+        for i in range(A):
+            for j in range(A):
+                h, w = h0 + i, w0 + j
+                if 0 <= h < 12 and 0 <= w < 12:
+                    t[i, j] = d["plane"][h, w, c]
+        ol.oracle().orc_wino_tile_input_a(A, int(border), ol.ptr(t), ol.ptr(v))
+        out[:, :, c] = v.reshape(A, A)
+    return out
+
+
+def winoa_out_inputs(A, kind, with_bias, with_relu, h_end, w_end, seed):
+    rng = np.random.default_rng(seed)
+    return dict(A=np.int32(A), kind=np.int32(kind), with_bias=np.int32(with_bias), with_relu=np.int32(with_relu),
+                h_end=np.int32(h_end), w_end=np.int32(w_end), m=rng.normal(0, 3, (A, A, 16)).astype(np.float32),
+                bias=rng.normal(0, 1, 16).astype(np.float32), out_scale=np.float32(0.0437),
+                out_z=np.float32(3.0 if kind == ol.U8 else 0.0))
+
+
+def winoa_out_reference(d, ref):
+    A, kind = int(d["A"]), int(d["kind"])
+    M = A - 2
+    fill = -777.0 if kind == ol.F32 else 99
+    out = ol.aligned((8, 8, 16), ol.NP_OF[kind], fill)
+    h_end, w_end = int(d["h_end"]), int(d["w_end"])
+    border = not (h_end == M - 1 and w_end == M - 1)
+    m, bias = _al(d["m"]), _al(d["bias"])
+    rep = np.float32(1.0) / d["out_scale"]
+    assert ref.ref_wino_trans_output_a(A, KIND_ID[kind], int(border), int(d["with_bias"]), int(d["with_relu"]), 8, 8,
+                                       ol.ptr(out), ol.ptr(m), ol.ptr(bias), h_end, w_end, float(rep),
+                                       float(np.ceil(d["out_z"]))) == 0
+    return np.array(out[:M, :M, :])
+
+
+def winoa_out_oracle(d):
+    A, kind = int(d["A"]), int(d["kind"])
+    M = A - 2
+    out = np.full((M, M, 16), -777.0 if kind == ol.F32 else 99, ol.NP_OF[kind])
+    y = np.zeros(M * M, np.float32)
+    for c in range(16):
+        mm = np.ascontiguousarray(d["m"][:, :, c].ravel())
+        ol.oracle().orc_wino_tile_output_a(A, ol.ptr(mm), ol.ptr(y))
+        for i in range(M):
+            for j in range(M):
+                if i > int(d["h_end"]) or j > int(d["w_end"]):
+                    continue
+                r = ctypes.c_float()
+                q = ol.oracle().orc_wino_output_value_a(A, float(y[M * i + j]), int(d["with_bias"]), float(d["bias"][c]), kind,
+                                                        float(d["out_scale"]), float(d["out_z"]), int(d["with_relu"]),
+                                                        ctypes.byref(r))
+                out[i, j, c] = r.value if kind == ol.F32 else np.array(q).astype(ol.NP_OF[kind])
+    return out
+
+
+for _A in (4, 5):
+    CASES["wino%d_weights" % _A] = (lambda A=_A: winoa_w_inputs(A, 21 + A), winoa_w_reference, winoa_w_oracle)
+    for _h0, _w0 in ((2, 2), (1, 3), (-1, -1), (-1, 4), (3, -1), (9, 9), (8, 2), (-1, 9)):
+        CASES["wino%d_input_h%d_w%d" % (_A, _h0, _w0)] = (
+            lambda A=_A, h=_h0, w=_w0: winoa_in_inputs(A, h, w, h * 13 + w + 50 + A), winoa_in_reference, winoa_in_oracle)
+    for _k, _kn in ((ol.F32, "f32"), (ol.U8, "u8"), (ol.S8, "s8")):
+        for _b, _r, _he, _we in ((1, 1, _A - 3, _A - 3), (1, 0, 0, _A - 3), (0, 0, _A - 3, _A - 4)):
+            CASES["wino%d_output_%s_b%d_r%d_h%d_w%d" % (_A, _kn, _b, _r, _he, _we)] = (
+                lambda A=_A, k=_k, b=_b, r=_r, he=_he, we=_we: winoa_out_inputs(A, k, b, r, he, we, 700 + 16 * k + 8 * b + he + we + A),
+                winoa_out_reference, winoa_out_oracle)

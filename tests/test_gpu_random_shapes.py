@@ -96,7 +96,7 @@ def test_random_depthwise(seed):
                           seed=seed, w_sigma=0.1, T=T))
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(16))
 def test_random_winograd(seed):
     import torch
     from gpu_common import bits, dev, host
@@ -107,11 +107,12 @@ def test_random_winograd(seed):
     u8_in = bool(r.integers(0, 2))
     out_type = [ol.F32, ol.U8, ol.S8][int(r.integers(0, 3))] if u8_in else ol.F32
     bias_on, relu_on = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+    tile = int(r.choice([6, 4, 5]))   # F(4x4,3x3), F(2x2,3x3), F(3x3,3x3)
     if u8_in:
-        E, p, d, x, wb, bias = make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=bias_on, with_relu=relu_on)
+        E, p, d, x, wb, bias = make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=bias_on, with_relu=relu_on, tile=tile)
         xf = x.astype(np.float32)
     else:
-        E, p, d, x, wb, bias = make_wino(n, ic, oc, hw, seed, with_bias=bias_on, with_relu=relu_on)
+        E, p, d, x, wb, bias = make_wino(n, ic, oc, hw, seed, with_bias=bias_on, with_relu=relu_on, tile=tile)
         xf = x
     p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
     d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def make_wino(n, ic, oc, hw, seed, with_bias=True, with_relu=True):
+def make_wino(n, ic, oc, hw, seed, with_bias=True, with_relu=True, tile=6):
     E = pkg()
     rng = np.random.default_rng(seed)
     x = rng.uniform(0, 1, (n, ic, hw, hw)).astype(f32)
@@ -20,18 +20,20 @@ def make_wino(n, ic, oc, hw, seed, with_bias=True, with_relu=True):
     bias[:oc] = rng.normal(0, 0.01, oc)
     xb, wb = ol.to_blocked(x), ol.weights_to_blocked(w)
     p = ol.make_params(n, ic, oc, hw, hw, 3, 3, 1, out_type=ol.F32, in_scale=1.0, with_bias=with_bias,
-                       with_relu=with_relu)
+                       with_relu=with_relu, wino_tile=tile)
     d = E.make_desc(n, ic, oc, hw, hw, 3, 3, 1, algorithm=E.CONV_WINOGRAD, input_type=E.F32, output_type=E.F32,
-                    with_bias=with_bias, with_relu=with_relu, input_quant=(1.0, 0.0), tile_size=6,
+                    with_bias=with_bias, with_relu=with_relu, input_quant=(1.0, 0.0), tile_size=tile,
                     execution_mode=0xa161, wino_tinput_quant=(1.0, 0.0))
     return E, p, d, xb, wb, bias
 
 
+@pytest.mark.parametrize("tile", [6, 4, 5])
 @pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 10), (1, 64, 48, 12), (3, 16, 80, 7), (1, 32, 32, 28)])
-def test_wino_pipeline(n, ic, oc, hw, monkeypatch):
+def test_wino_pipeline(n, ic, oc, hw, tile, monkeypatch):
+    """tile 6 = F(4x4,3x3), 4 = F(2x2,3x3), 5 = F(3x3,3x3) (src/eld_conv.cpp:257-270)"""
     import torch
     monkeypatch.setenv("EHIP_WINO_FUSED", "0")   # three kernels: every stage can be inspected
-    E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 100 + hw)
+    E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 100 + hw, tile=tile)
     d_x = dev(xb)
     # calibration of wino_tinput_quant from the fp32 transformed input
     mn, mx = E.wino_tinput_range(d, d_x)
@@ -89,7 +91,7 @@ def test_wino_fused_gemm_and_output_transform(n, ic, oc, hw):
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
-def make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=True, with_relu=True, out_scale=None, out_z=0.0):
+def make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=True, with_relu=True, out_scale=None, out_z=0.0, tile=6):
     """u8 user input (codes of U[0,1) at scale 1/255), f32 / u8 / s8 user output: the data-type
     configurations U8F32F32F32, U8F32U8F32, U8F32S8F32 of the reference (src/eld_conv.cpp:275-281)."""
     E = pkg()
@@ -103,9 +105,9 @@ def make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=True, with_relu=True, 
     if out_scale is None:
         out_scale = 4.0 * 0.02 * np.sqrt(9 * ic / 3.0) / (127.0 if out_type == ol.S8 else 255.0)
     p = ol.make_params(n, ic, oc, hw, hw, 3, 3, 1, out_type=out_type, in_scale=1.0 / 255.0, with_bias=with_bias,
-                       with_relu=with_relu, out_scale=out_scale, out_z=out_z)
+                       with_relu=with_relu, out_scale=out_scale, out_z=out_z, wino_tile=tile)
     d = E.make_desc(n, ic, oc, hw, hw, 3, 3, 1, algorithm=E.CONV_WINOGRAD, input_type=E.U8, output_type=out_type,
-                    with_bias=with_bias, with_relu=with_relu, input_quant=(1.0 / 255.0, 0.0), tile_size=6,
+                    with_bias=with_bias, with_relu=with_relu, input_quant=(1.0 / 255.0, 0.0), tile_size=tile,
                     execution_mode=0xa161, wino_tinput_quant=(1.0, 0.0), output_quant=(out_scale, out_z))
     return E, p, d, xq, wb, bias
 
@@ -182,4 +184,62 @@ def test_wino_no_bias_no_relu():
     d_out = torch.zeros(exp.shape, dtype=torch.float32, device="cuda")
     conv.execute(d_out, dev(xb), dev(wb), None)
     torch.cuda.synchronize()
+    assert np.array_equal(bits(host(d_out)), bits(exp))
+
+
+# ---- tile sizes 4 (F(2x2,3x3)) and 5 (F(3x3,3x3)) with u8 input and every user output type ------------
+@pytest.mark.parametrize("tile", [4, 5])
+@pytest.mark.parametrize("out_type", [ol.F32, ol.U8, ol.S8])
+@pytest.mark.parametrize("n,ic,oc,hw,with_relu", [(2, 32, 32, 10, True), (1, 64, 80, 13, True), (1, 48, 32, 7, False),
+                                                  (2, 16, 16, 4, True)])
+def test_wino_other_tiles_u8_input_quantized_output(tile, out_type, n, ic, oc, hw, with_relu):
+    """The F(2x2,3x3) store rounds toward minus infinity, the others to nearest even; without ReLU negative
+    values of a u8 output end as 255 (src/kernel/elk_conv_wino_2x2_3x3_output.hxx:142-151,
+    src/kernel/elk_conv_wino_3x3_3x3_output.hxx:74-86)."""
+    import torch
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=9 * n + hw + ic + out_type + tile, out_type=out_type,
+                                         with_relu=with_relu, out_z=0.0 if out_type == ol.S8 else 2.4, tile=tile)
+    d_x = dev(xq)
+    mn, mx = E.wino_tinput_range(d, d_x)
+    omn, omx = ol.wino_tinput_range(p, xq.astype(f32))
+    assert (f32(mn), f32(mx)) == (f32(omn), f32(omx))
+    diff = (f32(mx) - f32(mn)) * f32(1.0 / 255.0) + f32(0.000001)
+    s_t, z_t = float(diff / f32(255.0)), float(-f32(mn) * f32(1.0 / 255.0) * f32(255.0) / diff)
+    p.tin_scale, p.tin_z = s_t, z_t
+    d.tinput_scale, d.tinput_z = s_t, z_t
+    tin, exp = _oracle_u8(p, xq, wb, bias)
+    assert tin.shape[0] == tile * tile
+    conv = E.Conv(d)
+    assert conv.kernel_name.endswith("k_wino_trans_output")   # three-kernel schedule
+    tdt = {ol.F32: torch.float32, ol.U8: torch.uint8, ol.S8: torch.int8}[out_type]
+    d_out = torch.full(exp.shape, 5, dtype=tdt, device="cuda")
+    d_b = dev(bias)
+    conv.execute(d_out, d_x, dev(wb), d_b)
+    torch.cuda.synchronize()
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    assert np.array_equal(conv.query(E.Q_WEIGHTS_S8), twq.ravel()), "transformed weights differ"
+    assert np.array_equal(bits(conv.query(E.Q_SCALE)), bits(tscale))
+    g_tin = conv.query(E.Q_TINPUT_U8).reshape(tin.shape)
+    assert np.array_equal(g_tin, tin), "u8 transformed input differs at %d cells" % int((g_tin != tin).sum())
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
+def test_wino_automatic_tile_size():
+    """tile_size 0: the reference picks 6 or 4 from the layer's multiply-accumulates per byte read
+    (src/eld_conv.cpp:231-236); a small layer gets F(2x2,3x3)."""
+    import torch
+    E, p, d, xb, wb, bias = make_wino(1, 16, 16, 8, seed=3, tile=4)
+    d.tile_size = 0
+    p.tin_scale, p.tin_z = 6.0 / 255.0, 120.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xb), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias)
+    conv = E.Conv(d)
+    d_out = torch.zeros(exp.shape, dtype=torch.float32, device="cuda")
+    d_b = dev(bias)
+    conv.execute(d_out, dev(xb), dev(wb), d_b)
+    torch.cuda.synchronize()
+    assert conv.query(E.Q_WEIGHTS_S8).size == 16 * twq.shape[1] * twq.shape[2]
     assert np.array_equal(bits(host(d_out)), bits(exp))
