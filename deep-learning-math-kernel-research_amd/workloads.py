@@ -19,11 +19,12 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 class Workload:
     def __init__(self, key, title, n, ic, oc, hw, k=1, pad=0, stride=1, algorithm=CONV_DIRECT, in_type=U8,
                  out_type=U8, with_sum=False, depthwise=False, w_sigma=0.05, T=0, relu6=False, nhwc=False, oh=None, in_z=0.0, nhwc_out=False,
-                 nhwc_in=False):
+                 nhwc_in=False, tile=6):
         self.key, self.title = key, title
         self.n, self.ic, self.oc, self.hw, self.k, self.pad, self.stride = n, ic, oc, hw, k, pad, stride
         self.algorithm, self.in_type, self.out_type = algorithm, in_type, out_type
         self.with_sum, self.depthwise, self.w_sigma, self.T, self.relu6 = with_sum, depthwise, w_sigma, T, relu6
+        self.tile = tile   # Winograd tile size: 6 = F(4x4,3x3), 4 = F(2x2,3x3), 5 = F(3x3,3x3)
         self.in_z = in_z   # input zero point (the reference's "...z" data-type configurations)
         self.nhwc = nhwc   # activations [n][h][w][c] on both sides instead of nChw16c
         self.nhwc_in, self.nhwc_out = nhwc or nhwc_in, nhwc or nhwc_out
@@ -54,7 +55,7 @@ class Workload:
         if self.depthwise:
             w = up16(self.oc) * 9
         elif self.algorithm == CONV_WINOGRAD:
-            w = 36 * up16(self.ic) * up16(self.oc)
+            w = self.tile * self.tile * up16(self.ic) * up16(self.oc)
         else:
             w = up16(self.ic) * up16(self.oc) * self.k * self.k
         b = n_in * esz[self.in_type] + w + n_out * esz[self.out_type] + 8 * up16(self.oc)
@@ -85,7 +86,7 @@ class Workload:
                       input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, self.in_z),
                       output_quant=(out_scale, 0.0), sum_quant=(0.7, 0.0) if self.with_sum else (0.0, 0.0),
                       wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
-                      tile_size=6 if self.algorithm == CONV_WINOGRAD else 0,
+                      tile_size=self.tile if self.algorithm == CONV_WINOGRAD else 0,
                       execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
         if self.nhwc_in:
             d.input_fmt = NHWC
@@ -137,6 +138,10 @@ WORKLOADS = {w.key: w for w in [
              k=3, pad=1, algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02),
     Workload("C4b_i8", "Winograd F(4,3) 512->512 @28x28 N=64, u8 in / s8 out (VGG-16 conv4, U8F32S8F32)", 64, 512, 512, 28,
              k=3, pad=1, algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02),
+    Workload("C4b_i8_t4", "Winograd F(2,3) (tile size 4) 512->512 @28x28 N=64, u8 in / s8 out", 64, 512, 512, 28,
+             k=3, pad=1, algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02, tile=4),
+    Workload("C4b_i8_t5", "Winograd F(3,3) (tile size 5) 512->512 @28x28 N=64, u8 in / s8 out", 64, 512, 512, 28,
+             k=3, pad=1, algorithm=CONV_WINOGRAD, in_type=U8, out_type=S8, w_sigma=0.02, tile=5),
     Workload("C5a", "depthwise 3x3 C=144 @56x56 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 144, 144, 56, k=3, pad=1,
              depthwise=True, w_sigma=0.1, T=14, relu6=True),
     Workload("C5b", "depthwise 3x3 C=960 @7x7 N=64, bias+ReLU6, u8 out (MobileNet-v2)", 64, 960, 960, 7, k=3, pad=1,

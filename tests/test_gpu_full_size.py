@@ -74,12 +74,12 @@ def test_configured_winograd_layer(key, check_images):
     assert float(got.max()) > 0.0
 
 
-@pytest.mark.parametrize("key,check_images", [("C4a_i8", 2), ("C4b_i8", 4)])
+@pytest.mark.parametrize("key,check_images", [("C4a_i8", 2), ("C4b_i8", 4), ("C4b_i8_t4", 2), ("C4b_i8_t5", 2)])
 def test_configured_winograd_layer_u8_in_s8_out(key, check_images):
     """The VGG layers as the reference's tuned int8 run feeds them (u8 input, s8 output)."""
     import torch
     wl = W.WORKLOADS[key]
-    E, p, d, xq, wb, bias = make_wino_u8(wl.n, wl.ic, wl.oc, wl.hw, seed=91 + wl.hw, out_type=ol.S8)
+    E, p, d, xq, wb, bias = make_wino_u8(wl.n, wl.ic, wl.oc, wl.hw, seed=91 + wl.hw, out_type=ol.S8, tile=wl.tile)
     s_t, z_t = 22.0 / 255.0, 104.0
     d.tinput_scale, d.tinput_z = s_t, z_t
     conv = E.Conv(d)
@@ -91,7 +91,7 @@ def test_configured_winograd_layer_u8_in_s8_out(key, check_images):
     got = host(d_out)
     k = check_images
     pk = ol.make_params(k, wl.ic, wl.oc, wl.hw, wl.hw, 3, 3, 1, out_type=ol.S8, in_scale=1.0 / 255.0, with_bias=True,
-                        with_relu=True, out_scale=p.out_scale, out_z=p.out_z)
+                        with_relu=True, out_scale=p.out_scale, out_z=p.out_z, wino_tile=wl.tile)
     pk.tin_scale, pk.tin_z = s_t, z_t
     twq, tscale, tshift = ol.wino_prepare(pk, wb)
     tin = ol.wino_trans_input(pk, np.ascontiguousarray(xq[:k]).astype(np.float32))
