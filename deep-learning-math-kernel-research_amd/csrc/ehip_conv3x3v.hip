@@ -23,6 +23,8 @@
 // weight operands (9 taps x TM) live in registers and every slot is refilled with the next channel
 // pair's operand right after its last use, i.e. nine taps ahead; pixel operands come from LDS one
 // tap ahead.  Two workgroups share a CU.
+#include <type_traits>
+
 #include "ehip_internal.hpp"
 
 // Development aid (compile with -DEHIP_TRACE): lane 0 of every wave records the shader clock at
@@ -124,14 +126,40 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
     }
   };
 
-  v16i acc[TM][TN];
+  // The first fill: nothing else is live yet, so the loads of ALL passes travel together, up to 16
+  // per thread -- a workgroup's staging time is the number of round trips, not the number of cells
+  // (a 3-pass tile of a 224-wide image: three trips before, one now).
+  auto stage_first = [&](auto kb) {
+    constexpr int KB = decltype(kb)::value;   // units per thread and round trip
+    for (int k0 = 0; k0 < nk; k0 += KB) {
+      v4i t[NPASS][KB];
 #pragma unroll
-  for (int mt = 0; mt < TM; ++mt)
+      for (int p = 0; p < NPASS; ++p)
 #pragma unroll
-    for (int nt = 0; nt < TN; ++nt)
+        for (int j = 0; j < KB; ++j) {
+          const int k = k0 + j < nk ? k0 + j : nk - 1;
+          int u = ug + G * k;
+          u = u < a.ic2 ? u : a.ic2 - 1;   // padded units multiply zero weights
+          t[p][j] = *reinterpret_cast<const v4i *>(inb + (long long)u * plane + goff[p]);
+        }
+      if (k0 == 0) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
+        for (int tap = 0; tap < 9; ++tap) load_a(tap, 0);
+      }
+#pragma unroll
+      for (int p = 0; p < NPASS; ++p)
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+          if (k0 + j < nk) {
+            const v4i x = t[p][j] ^ (int)0x80808080;
+            const v4i z = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+            lds[(ug + G * (k0 + j)) * STRIDE + tid % CT + p * CT] = gin[p] ? x : z;
+          }
+        }
+    }
+  };
 
+  v16i acc[TM][TN];
   // one channel pair (32 input channels) x nine taps; `last` = nothing left to prefetch
   auto pair_taps = [&](int pl, int pair, bool last) {
     const v4i *tile = lds + (2 * pl + lh) * STRIDE + pw0 + l32;
@@ -161,7 +189,18 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   const int nchunks = a.units_pad / a.chunk_units;
   const long long cidx = oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
   OcConsts k0;
-  stage(0, true);
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
+  // as few loads per trip as cover the fill (unused slots repeat the last unit's load), at most 16
+  constexpr int KBMAX = NPASS == 1 ? 16 : (NPASS == 2 ? 8 : 4);
+  if (nk <= 2) stage_first(std::integral_constant<int, 2>());
+  else if (nk <= 4 || KBMAX == 4) stage_first(std::integral_constant<int, 4>());
+  else if (nk <= 8 || KBMAX == 8) stage_first(std::integral_constant<int, (KBMAX < 8 ? KBMAX : 8)>());
+  else stage_first(std::integral_constant<int, KBMAX>());
   TRACE_POINT(2);
   __syncthreads();
   TRACE_POINT(3);
