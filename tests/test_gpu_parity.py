@@ -225,6 +225,19 @@ def test_direct_few_input_channels_strip_heights(rows, monkeypatch):
     run_and_compare(Layer(2, 3, 32, 13, k=3, pad=1, stride=1, out_type=ol.U8, seed=195 + rows, in_nhwc=True))
 
 
+def test_direct_few_input_channels_rows_too_wide_for_lds():
+    """7 staged rows of a 3000-pixel image do not fit the first-layer kernel's LDS: blocked input takes the
+    general k x k form, compact nhwc input is refused (nothing else reads that layout)."""
+    E = pkg()
+    d = E.make_desc(1, 3, 16, 8, 3000, 7, 7, 3, algorithm=E.CONV_DIRECT, output_type=E.U8, output_quant=(0.05, 0.0),
+                    input_quant=(1.0 / 255.0, 128.0))
+    conv = E.Conv(d)
+    assert conv.kernel_name.startswith("k_gemm_u8s8")
+    d.input_fmt = E.NHWC
+    with pytest.raises(E.EulerHipError):
+        E.Conv(d)
+
+
 @pytest.mark.parametrize("variant", range(7))
 def test_direct_3x3_stride2_every_kernel_variant(variant, monkeypatch):
     monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
