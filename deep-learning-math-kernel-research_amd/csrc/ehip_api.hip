@@ -132,11 +132,11 @@ int classify(ehip_conv *c)
     const bool in_ok = d.input_fmt == EHIP_NCHW16C || d.input_fmt == EHIP_NHWC;
     const bool out_ok = d.output_fmt == EHIP_NCHW16C || d.output_fmt == EHIP_NHWC;
     if (!in_ok || !out_ok) return fail(EHIP_UNIMPLEMENTED, "activation formats: nChw16c or nhwc");
-    // nhwc input: 1x1, and kh x kw over at most four channels (the first layer of an image network,
-    // whose nhwc input is compact: ic bytes per pixel); nhwc output: 1x1 and kh x kw direct
+    // nhwc on either side of the 1x1 and kh x kw direct executors; with at most four channels (the
+    // first layer of an image network) the nhwc input is compact: ic bytes per pixel
     const bool fewch = d.algorithm == EHIP_CONV_DIRECT && !depthwise && conv_fewch_applies(d.ic, d.kh, d.kw);
-    if (d.input_fmt == EHIP_NHWC && !(d.kh == 1 && d.kw == 1 && !depthwise) && !fewch)
-      return fail(EHIP_UNIMPLEMENTED, "nhwc input is only built for 1x1 convolutions and for kh x kw over at most 4 channels");
+    if (d.input_fmt == EHIP_NHWC && depthwise)
+      return fail(EHIP_UNIMPLEMENTED, "nhwc input is not built for depthwise convolutions");
     if (d.output_fmt == EHIP_NHWC && (depthwise || d.algorithm == EHIP_CONV_WINOGRAD))
       return fail(EHIP_UNIMPLEMENTED, "nhwc output is only built for the direct 1x1 and kh x kw executors");
     if ((d.input_fmt == EHIP_NHWC && d.ic % 16 && !fewch) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
@@ -208,7 +208,8 @@ int classify(ehip_conv *c)
           d.ow == d.iw + d.pad_l + d.pad_r - 2 && d.oh == d.ih + d.pad_t + d.pad_b - 2;
       // the GEMM family walks [tap][unit] for kh x kw; it also owns the per-pixel shift that a zero
       // point with padding needs
-      c->family = (s1_3x3 && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC) ? FAM_CONV_3X3 : FAM_GEMM_1X1;
+      c->family = (s1_3x3 && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC && d.input_fmt != EHIP_NHWC)
+          ? FAM_CONV_3X3 : FAM_GEMM_1X1;
       {
         // at most four input channels: several pixels per operand cell, weights in registers
         const char *env = getenv("EHIP_FEWCH");

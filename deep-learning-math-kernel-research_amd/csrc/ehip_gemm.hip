@@ -44,7 +44,7 @@ namespace ehip {
 template <int WM, int WN, int TM, int TN, int KC, int D, bool NHWC, int CONV>
 __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 {
-  static_assert(!(NHWC && CONV), "the kh x kw form is built for blocked input only");
+  static_assert(!(NHWC && CONV == 1), "nhwc kh x kw input works the tap out per cell");
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
   constexpr int KS = KC / 2;               // MFMA k-steps per fill
@@ -88,9 +88,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   // Byte offset of output pixel gp's first input cell (unit 0); nhwc: the pixel's channel vector.
   // kh x kw form (CONV): the cell under tap (0, 0), which may lie outside the image, and the set of
   // taps that fall inside it.
-  unsigned long long tapmask = 0;
   long long safe_off = 0;   // a cell of the same image that every unit offset keeps in bounds
-  auto input_pixel = [&](int gp) -> long long {
+  auto input_pixel = [&](int gp, unsigned long long &tapmask) -> long long {
     gp = gp < a.p_total ? gp : a.p_total - 1;
     const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic);
     const int r = gp - n * a.ohw;
@@ -103,6 +102,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
       const int ih0 = oh * a.stride_h - (CONV ? a.pad_t : 0), iw0 = ow * a.stride_w - (CONV ? a.pad_l : 0);
       sp = (long long)ih0 * a.iw + iw0;
       if (CONV) {
+        tapmask = 0;
         for (int kh = 0; kh < a.kh; ++kh)
           for (int kw = 0; kw < a.kw; ++kw)
             if (ih0 + kh >= 0 && ih0 + kh < a.ih && iw0 + kw >= 0 && iw0 + kw < a.iw) tapmask |= 1ull << (kh * a.kw + kw);
@@ -116,9 +116,15 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   // id / KC, unit id % KC (a pixel's units are contiguous: KC lanes read 16 * KC consecutive bytes).
   constexpr int NPIX = NHWC ? NB : 1;
   const uint8_t *inb[NPIX];
+  unsigned long long tapmask[NPIX];   // CONV: the taps of the thread's pixel(s) that fall inside the image
 #pragma unroll
-  for (int j = 0; j < NPIX; ++j)
-    inb[j] = a.in + (long long)b * a.in_batch_stride + input_pixel(pix0 + (NHWC ? (tid + j * kBlock) / KC : tid % P_T));
+  for (int j = 0; j < NPIX; ++j) {
+    tapmask[j] = 0;
+    inb[j] = a.in + (long long)b * a.in_batch_stride +
+        input_pixel(pix0 + (NHWC ? (tid + j * kBlock) / KC : tid % P_T), tapmask[j]);
+  }
+  // bytes between horizontally adjacent taps of a pixel: a cell (blocked), a whole channel vector (nhwc)
+  const long long tap_stride = NHWC ? (long long)a.ic2 * 16 : 16;
   const uint8_t *safe = a.in + safe_off;
   const int bu0 = NHWC ? tid % KC : tid / P_T;
   const long long unit_stride = NHWC ? 16 : (long long)a.ihw * 16;
@@ -147,7 +153,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
       const int tap = fastdiv(chunk * KC, a.ic2, a.ic2_magic);
       const int ub = chunk * KC - tap * a.ic2;
       const int kh = fastdiv(tap, a.kw, a.kw_magic);
-      const bool inside = (tapmask >> tap) & 1;
+      const bool inside = (tapmask[0] >> tap) & 1;
       stz[d] = inside ? 0u : ~0u;
       const uint8_t *src = inside ? inb[0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * 16 : safe;
 #pragma unroll
@@ -165,9 +171,9 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
         const int tap = fastdiv(u, a.ic2, a.ic2_magic);
         u -= tap * a.ic2;
         const int kh = fastdiv(tap, a.kw, a.kw_magic);
-        const bool inside = (tapmask >> tap) & 1;
+        const bool inside = (tapmask[NHWC ? j : 0] >> tap) & 1;
         stz[d] |= inside ? 0u : 1u << j;
-        src = inside ? inb[0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * 16 : safe;
+        src = inside ? inb[NHWC ? j : 0] + (long long)(kh * a.iw + (tap - kh * a.kw)) * tap_stride : safe;
       } else {
         u = u < a.ic2 ? u : a.ic2 - 1;  // padded units multiply zero weights: any valid cell will do
       }
@@ -415,8 +421,9 @@ namespace {
 struct Variant {
   const char *name;
   int oc_t, p_t, kc;
-  // [blocked | nhwc | blocked kh x kw, ic2 % KC == 0 | blocked kh x kw, any ic2][prefetch depth 1, 2, 4] (null: not built)
-  void (*kernel[4][3])(GemmArgs);
+  // [blocked | nhwc | blocked kh x kw, ic2 % KC == 0 | blocked kh x kw, any ic2 | nhwc kh x kw][prefetch depth 1, 2, 4]
+  // (null: not built)
+  void (*kernel[5][3])(GemmArgs);
 };
 // depth 4 only where four fills of staging fit in 96 registers
 template <int WM, int WN, int TM, int TN, int KC, bool NHWC>
@@ -432,7 +439,8 @@ constexpr void (*deep_or_null())(GemmArgs)
       { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true, 0>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true, 0>,                   \
         deep_or_null<WM, WN, TM, TN, KC, true>() },                                                               \
       { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, 1>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, 1>, nullptr },      \
-      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, 2>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, 2>, nullptr } } }
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, false, 2>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, false, 2>, nullptr },      \
+      { k_gemm_u8s8<WM, WN, TM, TN, KC, 1, true, 2>, k_gemm_u8s8<WM, WN, TM, TN, KC, 2, true, 2>, nullptr } } }
 const Variant kVariants[] = {
     V(2, 2, 2, 2, 8),  // 0: 128 oc x 128 px
     V(2, 2, 2, 1, 8),  // 1: 128 oc x  64 px
@@ -539,8 +547,8 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   int dl = 1;
   const char *env = getenv("EHIP_GEMM_DEPTH");
   if (env && env[0]) dl = atoi(env) >= 4 ? 2 : (atoi(env) >= 2 ? 1 : 0);
-  if (taps > 1 && (a.in_nhwc || taps > 64 || nbatch != 1)) return hipErrorInvalidValue;
-  const int fmt = taps > 1 ? (a.ic2 % k.kc == 0 ? 2 : 3) : (a.in_nhwc ? 1 : 0);
+  if (taps > 1 && (taps > 64 || nbatch != 1)) return hipErrorInvalidValue;
+  const int fmt = taps > 1 ? (a.in_nhwc ? 4 : (a.ic2 % k.kc == 0 ? 2 : 3)) : (a.in_nhwc ? 1 : 0);
   while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[fmt][dl])) --dl;
   hipLaunchKernelGGL(k.kernel[fmt][dl], grid, dim3(kBlock), 0, s, a);
   return hipGetLastError();

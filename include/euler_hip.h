@@ -85,9 +85,9 @@ EHIP_API const char *ehip_last_error(void);
  *    no padding, sum fusion; activations nChw16c or nhwc on either side (nhwc: channels % 16 == 0);
  *  - CONV_DIRECT with a 1x1 kernel (a160, src/elx_int8_conv_direct.cpp:574-718): also f32 output;
  *  - CONV_DIRECT with a 3/5/7 kernel (c160, src/elx_int8_conv_direct.cpp:66-77): stride 1 or 2, every
- *    pad k/2 or k/2 - 1 (right/bottom pads follow from oh/ow), ow % flatting_t == 0; nChw16c input, or --
- *    with at most 4 input channels, a network's first layer -- nhwc input of ic bytes per pixel (4-byte
- *    aligned base address); nChw16c or nhwc output;
+ *    pad k/2 or k/2 - 1 (right/bottom pads follow from oh/ow), ow % flatting_t == 0; nChw16c or nhwc on
+ *    either side (nhwc: channels % 16 == 0, except that a layer with at most 4 input channels -- a
+ *    network's first layer -- takes nhwc input of ic bytes per pixel at a 4-byte aligned address);
  *  - depthwise 3x3 (g == ic == oc, src/elx_int8_conv_direct_depthwise.cpp): stride 1 or 2, pads 0/1,
  *    u8/s8 output, weights goihw;
  *  - CONV_WINOGRAD tile_size 4, 5 or 6 (0: the reference's automatic choice; src/elx_int8_conv_wino.cpp, src/eld_conv.cpp:231-270): f32 tensors with execution_mode 0xa1xx, or

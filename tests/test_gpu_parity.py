@@ -106,8 +106,8 @@ def test_nhwc_is_refused_where_it_is_not_built():
     d.input_fmt = E.NHWC   # channel tail
     with pytest.raises(E.EulerHipError):
         E.Conv(d)
-    d = E.make_desc(1, 64, 64, 8, 8, 3, 3, 1, algorithm=E.CONV_DIRECT)
-    d.input_fmt = E.NHWC   # nhwc input of a 3x3
+    d = E.make_desc(1, 64, 64, 8, 8, 3, 3, 1, g=64, algorithm=E.CONV_DIRECT)
+    d.input_fmt = E.NHWC   # nhwc input of a depthwise layer
     with pytest.raises(E.EulerHipError):
         E.Conv(d)
 
@@ -116,6 +116,24 @@ def test_nhwc_is_refused_where_it_is_not_built():
 def test_direct_kxk_nhwc_output(k, pad, stride):
     res = run_and_compare(Layer(2, 32, 48, 13, k=k, pad=pad, stride=stride, out_type=ol.S8, seed=160 + k + stride, out_nhwc=True))
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
+# nhwc INPUT of a k x k layer (src/elx_int8_conv_direct.cpp:596-668, input_as_bfmt_ false): the tap offset
+# is a whole channel vector per pixel, every thread keeps the valid-tap mask of each pixel it stages
+@pytest.mark.parametrize("in_z", [0.0, 128.0])
+@pytest.mark.parametrize("out_nhwc", [False, True])
+@pytest.mark.parametrize("n,ic,oc,hw,k,pad,stride", [(2, 32, 48, 13, 3, 1, 1), (1, 64, 64, 14, 3, 1, 2), (2, 16, 32, 17, 7, 3, 2),
+                                                     (1, 144, 32, 9, 5, 2, 1), (2, 48, 80, 12, 3, 0, 1)])
+def test_direct_kxk_nhwc_input(in_z, out_nhwc, n, ic, oc, hw, k, pad, stride):
+    res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=ol.U8, seed=260 + k + stride + ic,
+                                in_nhwc=True, out_nhwc=out_nhwc, in_z=in_z))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
+@pytest.mark.parametrize("variant", range(7))
+def test_direct_kxk_nhwc_input_every_kernel_variant(variant, monkeypatch):
+    monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
+    run_and_compare(Layer(2, 80, 96, 13, k=3, pad=1, stride=2, out_type=ol.S8, seed=270 + variant, in_nhwc=True))
 
 
 # ---- 3x3 direct (c160) ------------------------------------------------------------------------------

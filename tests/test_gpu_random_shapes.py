@@ -47,8 +47,10 @@ def test_random_kxk(seed):
         if r.integers(0, 2):
             out_hw = natural + 1
     out_type = OUT_TYPES[int(r.integers(0, 4))]
+    nhwc_in = ic % 16 == 0 and bool(r.integers(0, 2))
+    nhwc_out = oc % 16 == 0 and bool(r.integers(0, 2))
     run_and_compare(Layer(int(r.integers(1, 3)), ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=seed,
-                          out_hw=out_hw))
+                          out_hw=out_hw, in_nhwc=nhwc_in, out_nhwc=nhwc_out))
 
 
 @pytest.mark.parametrize("seed", range(24))
