@@ -242,7 +242,6 @@ int classify(ehip_conv *c)
     if (d.tinput_scale == kNoCali || d.tinput_scale == 0.0f) return fail(EHIP_GENERAL_ERROR, "wino_tinput_quant is not set");
     if (d.input_fmt != EHIP_NCHW16C || d.output_fmt != EHIP_NCHW16C || d.weights_fmt != EHIP_OIHW16I16O)
       return fail(EHIP_UNIMPLEMENTED, "winograd: only blocked formats are built");
-    if (d.with_ip_sum) return fail(EHIP_UNIMPLEMENTED, "winograd: sum fusion is not built");
     if (d.pad_t > 1 || d.pad_l > 1) return fail(EHIP_UNIMPLEMENTED, "winograd: pads > 1");
     c->family = FAM_WINOGRAD;
     return EHIP_OK;
@@ -369,7 +368,8 @@ int setup_workspace(ehip_conv *c)
       const char *env = getenv("EHIP_WINO_FUSED");
       // the fused GEMM + output transform is built for F(4x4,3x3); the other tile sizes run the
       // three-kernel schedule
-      c->fused = !(env && env[0] == '0') && d.tile_size == 6;
+      // ... and so does the in-place sum (the stand-alone output transform reads the old output)
+      c->fused = !(env && env[0] == '0') && d.tile_size == 6 && !d.with_ip_sum;
     }
     c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
                               : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output";
@@ -429,7 +429,7 @@ WinoArgs make_wino_args(const ehip_conv_desc_t &d, int ic2, int oc2)
   w.ht = (d.oh + w.tile - 3) / (w.tile - 2); w.wt = (d.ow + w.tile - 3) / (w.tile - 2);
   w.nt = w.ht * w.wt; w.t = w.nt * d.n;
   w.pad_t = d.pad_t; w.pad_l = d.pad_l;
-  w.with_bias = d.with_bias; w.with_relu = d.with_relu;
+  w.with_bias = d.with_bias; w.with_relu = d.with_relu; w.with_sum = d.with_ip_sum;
   w.in_u8 = d.input_type == EHIP_U8;
   w.out_type = d.output_type;
   if (d.output_type == EHIP_U8 || d.output_type == EHIP_S8) {

@@ -105,6 +105,7 @@ struct WinoArgs {
   int blocks_interior;  // set by the input-transform launcher: blocks over tiles off the rim
   float mrepS, mz;      // input_S / tinput_S, ceil(tinput_z)
   int with_bias, with_relu;
+  int with_sum;         // in-place sum: the old output is added before the ReLU (stand-alone output transform only)
 };
 
 struct WinoFusedArgs {

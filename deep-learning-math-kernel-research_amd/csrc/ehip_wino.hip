@@ -255,12 +255,37 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
 // ends as 255.  Border tiles write their valid rows and columns only.
 // The F(2x2,3x3) kernel converts toward minus infinity in its u8 / s8 store
 // (src/kernel/elk_conv_wino_2x2_3x3_output.hxx:142-151), the others to nearest even.
+// with_sum (in-place sum): the old output -- an f32, or the u8 / s8 code as a float, no scale -- is added
+// after the output quantization and before the ReLU (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:168-187).
 template <int OUT, int A = 6>
 __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias, bool with_bias, bool with_relu,
-                                            float repS, float z, void *plane, int q, int th, int tw, int oh_n, int ow_n)
+                                            float repS, float z, void *plane, int q, int th, int tw, int oh_n, int ow_n,
+                                            bool with_sum = false)
 {
   constexpr int AA = A * A, M = A - 2;
   float y[4][M * M];
+  float old[4][M * M];
+  if (with_sum) {
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+      for (int j = 0; j < M; ++j) {
+        const int oh = M * th + i, ow = M * tw + j;
+        const bool in = oh < oh_n && ow < ow_n;
+        const size_t cell = in ? ((size_t)oh * ow_n + ow) * 16 + 4 * q : 0;
+        if (OUT == EHIP_F32) {
+          const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(plane) + cell);
+          old[0][M * i + j] = v.x; old[1][M * i + j] = v.y; old[2][M * i + j] = v.z; old[3][M * i + j] = v.w;
+        } else {
+          const unsigned v = *reinterpret_cast<const unsigned *>(static_cast<const uint8_t *>(plane) + cell);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const unsigned b = (v >> (8 * k)) & 0xffu;
+            old[k][M * i + j] = OUT == EHIP_U8 ? (float)b : (float)(int)(signed char)b;
+          }
+        }
+      }
+  }
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     float f[AA], o[M * M];
@@ -273,6 +298,7 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
       float r = o[e];
       if (with_bias) r = r + b;
       if (OUT != EHIP_F32) r = __builtin_fmaf(r, repS, z);
+      if (with_sum) r = r + old[k][e];
       if (with_relu) r = r > 0.0f ? r : 0.0f;
       y[k][e] = r;
     }
@@ -335,7 +361,8 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
   const size_t plane = ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 16;
   void *dst = OUT == EHIP_F32 ? static_cast<void *>(static_cast<float *>(a.out) + plane)
                               : static_cast<void *>(static_cast<uint8_t *>(a.out) + plane);
-  output_tile<OUT, A>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z, dst, q, th, tw, a.oh, a.ow);
+  output_tile<OUT, A>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z, dst, q, th, tw, a.oh, a.ow,
+                      a.with_sum != 0);
 }
 
 // ---- the 36 GEMMs and the output transform in one kernel ----------------------------------------

@@ -998,9 +998,19 @@ int orc_wino_output_value(float y, int with_bias, float bias, int out_type, floa
 int orc_wino_output_value_a(int A, float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
                             int with_relu, float *f32_out)
 {
+  return orc_wino_output_value_sum(A, y, with_bias, bias, out_type, out_scale, out_z, with_relu, 0, 0.0f, f32_out);
+}
+
+// ... and with the in-place sum (with_ip_sum): the old output -- an f32, or the u8 / s8 code as a float,
+// no scale -- is added after the output quantization and before the ReLU
+// (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:168-187)
+int orc_wino_output_value_sum(int A, float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
+                              int with_relu, int with_sum, float old, float *f32_out)
+{
   float r = y;
   if (with_bias) r += bias;
   if (out_type == ORC_U8 || out_type == ORC_S8) r = fmaf(r, 1.0f / out_scale, std::ceil(out_z));
+  if (with_sum) r += old;
   if (with_relu) r = r > 0.0f ? r : 0.0f;  // vmaxps(p, 0): no upper bound here
   if (f32_out) *f32_out = r;
   if (out_type == ORC_U8) return usat8(A == 4 ? cvt_u32_floor(r) : cvt_u32_rne(r));
@@ -1027,10 +1037,14 @@ int orc_wino_trans_output(const orc_conv_params *p, const float *toutput, const 
                 int oh = g.M * th + i, ow = g.M * tw + j;
                 if (oh >= p->oh || ow >= p->ow) continue;
                 float r;
-                const int q = orc_wino_output_value_a(g.A, y[g.M * i + j], p->with_bias,
-                                                      p->with_bias ? bias[o2 * 16 + v] : 0.0f, p->out_type,
-                                                      p->out_scale, p->out_z, p->with_relu, &r);
                 const size_t oi = ((((size_t)n * g.OC2 + o2) * p->oh + oh) * p->ow + ow) * 16 + v;
+                float old = 0.0f;
+                if (p->with_sum)
+                  old = p->out_type == ORC_U8 ? (float)((uint8_t *)output)[oi]
+                      : (p->out_type == ORC_S8 ? (float)((int8_t *)output)[oi] : ((float *)output)[oi]);
+                const int q = orc_wino_output_value_sum(g.A, y[g.M * i + j], p->with_bias,
+                                                        p->with_bias ? bias[o2 * 16 + v] : 0.0f, p->out_type,
+                                                        p->out_scale, p->out_z, p->with_relu, p->with_sum, old, &r);
                 if (p->out_type == ORC_U8) ((uint8_t *)output)[oi] = (uint8_t)q;
                 else if (p->out_type == ORC_S8) ((int8_t *)output)[oi] = (int8_t)q;
                 else ((float *)output)[oi] = r;

@@ -131,6 +131,8 @@ void orc_wino_tile_weights_a(int A, const float g[9], float *u);
 void orc_wino_tile_output_a(int A, const float *m, float *y);
 int orc_wino_output_value_a(int A, float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
                             int with_relu, float *f32_out);
+int orc_wino_output_value_sum(int A, float y, int with_bias, float bias, int out_type, float out_scale, float out_z,
+                              int with_relu, int with_sum, float old, float *f32_out);
 
 /* epilogue on one value, exposed for the same reason (out_kind ORC_*; returns the f32 result
  * for ORC_F32 through *fout, else the quantized byte through the return value) */

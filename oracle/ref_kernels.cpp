@@ -444,4 +444,33 @@ int ref_wino_trans_output_a(int A, int out_kind, int border, int with_bias, int 
   return -1;
 }
 
+// The output transform with the in-place sum fused (with_ip_sum = true): the old output value -- an
+// f32, or a u8 / s8 code converted to float -- is added after the output quantization and before the
+// ReLU (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:112-131 and the same lines of the other tile sizes).
+int ref_wino_trans_output_sum(int A, int out_kind, int border, int with_bias, int with_relu, int oh,
+    int ow, void *out, float *toutput, float *bias, int h_end, int w_end, float repS, float z)
+{
+  elx_param_t ep;
+  fill_common(ep, 0.f, FLT_MAX, 0.f);
+  ep.oh = oh; ep.ow = ow;
+  ep.output_quant_repS = repS;
+  ep.output_quant_z = z;
+#define WS_CASE(a, k, OT, b, wb, wr)                                            \
+  if (A == a && out_kind == k && !!border == b && !!with_bias == wb && !!with_relu == wr) { \
+    elk_conv_wino_trans_output<float, OT, float, TKF_BLOCKED, b, wb, wr,        \
+        true, ISA_AVX512, a, 3, 16>::execute(ep, (OT *)out, toutput, bias,      \
+        h_end, w_end);                                                          \
+    return 0;                                                                   \
+  }
+#define WS_ALL(a, k, OT)                                                        \
+  WS_CASE(a, k, OT, false, true, true) WS_CASE(a, k, OT, false, false, false)   \
+  WS_CASE(a, k, OT, true, true, true) WS_CASE(a, k, OT, true, true, false)
+  WS_ALL(6, 0, float) WS_ALL(6, 1, uint8_t) WS_ALL(6, 2, int8_t)
+  WS_ALL(4, 0, float) WS_ALL(4, 1, uint8_t) WS_ALL(4, 2, int8_t)
+  WS_ALL(5, 0, float) WS_ALL(5, 1, uint8_t) WS_ALL(5, 2, int8_t)
+#undef WS_ALL
+#undef WS_CASE
+  return -1;
+}
+
 } // extern "C"

@@ -86,6 +86,9 @@ def oracle():
         lib.orc_wino_output_value_a.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int,
                                                 ctypes.c_float, ctypes.c_float, ctypes.c_int,
                                                 ctypes.POINTER(ctypes.c_float)]
+        lib.orc_wino_output_value_sum.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int,
+                                                  ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_int,
+                                                  ctypes.c_float, ctypes.POINTER(ctypes.c_float)]
         lib.orc_epilogue.argtypes = [ctypes.c_int, ctypes.c_int32, ctypes.c_float, ctypes.c_float, ctypes.c_int,
                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_float,
                                      ctypes.POINTER(ctypes.c_float)]
@@ -125,6 +128,8 @@ def ref_kernels():
             lib.ref_wino_trans_input_a.argtypes = [ci, ci, ci, ci, vp, vp, ci, ci, ci, ci]
             lib.ref_wino_trans_weights_a.argtypes = [ci, vp, vp]
             lib.ref_wino_trans_output_a.argtypes = [ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, ci, ci, fl, fl]
+        if hasattr(lib, "ref_wino_trans_output_sum"):
+            lib.ref_wino_trans_output_sum.argtypes = [ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, ci, ci, fl, fl]
         _ref = lib
     return _ref
 
@@ -266,8 +271,11 @@ def wino_gemm(p, tin, twq, tscale, tshift):
     return tout, acc
 
 
-def wino_trans_output(p, tout, bias):
+def wino_trans_output(p, tout, bias, out_init=None):
+    """out_init: the output tensor on entry (the sum operand when p.with_sum)"""
     out = np.zeros((p.n, up16(p.oc) // 16, p.oh, p.ow, 16), NP_OF[p.out_type])
+    if out_init is not None:
+        out[...] = out_init
     assert oracle().orc_wino_trans_output(ctypes.byref(p), ptr(tout), ptr(bias), ptr(out)) == 0
     return out
 

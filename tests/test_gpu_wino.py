@@ -243,3 +243,37 @@ def test_wino_automatic_tile_size():
     torch.cuda.synchronize()
     assert conv.query(E.Q_WEIGHTS_S8).size == 16 * twq.shape[1] * twq.shape[2]
     assert np.array_equal(bits(host(d_out)), bits(exp))
+
+
+# ---- in-place sum (with_ip_sum) in the output transform ------------------------------------------------
+@pytest.mark.parametrize("tile", [6, 4, 5])
+@pytest.mark.parametrize("out_type", [ol.F32, ol.U8, ol.S8])
+def test_wino_with_ip_sum(tile, out_type):
+    """The old output (f32, or the u8 / s8 code as it is) is added after the output quantization and before
+    the ReLU (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:168-187)."""
+    import torch
+    n, ic, oc, hw = 2, 32, 48, 11
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=31 + tile + out_type, out_type=out_type,
+                                         out_z=0.0 if out_type == ol.S8 else 1.6, tile=tile)
+    p.with_sum = 1
+    d.with_ip_sum = 1
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    rng = np.random.default_rng(77 + tile)
+    shape = (n, ol.up16(oc) // 16, hw, hw, 16)
+    if out_type == ol.F32:
+        old = rng.normal(0, 0.05, shape).astype(f32)
+    else:
+        old = rng.integers(-30 if out_type == ol.S8 else 0, 60, shape).astype(ol.NP_OF[out_type])
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xq.astype(f32)), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias, out_init=old)
+    assert not np.array_equal(exp, ol.wino_trans_output(p, tout, bias))   # the sum operand matters
+    conv = E.Conv(d)
+    assert conv.kernel_name.endswith("k_wino_trans_output")
+    d_out = dev(old)
+    d_b = dev(bias)
+    conv.execute(d_out, dev(xq), dev(wb), d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)

@@ -318,3 +318,44 @@ def test_wino_output_transform_bits_other_tiles(A, kind, with_bias, with_relu, e
                     assert np.float32(r.value).view(np.uint32) == out[i, j, c].view(np.uint32), (i, j, c)
                 else:
                     assert np_kind(q) == out[i, j, c], (i, j, c, q, out[i, j, c], r.value)
+
+
+# ---- in-place sum fused into the Winograd output transform (with_ip_sum) ----------------------------
+@pytest.mark.parametrize("A", [6, 4, 5])
+@pytest.mark.parametrize("kind", [ol.F32, ol.U8, ol.S8])
+@pytest.mark.parametrize("with_bias,with_relu,border", [(True, True, False), (False, False, False), (True, True, True),
+                                                        (True, False, True)])
+def test_wino_output_transform_with_sum_bits(A, kind, with_bias, with_relu, border):
+    M = A - 2
+    h_end, w_end = (M - 2, M - 1) if border else (M - 1, M - 1)
+    rng = np.random.default_rng(900 + A + kind + 2 * with_bias + with_relu + 4 * border)
+    m = ol.aligned((A, A, 16), np.float32)
+    m[...] = rng.normal(0, 3, m.shape)
+    bias = ol.aligned(16, np.float32)
+    bias[...] = rng.normal(0, 1, 16)
+    np_kind = ol.NP_OF[kind]
+    out = ol.aligned((8, 8, 16), np_kind)
+    out[...] = rng.normal(0, 2, out.shape) if kind == ol.F32 else rng.integers(-100 if kind == ol.S8 else 0, 100, out.shape)
+    old = np.array(out)
+    out_scale, out_z = 0.11, 3.0 if kind == ol.U8 else 0.0
+    rc = ref.ref_wino_trans_output_sum(A, {ol.F32: 0, ol.U8: 1, ol.S8: 2}[kind], int(border), int(with_bias), int(with_relu),
+                                       8, 8, ol.ptr(out), ol.ptr(m), ol.ptr(bias), h_end, w_end,
+                                       np.float32(1.0) / np.float32(out_scale), out_z)
+    assert rc == 0
+    y = np.zeros(M * M, np.float32)
+    for c in range(16):
+        mm = np.ascontiguousarray(m[:, :, c].ravel())
+        ol.oracle().orc_wino_tile_output_a(A, ol.ptr(mm), ol.ptr(y))
+        for i in range(M):
+            for j in range(M):
+                if i > h_end or j > w_end:
+                    assert out[i, j, c] == old[i, j, c]
+                    continue
+                r = ctypes.c_float()
+                q = ol.oracle().orc_wino_output_value_sum(A, float(y[M * i + j]), int(with_bias), float(bias[c]), kind,
+                                                          out_scale, out_z, int(with_relu), 1, float(old[i, j, c]),
+                                                          ctypes.byref(r))
+                if kind == ol.F32:
+                    assert np.float32(r.value).view(np.uint32) == out[i, j, c].view(np.uint32), (i, j, c)
+                else:
+                    assert np_kind(q) == out[i, j, c], (i, j, c, q, out[i, j, c], r.value)
