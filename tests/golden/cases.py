@@ -561,3 +561,59 @@ for _A in (4, 5):
             CASES["wino%d_output_%s_b%d_r%d_h%d_w%d" % (_A, _kn, _b, _r, _he, _we)] = (
                 lambda A=_A, k=_k, b=_b, r=_r, he=_he, we=_we: winoa_out_inputs(A, k, b, r, he, we, 700 + 16 * k + 8 * b + he + we + A),
                 winoa_out_reference, winoa_out_oracle)
+
+
+# ---- in-place sum fused into the Winograd output transform (with_ip_sum = true) -------------------
+def winos_out_inputs(A, kind, with_bias, with_relu, border, seed):
+    M = A - 2
+    h_end, w_end = (M - 2, M - 1) if border else (M - 1, M - 1)
+    d = winoa_out_inputs(A, kind, with_bias, with_relu, h_end, w_end, seed)
+    rng = np.random.default_rng(seed + 1)
+    if kind == ol.F32:
+        d["old"] = rng.normal(0, 2, (8, 8, 16)).astype(np.float32)
+    else:
+        d["old"] = rng.integers(-100 if kind == ol.S8 else 0, 100, (8, 8, 16)).astype(ol.NP_OF[kind])
+    return d
+
+
+def winos_out_reference(d, ref):
+    A, kind = int(d["A"]), int(d["kind"])
+    M = A - 2
+    out = ol.aligned((8, 8, 16), ol.NP_OF[kind])
+    out[...] = d["old"]
+    h_end, w_end = int(d["h_end"]), int(d["w_end"])
+    border = not (h_end == M - 1 and w_end == M - 1)
+    m, bias = _al(d["m"]), _al(d["bias"])
+    rep = np.float32(1.0) / d["out_scale"]
+    assert ref.ref_wino_trans_output_sum(A, KIND_ID[kind], int(border), int(d["with_bias"]), int(d["with_relu"]), 8, 8,
+                                         ol.ptr(out), ol.ptr(m), ol.ptr(bias), h_end, w_end, float(rep),
+                                         float(np.ceil(d["out_z"]))) == 0
+    return np.array(out[:M, :M, :])
+
+
+def winos_out_oracle(d):
+    A, kind = int(d["A"]), int(d["kind"])
+    M = A - 2
+    out = np.array(d["old"][:M, :M, :])
+    y = np.zeros(M * M, np.float32)
+    for c in range(16):
+        mm = np.ascontiguousarray(d["m"][:, :, c].ravel())
+        ol.oracle().orc_wino_tile_output_a(A, ol.ptr(mm), ol.ptr(y))
+        for i in range(M):
+            for j in range(M):
+                if i > int(d["h_end"]) or j > int(d["w_end"]):
+                    continue
+                r = ctypes.c_float()
+                q = ol.oracle().orc_wino_output_value_sum(A, float(y[M * i + j]), int(d["with_bias"]), float(d["bias"][c]), kind,
+                                                          float(d["out_scale"]), float(d["out_z"]), int(d["with_relu"]), 1,
+                                                          float(d["old"][i, j, c]), ctypes.byref(r))
+                out[i, j, c] = r.value if kind == ol.F32 else np.array(q).astype(ol.NP_OF[kind])
+    return out
+
+
+for _A in (6, 4, 5):
+    for _k, _kn in ((ol.F32, "f32"), (ol.U8, "u8"), (ol.S8, "s8")):
+        for _b, _r, _bd in ((1, 1, 0), (1, 0, 1)):
+            CASES["wino%d_output_sum_%s_b%d_r%d_border%d" % (_A, _kn, _b, _r, _bd)] = (
+                lambda A=_A, k=_k, b=_b, r=_r, bd=_bd: winos_out_inputs(A, k, b, r, bd, 800 + 16 * k + 8 * b + bd + A),
+                winos_out_reference, winos_out_oracle)
