@@ -137,8 +137,8 @@ int classify(ehip_conv *c)
     const bool fewch = d.algorithm == EHIP_CONV_DIRECT && !depthwise && conv_fewch_applies(d.ic, d.kh, d.kw);
     if (d.input_fmt == EHIP_NHWC && depthwise)
       return fail(EHIP_UNIMPLEMENTED, "nhwc input is not built for depthwise convolutions");
-    if (d.output_fmt == EHIP_NHWC && (depthwise || d.algorithm == EHIP_CONV_WINOGRAD))
-      return fail(EHIP_UNIMPLEMENTED, "nhwc output is only built for the direct 1x1 and kh x kw executors");
+    if (d.output_fmt == EHIP_NHWC && depthwise)
+      return fail(EHIP_UNIMPLEMENTED, "nhwc output is not built for depthwise convolutions");
     if ((d.input_fmt == EHIP_NHWC && d.ic % 16 && !fewch) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
       return fail(EHIP_UNIMPLEMENTED, "nhwc: channel counts must be multiples of 16");
   }
@@ -240,8 +240,12 @@ int classify(ehip_conv *c)
     if (d.input_scale == kNoCali || d.input_z == kNoCali)
       return fail(EHIP_UNIMPLEMENTED, "winograd: input_quant must be set (FINE sampling is not built)");
     if (d.tinput_scale == kNoCali || d.tinput_scale == 0.0f) return fail(EHIP_GENERAL_ERROR, "wino_tinput_quant is not set");
-    if (d.input_fmt != EHIP_NCHW16C || d.output_fmt != EHIP_NCHW16C || d.weights_fmt != EHIP_OIHW16I16O)
-      return fail(EHIP_UNIMPLEMENTED, "winograd: only blocked formats are built");
+    // activations nChw16c or nhwc (the reference has no channel tails with nhwc, src/elx_int8_conv_wino.cpp:120-125)
+    if ((d.input_fmt != EHIP_NCHW16C && d.input_fmt != EHIP_NHWC) || (d.output_fmt != EHIP_NCHW16C && d.output_fmt != EHIP_NHWC) ||
+        d.weights_fmt != EHIP_OIHW16I16O)
+      return fail(EHIP_UNIMPLEMENTED, "winograd: activations nChw16c or nhwc, weights OIhw16i16o");
+    if ((d.input_fmt == EHIP_NHWC && d.ic % 16) || (d.output_fmt == EHIP_NHWC && d.oc % 16))
+      return fail(EHIP_UNIMPLEMENTED, "Unimplemented: nhwc with a channel tail");
     if (d.pad_t > 1 || d.pad_l > 1) return fail(EHIP_UNIMPLEMENTED, "winograd: pads > 1");
     c->family = FAM_WINOGRAD;
     return EHIP_OK;
@@ -430,6 +434,7 @@ WinoArgs make_wino_args(const ehip_conv_desc_t &d, int ic2, int oc2)
   w.nt = w.ht * w.wt; w.t = w.nt * d.n;
   w.pad_t = d.pad_t; w.pad_l = d.pad_l;
   w.with_bias = d.with_bias; w.with_relu = d.with_relu; w.with_sum = d.with_ip_sum;
+  w.in_nhwc = d.input_fmt == EHIP_NHWC; w.out_nhwc = d.output_fmt == EHIP_NHWC;
   w.in_u8 = d.input_type == EHIP_U8;
   w.out_type = d.output_type;
   if (d.output_type == EHIP_U8 || d.output_type == EHIP_S8) {
@@ -645,6 +650,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.oh = d.oh; f.ow = d.ow; f.ht = w.ht; f.wt = w.wt; f.nt = w.nt; f.t = w.t;
         f.with_bias = d.with_bias; f.with_relu = d.with_relu;
         f.out_type = w.out_type; f.out_repS = w.out_repS; f.out_z = w.out_z;
+        f.out_nhwc = w.out_nhwc;
         f.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
         HIP_TRY(launch_wino_gemm_output(f, s));
         continue;
@@ -777,8 +783,9 @@ EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *in
   if (!desc || !input_dev || !min_out || !max_out) return fail(EHIP_GENERAL_ERROR, "null argument");
   const ehip_conv_desc_t &d = *desc;
   if (d.kh != 3 || d.kw != 3 || d.stride_h != 1 || d.stride_w != 1 ||
-      (d.input_type != EHIP_F32 && d.input_type != EHIP_U8) || d.input_fmt != EHIP_NCHW16C)
-    return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 or u8 blocked 3x3 stride-1 layers only");
+      (d.input_type != EHIP_F32 && d.input_type != EHIP_U8) ||
+      (d.input_fmt != EHIP_NCHW16C && !(d.input_fmt == EHIP_NHWC && d.ic % 16 == 0)))
+    return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 or u8 3x3 stride-1 layers, nChw16c or nhwc without a channel tail");
   if (d.tile_size != 0 && (d.tile_size < 4 || d.tile_size > 6)) return fail(EHIP_UNIMPLEMENTED, "Unimplemented tile size");
   WinoArgs w = make_wino_args(d, up(d.ic, 16) / 16, up(d.oc, 16) / 16);
   w.in = input_dev;

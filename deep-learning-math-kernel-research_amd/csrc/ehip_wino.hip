@@ -80,28 +80,31 @@ __device__ __forceinline__ TileCoord tile_coord(const WinoArgs &a, int t)
 template <int A>
 __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, float4 *d)
 {
+  // blocked: the 16-channel plane of (n, c2), 4 quads per pixel; nhwc: quad c2 * 4 + q of every pixel's vector
+  const size_t pq = a.in_nhwc ? (size_t)a.ic2 * 4 : 4;   // quads between neighbouring pixels
   const float4 *plane = reinterpret_cast<const float4 *>(a.in) +
-      ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4 + q;
+      (a.in_nhwc ? (size_t)c.n * a.ih * a.iw * pq + c2 * 4 : ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4) + q;
 #pragma unroll
   for (int i = 0; i < A; ++i)
 #pragma unroll
     for (int j = 0; j < A; ++j) {
       const int h = c.h0 + i, w = c.w0 + j;
-      d[A * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4]
+      d[A * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * pq]
                                                                    : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 template <int A>
 __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &c, int c2, int q, unsigned *d)
 {
+  const size_t pq = a.in_nhwc ? (size_t)a.ic2 * 4 : 4;
   const unsigned *plane = reinterpret_cast<const unsigned *>(a.in) +
-      ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4 + q;
+      (a.in_nhwc ? (size_t)c.n * a.ih * a.iw * pq + c2 * 4 : ((size_t)c.n * a.ic2 + c2) * a.ih * a.iw * 4) + q;
 #pragma unroll
   for (int i = 0; i < A; ++i)
 #pragma unroll
     for (int j = 0; j < A; ++j) {
       const int h = c.h0 + i, w = c.w0 + j;
-      d[A * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * 4] : 0u;   // the frame is 0.0f
+      d[A * i + j] = (h >= 0 && h < a.ih && w >= 0 && w < a.iw) ? plane[((size_t)h * a.iw + w) * pq] : 0u;   // the frame is 0.0f
     }
 }
 
@@ -260,8 +263,10 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
 template <int OUT, int A = 6>
 __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias, bool with_bias, bool with_relu,
                                             float repS, float z, void *plane, int q, int th, int tw, int oh_n, int ow_n,
-                                            bool with_sum = false)
+                                            bool with_sum = false, int px = 16)
 {
+  // px: elements between neighbouring pixels of `plane` (16 blocked; the channel count for nhwc, where
+  // `plane` points at the tile's 16-channel block inside the first pixel's vector)
   constexpr int AA = A * A, M = A - 2;
   float y[4][M * M];
   float old[4][M * M];
@@ -272,7 +277,7 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
       for (int j = 0; j < M; ++j) {
         const int oh = M * th + i, ow = M * tw + j;
         const bool in = oh < oh_n && ow < ow_n;
-        const size_t cell = in ? ((size_t)oh * ow_n + ow) * 16 + 4 * q : 0;
+        const size_t cell = in ? ((size_t)oh * ow_n + ow) * px + 4 * q : 0;
         if (OUT == EHIP_F32) {
           const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(plane) + cell);
           old[0][M * i + j] = v.x; old[1][M * i + j] = v.y; old[2][M * i + j] = v.z; old[3][M * i + j] = v.w;
@@ -312,7 +317,7 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
       const int ow = M * tw + j;
       if (ow >= ow_n) break;
       const int e = M * i + j;
-      const size_t cell = ((size_t)oh * ow_n + ow) * 16 + 4 * q;   // element index inside the plane
+      const size_t cell = ((size_t)oh * ow_n + ow) * px + 4 * q;   // element index inside the plane
       if (OUT == EHIP_F32) {
         *reinterpret_cast<float4 *>(static_cast<float *>(plane) + cell) = make_float4(y[0][e], y[1][e], y[2][e], y[3][e]);
       } else {
@@ -358,11 +363,11 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 
   float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
   if (a.with_bias) bias = reinterpret_cast<const float4 *>(a.bias)[o2 * 4 + q];
-  const size_t plane = ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 16;
+  const size_t plane = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + o2 * 16 : ((size_t)n * a.oc2 + o2) * a.oh * a.ow * 16;
   void *dst = OUT == EHIP_F32 ? static_cast<void *>(static_cast<float *>(a.out) + plane)
                               : static_cast<void *>(static_cast<uint8_t *>(a.out) + plane);
   output_tile<OUT, A>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z, dst, q, th, tw, a.oh, a.ow,
-                      a.with_sum != 0);
+                      a.with_sum != 0, a.out_nhwc ? a.oc2 * 16 : 16);
 }
 
 // ---- the 36 GEMMs and the output transform in one kernel ----------------------------------------
@@ -528,18 +533,20 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
       for (int e = 0; e < 36; ++e) m[e] = xl[(e * 32 + tile_l) * 8 + (q8 ^ ((tile_l >> 1) & 7))];
       float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
       if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
-      const size_t plane = ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 16;
+      const size_t plane = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (oc >> 4) * 16
+                                      : ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 16;
+      const int px = a.out_nhwc ? a.oc2 * 16 : 16;
       const int q = (oc >> 2) & 3;
       TRACE_POINT(4 + 4 * h);
       if (a.out_type == EHIP_U8)
         output_tile<EHIP_U8>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
-                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow);
+                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow, false, px);
       else if (a.out_type == EHIP_S8)
         output_tile<EHIP_S8>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
-                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow);
+                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow, false, px);
       else
         output_tile<EHIP_F32>(m, bias, a.with_bias != 0, a.with_relu != 0, 0.f, 0.f, static_cast<float *>(a.out) + plane, q,
-                              th, tw, a.oh, a.ow);
+                              th, tw, a.oh, a.ow, false, px);
     }
     TRACE_POINT(5 + 4 * h);
   }

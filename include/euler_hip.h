@@ -93,7 +93,8 @@ EHIP_API const char *ehip_last_error(void);
  *  - CONV_WINOGRAD tile_size 4, 5 or 6 (0: the reference's automatic choice; src/elx_int8_conv_wino.cpp, src/eld_conv.cpp:231-270): f32 tensors with execution_mode 0xa1xx, or
  *    u8 input with f32/u8/s8 output (U8F32F32F32 / U8F32U8F32 / U8F32S8F32, src/eld_conv.cpp:275-281);
  *    wino_tinput_quant must be set (calibrated sampling); with_ip_sum adds the old output (f32, or the
- *    u8 / s8 code, unscaled) before the ReLU as the reference's output transform does.
+ *    u8 / s8 code, unscaled) before the ReLU as the reference's output transform does; activations
+ *    nChw16c or nhwc on either side (nhwc: channels % 16 == 0).
  * A non-zero input zero point with padding is accepted by the 3/5/7 direct kernels (the shift then
  * depends on the output pixel's set of valid taps, src/elx_int8_conv_direct.cpp:227-423); depthwise and
  * Winograd accept it only where no tap falls on padding. */

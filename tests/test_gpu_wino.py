@@ -277,3 +277,78 @@ def test_wino_with_ip_sum(tile, out_type):
     torch.cuda.synchronize()
     got = host(d_out)
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
+# ---- nhwc activations -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("fused", ["1", "0"])
+@pytest.mark.parametrize("in_nhwc,out_nhwc", [(True, True), (True, False), (False, True)])
+@pytest.mark.parametrize("tile,out_type,with_sum", [(6, ol.F32, 0), (6, ol.U8, 0), (6, ol.S8, 1), (4, ol.U8, 0),
+                                                    (5, ol.F32, 1), (5, ol.S8, 0)])
+def test_wino_nhwc_activations(tile, out_type, with_sum, in_nhwc, out_nhwc, fused, monkeypatch):
+    """The transforms read and write [n][h][w][c] activations (the reference's nhwc variants of the
+    Winograd transforms, src/elx_conv_wino_trans_input.cpp:226-262, src/elx_conv_wino_trans_output.cpp:136-190):
+    the same values as with nChw16c, in the other layout."""
+    import torch
+    if fused == "0" and (tile != 6 or with_sum):
+        pytest.skip("only the 6x6 tile without a sum has a fused schedule to switch off")
+    monkeypatch.setenv("EHIP_WINO_FUSED", fused)
+    n, ic, oc, hw = 2, 48, 80, 13
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=91 + tile + out_type, out_type=out_type,
+                                         out_z=0.0 if out_type == ol.S8 else 2.4, tile=tile)
+    p.with_sum = with_sum
+    d.with_ip_sum = with_sum
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    if in_nhwc:
+        d.input_fmt = E.NHWC
+    if out_nhwc:
+        d.output_fmt = E.NHWC
+    rng = np.random.default_rng(5 + tile)
+    shape = (n, oc // 16, hw, hw, 16)
+    if out_type == ol.F32:
+        old = rng.normal(0, 0.05, shape).astype(f32)
+    else:
+        old = rng.integers(-30 if out_type == ol.S8 else 0, 60, shape).astype(ol.NP_OF[out_type])
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xq.astype(f32)), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias, out_init=old if with_sum else None)
+    conv = E.Conv(d)
+    d_x = dev(ol.blocked_to_nhwc(xq, ic) if in_nhwc else xq)
+    d_out = dev(ol.blocked_to_nhwc(old, oc) if out_nhwc else old)
+    d_b = dev(bias)
+    conv.execute(d_out, d_x, dev(wb), d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    if out_nhwc:
+        exp = ol.blocked_to_nhwc(exp, oc)
+    assert got.shape == exp.shape
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
+def test_wino_nhwc_f32_input_and_range():
+    """fp32 nhwc input: calibration range and the whole pipeline match the blocked layout's."""
+    import torch
+    E, p, d, xb, wb, bias = make_wino(2, 32, 48, 11, seed=3)
+    p.tin_scale, p.tin_z = 9.0 / 255.0, 100.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    d.input_fmt = d.output_fmt = E.NHWC
+    d_x = dev(ol.blocked_to_nhwc(xb, 32))
+    mn, mx = E.wino_tinput_range(d, d_x)
+    omn, omx = ol.wino_tinput_range(p, xb)
+    assert (f32(mn), f32(mx)) == (f32(omn), f32(omx))
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xb), twq, tscale, tshift)
+    exp = ol.blocked_to_nhwc(ol.wino_trans_output(p, tout, bias), 48)
+    conv = E.Conv(d)
+    d_out = torch.zeros(exp.shape, dtype=torch.float32, device="cuda")
+    d_b = dev(bias)
+    conv.execute(d_out, d_x, dev(wb), d_b)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(host(d_out)), bits(exp))
+
+
+def test_wino_nhwc_channel_tail_is_refused():
+    E, p, d, xq, wb, bias = make_wino_u8(1, 24, 32, 8, seed=1, out_type=ol.U8)
+    d.input_fmt = E.NHWC
+    with pytest.raises(E.EulerHipError, match="channel tail"):
+        E.Conv(d)
