@@ -169,7 +169,9 @@ int classify(ehip_conv *c)
       if (d.g % 16) return fail(EHIP_UNIMPLEMENTED, "conv: g blocking error for depthwise conv");
       if (d.weights_fmt != EHIP_GOIHW) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: format not supported");
       if (d.with_ip_sum) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: no sum fusion");
-      if (d.input_z != 0.0f) return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: input zero point with padding");
+      // a non-zero input zero point: as in the reference, a padded tap adds nothing to the sum while the
+      // shift takes z times all nine weights (src/elx_int8_conv_direct_depthwise.cpp:247-289,
+      // src/kernel/elk_u8s8_depthwise_conv.hxx:316-413) -- no border correction
       c->family = FAM_DEPTHWISE;
       return EHIP_OK;
     }

@@ -96,8 +96,10 @@ EHIP_API const char *ehip_last_error(void);
  *    u8 / s8 code, unscaled) before the ReLU as the reference's output transform does; activations
  *    nChw16c or nhwc on either side (nhwc: channels % 16 == 0).
  * A non-zero input zero point with padding is accepted by the 3/5/7 direct kernels (the shift then
- * depends on the output pixel's set of valid taps, src/elx_int8_conv_direct.cpp:227-423); depthwise and
- * Winograd accept it only where no tap falls on padding. */
+ * depends on the output pixel's set of valid taps, src/elx_int8_conv_direct.cpp:227-423).  The depthwise
+ * executor follows the reference: one shift of z times all nine weights, padded taps adding nothing
+ * (src/elx_int8_conv_direct_depthwise.cpp:247-289); the Winograd executor, like the reference's, uses
+ * the input scale only (src/elx_conv_wino_trans_input.cpp:367-368). */
 EHIP_API int ehip_conv_create(const ehip_conv_desc_t *desc, ehip_conv_t **out);
 EHIP_API int ehip_conv_destroy(ehip_conv_t *conv);
 

@@ -292,6 +292,15 @@ def test_depthwise_stride2(out_type, g, hw, pad, out_hw, T):
                           w_sigma=0.1, T=T, out_hw=out_hw))
 
 
+@pytest.mark.parametrize("stride,pad,hw", [(1, 1, 14), (1, 0, 9), (2, 1, 15), (2, 0, 14)])
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
+def test_depthwise_input_zero_point(out_type, stride, pad, hw):
+    """z != 0: the shift takes z x all nine weights, padded taps add nothing
+    (src/elx_int8_conv_direct_depthwise.cpp:247-289): the reference's values, border included."""
+    run_and_compare(Layer(2, 48, 48, hw, k=3, pad=pad, stride=stride, out_type=out_type, depthwise=True,
+                          seed=hw + stride + out_type, w_sigma=0.1, T=0, in_z=37.0))
+
+
 def test_depthwise_stride2_raw_sums():
     run_and_compare(Layer(1, 32, 32, 11, k=3, pad=1, stride=2, out_type=ol.S32, depthwise=True, seed=78, w_sigma=0.1, T=3))
 
