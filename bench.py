@@ -22,10 +22,20 @@ sys.path.insert(0, ROOT)
 PKG = "deep-learning-math-kernel-research_amd"
 
 
+PREHEAT_S = 0.1
+
+
 def measure(layer, steps, warmup):
     """(wall seconds per step, HIP-event seconds per step).  Both regions hold exactly `steps`
-    executions enqueued back to back on the stream the kernels run on (the default stream)."""
+    executions enqueued back to back on the stream the kernels run on (the default stream).
+    Before the warmup steps the layer runs untimed for PREHEAT_S seconds: an idle GPU takes tens of
+    milliseconds to reach its running clocks, far longer than `warmup` launches of a 10 us kernel
+    (the same layer reads 12 % slower when timed straight from idle)."""
     import torch
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < PREHEAT_S:
+        layer.run(200)
+        torch.cuda.synchronize()
     layer.run(warmup)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -131,6 +141,8 @@ def main():
                     help="with --network: run the 3x3 stride-1 layers with CONV_DIRECT instead of the Winograd "
                          "algorithm the reference's scripts ask for (on this GPU the direct kernel is the faster one; "
                          "its results are the reference's DIRECT results, not its Winograd results)")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="rate of v_mfma_i32_32x32x32_i8 from registers, nothing else in the way")
     ap.add_argument("--hbm-probe", action="store_true",
                     help="instead of a layer, time plain device copy / fill / read of 1 GiB (the HBM rates a "
                          "trivial kernel reaches on this box)")
@@ -186,6 +198,23 @@ def main():
                           "fill_write_GBs": rate(lambda: a.zero_(), n), "sum_read_GBs": rate(lambda: af.sum(), n)}))
         return
 
+    if args.mfma_probe:
+        out = torch.empty(4096 * 256, dtype=torch.int32, device="cuda")
+        res = {}
+        stream = torch.cuda.current_stream().cuda_stream
+        for wgs in (256, 512, 1024, 2048, 4096):   # 1, 2, 4, 8, 16 waves per SIMD's worth of workgroups
+            ops = E.probe_mfma_i8(wgs, 2000, out, stream)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                E.probe_mfma_i8(wgs, 2000, out, stream)
+            e1.record()
+            torch.cuda.synchronize()
+            res["wgs_%d" % wgs] = round(ops / (e0.elapsed_time(e1) * 1e-3 / 5) / 1e12, 1)
+        print(json.dumps({"mfma_i8_probe_TOPS": res, "instruction": "v_mfma_i32_32x32x32_i8", "published_peak_TOPS": 5000.0}))
+        return
+
     if args.network:
         net = W.NETWORKS[args.network]
         rows, total_s, total_ops = [], 0.0, 0.0
@@ -227,7 +256,8 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "%s: %s" % (wl.key, wl.title), "ops_per_step": wl.ops(),
-                   "algorithmic_bytes_per_step": wl.algorithmic_bytes(), "kernel": layer.conv.kernel_name},
+                   "algorithmic_bytes_per_step": wl.algorithmic_bytes(), "kernel": layer.conv.kernel_name,
+                   "untimed_preheat_ms": PREHEAT_S * 1e3},
         "images_per_s": round(wl.n / wall, 1),
         "single_launch_latency_us": round(lat * 1e6, 2),
         "event_ms_per_step": round(ev * 1e3, 6),

@@ -20,6 +20,7 @@ SOURCES = [
     "ehip_depthwise.hip",
     "ehip_wino.hip",
     "ehip_prepare.hip",
+    "ehip_probe.hip",
     "ehip_api.hip",
     "euler_api.hip",
 ]

@@ -316,7 +316,7 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
     const long long wgs = (long long)gx * gy * n;
     const double util = (double)(oh * ow) / ((double)gx * k.p_t);
     const double fill = wgs >= 256 ? 1.0 : (double)wgs / 256.0;
-    const double big = (k.p_t >= 128 && wgs >= 768) ? 1.15 : 1.0;   // enough work: amortise the weights
+    const double big = (k.p_t >= 128 && wgs >= 440) ? 1.15 : 1.0;   // enough work: amortise the weights
     const double score = util * fill * big * pref[v];
     if (score > best_score) { best_score = score; best = v; }
   }

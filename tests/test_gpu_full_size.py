@@ -74,21 +74,28 @@ def test_configured_winograd_layer(key, check_images):
     assert float(got.max()) > 0.0
 
 
-@pytest.mark.parametrize("key,check_images", [("C4a_i8", 2), ("C4b_i8", 4), ("C4b_i8_t4", 2), ("C4b_i8_t5", 2)])
-def test_configured_winograd_layer_u8_in_s8_out(key, check_images):
-    """The VGG layers as the reference's tuned int8 run feeds them (u8 input, s8 output)."""
+@pytest.mark.parametrize("key,check_images,nhwc", [("C4a_i8", 2, False), ("C4b_i8", 4, False), ("C4b_i8_t4", 2, False),
+                                                   ("C4b_i8_t5", 2, False), ("C4b_i8", 2, True), ("C4b_i8_t4", 2, True)])
+def test_configured_winograd_layer_u8_in_s8_out(key, check_images, nhwc):
+    """The VGG layers as the reference's tuned int8 run feeds them (u8 input, s8 output); `nhwc`: the same
+    layer with [n][h][w][c] activations on both sides."""
     import torch
     wl = W.WORKLOADS[key]
     E, p, d, xq, wb, bias = make_wino_u8(wl.n, wl.ic, wl.oc, wl.hw, seed=91 + wl.hw, out_type=ol.S8, tile=wl.tile)
     s_t, z_t = 22.0 / 255.0, 104.0
     d.tinput_scale, d.tinput_z = s_t, z_t
+    if nhwc:
+        d.input_fmt = d.output_fmt = E.NHWC
     conv = E.Conv(d)
-    d_out = torch.full((wl.n, ol.up16(wl.oc) // 16, wl.hw, wl.hw, 16), -7, dtype=torch.int8, device="cuda")
+    d_out = torch.full((wl.n, wl.hw, wl.hw, wl.oc) if nhwc else (wl.n, ol.up16(wl.oc) // 16, wl.hw, wl.hw, 16), -7,
+                       dtype=torch.int8, device="cuda")
     d_b = dev(bias)
     conv.prepare(dev(wb), d_b)
-    conv.execute(d_out, dev(xq), None, d_b)
+    conv.execute(d_out, dev(ol.blocked_to_nhwc(xq, wl.ic) if nhwc else xq), None, d_b)
     torch.cuda.synchronize()
     got = host(d_out)
+    if nhwc:   # back to nChw16c for the comparison
+        got = np.ascontiguousarray(got.reshape(wl.n, wl.hw, wl.hw, wl.oc // 16, 16).transpose(0, 3, 1, 2, 4))
     k = check_images
     pk = ol.make_params(k, wl.ic, wl.oc, wl.hw, wl.hw, 3, 3, 1, out_type=ol.S8, in_scale=1.0 / 255.0, with_bias=True,
                         with_relu=True, out_scale=p.out_scale, out_z=p.out_z, wino_tile=wl.tile)
