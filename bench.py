@@ -141,6 +141,9 @@ def main():
                     help="with --network: run the 3x3 stride-1 layers with CONV_DIRECT instead of the Winograd "
                          "algorithm the reference's scripts ask for (on this GPU the direct kernel is the faster one; "
                          "its results are the reference's DIRECT results, not its Winograd results)")
+    ap.add_argument("--preheat-ms", type=float, default=100.0,
+                    help="untimed run of the layer before the warmup steps, so that the GPU is at its running clocks "
+                         "(profiler runs pass a small value to keep their traces short)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="rate of v_mfma_i32_32x32x32_i8 from registers, nothing else in the way")
     ap.add_argument("--hbm-probe", action="store_true",
@@ -156,6 +159,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    global PREHEAT_S
+    PREHEAT_S = args.preheat_ms * 1e-3
     import torch
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
