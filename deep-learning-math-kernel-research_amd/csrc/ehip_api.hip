@@ -538,6 +538,18 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const vo
   return EHIP_OK;
 }
 
+// Development aid: a build with -DEHIP_TRACE takes the address of a device buffer for the kernels' clock
+// stamps from the environment; the product build passes null and never looks.
+static long long *trace_buffer()
+{
+#ifdef EHIP_TRACE
+  const char *env = getenv("EHIP_TRACE_PTR");
+  return reinterpret_cast<long long *>(env ? strtoull(env, nullptr, 0) : 0ull);
+#else
+  return nullptr;
+#endif
+}
+
 EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *input_dev, const void *weights_dev,
                                const void *bias_dev, void *hip_stream)
 {
@@ -568,7 +580,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       a.ep.shift_tab = c->shift_tab; a.ep.tab_stride = c->ocpp;
       a.cls_h = c->cls_h; a.cls_w = c->cls_w; a.ncls_w = c->ncls_w;
     }
-    a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
+    a.trace = trace_buffer();
     HIP_TRY(launch_gemm(a, 1, c->variant, s));
     break;
   }
@@ -605,7 +617,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.chunk_units = c->chunk_units;
     a.vw = d.ow + 2;
     a.vw_magic = div_magic(a.vw);
-    a.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
+    a.trace = trace_buffer();
     HIP_TRY(launch_conv3x3v(a, d.n, c->variant, s));
     break;
   }
@@ -653,7 +665,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.with_bias = d.with_bias; f.with_relu = d.with_relu;
         f.out_type = w.out_type; f.out_repS = w.out_repS; f.out_z = w.out_z;
         f.out_nhwc = w.out_nhwc;
-        f.trace = reinterpret_cast<long long *>(getenv("EHIP_TRACE_PTR") ? strtoull(getenv("EHIP_TRACE_PTR"), nullptr, 0) : 0ull);
+        f.trace = trace_buffer();
         HIP_TRY(launch_wino_gemm_output(f, s));
         continue;
       }
