@@ -380,6 +380,57 @@ def test_three_layers_chained_on_the_device():
     assert np.array_equal(host(bufs[2]), o3)
 
 
+def test_chain_replayed_from_a_hip_graph():
+    """execute() of a prepared handle only launches kernels (no allocation, no memset, no synchronisation), so a
+    chain of layers can be captured into a HIP graph: three replays with fresh inputs, eager work and
+    synchronisations between them, each compared with the eager chain on the same input."""
+    import torch
+    E = pkg()
+    rng = np.random.default_rng(5)
+    l1 = Layer(2, 64, 96, 14, k=3, pad=1, out_type=ol.U8, seed=311, T=14)
+    l2 = Layer(2, 96, 96, 14, k=3, pad=1, out_type=ol.U8, depthwise=True, seed=312, w_sigma=0.1, T=14)
+    l3 = Layer(2, 96, 48, 14, stride=2, out_type=ol.S8, seed=313)
+    l4 = Layer(2, 48, 64, 7, k=3, pad=1, stride=1, out_type=ol.F32, seed=314, in_nhwc=False)
+    layers = (l1, l2, l3, l4)
+    convs, bufs = [], []
+    for l in layers:
+        c = E.Conv(l.desc)
+        c.prepare(dev(l.wb), dev(l.bias))
+        convs.append(c)
+        shape = (l.p.n, ol.up16(l.p.oc) // 16, l.p.oh, l.p.ow, 16)
+        bufs.append(torch.zeros(shape, dtype={ol.S8: torch.int8, ol.U8: torch.uint8, ol.F32: torch.float32}[l.p.out_type],
+                                device="cuda"))
+    x = dev(l1.xb)
+
+    def chain(stream=0):
+        src = x
+        for c, l, b in zip(convs, layers, bufs):
+            # the s8 codes of layer 3 are layer 4's u8 input bytes as they are: only the chaining is under test
+            c.execute(b, src, stream=stream)
+            src = b
+
+    inputs = [rng.integers(0, 256, l1.xb.shape).astype(np.uint8) for _ in range(3)]
+    eager = []
+    for xi in inputs:
+        x.copy_(dev(xi))
+        chain()
+        torch.cuda.synchronize()
+        eager.append([host(b).copy() for b in bufs])
+    assert not np.array_equal(eager[0][3], eager[1][3])
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        chain(torch.cuda.current_stream().cuda_stream)
+    for xi, exp in zip(inputs, eager):
+        x.copy_(dev(xi))
+        for b in bufs:
+            b.fill_(7)                       # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for b, e in zip(bufs, exp):
+            assert np.array_equal(bits(host(b)), bits(e))
+
+
 # ---- error behaviour of setup ---------------------------------------------------------------------------
 def test_setup_rejects_what_the_reference_rejects():
     E = pkg()

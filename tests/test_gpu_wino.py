@@ -352,3 +352,37 @@ def test_wino_nhwc_channel_tail_is_refused():
     d.input_fmt = E.NHWC
     with pytest.raises(E.EulerHipError, match="channel tail"):
         E.Conv(d)
+
+
+@pytest.mark.parametrize("tile", [6, 4])
+def test_wino_replayed_from_a_hip_graph(tile):
+    """The Winograd execute of a prepared handle (input transform, GEMMs, output transform over the handle's
+    own workspace) launches kernels only, so it can be captured: three replays with fresh inputs, eager work
+    and synchronisations between them, each equal to the eager result."""
+    import torch
+    E, p, d, xq, wb, bias = make_wino_u8(3, 48, 80, 13, seed=17 + tile, out_type=ol.S8, tile=tile)
+    d.tinput_scale, d.tinput_z = 22.0 / 255.0, 104.0
+    conv = E.Conv(d)
+    d_b = dev(bias)
+    conv.prepare(dev(wb), d_b)
+    rng = np.random.default_rng(3)
+    inputs = [rng.integers(0, 256, xq.shape).astype(np.uint8) for _ in range(3)]
+    x = dev(xq)
+    out = torch.zeros((3, 5, 13, 13, 16), dtype=torch.int8, device="cuda")
+    eager = []
+    for xi in inputs:
+        x.copy_(dev(xi))
+        conv.execute(out, x, None, d_b)
+        torch.cuda.synchronize()
+        eager.append(host(out).copy())
+    assert not np.array_equal(eager[0], eager[1])
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        conv.execute(out, x, None, d_b, stream=torch.cuda.current_stream().cuda_stream)
+    for xi, exp in zip(inputs, eager):
+        x.copy_(dev(xi))
+        out.fill_(9)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(out), exp)
