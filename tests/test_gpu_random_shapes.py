@@ -94,11 +94,12 @@ def test_random_depthwise(seed):
     divs = [t for t in range(1, oh + 1) if oh % t == 0]
     T = int(r.choice(divs + [0, oh]))
     out_type = [ol.U8, ol.S8, ol.S32][int(r.integers(0, 3))]
+    in_z = float(r.choice([0.0, 0.0, 3.0, 128.0]))
     run_and_compare(Layer(int(r.integers(1, 4)), g, g, hw, k=3, pad=pad, stride=stride, out_type=out_type, depthwise=True,
-                          seed=seed, w_sigma=0.1, T=T))
+                          seed=seed, w_sigma=0.1, T=T, in_z=in_z))
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(24))
 def test_random_winograd(seed):
     import torch
     from gpu_common import bits, dev, host
@@ -110,6 +111,9 @@ def test_random_winograd(seed):
     out_type = [ol.F32, ol.U8, ol.S8][int(r.integers(0, 3))] if u8_in else ol.F32
     bias_on, relu_on = bool(r.integers(0, 2)), bool(r.integers(0, 2))
     tile = int(r.choice([6, 4, 5]))   # F(4x4,3x3), F(2x2,3x3), F(3x3,3x3)
+    with_sum = bool(r.integers(0, 3) == 0)
+    in_nhwc = bool(r.integers(0, 3) == 0) and ic % 16 == 0
+    out_nhwc = bool(r.integers(0, 3) == 0) and oc % 16 == 0
     if u8_in:
         E, p, d, x, wb, bias = make_wino_u8(n, ic, oc, hw, seed, out_type, with_bias=bias_on, with_relu=relu_on, tile=tile)
         xf = x.astype(np.float32)
@@ -120,12 +124,26 @@ def test_random_winograd(seed):
     d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
     twq, tscale, tshift = ol.wino_prepare(p, wb)
     tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xf), twq, tscale, tshift)
-    exp = ol.wino_trans_output(p, tout, bias)
+    old = None
+    if with_sum:
+        p.with_sum = d.with_ip_sum = 1
+        shape = (n, ol.up16(oc) // 16, hw, hw, 16)
+        old = (r.normal(0, 0.05, shape).astype(np.float32) if out_type == ol.F32 else
+               r.integers(-30 if out_type == ol.S8 else 0, 60, shape).astype(ol.NP_OF[out_type]))
+    exp = ol.wino_trans_output(p, tout, bias, out_init=old)
+    if in_nhwc:
+        d.input_fmt = E.NHWC
+        x = ol.blocked_to_nhwc(x, ic)
+    if out_nhwc:
+        d.output_fmt = E.NHWC
+        exp = ol.blocked_to_nhwc(exp, oc)
+        old = ol.blocked_to_nhwc(old, oc) if with_sum else None
     conv = E.Conv(d)
     tdt = {ol.F32: torch.float32, ol.U8: torch.uint8, ol.S8: torch.int8}[out_type]
-    d_out = torch.full(exp.shape, 3, dtype=tdt, device="cuda")
+    d_out = dev(old) if with_sum else torch.full(exp.shape, 3, dtype=tdt, device="cuda")
     d_b = dev(bias) if bias_on else None
     conv.execute(d_out, dev(x), dev(wb), d_b)
     torch.cuda.synchronize()
     got = host(d_out)
+    assert got.shape == exp.shape
     assert np.array_equal(bits(got), bits(exp)), "%d of %d values differ" % (int((got != exp).sum()), got.size)
