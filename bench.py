@@ -74,6 +74,17 @@ def roofline_of(wl, sec_per_launch, traffic):
             "frac": round(achieved / peak, 5), "traffic": traffic}
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(wl, budget_s=12.0):
     """The CPU oracle (a port of the reference's loop nest; AVX-512-VNNI inner loop when the host
     has it) timed on this host's cores on the same layer.  Bounded: as many passes as fit ~budget."""
@@ -112,7 +123,7 @@ def cpu_baseline(wl, budget_s=12.0):
             "isa": "avx512-vnni" if vnni else "scalar/auto-vectorised",
             "sample": "%d passes of %s with N=%d of %d in %.1f s (weight preparation excluded)" % (
                 passes, wl.key, n, wl.n, el),
-            "ms_per_pass": round(sec * 1e3, 3), "images_per_s": round(n / sec, 1)}
+            "ms_per_pass": round(sec * 1e3, 3), "images_per_s": round(n / sec, 1), "cpu_model": cpu_model()}
 
 
 def load_traffic():
