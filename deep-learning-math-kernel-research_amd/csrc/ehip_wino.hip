@@ -181,13 +181,15 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   unsigned packed[AA];
 #pragma unroll
   for (int k = 0; k < AA; ++k) packed[k] = 0u;
-  auto channels = [&](bool border) {
+  // mixed: the wave holds interior and rim tiles -- the per-lane, branch-free form of the transform
+  auto channels = [&](bool mixed) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       float f[AA], v[AA];
 #pragma unroll
       for (int e = 0; e < AA; ++e) f[e] = comp_of(d[e], k);
-      wino::tile_input<A>(f, v, border);
+      if (mixed) wino::tile_input_lanes<A>(f, v, c.border);
+      else wino::tile_input<A>(f, v, false);
 #pragma unroll
       for (int e = 0; e < AA; ++e) {
         // sat_u8(rne_to_u32(V * (in_S / tin_S) + tin_z)), one rounding in the multiply-add.  The
@@ -198,12 +200,8 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
       }
     }
   };
-  if (blockIdx.x < a.blocks_interior) {
-    channels(false);
-  } else {
-    if (c.border) channels(true);
-    else channels(false);
-  }
+  if (__ballot(c.border) != 0) channels(true);   // wave-uniform
+  else channels(false);
   unsigned *dst = reinterpret_cast<unsigned *>(a.tin) + ((size_t)c2 * a.t + t) * 4 + q;
   const size_t pos_stride = (size_t)a.ic2 * a.t * 4;
 #pragma unroll
@@ -229,8 +227,7 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
       float f[AA], v[AA];
 #pragma unroll
       for (int e = 0; e < AA; ++e) f[e] = comp_of(d[e], k);
-      if (c.border) wino::tile_input<A>(f, v, true);
-      else wino::tile_input<A>(f, v, false);
+      wino::tile_input_lanes<A>(f, v, c.border);
 #pragma unroll
       for (int e = 0; e < AA; ++e) {
         mn = v[e] < mn ? v[e] : mn;

@@ -41,6 +41,31 @@ __device__ __forceinline__ void in6_1d(const float f[6], float o[6], bool raw_un
   o[3] = __builtin_fmaf(t3, z5, t2);
   o[4] = __builtin_fmaf(-t3, z5, t2);
 }
+// The same with the choice made per LANE and without a branch, for waves that hold tiles of both kinds:
+// fma(p, 1, g) with p = f * z already rounded IS the rounded sum p + g, so a term is
+// fma(unfused ? p : f, unfused ? 1 : z, g) -- one multiply and one select more than the plain form
+// instead of running the whole transform twice under complementary masks.
+__device__ __forceinline__ float fma_or_mul_add(float f, float z, float g, bool unfused)
+{
+  const float p = f * z;
+  return __builtin_fmaf(unfused ? p : f, unfused ? 1.0f : z, g);
+}
+__device__ __forceinline__ void in6_1d_lanes(const float f[6], float o[6], bool raw_unfused, bool t4_unfused)
+{
+  const float z0 = -2.25f, z1 = -0.390625f, z2 = 0.87890625f, z3 = -2.640625f, z4 = 0.625f, z5 = 1.5f;
+  const float t0 = fma_or_mul_add(f[2], z0, f[4], raw_unfused);
+  const float t1 = fma_or_mul_add(f[1], z0, f[3], raw_unfused);
+  const float t2 = fma_or_mul_add(f[2], z1, f[4], raw_unfused);
+  const float t3 = fma_or_mul_add(f[1], z1, f[3], raw_unfused);
+  const float t4 = fma_or_mul_add(f[0], z2, f[4], raw_unfused || t4_unfused);
+  const float t5 = fma_or_mul_add(f[1], z2, f[5], raw_unfused);
+  o[0] = fma_or_mul_add(f[2], z3, t4, raw_unfused);
+  o[5] = fma_or_mul_add(f[3], z3, t5, raw_unfused);
+  o[1] = __builtin_fmaf(t1, z4, t0);
+  o[2] = __builtin_fmaf(-t1, z4, t0);
+  o[3] = __builtin_fmaf(t3, z5, t2);
+  o[4] = __builtin_fmaf(-t3, z5, t2);
+}
 __device__ __forceinline__ void out6_1d(const float f[6], float o[4])
 {
   const float z0 = 1.5f, z1 = 2.25f, z2 = 3.375f, z3 = 0.625f, z4 = 0.390625f, z5 = 0.244140625f;
@@ -83,6 +108,18 @@ __device__ __forceinline__ void in5_1d(const float f[5], float o[5], bool fuse15
   o[0] = f[0] * z0 - t1 - t2;
   o[1] = f[3] - t0 - t1;
   o[2] = (fuse15 ? __builtin_fmaf(f[2], z1, f[3]) : f[2] * z1 + f[3]) + t0;
+  o[3] = t2;
+  o[4] = f[3] * z0 + f[4] - f[2] - t0;
+}
+__device__ __forceinline__ void in5_1d_lanes(const float f[5], float o[5], bool unfused15)
+{
+  const float z0 = 0.5f, z1 = 1.5f;
+  const float t0 = f[1] * z0;
+  const float t1 = f[2] * z0;
+  const float t2 = f[3] - f[1];
+  o[0] = f[0] * z0 - t1 - t2;
+  o[1] = f[3] - t0 - t1;
+  o[2] = fma_or_mul_add(f[2], z1, f[3], unfused15) + t0;
   o[3] = t2;
   o[4] = f[3] * z0 + f[4] - f[2] - t0;
 }
@@ -174,6 +211,48 @@ __device__ __forceinline__ void tile_input<4>(const float *d, float *v, bool)
   V(3, 3) = (c1 - D(3, 1)) + D(3, 3);
 #undef D
 #undef V
+}
+
+// tile_input with the border flag per lane (see fma_or_mul_add): what a wave with both kinds of tile runs
+template <int A>
+__device__ __forceinline__ void tile_input_lanes(const float *d, float *v, bool border);
+template <>
+__device__ __forceinline__ void tile_input_lanes<6>(const float *d, float *v, bool border)
+{
+  float m[36];
+#pragma unroll
+  for (int j = 0; j < 6; ++j) {
+    float f[6], o[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) f[i] = d[6 * i + j];
+    in6_1d_lanes(f, o, border, false);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) m[6 * i + j] = o[i];
+  }
+#pragma unroll
+  for (int i = 0; i < 5; ++i) in6_1d(&m[6 * i], &v[6 * i], false, false);
+  in6_1d_lanes(&m[30], &v[30], false, border);
+}
+template <>
+__device__ __forceinline__ void tile_input_lanes<5>(const float *d, float *v, bool border)
+{
+  float m[25];
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    float f[5], o[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) f[i] = d[5 * i + j];
+    in5_1d_lanes(f, o, border);
+#pragma unroll
+    for (int i = 0; i < 5; ++i) m[5 * i + j] = o[i];
+  }
+#pragma unroll
+  for (int i = 0; i < 5; ++i) in5_1d(&m[5 * i], &v[5 * i], true);
+}
+template <>
+__device__ __forceinline__ void tile_input_lanes<4>(const float *d, float *v, bool border)
+{
+  tile_input<4>(d, v, border);
 }
 
 // g: [3][3] (kh, kw)
