@@ -32,7 +32,7 @@
 #ifdef EHIP_TRACE
 #define TRACE_POINT(i)                                                                             \
   do {                                                                                             \
-    if (a.trace && lane == 0) a.trace[((size_t)(blockIdx.z * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
+    if (a.trace && lane == 0) a.trace[((size_t)tile_id * 4 + wave) * 16 + (i)] = clock64(); \
   } while (0)
 #else
 #define TRACE_POINT(i) do { } while (0)
@@ -56,9 +56,18 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
-  const int n = blockIdx.z;
-  const int v0 = blockIdx.x * P_T;
-  const int oc0 = blockIdx.y * OC_T;
+  // Workgroups go round the eight XCDs (block b runs on XCD b % 8), each XCD with an L2 of its own.
+  // Tiles are numbered pixel tile first, then channel tile, then image, and XCD x takes the x-th
+  // eighth of that sequence: neighbouring pixel tiles share two rows of input, the channel tiles of an
+  // image share all of it, and what one of them has pulled into the XCD's L2 the others find there
+  // instead of fetching it from HBM again through another XCD.
+  const int tile_id = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+  if (tile_id >= a.tiles) return;   // whole workgroup
+  const int n = tile_id / (a.gx * a.gy);
+  const int txy = tile_id - n * (a.gx * a.gy);
+  const int ty = txy / a.gx;
+  const int v0 = (txy - ty * a.gx) * P_T;
+  const int oc0 = ty * OC_T;
   const int mw0 = (wave % WM) * TM * 32;
   const int pw0 = (wave / WM) * TN * 32;
   const int oc_real = a.oc2 * 16;
@@ -323,11 +332,21 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
   return best;
 }
 
-hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s)
+hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_t s)
 {
   const Variant &k = kVariants[variant];
+  Conv3x3Args a = a0;
   const size_t lds_bytes = (size_t)a.chunk_units * k.cells * 16;
-  dim3 grid((a.oh * a.vw + k.p_t - 1) / k.p_t, (a.oc2 * 16 + k.oc_t - 1) / k.oc_t, n);
+  a.gx = (a.oh * a.vw + k.p_t - 1) / k.p_t;
+  a.gy = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
+  const long long tiles = (long long)a.gx * a.gy * n;
+  if (tiles >= (1ll << 30)) {
+    set_error("direct 3x3: too many tiles");
+    return hipErrorInvalidValue;
+  }
+  a.tiles = (int)tiles;
+  a.tiles_per_xcd = (a.tiles + 7) / 8;
+  dim3 grid(8 * a.tiles_per_xcd, 1, 1);
   if (lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k.kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);

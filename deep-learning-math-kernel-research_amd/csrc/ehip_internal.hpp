@@ -75,6 +75,7 @@ struct Conv3x3Args {
   int vw;               // virtual row width ow + 2
   unsigned vw_magic;    // div_magic(vw)
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
+  int gx, gy, tiles, tiles_per_xcd;   // set by the launcher: pixel tiles per image, channel tiles, all tiles, ceil(tiles / 8)
 };
 
 struct DepthwiseArgs {
