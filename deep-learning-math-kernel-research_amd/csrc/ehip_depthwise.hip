@@ -45,16 +45,22 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 {
   constexpr int NPX = S == 1 ? 4 : 5;          // input pixels per row a lane touches
   constexpr int NROWS = S * (RB - 1) + 3;      // input rows
-  // grid: x = blocks over one plane's lanes (q fastest, then column pair, then row block),
-  // y = 16-channel block, z = image
+  // A plane (one image x one 16-channel block) is split into blocks over its lanes (q fastest, then
+  // column pair, then row block).  Workgroups go round the eight XCDs (block b runs on XCD b % 8), each
+  // with an L2 of its own, and neighbouring row blocks share two input rows: so all blocks of a plane
+  // are given to ONE XCD, one after the other -- plane = 8 * (seq / blocks_per_plane) + xcd.
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int pgrp = seq / a.blocks_per_plane;
+  const int plane_id = pgrp * 8 + xcd;
+  if (plane_id >= a.n * a.g2) return;   // whole workgroup
   const int wp = (a.ow + 1) >> 1;
-  const int local = blockIdx.x * blockDim.x + threadIdx.x;
+  const int local = (seq - pgrp * a.blocks_per_plane) * blockDim.x + threadIdx.x;
   if (local >= a.lanes_per_plane) return;
   const int q = local & 3;
   const int hb = fastdiv(local >> 2, wp, a.wp_magic);
   const int p = (local >> 2) - hb * wp;
-  const int g2 = blockIdx.y;
-  const unsigned ng = blockIdx.z * a.g2 + g2;
+  const int g2 = plane_id % a.g2;
+  const unsigned ng = plane_id;   // image * g2 + channel block
   const int oh0 = hb * RB;
   const int c0 = 2 * p;
   const int ch0 = g2 * 16 + 4 * q;  // first of the lane's 4 channels
@@ -221,7 +227,9 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s)
   if (a.out_type == EHIP_U8 && a.with_relu && a.lo >= 0.0f && a.hi <= 255.0f && a.hi >= a.lo)
     mode = (a.lo == 0.0f && a.hi == 255.0f) ? 2 : 1;
   const int block = a.lanes_per_plane >= kBlock ? kBlock : up(a.lanes_per_plane, kWave);
-  dim3 grid((a.lanes_per_plane + block - 1) / block, a.g2, a.n);
+  a.blocks_per_plane = (a.lanes_per_plane + block - 1) / block;
+  const long long planes = (long long)a.n * a.g2;
+  dim3 grid((unsigned)(8 * ((planes + 7) / 8) * a.blocks_per_plane), 1, 1);
   if (rb == 7) launch_rb<7>(a, mode, grid, dim3(block), s);
   else if (rb == 4) launch_rb<4>(a, mode, grid, dim3(block), s);
   else if (rb == 2) launch_rb<2>(a, mode, grid, dim3(block), s);

@@ -88,6 +88,7 @@ struct DepthwiseArgs {
   int stride;           // 1 or 2, both directions
   int T, Tr, wt;        // width blocking of the reference kernel (decides floor vs round per column)
   int lanes_per_plane;  // set by the launcher: row blocks x column pairs x 4
+  int blocks_per_plane; // set by the launcher: workgroups per plane
   unsigned wp_magic, T_magic;  // div_magic of the column pairs per row and of T
   int out_type, with_relu;
   float lo, hi;
