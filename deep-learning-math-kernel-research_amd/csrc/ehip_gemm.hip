@@ -70,11 +70,12 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   const int lh = lane >> 5;
   // Workgroups go to the 8 XCDs round-robin by their linear index.  The channel blocks of one pixel
   // block are numbered so that they follow each other on ONE XCD: the first one pulls the pixels
-  // into that XCD's L2, the others find them there.
+  // into that XCD's L2, the others find them there.  An XCD takes a contiguous eighth of the pixel
+  // blocks: in the kh x kw form neighbouring pixel blocks share input rows.
   const int b = blockIdx.y;
   const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
   const int by = seq % a.ny;
-  const int bx = (seq / a.ny) * 8 + xcd;
+  const int bx = xcd * ((a.nx + 7) >> 3) + seq / a.ny;
   if (bx >= a.nx) return;   // whole workgroup (grid padded to a multiple of 8 pixel blocks)
   const int pix0 = bx * P_T;
   const int oc0 = by * OC_T;
