@@ -104,7 +104,7 @@ struct WinoArgs {
   float out_repS, out_z;   // u8 / s8 output: 1 / output_S, ceil(output_z)
   int n, ic2, oc2, ih, iw, oh, ow, ht, wt, nt, t, pad_t, pad_l;
   int tile;             // tile size A: 6 (or 0) = F(4x4,3x3), 4 = F(2x2,3x3), 5 = F(3x3,3x3); 36 below reads A * A
-  int blocks_interior;  // set by the input-transform launcher: blocks over tiles off the rim
+  int nblocks, items_per_xcd;   // set by the input-transform launcher: blocks of 64 tiles; ceil(blocks x units / 8)
   float mrepS, mz;      // input_S / tinput_S, ceil(tinput_z)
   int with_bias, with_relu;
   int with_sum;         // in-place sum: the old output is added before the ReLU (stand-alone output transform only)

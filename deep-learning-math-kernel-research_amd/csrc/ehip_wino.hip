@@ -110,72 +110,24 @@ __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &
 
 }  // namespace
 
-// Measured: with the rim split off the kernel executes 38 % fewer vector instructions but writes
-// 26 % more bytes (the runs of tiles a wave stores per position no longer fill whole cache lines),
-// and it is the memory side that bounds it -- so the split is off.
-constexpr bool kSplitRim = false;
-
-// Tiles that touch the zero frame take the "border" arithmetic, all others the plain one; a wave
-// that holds both kinds would execute both.  So the grid is split: the first a.blocks_interior
-// blocks enumerate only tiles away from the rim of the tile grid (never border), the remaining
-// blocks enumerate the rim.  Returns false past the end of the group.
-template <int A>
-__device__ __forceinline__ bool grouped_tile(const WinoArgs &a, int block, int slot, TileCoord &c, int &t)
-{
-  if (!kSplitRim) {
-    t = block * 64 + slot;
-    if (t >= a.t) return false;
-    c = tile_coord<A>(a, t);
-    return true;
-  }
-  const int wi = a.wt - 2, hi = a.ht - 2;
-  const int ni = (wi > 0 && hi > 0) ? wi * hi : 0;   // interior tiles per image
-  int n, th, tw;
-  if (block < a.blocks_interior) {
-    const int idx = block * 64 + slot;
-    if (idx >= a.n * ni) return false;
-    n = idx / ni;
-    const int r = idx - n * ni;
-    th = 1 + r / wi;
-    tw = 1 + (r - (th - 1) * wi);
-  } else {
-    const int idx = (block - a.blocks_interior) * 64 + slot;
-    const int nr = a.nt - ni;                        // rim tiles per image
-    if (idx >= a.n * nr) return false;
-    n = idx / nr;
-    const int r = idx - n * nr;
-    if (ni == 0) {                                   // fewer than 3 tile rows or columns: all rim
-      th = r / a.wt;
-      tw = r - th * a.wt;
-    } else if (r < a.wt) {
-      th = 0; tw = r;
-    } else if (r < 2 * a.wt) {
-      th = a.ht - 1; tw = r - a.wt;
-    } else {
-      const int rr = r - 2 * a.wt;
-      th = 1 + (rr >> 1);
-      tw = (rr & 1) ? a.wt - 1 : 0;
-    }
-  }
-  t = n * a.nt + th * a.wt + tw;
-  c.n = n; c.th = th; c.tw = tw;
-  c.h0 = (A - 2) * th - a.pad_t;
-  c.w0 = (A - 2) * tw - a.pad_l;
-  c.border = c.h0 < 0 || c.w0 < 0 || c.h0 + A - 1 >= a.ih || c.w0 + A - 1 >= a.iw;
-  return true;
-}
-
-// grid: (interior blocks + rim blocks, ic2); block: 64 tiles x 4 channel quads.
+// block: 64 consecutive tiles x 4 channel quads of one 16-channel unit.  Work items are numbered tile
+// block first, then unit, and XCD x (workgroup b runs on XCD b % 8) takes the x-th eighth of them:
+// neighbouring tile blocks read the same two input rows where they meet, and find them in their XCD's L2.
+// Tiles that touch the zero frame take the reference's "border" arithmetic, the others the plain one; a
+// wave that holds both kinds (nearly every wave: two rim tiles per row of tiles) runs the per-lane,
+// branch-free form of the transform instead of both forms under complementary masks.
 // Cell = float4 (f32 user input) or unsigned (u8 user input: four codes per lane and pixel).
 template <typename Cell, int A = 6>
 __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
 {
   constexpr int AA = A * A;
   const int q = threadIdx.x & 3;
-  const int c2 = blockIdx.y;
-  TileCoord c;
-  int t;
-  if (!grouped_tile<A>(a, blockIdx.x, threadIdx.x >> 2, c, t)) return;
+  const int item = (blockIdx.x & 7) * a.items_per_xcd + (blockIdx.x >> 3);
+  if (item >= a.nblocks * a.ic2) return;   // whole workgroup
+  const int c2 = item / a.nblocks;
+  const int t = (item - c2 * a.nblocks) * 64 + (threadIdx.x >> 2);
+  if (t >= a.t) return;
+  const TileCoord c = tile_coord<A>(a, t);
   Cell d[AA];
   gather_tile<A>(a, c, c2, q, d);
   unsigned packed[AA];
@@ -552,14 +504,9 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s)
 {
   WinoArgs a = a0;
-  const int ni = (a.wt > 2 && a.ht > 2) ? (a.wt - 2) * (a.ht - 2) : 0;
-  a.blocks_interior = (a.n * ni + 63) / 64;
-  int blocks_rim = (a.n * (a.nt - ni) + 63) / 64;
-  if (!kSplitRim) {   // one group: tiles in memory order
-    a.blocks_interior = 0;
-    blocks_rim = (a.t + 63) / 64;
-  }
-  dim3 grid(a.blocks_interior + blocks_rim, a.ic2);
+  a.nblocks = (a.t + 63) / 64;
+  a.items_per_xcd = (int)(((long long)a.nblocks * a.ic2 + 7) / 8);
+  dim3 grid(8 * a.items_per_xcd, 1);
   void (*kern)(WinoArgs) = nullptr;
   if (a.tile == 4) kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 4> : k_wino_trans_input_u8<float4, 4>;
   else if (a.tile == 5) kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 5> : k_wino_trans_input_u8<float4, 5>;
