@@ -91,13 +91,13 @@ void run_dw(elx_param_t &ep, void *routput, uint8_t *input, int8_t *weights,
       wscale, wshift, khs, khe, 0, 3, pad_l, pad_r, attr);
 }
 
-template <typename OT, int T, int S = 1>
+template <typename OT, int T, int S = 1, int K = 3>
 void run_conv3(elx_param_t &ep, float *toutput, void *routput, uint8_t *input,
     int8_t *weights, float *wscale, float *wshift, int khs, int khe, int kws,
     int kwe, int pad_l, int pad_r, int attr)
 {
   using ker = u8s8_conv_kernel<conv_impl::INT8_F32, OT, 16, 4, ISA_AVX512,
-      estl::integer_sequence<S, GKF_DCD, 1, T, 3>>;
+      estl::integer_sequence<S, GKF_DCD, 1, T, K>>;
   ker::conv(ep, toutput, (OT *)routput, input, weights, nullptr, nullptr, nullptr,
       wscale, wshift, khs, khe, kws, kwe, pad_l, pad_r, attr);
 }
@@ -262,6 +262,50 @@ int ref_u8s8_conv3x3_s2(int out_kind, int T, int I2, int ih, int iw, int oh, int
     return 0;                                                                   \
   }
   CV_CASE(0, float, 7) CV_CASE(1, uint8_t, 7) CV_CASE(2, int8_t, 7)
+#undef CV_CASE
+  return -1;
+}
+
+// The micro-kernel template for the other kernel sizes (5x5 and 7x7: the generic branch,
+// src/kernel/elk_u8s8_conv.hxx:254-677), stride 1 or 2, set up and bound as above for any K
+// (src/elx_int8_conv_direct.cpp:502-571, src/elx_int8_conv_direct_bind.hpp:108-117).  T = 7, one
+// width block (_wt = 0, wt = 1): pads lp on the left and rp on the right of that block.
+int ref_u8s8_convk(int K, int S, int out_kind, int I2, int ih, int iw, int oh, int ow, int _ht,
+    int tp, int lp, int rp, int with_relu, float relu_lo, float relu_hi, float *toutput,
+    void *routput, uint8_t *input, int8_t *weights, float *wscale, float *wshift)
+{
+  const int T = 7;
+  if (ow != T) return -2;
+  elx_param_t ep;
+  fill_common(ep, relu_lo, relu_hi, 0.f);
+  ep.kh = ep.kw = K; ep.I2 = I2; ep.ic2 = I2; ep.IC = ep.ic = 16 * I2;
+  ep.OC = ep.oc = 16; ep.oc2 = 1;
+  ep.ih = ih; ep.iw = iw; ep.oh = oh; ep.ow = ow; ep.T = T;
+  ep.hs = ep.ws = S;
+  ep.tp = tp; ep.lp = lp; ep.rp = rp; ep.bp = 0;
+  int khs = tp - S * _ht > 0 ? tp - S * _ht : 0;
+  int khe = K < ih + tp - S * _ht ? K : ih + tp - S * _ht;
+  int kws = lp, kwe = K - rp;
+  int cih = S * _ht + K / 2 - tp, ciw = K / 2 - lp;
+  uint8_t *in = input + ((long)cih * iw + ciw) * 16;
+  size_t ooff = (size_t)_ht * ow * 16;
+  int attr = AT_CLEAR_OUTPUT_MASK | AT_RESTORE_OUTPUT_MASK
+      | (with_relu ? (int)AT_RELU_MASK : 0);
+#define CV_CASE(kk, ss, k, OT)                                                  \
+  if (K == kk && S == ss && out_kind == k) {                                    \
+    if (ss == 2 && lp > rp)                                                     \
+      run_conv3<OT, 7, (ss == 2 ? S2_LLP : 1), kk>(ep, toutput ? toutput + ooff : nullptr, \
+          routput ? (char *)routput + ooff * sizeof(OT) : nullptr, in, weights, \
+          wscale, wshift, khs, khe, kws, kwe, lp, rp, attr);                    \
+    else                                                                        \
+      run_conv3<OT, 7, ss, kk>(ep, toutput ? toutput + ooff : nullptr,          \
+          routput ? (char *)routput + ooff * sizeof(OT) : nullptr, in, weights, \
+          wscale, wshift, khs, khe, kws, kwe, lp, rp, attr);                    \
+    return 0;                                                                   \
+  }
+  CV_CASE(5, 1, 0, float) CV_CASE(5, 1, 1, uint8_t) CV_CASE(5, 1, 2, int8_t)
+  CV_CASE(7, 2, 0, float) CV_CASE(7, 2, 1, uint8_t) CV_CASE(7, 2, 2, int8_t)
+  CV_CASE(5, 2, 1, uint8_t) CV_CASE(7, 1, 2, int8_t)
 #undef CV_CASE
   return -1;
 }

@@ -214,6 +214,58 @@ def conv_s2_reference(d, ref):
     return np.array(tout if kind == ol.F32 else rout)
 
 
+# 5x5 and 7x7 kernels: the reference's generic micro-kernel template, stride 1 or 2, one width block of 7
+def convk_inputs(kind, K, S, iw, lp, rp, seed):
+    rng = np.random.default_rng(seed)
+    I2 = 2
+    return dict(kind=np.int32(kind), K=np.int32(K), S=np.int32(S), iw=np.int32(iw), lp=np.int32(lp), rp=np.int32(rp),
+                x=rng.integers(0, 256, (1, I2, iw, iw, 16)).astype(np.uint8),
+                w=rng.normal(0, 0.03, (16, 16 * I2, K, K)).astype(np.float32),
+                bias=rng.normal(0, 0.3, 16).astype(np.float32))
+
+
+def _convk_geometry(d):
+    K, S, iw, lp, rp = (int(d[k]) for k in ("K", "S", "iw", "lp", "rp"))
+    ow = (iw + lp + rp - K) // S + 1
+    assert ow == 7 and (ow - 1) * S + K == iw + lp + rp
+    return K, S, iw, lp, rp, ow
+
+
+def _convk_params(d):
+    K, S, iw, lp, rp, ow = _convk_geometry(d)
+    return ol.make_params(1, 32, 16, iw, iw, K, K, stride=S, out_type=int(d["kind"]), out_scale=0.02,
+                          relu_hi=ol.FLT_MAX, pad_tl=lp, out_hw=(ow, ow))
+
+
+def convk_oracle(d):
+    p = _convk_params(d)
+    wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(d["w"]), d["bias"])
+    out, _ = ol.direct_execute(p, d["x"], wq, scale, shift)
+    return out.reshape(p.oh * p.ow, 16)
+
+
+def convk_reference(d, ref):
+    p = _convk_params(d)
+    K, S, iw, lp, rp, ow = _convk_geometry(d)
+    kind, I2, T = int(d["kind"]), 2, 7
+    wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(d["w"]), d["bias"])
+    xb = ol.aligned(d["x"].size + 1024, np.uint8)
+    xb[:d["x"].size] = d["x"].ravel()
+    wr = ol.aligned((K, K, I2, 4, 16, 4), np.int8)
+    wr[...] = wq.reshape(16, I2, 4, 4, K, K).transpose(4, 5, 1, 2, 0, 3)
+    sc = _al(scale[:16])
+    sh = ol.aligned((T, 16), np.float32)
+    sh[...] = shift[None, :16]
+    tout = ol.aligned((ow * ow, 16), np.float32)
+    rout = ol.aligned((ow * ow, 16), ol.NP_OF[kind])
+    for ht in range(ow):
+        rc = ref.ref_u8s8_convk(K, S, KIND_ID[kind], I2, iw, iw, ow, ow, ht, lp, lp, rp, 1, 0.0, ol.FLT_MAX,
+                                ol.ptr(tout), ol.ptr(rout) if kind != ol.F32 else None, ol.ptr(xb), ol.ptr(wr),
+                                ol.ptr(sc), ol.ptr(sh))
+        assert rc == 0, rc
+    return np.array(tout if kind == ol.F32 else rout)
+
+
 def dw_s2_inputs(kind, iw, lp, rp, T, seed):
     rng = np.random.default_rng(seed)
     return dict(kind=np.int32(kind), iw=np.int32(iw), lp=np.int32(lp), rp=np.int32(rp), T=np.int32(T),
@@ -420,6 +472,19 @@ for _k, _kn, _iw, _lp, _rp in ((ol.U8, "u8", 15, 0, 0), (ol.S8, "s8", 14, 1, 0),
     CASES["conv3x3_s2_%s_w%d_l%d_r%d" % (_kn, _iw, _lp, _rp)] = (
         lambda k=_k, iw=_iw, lp=_lp, rp=_rp: conv_s2_inputs(k, iw, lp, rp, 300 + iw + 2 * lp + rp + k), conv_s2_reference,
         conv_s2_oracle)
+# 5x5 / 7x7.  The template takes its column bounds per tap from k/2 and the stride, not from the pads it
+# is given (src/kernel/elk_u8s8_conv.hxx:312-470), so it is the convolution only for the pad sets it was
+# written for: stride 1 with k/2 on both sides; stride 2 with (k/2, k/2 - 1) -- the "lean left padding"
+# instantiation -- or (k/2 - 1, k/2), and 5x5 with (1, 1).  Elsewhere it reads a pixel of the neighbouring
+# row or drops a valid tap (7x7 s2 pads (2, 2): column 5 differs; (3, 3): column 1; stride 1 pads (3, 2):
+# columns 4-5), and the oracle and the product compute the convolution.  The cases below are the exact ones,
+# which include every shape of the reference's tuned runs.
+for _k, _kn, _K, _S, _iw, _lp, _rp in ((ol.U8, "u8", 5, 1, 7, 2, 2), (ol.S8, "s8", 5, 1, 7, 2, 2), (ol.F32, "f32", 5, 1, 7, 2, 2),
+                                       (ol.U8, "u8", 7, 2, 14, 3, 2), (ol.S8, "s8", 7, 2, 14, 2, 3), (ol.F32, "f32", 7, 2, 14, 3, 2),
+                                       (ol.U8, "u8", 5, 2, 15, 1, 1), (ol.S8, "s8", 7, 1, 7, 3, 3)):
+    CASES["conv%dx%d_s%d_%s_w%d_l%d_r%d" % (_K, _K, _S, _kn, _iw, _lp, _rp)] = (
+        lambda k=_k, K=_K, S=_S, iw=_iw, lp=_lp, rp=_rp: convk_inputs(k, K, S, iw, lp, rp, 500 + 10 * K + iw + 2 * lp + rp + k),
+        convk_reference, convk_oracle)
 for _k, _kn, _iw, _lp, _rp, _T in ((ol.U8, "u8", 15, 0, 0, 7), (ol.U8, "u8", 14, 0, 1, 7), (ol.S8, "s8", 13, 1, 1, 7),
                                    (ol.U8, "u8", 21, 1, 1, 7)):
     CASES["depthwise_s2_%s_w%d_l%d_r%d" % (_kn, _iw, _lp, _rp)] = (

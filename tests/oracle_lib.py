@@ -116,6 +116,8 @@ def ref_kernels():
         lib.ref_u8s8_gemm.argtypes = [ci, ci, ci, ci, ci, fl, fl, fl, vp, vp, vp, vp, vp, vp]
         lib.ref_u8s8_depthwise.argtypes = [ci] * 14 + [fl, fl, vp, vp, vp, vp, vp]
         lib.ref_u8s8_conv3x3.argtypes = [ci] * 11 + [fl, fl, vp, vp, vp, vp, vp, vp]
+        if hasattr(lib, "ref_u8s8_convk"):
+            lib.ref_u8s8_convk.argtypes = [ci] * 13 + [fl, fl, vp, vp, vp, vp, vp, vp]
         if hasattr(lib, "ref_u8s8_conv3x3_s2"):
             lib.ref_u8s8_conv3x3_s2.argtypes = [ci] * 13 + [fl, fl, vp, vp, vp, vp, vp, vp]
             lib.ref_u8s8_depthwise_s2.argtypes = [ci] * 14 + [fl, fl, vp, vp, vp, vp, vp]

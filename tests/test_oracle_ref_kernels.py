@@ -359,3 +359,32 @@ def test_wino_output_transform_with_sum_bits(A, kind, with_bias, with_relu, bord
                     assert np.float32(r.value).view(np.uint32) == out[i, j, c].view(np.uint32), (i, j, c)
                 else:
                     assert np_kind(q) == out[i, j, c], (i, j, c, q, out[i, j, c], r.value)
+
+
+# ---- 5x5 / 7x7: the reference's generic k x k micro-kernel template ---------------------------------------
+@pytest.mark.parametrize("kind", [ol.F32, ol.U8, ol.S8])
+@pytest.mark.parametrize("K,S,iw,lp,rp", [(5, 1, 7, 2, 2), (7, 1, 7, 3, 3), (5, 2, 15, 1, 1), (7, 2, 14, 3, 2), (7, 2, 14, 2, 3)])
+def test_conv_kxk_kernel(kind, K, S, iw, lp, rp):
+    """The oracle's k x k path against the compiled template on the pad sets for which the template is
+    the convolution (stride 1: k/2 on both sides; stride 2: (k/2, k/2 - 1) bound as S2_LLP, or
+    (k/2 - 1, k/2)): every shape of the reference's tuned runs, ResNet's 7x7 s2 first layer included."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    import cases
+    d = cases.convk_inputs(kind, K, S, iw, lp, rp, 900 + K + S + iw + kind)
+    got, exp = cases.convk_oracle(d), cases.convk_reference(d, ref)
+    assert got.dtype == exp.dtype
+    assert np.array_equal(np.ascontiguousarray(got).view(np.uint8), np.ascontiguousarray(exp).view(np.uint8))
+
+
+def test_conv_kxk_template_is_not_the_convolution_for_other_pad_sets():
+    """Why the k x k golden cases stop where they do: with pads (2, 2) at stride 2 the 7x7 template differs
+    from the convolution in its second-to-last column only (a valid tap dropped), which the oracle and
+    the product do not imitate."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    import cases
+    d = cases.convk_inputs(ol.S8, 7, 2, 15, 2, 2, 77)
+    got, exp = cases.convk_oracle(d).reshape(7, 7, 16), cases.convk_reference(d, ref).reshape(7, 7, 16)
+    cols = np.unique(np.argwhere(got != exp)[:, 1])
+    assert list(cols) == [5]
