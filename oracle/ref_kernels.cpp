@@ -305,7 +305,8 @@ int ref_u8s8_convk(int K, int S, int out_kind, int I2, int ih, int iw, int oh, i
   }
   CV_CASE(5, 1, 0, float) CV_CASE(5, 1, 1, uint8_t) CV_CASE(5, 1, 2, int8_t)
   CV_CASE(7, 2, 0, float) CV_CASE(7, 2, 1, uint8_t) CV_CASE(7, 2, 2, int8_t)
-  CV_CASE(5, 2, 1, uint8_t) CV_CASE(7, 1, 2, int8_t)
+  CV_CASE(5, 2, 0, float) CV_CASE(5, 2, 1, uint8_t) CV_CASE(5, 2, 2, int8_t)
+  CV_CASE(7, 1, 0, float) CV_CASE(7, 1, 1, uint8_t) CV_CASE(7, 1, 2, int8_t)
 #undef CV_CASE
   return -1;
 }
