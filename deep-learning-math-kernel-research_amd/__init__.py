@@ -75,6 +75,7 @@ def _load():
     lib.ehip_conv_query.argtypes = [vp, ci, vp, ctypes.POINTER(sz)]
     lib.ehip_quantize_input_u8.argtypes = [vp, vp, sz, fl, fl, vp]
     lib.ehip_wino_tinput_range.argtypes = [ctypes.POINTER(ConvDesc), vp, ctypes.POINTER(fl), ctypes.POINTER(fl)]
+    lib.ehip_wino_tinput_range_noalloc.argtypes = [ctypes.POINTER(ConvDesc), vp, vp, vp]
     lib.ehip_reorder_nchw_to_blocked.argtypes = [vp, vp, ci, ci, ci, ci, ci, vp]
     lib.ehip_reorder_blocked_to_nchw.argtypes = [vp, vp, ci, ci, ci, ci, ci, vp]
     lib.ehip_reorder_oihw_to_blocked.argtypes = [vp, vp, ci, ci, ci, ci, vp]
@@ -87,7 +88,7 @@ lib = _load()
 EXPORTED_SYMBOLS = (
     "ehip_init", "ehip_last_error", "ehip_conv_create", "ehip_conv_destroy", "ehip_conv_prepare",
     "ehip_conv_execute", "ehip_conv_execute_repeat", "ehip_conv_query", "ehip_conv_kernel_name", "ehip_quantize_input_u8",
-    "ehip_wino_tinput_range", "ehip_reorder_nchw_to_blocked", "ehip_reorder_blocked_to_nchw",
+    "ehip_wino_tinput_range", "ehip_wino_tinput_range_noalloc", "ehip_reorder_nchw_to_blocked", "ehip_reorder_blocked_to_nchw",
     "ehip_reorder_oihw_to_blocked", "ehip_probe_mfma_i8",
 )
 
@@ -190,6 +191,11 @@ def wino_tinput_range(desc, input):
     mn, mx = ctypes.c_float(), ctypes.c_float()
     _check(lib.ehip_wino_tinput_range(ctypes.byref(desc), _ptr(input), ctypes.byref(mn), ctypes.byref(mx)))
     return mn.value, mx.value
+
+
+def wino_tinput_range_noalloc(desc, input, minmax_out, stream=0):
+    """min / max into two floats of device memory (minmax_out), asynchronous, no device allocation"""
+    _check(lib.ehip_wino_tinput_range_noalloc(ctypes.byref(desc), _ptr(input), _ptr(minmax_out), ctypes.c_void_p(stream)))
 
 
 def probe_mfma_i8(workgroups, iters, out, stream=0):

@@ -460,6 +460,9 @@ EHIP_API int ehip_init(int device)
   HIP_TRY(hipGetDeviceProperties(&prop, device));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(EHIP_GENERAL_ERROR, std::string("this library is built for gfx950 only, device is ") + prop.gcnArchName);
+  // the device's address of the static range scratch, so that the first allocation-free call need not ask
+  unsigned *scratch_dev = nullptr;
+  HIP_TRY(wino_range_scratch(&scratch_dev));
   return EHIP_OK;
 }
 
@@ -791,35 +794,58 @@ EHIP_API int ehip_quantize_input_u8(void *dst_dev, const void *src_dev, size_t c
   return EHIP_OK;
 }
 
-EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev, float *min_out,
-                                    float *max_out)
+// shared by the two range entry points: descriptor checks and the kernel's arguments
+static int range_args(const ehip_conv_desc_t *desc, const void *input_dev, WinoArgs *w)
 {
-  if (!desc || !input_dev || !min_out || !max_out) return fail(EHIP_GENERAL_ERROR, "null argument");
+  if (!desc || !input_dev) return fail(EHIP_GENERAL_ERROR, "null argument");
   const ehip_conv_desc_t &d = *desc;
   if (d.kh != 3 || d.kw != 3 || d.stride_h != 1 || d.stride_w != 1 ||
       (d.input_type != EHIP_F32 && d.input_type != EHIP_U8) ||
       (d.input_fmt != EHIP_NCHW16C && !(d.input_fmt == EHIP_NHWC && d.ic % 16 == 0)))
     return fail(EHIP_UNIMPLEMENTED, "tinput range: fp32 or u8 3x3 stride-1 layers, nChw16c or nhwc without a channel tail");
   if (d.tile_size != 0 && (d.tile_size < 4 || d.tile_size > 6)) return fail(EHIP_UNIMPLEMENTED, "Unimplemented tile size");
-  WinoArgs w = make_wino_args(d, up(d.ic, 16) / 16, up(d.oc, 16) / 16);
-  w.in = input_dev;
+  if (d.n < 1 || d.ic < 1 || d.oh < 1 || d.ow < 1 || d.ih < 1 || d.iw < 1) return fail(EHIP_GENERAL_ERROR, "tinput range: empty tensor");
+  *w = make_wino_args(d, up(d.ic, 16) / 16, up(d.oc, 16) / 16);
+  if ((long long)w->nt * d.n >= (1ll << 31) / 64) return fail(EHIP_UNIMPLEMENTED, "tinput range: too many tiles");
+  if (w->ic2 > 65535) return fail(EHIP_UNIMPLEMENTED, "tinput range: more than 65535 x 16 input channels");
+  w->in = input_dev;
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev, float *min_out,
+                                    float *max_out)
+{
+  if (!min_out || !max_out) return fail(EHIP_GENERAL_ERROR, "null argument");
+  WinoArgs w;
+  int rc = range_args(desc, input_dev, &w);
+  if (rc != EHIP_OK) return rc;
+  // per-unit partial results and, behind them, the two floats of the result
   unsigned *mm = nullptr;
-  HIP_TRY(hipMalloc(reinterpret_cast<void **>(&mm), 2 * sizeof(unsigned)));
-  const unsigned init[2] = {0xffffffffu, 0u};
-  hipError_t e = hipMemcpy(mm, init, sizeof(init), hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = launch_wino_range(w, d.ic, mm, nullptr);
-  unsigned res[2] = {0, 0};
-  if (e == hipSuccess) e = hipMemcpy(res, mm, sizeof(res), hipMemcpyDeviceToHost);
+  HIP_TRY(hipMalloc(reinterpret_cast<void **>(&mm), (2 * (size_t)w.ic2 + 2) * sizeof(unsigned)));
+  hipError_t e = launch_wino_range(w, desc->ic, mm, reinterpret_cast<float *>(mm + 2 * (size_t)w.ic2), nullptr);
+  float res[2] = {0.f, 0.f};
+  if (e == hipSuccess) e = hipMemcpy(res, mm + 2 * (size_t)w.ic2, sizeof(res), hipMemcpyDeviceToHost);
   (void)hipFree(mm);
   HIP_TRY(e);
-  auto ord2f = [](unsigned u) {
-    u = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
-    float f;
-    memcpy(&f, &u, 4);
-    return f;
-  };
-  *min_out = ord2f(res[0]);
-  *max_out = ord2f(res[1]);
+  *min_out = res[0];
+  *max_out = res[1];
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_wino_tinput_range_noalloc(const ehip_conv_desc_t *desc, const void *input_dev, float *minmax_out_dev,
+                                            void *hip_stream)
+{
+  if (!minmax_out_dev) return fail(EHIP_GENERAL_ERROR, "null argument");
+  WinoArgs w;
+  int rc = range_args(desc, input_dev, &w);
+  if (rc != EHIP_OK) return rc;
+  if (w.ic2 > kRangeScratchUnits)
+    return fail(EHIP_UNIMPLEMENTED, "tinput range without allocation: at most " + std::to_string(kRangeScratchUnits * 16) +
+                " input channels (the static scratch holds " + std::to_string(kRangeScratchUnits) + " units); got " +
+                std::to_string(desc->ic));
+  unsigned *partials = nullptr;
+  HIP_TRY(wino_range_scratch(&partials));
+  HIP_TRY(launch_wino_range(w, desc->ic, partials, minmax_out_dev, static_cast<hipStream_t>(hip_stream)));
   return EHIP_OK;
 }
 

@@ -145,7 +145,13 @@ hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s);
 hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s);
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s);
 hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s);
-hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_dev, hipStream_t s);
+// min / max of the transformed input: partials = 2 * a.ic2 dwords of device scratch, result = two floats
+// of device memory (min, max); three launches on `s`, nothing else
+hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *partials, float *minmax_out_dev, hipStream_t s);
+// the current device's copy of the library's static range scratch (2 * kRangeScratchUnits dwords);
+// resolved once per device, no allocation
+constexpr int kRangeScratchUnits = 4096;   // 16-channel units: up to 65536 input channels, 32 KB
+hipError_t wino_range_scratch(unsigned **ptr);
 
 // weight preparation
 hipError_t launch_prepare_direct(const float *w_blocked, const float *bias, int oc, int ic, int kh, int kw,

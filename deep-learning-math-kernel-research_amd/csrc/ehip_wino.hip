@@ -23,6 +23,8 @@
 // with -ffp-contract=off.  Tiles that touch the zero frame go through the reference's "border"
 // kernel, whose compiled form rounds the products of raw inputs in the column pass (and one
 // product of the last row pass) separately.
+#include <mutex>
+
 #include "ehip_internal.hpp"
 #include "ehip_wino_tiles.hpp"
 
@@ -160,9 +162,10 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   for (int e = 0; e < AA; ++e) dst[e * pos_stride] = packed[e];
 }
 
-// minmax_dev[0] = ordered-min, [1] = ordered-max (see f2ord); real channels only
+// partials[2 * c2] = ordered-min, [2 * c2 + 1] = ordered-max (see f2ord) of 16-channel unit c2; real
+// channels only.  One pair per unit keeps the atomics of different units on different addresses.
 template <typename Cell, int A = 6>
-__global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic_real, unsigned *minmax_dev)
+__global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic_real, unsigned *partials)
 {
   constexpr int AA = A * A;
   const int q = threadIdx.x & 3;
@@ -194,8 +197,36 @@ __global__ __launch_bounds__(kBlock) void k_wino_tinput_range(WinoArgs a, int ic
     mx = omx > mx ? omx : mx;
   }
   if ((threadIdx.x & 63) == 0) {
-    atomicMin(&minmax_dev[0], f2ord(mn));
-    atomicMax(&minmax_dev[1], f2ord(mx));
+    atomicMin(&partials[2 * c2], f2ord(mn));
+    atomicMax(&partials[2 * c2 + 1], f2ord(mx));
+  }
+}
+
+// every pair starts as (largest, smallest) ordered value
+__global__ __launch_bounds__(kBlock) void k_wino_range_init(unsigned *partials, int units)
+{
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < 2 * units) partials[i] = (i & 1) ? 0u : 0xffffffffu;
+}
+
+// one wave: min / max over the units' pairs, back to floats, to out[0] = min, out[1] = max
+__global__ __launch_bounds__(kWave) void k_wino_range_finish(const unsigned *partials, int units, float *out)
+{
+  unsigned mn = 0xffffffffu, mx = 0u;
+  for (int i = threadIdx.x; i < units; i += kWave) {
+    const unsigned a = partials[2 * i], b = partials[2 * i + 1];
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned omn = __shfl_xor(mn, off), omx = __shfl_xor(mx, off);
+    mn = omn < mn ? omn : mn;
+    mx = omx > mx ? omx : mx;
+  }
+  if (threadIdx.x == 0) {
+    out[0] = __uint_as_float((mn & 0x80000000u) ? (mn & 0x7fffffffu) : ~mn);
+    out[1] = __uint_as_float((mx & 0x80000000u) ? (mx & 0x7fffffffu) : ~mx);
   }
 }
 
@@ -550,15 +581,48 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s)
   return hipGetLastError();
 }
 
-hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *minmax_dev, hipStream_t s)
+// partials: 2 * a.ic2 dwords of device memory; minmax_out_dev: two floats of device memory
+hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *partials, float *minmax_out_dev, hipStream_t s)
 {
+  hipLaunchKernelGGL(k_wino_range_init, dim3((2 * a.ic2 + kBlock - 1) / kBlock), dim3(kBlock), 0, s, partials, a.ic2);
   dim3 grid((a.t + 63) / 64, a.ic2);
   void (*kern)(WinoArgs, int, unsigned *) = nullptr;
   if (a.tile == 4) kern = a.in_u8 ? k_wino_tinput_range<unsigned, 4> : k_wino_tinput_range<float4, 4>;
   else if (a.tile == 5) kern = a.in_u8 ? k_wino_tinput_range<unsigned, 5> : k_wino_tinput_range<float4, 5>;
   else kern = a.in_u8 ? k_wino_tinput_range<unsigned, 6> : k_wino_tinput_range<float4, 6>;
-  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a, ic_real, minmax_dev);
+  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a, ic_real, partials);
+  hipLaunchKernelGGL(k_wino_range_finish, dim3(1), dim3(kWave), 0, s, partials, a.ic2, minmax_out_dev);
   return hipGetLastError();
+}
+
+// ---- the range without an allocation ------------------------------------------------------------
+// The per-unit partial results of the range live in this array instead of in memory from hipMalloc.
+// Every GPU of the process holds its own copy at its own address; host code never uses the array's
+// name as a pointer, only the address hipGetSymbolAddress returned for the device in question.
+static __device__ __align__(256) unsigned scratch[2 * kRangeScratchUnits];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned *g_scratch_ptr[kMaxDevices];   // by device ordinal; null until resolved
+}  // namespace
+
+hipError_t wino_range_scratch(unsigned **ptr)
+{
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = static_cast<unsigned *>(p);
+  }
+  *ptr = g_scratch_ptr[dev];
+  return hipSuccess;
 }
 
 }  // namespace ehip

@@ -146,6 +146,19 @@ EHIP_API int ehip_quantize_input_u8(void *dst_dev, const void *src_dev, size_t c
 EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev,
                                     float *min_out, float *max_out);
 
+/* No counterpart in the reference.  ehip_wino_tinput_range for callers that cannot allocate device
+ * memory (a stream under HIP graph capture, a serving loop or a harness that forbids hipMalloc): the
+ * per-unit partial minima / maxima go to a static device array of the library (32 KB on every GPU the
+ * library runs on, held until the process ends) instead of to memory from hipMalloc, the result goes to
+ * minmax_out_dev[0] = min, [1] = max (two floats of DEVICE memory owned by the caller), and the three
+ * kernels are enqueued on `hip_stream` without a synchronisation.  Calls no hipMalloc / hipFree.
+ * Limit: at most 65536 input channels (4096 units of 16), else EHIP_UNIMPLEMENTED.  All calls on one
+ * GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;
+ * calls on one stream are safe, each one re-initialises what it uses.  ehip_init(device) resolves the
+ * array's address for the device ahead of the first call (otherwise the first call does). */
+EHIP_API int ehip_wino_tinput_range_noalloc(const ehip_conv_desc_t *desc, const void *input_dev,
+                                            float *minmax_out_dev, void *hip_stream);
+
 /* Device-side layout reorders with the index maps of src/elx_reorder.cpp:35-93
  * (elem_size 1 or 4).  nchw <-> nChw16c and oihw -> OIhw16i16o; channel tails are zero-filled. */
 EHIP_API int ehip_reorder_nchw_to_blocked(void *dst_dev, const void *src_dev, int elem_size, int n,
