@@ -36,7 +36,17 @@ FLAGS = [
 ]
 
 
-def build(verbose=True, jobs=8):
+def _stale(obj, src):
+    """an object is reused only when it is newer than its source and every header"""
+    if not os.path.exists(obj):
+        return True
+    deps = [src] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")] + \
+        [os.path.join(ROOT, "include", f) for f in os.listdir(os.path.join(ROOT, "include"))] + [__file__]
+    return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps)
+
+
+def build(verbose=True, jobs=8, incremental=False):
+    """incremental: recompile only what changed (development); the default compiles everything"""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
@@ -45,6 +55,8 @@ def build(verbose=True, jobs=8):
     for src in SOURCES:
         obj = os.path.join(objdir, src + ".o")
         objs.append(obj)
+        if incremental and not _stale(obj, os.path.join(CSRC, src)):
+            continue
         cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -84,5 +96,5 @@ def _wait(procs):
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv)
     print("built", LIB)

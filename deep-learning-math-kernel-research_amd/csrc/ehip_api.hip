@@ -235,6 +235,9 @@ int classify(ehip_conv *c)
       return fail(EHIP_UNIMPLEMENTED, "winograd: only the int8 implementation (execution_mode 0xa1xx) is built");
     if (out_q && (d.output_scale == kNoCali || d.output_z == kNoCali || d.output_scale == 0.0f))
       return fail(EHIP_GENERAL_ERROR, "output_quant is not set");
+    // the reference stops here (el_error, src/eld_conv.cpp:223-228): its transform never reads the zero point
+    if (u8_user && d.input_z != 0.0f)
+      return fail(EHIP_UNIMPLEMENTED, "Support abs-max scaling for input only in Conv Winograd ...");
     if (d.tile_size == 0) d.tile_size = wino_auto_tile(d);
     // src/eld_conv.cpp:257-270: the int8 executor exists for tile sizes 4, 5 and 6
     if (d.tile_size < 4 || d.tile_size > 6) return fail(EHIP_UNIMPLEMENTED, "Unimplemented tile size");

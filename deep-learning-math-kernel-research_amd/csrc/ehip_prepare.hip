@@ -45,7 +45,9 @@ __device__ __forceinline__ void fold(const FoldParams &p, float absmax, float ws
     s = p.in_S * w_S * p.out_repS;
     z = __builtin_fmaf(-(p.in_z * wsum), s, __builtin_fmaf(bias, p.out_repS, p.out_z));
   }
-  if (p.with_sum) z = __builtin_fmaf(-p.sum_z, p.sum_S, z);
+  // sum_z * sum_S is a product of two scalars that the reference's compiled code rounds on its own and
+  // then subtracts (src/elx_int8_conv_direct_1x1.cpp:349-353: vmulss, broadcast, vsubps) -- two roundings
+  if (p.with_sum) z = z - p.sum_z * p.sum_S;
   *scale = s;
   *shift = z;
 }

@@ -98,8 +98,9 @@ EHIP_API const char *ehip_last_error(void);
  * A non-zero input zero point with padding is accepted by the 3/5/7 direct kernels (the shift then
  * depends on the output pixel's set of valid taps, src/elx_int8_conv_direct.cpp:227-423).  The depthwise
  * executor follows the reference: one shift of z times all nine weights, padded taps adding nothing
- * (src/elx_int8_conv_direct_depthwise.cpp:247-289); the Winograd executor, like the reference's, uses
- * the input scale only (src/elx_conv_wino_trans_input.cpp:367-368). */
+ * (src/elx_int8_conv_direct_depthwise.cpp:247-289); the Winograd executor uses the input scale only
+ * (src/elx_conv_wino_trans_input.cpp:367-368) and, like the reference's setup, refuses u8 input with a
+ * non-zero zero point (src/eld_conv.cpp:223-228). */
 EHIP_API int ehip_conv_create(const ehip_conv_desc_t *desc, ehip_conv_t **out);
 EHIP_API int ehip_conv_destroy(ehip_conv_t *conv);
 

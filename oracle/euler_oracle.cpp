@@ -65,7 +65,9 @@ inline float epilogue_f32(int32_t acc, float scale, float shift, bool with_sum, 
 }
 
 // g++ contracts `a - b * c` where b*c is (iz*wsum)*scale: the last product fuses into the
-// subtraction (src/elx_int8_conv_direct_1x1.cpp:337-343, src/elx_int8_conv_direct.cpp:410-414).
+// subtraction (src/elx_int8_conv_direct_1x1.cpp:337-343, src/elx_int8_conv_direct.cpp:410-414): the
+// reference's translation units compiled with its own flags hold vmulps (iz * wsum), vfmadd132ps
+// (bias * out_repS + out_z), vfnmadd132ps (that - product * scale) for the 1x1, k x k and depthwise folds.
 inline void fold_scale_shift(const orc_conv_params *p, float w_S, float wsum, float bias,
                              float *scale, float *shift)
 {
@@ -78,7 +80,9 @@ inline void fold_scale_shift(const orc_conv_params *p, float w_S, float wsum, fl
     s = p->in_scale * w_S * out_repS;
     z = fmaf(-(p->in_z * wsum), s, fmaf(bias, out_repS, p->out_z));
   }
-  if (p->with_sum) z = fmaf(-p->sum_z, p->sum_scale, z);
+  // `mmqf -= sum_z * sum_S` (src/elx_int8_conv_direct_1x1.cpp:349-353): both factors are broadcast scalars,
+  // g++ multiplies them once as scalars (vmulss), broadcasts and subtracts (vsubps) -- two roundings
+  if (p->with_sum) z = z - p->sum_z * p->sum_scale;
   *scale = s;
   *shift = z;
 }

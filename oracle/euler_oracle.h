@@ -14,17 +14,24 @@
  *     (g++ -O2, default -ffp-contract=fast) performs one fused rounding; this file is built
  *     with -ffp-contract=off so nothing else fuses.
  *
- * Pinning status (what checks each part; see tests/test_oracle_*.py):
+ * Pinning status (what checks each part; see tests/test_oracle_*.py, tests/test_golden.py):
  *   - fused-rounding pattern of the GEMM/conv/depthwise epilogues, depthwise floor/round split,
- *     unsigned saturation, Winograd F(4,3) input/weights/output transforms: pinned against the
+ *     unsigned saturation, Winograd tile transforms (tile sizes 4, 5, 6): pinned against the
  *     reference's own kernel templates compiled from /root/reference (oracle/ref_kernels.cpp).
+ *   - Winograd glue -- tile gather and border handling, the quantization fma(V, in_S / tin_S, ceil(z)) ->
+ *     unsigned conversion -> saturation, the calibration range, per-(position, oc) weight quantization,
+ *     scale and shift: pinned against the reference's two transform translation units compiled from
+ *     /root/reference (oracle/ref_wino_glue.cpp), including inputs searched so that a dropped fusion
+ *     changes the code.
  *   - integer contractions: pinned by brute-force integer convolution in numpy.
- *   - weight quantization (abs-max, (w*127)/absmax, round-half-even) and scale/shift folding:
- *     pure IEEE mul/div/rint sequences, pinned by an independent numpy float32 evaluation.
- *     For input_z != 0 or sum_z != 0 the folding contains a product-difference whose fusion
- *     is compiler-chosen and no compiled reference code is available for it here:
- *     PARITY UNPINNED for non-zero input/sum zero points (all configured layers use 0).
+ *   - direct / depthwise weight quantization (abs-max, (w*127)/absmax, round-half-even) and scale/shift
+ *     folding with every zero point non-zero, and the per-pixel shift rows of a zero point with padding:
+ *     the executors that hold these folds do not link without tables the reference's build generates, so
+ *     they are pinned by an independent long-double evaluation of the contraction pattern their compiled
+ *     objects hold (vfmadd bias*repS+z, vfnmadd of the zero-point term, unfused sum_z*sum_S), on data
+ *     checked to tell that pattern from its neighbours.
  *   - reorders: closed-form index maps, pinned by numpy transposes.
+ *   - not pinned by anything but the source: the ORDER of exact integer additions in the executors.
  */
 #ifndef EULER_ORACLE_H
 #define EULER_ORACLE_H

@@ -682,3 +682,157 @@ for _A in (6, 4, 5):
             CASES["wino%d_output_sum_%s_b%d_r%d_border%d" % (_A, _kn, _b, _r, _bd)] = (
                 lambda A=_A, k=_k, b=_b, r=_r, bd=_bd: winos_out_inputs(A, k, b, r, bd, 800 + 16 * k + 8 * b + bd + A),
                 winos_out_reference, winos_out_oracle)
+
+
+# ---- Winograd quantization glue: whole small layers through the reference's transform CLASSES ------
+# (src/elx_conv_wino_trans_input.cpp:599-654: tile gather, interior / border kernels, a * mrepS + mz ->
+#  cvt_roundps_epu32 -> saturate; src/elx_conv_wino_trans_weights.cpp:175-195,437-535: U = G g Gt, per
+#  (position, oc) abs-max quantization, scale = absmax / 127 * tin_S, shift = -sum * scale * ceil(tin_z)).
+# The reference side is the pair of translation units compiled from the reference tree
+# (oracle/ref_wino_glue.cpp); the `ref` argument of the other cases is not used here.
+def glue_in_inputs(A, in_u8, n, ic, hw, pad, T, tin_scale, tin_z, seed, lo=-1.0, hi=2.0):
+    rng = np.random.default_rng(seed)
+    if in_u8:
+        x = rng.integers(0, 256, (n, ic, hw, hw)).astype(np.float32)
+    else:
+        x = rng.uniform(lo, hi, (n, ic, hw, hw)).astype(np.float32)
+    return dict(A=np.int32(A), in_u8=np.int32(in_u8), n=np.int32(n), ic=np.int32(ic), hw=np.int32(hw), pad=np.int32(pad),
+                T=np.int32(T), in_scale=np.float32(1.0 / 255.0 if in_u8 else 1.0), tin_scale=np.float32(tin_scale),
+                tin_z=np.float32(tin_z), x=ol.to_blocked(x))
+
+
+def _glue_params(d):
+    hw, pad = int(d["hw"]), int(d["pad"])
+    return ol.make_params(int(d["n"]), int(d["ic"]), 16, hw, hw, 3, 3, pad, out_type=ol.F32, in_scale=float(d["in_scale"]),
+                          tin_scale=float(d["tin_scale"]), tin_z=float(d["tin_z"]), wino_tile=int(d["A"]))
+
+
+def glue_in_reference(d, ref):
+    glue = ol.ref_wino_glue()
+    assert glue is not None, "oracle/_ref/libeuler_ref_wino_glue.so is not built"
+    p = _glue_params(d)
+    A, t = int(d["A"]), ol.wino_tiles(p)
+    out = np.zeros((A * A, ol.up16(p.ic) // 16, t, 16), np.uint8)
+    x = _al(d["x"].astype(np.uint8) if int(d["in_u8"]) else d["x"])
+    assert glue.ref_wino_glue_trans_input(A, int(d["in_u8"]), p.n, p.ic, p.ih, p.iw, p.oh, p.ow, p.pad_t, p.pad_l, int(d["T"]),
+                                          float(d["in_scale"]), float(d["tin_scale"]), float(d["tin_z"]), ol.ptr(x),
+                                          ol.ptr(out)) == 0
+    return out
+
+
+def glue_in_oracle(d):
+    return ol.wino_trans_input(_glue_params(d), np.ascontiguousarray(d["x"], np.float32))
+
+
+def glue_range_reference(d, ref):
+    glue = ol.ref_wino_glue()
+    assert glue is not None, "oracle/_ref/libeuler_ref_wino_glue.so is not built"
+    p = _glue_params(d)
+    A, t = int(d["A"]), ol.wino_tiles(p)
+    tin = np.zeros((A * A, ol.up16(p.ic) // 16, t, 16), np.float32)
+    x = _al(d["x"])
+    assert glue.ref_wino_glue_trans_input_f32(A, p.n, p.ic, p.ih, p.iw, p.oh, p.ow, p.pad_t, p.pad_l, int(d["T"]), ol.ptr(x),
+                                              ol.ptr(tin)) == 0
+    # min / max over the transformed input as the harness takes it (tests/elt_conv_utils.cpp:222-262); the
+    # zero-filled channel tail of the last 16-channel unit is not part of the tensor
+    c = np.arange(tin.shape[1] * 16).reshape(tin.shape[1], 1, 16) < p.ic
+    real = tin[np.broadcast_to(c[None], tin.shape)]
+    return np.array([real.min(), real.max()], np.float32)
+
+
+def glue_range_oracle(d):
+    mn, mx = ol.wino_tinput_range(_glue_params(d), np.ascontiguousarray(d["x"], np.float32))
+    return np.array([mn, mx], np.float32)
+
+
+def glue_w_inputs(A, ic, oc, tin_scale, tin_z, seed):
+    rng = np.random.default_rng(seed)
+    w = rng.normal(0, 0.02, (oc, ic, 3, 3)).astype(np.float32)
+    return dict(A=np.int32(A), ic=np.int32(ic), oc=np.int32(oc), tin_scale=np.float32(tin_scale), tin_z=np.float32(tin_z),
+                w=ol.weights_to_blocked(w))
+
+
+def _pack3(twq, tscale, tshift):
+    return np.concatenate([np.ascontiguousarray(a).ravel().view(np.uint8) for a in (twq, tscale, tshift)])
+
+
+def glue_w_reference(d, ref):
+    glue = ol.ref_wino_glue()
+    assert glue is not None, "oracle/_ref/libeuler_ref_wino_glue.so is not built"
+    A, ic, oc = int(d["A"]), int(d["ic"]), int(d["oc"])
+    twq = np.zeros((A * A, ol.up16(oc), ol.up16(ic)), np.int8)
+    tscale = np.zeros((A * A, ol.up16(oc)), np.float32)
+    tshift = np.zeros((A * A, ol.up16(oc)), np.float32)
+    w = _al(d["w"])
+    assert glue.ref_wino_glue_trans_weights(A, ic, oc, float(d["tin_scale"]), float(d["tin_z"]), ol.ptr(w), ol.ptr(twq),
+                                            ol.ptr(tscale), ol.ptr(tshift)) == 0
+    return _pack3(twq, tscale, tshift)
+
+
+def glue_w_oracle(d):
+    p = ol.make_params(1, int(d["ic"]), int(d["oc"]), 8, 8, 3, 3, 1, out_type=ol.F32, in_scale=1.0,
+                       tin_scale=float(d["tin_scale"]), tin_z=float(d["tin_z"]), wino_tile=int(d["A"]))
+    return _pack3(*ol.wino_prepare(p, np.ascontiguousarray(d["w"])))
+
+
+def tie_values(m, z):
+    """f32 values v for which fma(v, m, z) (one rounding) and (v * m) + z (two roundings) land on different
+    sides of a rounding boundary of the final float -> integer conversion: one candidate search around every
+    code k + 0.5.  Evaluated in 64-bit-mantissa long doubles, where v * m + z is exact."""
+    L = np.longdouble
+    m, z, out = np.float32(m), np.float32(z), []
+    for k in range(0, 255):
+        base = np.float32((np.float64(k) + 0.5 - np.float64(z)) / np.float64(m))
+        bits = np.array([base], np.float32).view(np.int32)[0]
+        cand = (bits + np.arange(-64, 65, dtype=np.int32)).view(np.float32)
+        fused = (cand.astype(L) * L(m) + L(z)).astype(np.float32)
+        unfused = (cand * m).astype(np.float32) + z
+        hit = np.rint(fused) != np.rint(unfused)
+        out.extend(cand[hit][:1].tolist())
+    return np.array(out, np.float32)
+
+
+def glue_ties_sites(A, hw):
+    """pixels that are element (A-1, A-1) of an even-numbered tile and element (1, 1) of none that holds
+    another such pixel (pad 1): rows / columns M * (2a + 1)"""
+    M = A - 2
+    r = np.arange(M, hw, 2 * M)
+    return [(int(h), int(w)) for h in r for w in r]
+
+
+def glue_ties_inputs(A, tin_scale, tin_z):
+    """all-zero image except single pixels that carry tie_values: the transform hands such a value through
+    unchanged to position (A-1, A-1) of its tile, so the quantization a * mrepS + mz sees exactly it"""
+    M = A - 2
+    hw = 8 * M
+    v = tie_values(np.float32(1.0) * (np.float32(1.0) / np.float32(tin_scale)), np.ceil(np.float32(tin_z)))
+    x = np.zeros((1, 16, hw, hw), np.float32)
+    sites = glue_ties_sites(A, hw)
+    for i, val in enumerate(v[:16 * len(sites)]):
+        h, w = sites[i % len(sites)]
+        x[0, i // len(sites), h, w] = val
+    return dict(A=np.int32(A), in_u8=np.int32(0), n=np.int32(1), ic=np.int32(16), hw=np.int32(hw), pad=np.int32(1),
+                T=np.int32(6), in_scale=np.float32(1.0), tin_scale=np.float32(tin_scale), tin_z=np.float32(tin_z),
+                x=ol.to_blocked(x))
+
+
+for _A in (6, 4, 5):
+    # values chosen so that a dropped fusion in a * mrepS + mz changes the code
+    CASES["wino_glue_input%d_ties" % _A] = (lambda A=_A: glue_ties_inputs(A, 0.0283, 40.37), glue_in_reference, glue_in_oracle)
+    # f32 input with negative values, ragged last block of tiles (T = 5), every border kind (the image is not
+    # a multiple of the output tile), a zero point with a fractional part (ceil) placed so that part of the
+    # values round below zero (the float -> unsigned conversion's 255) and part saturate at 255
+    CASES["wino_glue_input%d_f32" % _A] = (lambda A=_A: glue_in_inputs(A, 0, 2, 24, 10, 1, 5, 0.0283, 40.37, 900 + A),
+                                           glue_in_reference, glue_in_oracle)
+    # no padding: only right / bottom borders
+    CASES["wino_glue_input%d_f32_nopad" % _A] = (lambda A=_A: glue_in_inputs(A, 0, 1, 16, 11, 0, 4, 0.05, 63.5, 910 + A),
+                                                 glue_in_reference, glue_in_oracle)
+    # u8 codes as input (U8F32*F32 user types): in_S / tin_S enters the factor
+    CASES["wino_glue_input%d_u8" % _A] = (lambda A=_A: glue_in_inputs(A, 1, 2, 32, 9, 1, 7, 0.1171, 101.2, 920 + A),
+                                          glue_in_reference, glue_in_oracle)
+    CASES["wino_glue_range%d" % _A] = (lambda A=_A: glue_in_inputs(A, 0, 2, 24, 10, 1, 5, 1.0, 0.0, 930 + A, -3.0, 5.0),
+                                       glue_range_reference, glue_range_oracle)
+    CASES["wino_glue_weights%d" % _A] = (lambda A=_A: glue_w_inputs(A, 24, 32, 0.0283, 40.37, 940 + A),
+                                         glue_w_reference, glue_w_oracle)
+    CASES["wino_glue_weights%d_negz" % _A] = (lambda A=_A: glue_w_inputs(A, 48, 16, 0.4071, -12.6, 950 + A),
+                                              glue_w_reference, glue_w_oracle)

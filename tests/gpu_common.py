@@ -34,7 +34,7 @@ class Layer:
 
     def __init__(self, n, ic, oc, hw, k=1, pad=0, stride=1, out_type=ol.U8, algorithm=None, with_sum=False,
                  depthwise=False, seed=0, w_sigma=0.05, T=0, with_bias=True, with_relu=True, relu_hi=None,
-                 in_nhwc=False, out_nhwc=False, out_hw=None, x_blocked=None, in_z=0.0):
+                 in_nhwc=False, out_nhwc=False, out_hw=None, x_blocked=None, in_z=0.0, out_z=0.0, sum_z=0.0):
         E = pkg()
         rng = np.random.default_rng(seed)
         self.E = E
@@ -77,12 +77,12 @@ class Layer:
             sum_scale = float(f32(s_r) / f32(out_scale))
         self.p = ol.make_params(n, ic, oc, hw, hw, k, k, pad, stride, g=g, out_type=out_type, with_bias=with_bias,
                                 with_relu=with_relu, with_sum=with_sum, T=T, out_scale=out_scale, sum_scale=sum_scale,
-                                relu_hi=relu_hi, in_z=in_z)
+                                relu_hi=relu_hi, in_z=in_z, out_z=out_z, sum_z=sum_z)
         if algorithm is None:
             algorithm = E.CONV_DIRECT_1X1 if (k == 1 and out_type in (ol.U8, ol.S8, ol.S32)) else E.CONV_DIRECT
         self.desc = E.make_desc(n, ic, oc, hw, hw, k, k, pad, stride, g=g, algorithm=algorithm,
                                 output_type=out_type, with_bias=with_bias, with_relu=with_relu, with_ip_sum=with_sum,
-                                output_quant=(out_scale, 0.0), sum_quant=(sum_scale, 0.0),
+                                output_quant=(out_scale, out_z), sum_quant=(sum_scale, sum_z),
                                 relu_bound=(0.0, relu_hi), flatting_t=T, input_quant=(1.0 / 255.0, in_z))
         if out_hw is not None:
             # output size given by the caller: right / bottom pads follow from it, as the reference

@@ -13,6 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 ORACLE_SO = os.path.join(ORACLE_DIR, "libeuler_oracle.so")
 REF_SO = os.path.join(ORACLE_DIR, "_ref", "libeuler_ref_kernels.so")
+REF_GLUE_SO = os.path.join(ORACLE_DIR, "_ref", "libeuler_ref_wino_glue.so")
 
 F32, U8, S8, S32 = 1, 3, 4, 5
 NP_OF = {F32: np.float32, U8: np.uint8, S8: np.int8, S32: np.int32}
@@ -70,6 +71,7 @@ def ptr(a):
 
 _oracle = None
 _ref = None
+_ref_glue = None
 
 
 def oracle():
@@ -134,6 +136,29 @@ def ref_kernels():
             lib.ref_wino_trans_output_sum.argtypes = [ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, ci, ci, fl, fl]
         _ref = lib
     return _ref
+
+
+def ref_wino_glue():
+    """The reference's Winograd input / weight transform classes with their quantization glue
+    (src/elx_conv_wino_trans_input.cpp, src/elx_conv_wino_trans_weights.cpp compiled from the reference
+    tree by oracle/Makefile), or None where oracle/_ref was not built or the host lacks AVX-512."""
+    global _ref_glue
+    if _ref_glue is None:
+        if not os.path.exists(REF_GLUE_SO):
+            return None
+        try:
+            flags = open("/proc/cpuinfo").read()
+        except OSError:
+            flags = ""
+        if "avx512_vnni" not in flags or "avx512bw" not in flags:
+            return None
+        lib = ctypes.CDLL(REF_GLUE_SO)
+        fl, ci, vp = ctypes.c_float, ctypes.c_int, ctypes.c_void_p
+        lib.ref_wino_glue_trans_input.argtypes = [ci] * 11 + [fl, fl, fl, vp, vp]
+        lib.ref_wino_glue_trans_input_f32.argtypes = [ci] * 10 + [vp, vp]
+        lib.ref_wino_glue_trans_weights.argtypes = [ci, ci, ci, fl, fl, vp, vp, vp, vp]
+        _ref_glue = lib
+    return _ref_glue
 
 
 # --------------------------------------------------------------------------------------------

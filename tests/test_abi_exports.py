@@ -64,3 +64,9 @@ def test_create_rejects_bad_descriptors_without_a_gpu():
     assert pkg.lib.ehip_conv_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EHIP_UNIMPLEMENTED
     d = pkg.make_desc(1, 60, 64, 8, 8, 3, 3, pad=1, g=7, algorithm=pkg.CONV_DIRECT)
     assert pkg.lib.ehip_conv_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EHIP_GENERAL_ERROR
+    # Winograd with u8 input takes abs-max scaling only: a zero point is refused, as the reference does
+    # (src/eld_conv.cpp:223-228)
+    d = pkg.make_desc(1, 32, 32, 8, 8, 3, 3, pad=1, algorithm=pkg.CONV_WINOGRAD, input_type=pkg.U8, output_type=pkg.F32,
+                      input_quant=(0.02, 128.0), tile_size=6, wino_tinput_quant=(1.0, 0.0))
+    assert pkg.lib.ehip_conv_create(ctypes.byref(d), ctypes.byref(h)) == pkg.EHIP_UNIMPLEMENTED
+    assert b"abs-max scaling" in pkg.lib.ehip_last_error()

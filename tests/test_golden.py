@@ -33,3 +33,32 @@ def test_oracle_matches_golden(path):
     fresh = cases.CASES[name][0]()
     for k, v in fresh.items():
         assert np.array_equal(np.asarray(v), d[k]), k
+
+
+@pytest.mark.parametrize("A", [6, 4, 5])
+def test_tie_fixtures_tell_the_fused_quantization_from_the_unfused(A):
+    """wino_glue_input*_ties: every injected value reaches position (A-1, A-1) of its tile unchanged, and the
+    stored code of the reference's compiled transform is the one of fma(v, mrepS, mz) -- never that of
+    (v * mrepS) + mz, which these values were searched to separate."""
+    path = os.path.join(HERE, "golden", "wino_glue_input%d_ties.npz" % A)
+    with np.load(path, allow_pickle=False) as z:
+        d = {k: z[k] for k in z.files}
+    f32, L = np.float32, np.longdouble
+    M, hw = A - 2, int(d["hw"])
+    wt = (hw + M - 1) // M
+    m = f32(1.0) * (f32(1.0) / f32(d["tin_scale"]))
+    mz = f32(np.ceil(d["tin_z"]))
+    x = d["x"].transpose(0, 1, 4, 2, 3).reshape(1, 16, hw, hw)
+    sites = 0
+    for h, w in cases.glue_ties_sites(A, hw):
+        t = ((h + 1 - (A - 1)) // M) * wt + (w + 1 - (A - 1)) // M
+        for c in range(16):
+            v = x[0, c, h, w]
+            if v == 0:
+                continue
+            fused = int(np.clip(np.rint((L(v) * L(m) + L(mz)).astype(f32)), 0, 255))
+            unfused = int(np.clip(np.rint(f32(v * m) + mz), 0, 255))
+            assert fused != unfused
+            assert int(d["expected"][A * A - 1, 0, t, c]) == fused
+            sites += 1
+    assert sites >= 32

@@ -45,6 +45,21 @@ def test_conv1x1_sum_relu(out_type):
     run_and_compare(Layer(2, 96, 64, 14, out_type=out_type, with_sum=True, seed=5))
 
 
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
+@pytest.mark.parametrize("with_sum", [False, True])
+def test_conv1x1_every_zero_point(out_type, with_sum):
+    """input, output and sum zero points all non-zero: the folded shift (compared bit for bit with the
+    oracle's, whose contraction pattern is that of the reference's compiled fold) and the result"""
+    run_and_compare(Layer(2, 96, 256, 9, out_type=out_type, with_sum=with_sum, seed=15 + out_type, in_z=113.0, out_z=3.0,
+                          sum_z=-97.0))
+
+
+def test_conv3x3_and_depthwise_output_zero_point():
+    run_and_compare(Layer(2, 32, 64, 9, k=3, pad=0, out_type=ol.S8, seed=16, in_z=113.0, out_z=-2.0))
+    run_and_compare(Layer(2, 64, 64, 9, k=3, pad=1, out_type=ol.U8, depthwise=True, T=3, w_sigma=0.1, seed=17, in_z=37.0,
+                          out_z=2.0))
+
+
 @pytest.mark.parametrize("out_type", [ol.S32, ol.S8])
 def test_conv1x1_stride2(out_type):
     run_and_compare(Layer(2, 64, 96, 14, stride=2, out_type=out_type, with_sum=(out_type == ol.S8), seed=6))

@@ -262,3 +262,118 @@ def test_zero_point_with_padding_matches_the_real_valued_convolution(k, pad, str
         assert np.abs(got - np.clip(exp, -128 * out_scale, 127 * out_scale)).max() <= 0.5 * out_scale + 1e-4
     else:
         assert np.abs(got - exp).max() <= 2e-4 * max(1.0, np.abs(exp).max())
+
+
+# ---- scale / shift folding with non-zero zero points -------------------------------------------------
+# What the reference's translation units hold when compiled with its own flags (g++ -O2, default
+# contraction; src/elx_int8_conv_direct_1x1.cpp:324-354, src/elx_int8_conv_direct.cpp:357-419,
+# src/elx_int8_conv_direct_depthwise.cpp:261-291):
+#   scale = (in_S * w_S) * out_repS                      vmulps, vmulps
+#   t     = in_z * wsum                                  vmulps
+#   shift = fma(bias, out_repS, out_z)                   vfmadd132ps
+#   shift = fma(-t, scale, shift)                        vfnmadd132ps
+#   shift = shift - (sum_z * sum_S)   (1x1 with sum)     vmulss, vbroadcastss, vsubps: NOT fused
+# The executors themselves cannot be linked here (their kernel tables are generated by the reference's
+# build), so these folds are evaluated independently in long doubles, where a product of two floats plus a
+# float is exact, and rounded once -- and the inputs are checked to tell every other contraction apart.
+L = np.longdouble
+
+
+def _fma(a, b, c):
+    return (np.asarray(a, f32).astype(L) * np.asarray(b, f32).astype(L) + np.asarray(c, f32).astype(L)).astype(f32)
+
+
+def fold_variants(in_S, in_z, w_S, wsum, bias, rep, out_z, sum_S=None, sum_z=None):
+    """{name: (scale, shift)}: "compiled" is the reference's compiled form, the others drop or add one fusion"""
+    scale = ((f32(in_S) * w_S).astype(f32) * f32(rep)).astype(f32)
+    t = (f32(in_z) * wsum.astype(f32)).astype(f32)
+    fused_b = _fma(bias, f32(rep), f32(out_z))
+    plain_b = ((bias * f32(rep)).astype(f32) + f32(out_z)).astype(f32)
+    v = {"compiled": _fma(-t, scale, fused_b),
+         "bias_unfused": _fma(-t, scale, plain_b),
+         "zero_point_unfused": (fused_b - (t * scale).astype(f32)).astype(f32)}
+    if sum_S is not None:
+        prod = f32(f32(sum_z) * f32(sum_S))
+        c = v["compiled"]
+        v = {k: (s - prod).astype(f32) for k, s in v.items()}
+        v["sum_fused"] = _fma(f32(-sum_z), f32(sum_S), c)
+    return scale, v
+
+
+@pytest.mark.parametrize("k,with_sum,out_type", [(1, True, ol.S8), (1, True, ol.U8), (1, False, ol.U8), (3, False, ol.S8),
+                                                 (3, False, ol.U8)])
+def test_direct_fold_with_zero_points_is_the_compiled_contraction(k, with_sum, out_type):
+    rng = np.random.default_rng(70 + k + 2 * with_sum + out_type)
+    ic, oc = 48, 256
+    w = rng.normal(0, 0.05, (oc, ic, k, k)).astype(f32)
+    b = rng.normal(0, 0.7, oc).astype(f32)
+    in_S, in_z, out_S, out_z, sum_S, sum_z = 0.0173, 113.0, 0.0371, 3.0, 0.6113, -97.0
+    p = ol.make_params(1, ic, oc, 8, 8, k, k, 0, out_type=out_type, with_sum=with_sum, in_scale=in_S, in_z=in_z,
+                       out_scale=out_S, out_z=out_z, sum_scale=sum_S, sum_z=sum_z)
+    wq, scale, shift, wsum = ol.direct_prepare(p, ol.weights_to_blocked(w), b)
+    wq_np, absmax = quant_weights_numpy(w)
+    assert np.array_equal(wq, wq_np)
+    w_S = (absmax / f32(127.0)).astype(f32)
+    rep = f32(1.0) / f32(out_S)
+    exp_scale, v = fold_variants(in_S, in_z, w_S, wq_np.reshape(oc, -1).sum(axis=1), b, rep, out_z,
+                                 sum_S if with_sum else None, sum_z if with_sum else None)
+    assert np.array_equal(scale.view(np.uint32), exp_scale.view(np.uint32))
+    assert np.array_equal(shift.view(np.uint32), v["compiled"].view(np.uint32))
+    for name, alt in v.items():   # the data tells the compiled form from every neighbour
+        assert name == "compiled" or (alt.view(np.uint32) != v["compiled"].view(np.uint32)).sum() >= 4, name
+
+
+def test_depthwise_fold_with_zero_points_is_the_compiled_contraction():
+    rng = np.random.default_rng(77)
+    g = 256
+    w = rng.normal(0, 0.1, (g, 3, 3)).astype(f32)
+    b = rng.normal(0, 0.7, g).astype(f32)
+    in_S, in_z, out_S, out_z = 0.0173, 113.0, 0.0371, 3.0
+    p = ol.make_params(1, g, g, 8, 8, 3, 3, 1, g=g, out_type=ol.S8, T=4, in_scale=in_S, in_z=in_z, out_scale=out_S,
+                       out_z=out_z, relu_hi=127.0)
+    wq, scale, shift, wsum = ol.depthwise_prepare(p, w, b)
+    wq_np, absmax = quant_weights_numpy(w.reshape(g, 1, 3, 3))
+    exp_scale, v = fold_variants(in_S, in_z, (absmax / f32(127.0)).astype(f32), wq_np.reshape(g, -1).sum(axis=1), b,
+                                 f32(1.0) / f32(out_S), out_z)
+    assert np.array_equal(scale.view(np.uint32), exp_scale.view(np.uint32))
+    assert np.array_equal(shift.view(np.uint32), v["compiled"].view(np.uint32))
+    for name, alt in v.items():
+        assert name == "compiled" or (alt.view(np.uint32) != v["compiled"].view(np.uint32)).sum() >= 4, name
+
+
+@pytest.mark.parametrize("k,pad,stride,hw,out_hw", [(3, 1, 1, 9, None), (3, 0, 2, 12, 6), (7, 3, 2, 15, None), (5, 2, 1, 8, None),
+                                                    (3, 1, 2, 11, None)])
+@pytest.mark.parametrize("out_type", [ol.F32, ol.U8])
+def test_border_shift_rows_fold_exactly_the_valid_taps(k, pad, stride, hw, out_hw, out_type):
+    """Every row of the oracle's per-pixel shift map equals the fold above applied to the sum of the quantized
+    weights of exactly the taps that fall inside the image for that pixel (taps found here by testing the
+    input coordinate, not through the reference's range tables, src/elx_int8_conv_direct.cpp:227-309)."""
+    rng = np.random.default_rng(k * 10 + stride + out_type)
+    ic, oc = 24, 32
+    in_S, in_z, out_S, out_z = 0.017, 113.0, 0.05, 2.0
+    w = rng.normal(0, 0.05, (oc, ic, k, k)).astype(f32)
+    b = rng.normal(0, 0.3, oc).astype(f32)
+    p = ol.make_params(1, ic, oc, hw, hw, k, k, stride=stride, out_type=out_type, in_scale=in_S, in_z=in_z, out_scale=out_S,
+                       out_z=out_z, with_relu=False, pad_tl=pad, out_hw=None if out_hw is None else (out_hw, out_hw),
+                       pad=pad)
+    wb = ol.weights_to_blocked(w)
+    wq, scale, shift, _ = ol.direct_prepare(p, wb, b)
+    smap = np.zeros((p.oh, p.ow, ol.up16(oc)), f32)
+    assert ol.oracle().orc_direct_border_shifts(ctypes.byref(p), ol.ptr(wb), ol.ptr(b), ol.ptr(smap)) == 0
+    wq_np, absmax = quant_weights_numpy(w)
+    w_S = (absmax / f32(127.0)).astype(f32)
+    seen = set()
+    for oh in range(p.oh):
+        for ow in range(p.ow):
+            vh = [a for a in range(k) if 0 <= oh * stride + a - pad < hw]
+            vw = [c for c in range(k) if 0 <= ow * stride + c - pad < hw]
+            seen.add((tuple(vh), tuple(vw)))
+            wsum = wq_np[:, :, vh][:, :, :, vw].reshape(oc, -1).astype(np.int64).sum(axis=1)
+            if out_type == ol.F32:
+                sc = (f32(in_S) * w_S).astype(f32)
+                exp = _fma(-(f32(in_z) * wsum.astype(f32)).astype(f32), sc, b)
+            else:
+                sc, v = fold_variants(in_S, in_z, w_S, wsum, b, f32(1.0) / f32(out_S), out_z)
+                exp = v["compiled"]
+            assert np.array_equal(smap[oh, ow, :oc].view(np.uint32), exp.view(np.uint32)), (oh, ow)
+    assert len(seen) >= (4 if pad else 1)
