@@ -32,7 +32,7 @@
 #ifdef EHIP_TRACE
 #define TRACE_POINT(i)                                                                             \
   do {                                                                                             \
-    if (a.trace && lane == 0) a.trace[((size_t)tile_id * 4 + wave) * 16 + (i)] = clock64(); \
+    if (a.trace && lane == 0) a.trace[((size_t)tile_id * 4 + wave) * 16 + (i)] = wall_clock64(); \
   } while (0)
 #else
 #define TRACE_POINT(i) do { } while (0)
@@ -40,20 +40,50 @@
 
 namespace ehip {
 
-template <int WM, int WN, int TM, int TN, int CT, int NPASS>
+// PAIRS > 0: the layer has exactly PAIRS pairs of 16-channel units and they are staged in one fill; the
+// whole K loop is then straight-line code.  The weight operands are requested nine taps ahead of their
+// use; inside a loop the compiler waits for ALL outstanding loads at the loop's head (its counter model
+// does not survive the back edge), which exposes a full trip to L2 once per pair.  Unrolled, every wait
+// names exactly the load it needs.
+//
+// SP ("strided pixels"): lane l32 of pixel tile nt owns virtual pixel TN * l32 + nt of the wave's run
+// instead of 32 * nt + l32.  The pixel operand of tap (kh, kw) and tile nt is then the staged run read
+// at offset kh * VW + (nt + kw) with a lane stride of TN cells -- it depends on nt + kw only, so one
+// kernel row needs TN + 2 operand reads for its 3 * TN pixel operands (18 instead of 36 per channel
+// pair at TN = 4), and they are requested a whole kernel row (3 * TM * TN MFMAs) ahead of their use.
+// The staged cells of a unit are stored by residue: cell c at (c % TN) * R + c / TN, which makes the
+// strided read a read of consecutive 16-byte slots; R is chosen so that neighbouring cells written by
+// neighbouring threads land in different banks.
+constexpr int conv3x3v_unit_stride(int cells, int tn, bool sp)
+{
+  if (!sp || tn == 1) return cells;
+  int r = (cells + tn - 1) / tn;
+  const int want = tn == 4 ? 2 : 4;   // R * 16 bytes = 32 (TN 4) or 64 (TN 2) modulo 128
+  while (r % 8 != want) ++r;
+  return r * tn;
+}
+
+template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS = 0, bool SP = false>
 __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
 {
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
-  constexpr int STRIDE = CT * NPASS;   // LDS cells per unit
+  constexpr int STRIDE = conv3x3v_unit_stride(CT * NPASS, TN, SP);   // LDS cells per unit
+  constexpr int RSP = STRIDE / TN;
+  static_assert(!SP || TN == 2 || TN == 4, "strided pixels: two or four pixel tiles per wave");
+  // where staged cell c of a unit lives
+  auto slot = [](int c) { return SP ? (c % TN) * RSP + c / TN : c; };
   constexpr int G = kBlock / CT;       // thread groups that split the units of a fill
   static_assert(WM * WN == 4, "four waves per workgroup");
   static_assert(kBlock % CT == 0, "cells per pass");
   extern __shared__ v4i lds[];         // [chunk_units][STRIDE]
+#ifdef EHIP_TRACE
+  const long long t_entry = wall_clock64();
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   // Workgroups go round the eight XCDs (block b runs on XCD b % 8), each XCD with an L2 of its own.
@@ -76,6 +106,12 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   const long long plane = (long long)a.ih * a.iw * 16;
   const uint8_t *inb = a.in + (long long)n * a.ic2 * plane;
   TRACE_POINT(0);
+#ifdef EHIP_TRACE
+  if (a.trace && lane == 0) {   // wall clock at the wave's first instruction and once the arguments are in
+    a.trace[((size_t)tile_id * 4 + wave) * 16 + 0] = t_entry;
+    a.trace[((size_t)tile_id * 4 + wave) * 16 + 1] = wall_clock64();
+  }
+#endif
 
   // ---- staging plan: the same cells for every fill ------------------------------------------
   const int ug = tid / CT;
@@ -97,6 +133,9 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   const long long w_tap = (long long)a.units_pad * w_unit;
   v4i a_reg[9][TM];
   auto load_a = [&](int tap, int pair) {
+#if defined(EHIP_KO) && (EHIP_KO & 1)
+    if (pair > 0) return;   // knock-out (development): the weight operands of pair 0 are used throughout
+#endif
     const int8_t *p = wb + tap * w_tap + (long long)(2 * pair) * w_unit;
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) a_reg[tap][mt] = *reinterpret_cast<const v4i *>(p + mt * 512);
@@ -128,7 +167,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
           if (k0 + j < nk) {
             const v4i x = t[j] ^ (int)0x80808080;
             const v4i z = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
-            lds[(ug + G * (k0 + j)) * STRIDE + tid % CT + p * CT] = gin[p] ? x : z;
+            lds[(ug + G * (k0 + j)) * STRIDE + slot(tid % CT + p * CT)] = gin[p] ? x : z;
           }
         }
       }
@@ -162,7 +201,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
           if (k0 + j < nk) {
             const v4i x = t[p][j] ^ (int)0x80808080;
             const v4i z = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
-            lds[(ug + G * (k0 + j)) * STRIDE + tid % CT + p * CT] = gin[p] ? x : z;
+            lds[(ug + G * (k0 + j)) * STRIDE + slot(tid % CT + p * CT)] = gin[p] ? x : z;
           }
         }
     }
@@ -170,40 +209,121 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
 
   v16i acc[TM][TN];
   // one channel pair (32 input channels) x nine taps; `last` = nothing left to prefetch
-  auto pair_taps = [&](int pl, int pair, bool last) {
+  // Issue order matters more than bandwidth here: a wave issues in order, an MFMA occupies the matrix
+  // pipe for 32 clocks, and an LDS read or a global load takes the wave's issue slot for several clocks.
+  // Four reads issued in a row between two groups of MFMAs leave the pipe idle behind them (measured:
+  // 46 instead of 32 clocks per MFMA); ONE memory instruction behind EACH MFMA hides in its shadow
+  // (34 clocks).  So every MFMA is followed by at most one pixel-operand read for the next tap, and the
+  // tap's last MFMA by the weight request for the next channel pair; sched_barrier pins that order.
+  v4i bq[2][TN];
+  auto read_b = [&](int par, int pl, int tap, int nt) {
     const v4i *tile = lds + (2 * pl + lh) * STRIDE + pw0 + l32;
-    v4i bq[2][TN];
+    bq[par][nt] = tile[nt * 32 + (tap / 3) * VW + tap % 3];
+  };
+  // one tap of one channel pair out of operand buffer par; next_pl >= 0: the operands of (next_pl,
+  // next_tap) are read into the other buffer on the way
+  auto tap_mfmas = [&](int par, int tap, int pair, bool last, int next_pl, int next_tap) {
 #pragma unroll
-    for (int nt = 0; nt < TN; ++nt) bq[0][nt] = tile[nt * 32];
+    for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
-    for (int tap = 0; tap < 9; ++tap) {
-      if (tap < 8) {
-        const int toff = ((tap + 1) / 3) * VW + (tap + 1) % 3;
-#pragma unroll
-        for (int nt = 0; nt < TN; ++nt) bq[(tap + 1) & 1][nt] = tile[nt * 32 + toff];
+      for (int nt = 0; nt < TN; ++nt) {
+        acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[tap][mt], bq[par][nt], acc[mt][nt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (mt == 0 && next_pl >= 0) read_b(par ^ 1, next_pl, next_tap, nt);
+        if (mt == TM - 1 && nt == TN - 1 && !last) load_a(tap, pair + 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      // keep the compiler from sinking these reads next to their use
-      __builtin_amdgcn_sched_barrier(0);
+  };
+  // loop form: the operands of a pair's first tap are read at its start
+  auto pair_taps = [&](int pl, int pair, bool last) {
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) read_b(0, pl, 0, nt);
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) tap_mfmas(tap & 1, tap, pair, last, tap < 8 ? pl : -1, tap + 1);
+  };
+
+  // strided pixels: LDS slot offsets of the TN + 2 operands of each kernel row (wave-uniform)
+  int soff[3][TN + 2];
+  if (SP) {
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+      for (int o = 0; o < TN + 2; ++o) {
+        const int b = kh * VW + o;   // pw0 is a multiple of TN
+        soff[kh][o] = (b % TN) * RSP + b / TN + pw0 / TN;
+      }
+  }
+  v4i q[2][TN + 2];
+  // operands of kernel row kh of the pair staged at pl, into buffer par
+  auto load_q = [&](int par, int pl, int kh) {
+    const v4i *ub = lds + (2 * pl + lh) * STRIDE + l32;
+#pragma unroll
+    for (int o = 0; o < TN + 2; ++o) q[par][o] = ub[soff[kh][o]];
+  };
+  // one kernel row of one channel pair: 3 taps x TM x TN MFMAs out of buffer par; next_pl >= 0: the
+  // TN + 2 operands of row (next_pl, next_kh) are read into the other buffer, one behind each MFMA
+  auto row_taps = [&](int par, int kh, int pair, bool last, int next_pl, int next_kh) {
+    int issued = 0;
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw) {
+      const int tap = kh * 3 + kw;
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < TN; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[tap][mt], bq[tap & 1][nt], acc[mt][nt], 0, 0, 0);
-      if (!last) load_a(tap, pair + 1);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int nt = 0; nt < TN; ++nt) {
+          acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[tap][mt], q[par][nt + kw], acc[mt][nt], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (next_pl >= 0 && issued < TN + 2) {
+            const v4i *ub = lds + (2 * next_pl + lh) * STRIDE + l32;
+            q[par ^ 1][issued] = ub[soff[next_kh][issued]];
+            ++issued;
+          }
+          if (mt == TM - 1 && nt == TN - 1 && !last) load_a(tap, pair + 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
     }
+  };
+  // generic loop form: the operands of a pair's first row are requested at its start
+  auto pair_taps_sp = [&](int pl, int pair, bool last) {
+    load_q(0, pl, 0);
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh) row_taps(kh & 1, kh, pair, last, kh < 2 ? pl : -1, kh + 1);
   };
 
   const int ppc = a.chunk_units / 2;
   const int nchunks = a.units_pad / a.chunk_units;
   const long long cidx = oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
   OcConsts k0;
+  // The accumulators start from the compensation 128 * sum(weights) of their channel instead of zero:
+  // it is requested before the staging loads and costs the epilogue nothing.
 #pragma unroll
-  for (int mt = 0; mt < TM; ++mt)
+  for (int mt = 0; mt < TM; ++mt) {
+    v4i c4[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) c4[qq] = *reinterpret_cast<const v4i *>(a.ep.comp + cidx + 32 * mt + 4 * qq);
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = c4[v >> 2][v & 3];
+  }
+  // Lean epilogue (a.lean, decided by the launcher): u8 / s8 output, ReLU with bounds 0 <= lo <= hi, no
+  // sum -- the case of every direct 3x3 layer of the tuned networks.  Scale and shift of the lane's
+  // channels travel during the last channel pair; a value then costs a convert, a multiply-add, a
+  // clamp (none when the bounds are exactly the u8 code range) and a byte pack.
+  float4 lsc[TM][4], lsh[TM][4];
+  auto load_lean_consts = [&]() {
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq) {
+        lsc[mt][qq] = *reinterpret_cast<const float4 *>(a.ep.scale + cidx + 32 * mt + 4 * qq);
+        lsh[mt][qq] = *reinterpret_cast<const float4 *>(a.ep.shift + cidx + 32 * mt + 4 * qq);
+      }
+  };
+  auto load_epilogue_consts = [&]() {
+    if (a.lean) load_lean_consts();
+    else load_consts(k0, a.ep, cidx);
+  };
   // as few loads per trip as cover the fill (unused slots repeat the last unit's load), at most 16
   constexpr int KBMAX = NPASS == 1 ? 16 : (NPASS == 2 ? 8 : 4);
   if (nk <= 2) stage_first(std::integral_constant<int, 2>());
@@ -213,6 +333,26 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   TRACE_POINT(2);
   __syncthreads();
   TRACE_POINT(3);
+  if (PAIRS > 0 && SP) {
+    // straight line over the 3 * PAIRS kernel rows, each one's operands requested a row ahead
+    load_q(0, 0, 0);
+#pragma unroll
+    for (int st = 0; st < 3 * PAIRS; ++st) {
+      const int pl = st / 3, kh = st % 3;
+      if (st == 3 * PAIRS - 3) load_epilogue_consts();
+      row_taps(st & 1, kh, pl, pl == PAIRS - 1, st + 1 < 3 * PAIRS ? (st + 1) / 3 : -1, (st + 1) % 3);
+    }
+  } else if (PAIRS > 0) {
+    // straight line over the 9 * PAIRS taps, each one's pixel operands read during the tap before
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) read_b(0, 0, 0, nt);
+#pragma unroll
+    for (int st = 0; st < 9 * PAIRS; ++st) {
+      const int pl = st / 9, tap = st % 9;
+      if (st == 9 * (PAIRS - 1)) load_epilogue_consts();
+      tap_mfmas(st & 1, tap, pl, pl == PAIRS - 1, st + 1 < 9 * PAIRS ? (st + 1) / 9 : -1, (st + 1) % 9);
+    }
+  } else
   for (int chunk = 0; chunk < nchunks; ++chunk) {
     if (chunk) {
       __syncthreads();
@@ -220,22 +360,68 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
       __syncthreads();
     }
     const int npl = chunk + 1 < nchunks ? ppc : ppc - 1;
-    for (int pl = 0; pl < npl; ++pl) pair_taps(pl, chunk * ppc + pl, false);
+    for (int pl = 0; pl < npl; ++pl) {
+      if (SP) pair_taps_sp(pl, chunk * ppc + pl, false);
+      else pair_taps(pl, chunk * ppc + pl, false);
+    }
     TRACE_POINT(4);
     if (chunk + 1 == nchunks) {
       // the epilogue's per-channel constants travel while the last pair is multiplied
-      load_consts(k0, a.ep, cidx);
-      pair_taps(ppc - 1, chunk * ppc + ppc - 1, true);
+      load_epilogue_consts();
+      if (SP) pair_taps_sp(ppc - 1, chunk * ppc + ppc - 1, true);
+      else pair_taps(ppc - 1, chunk * ppc + ppc - 1, true);
     }
   }
   TRACE_POINT(5);
 
   // ---- epilogue ------------------------------------------------------------------------------
+  if (a.lean) {
+    // byte offset of the lane's cell inside the (image, first channel block of the wave) plane pair: the
+    // lane's 16 channels are block lh of the wave's two; everything else about the address is scalar
+    uint8_t *outb = static_cast<uint8_t *>(a.out) + ((size_t)n * a.oc2 + ((oc0 + mw0) >> 4)) * ohw * 16;
+    const float hi = a.ep.out_type == EHIP_S8 ? __builtin_fminf(a.ep.hi, 127.0f) : a.ep.hi;
+    // CLAMP as a compile-time choice: two straight copies of the loop behind one uniform branch
+    auto lean_store = [&](auto clamp) {
+      constexpr bool CLAMP = decltype(clamp)::value;
+#pragma unroll
+      for (int nt = 0; nt < TN; ++nt) {
+        const int v = SP ? v0 + pw0 + TN * l32 + nt : v0 + pw0 + nt * 32 + l32;
+        const int r = fastdiv(v, VW, a.vw_magic);
+        const int c = v - r * VW;
+        const bool pv = r < a.oh && c < a.ow;
+        const unsigned off = (unsigned)(lh * ohw + r * a.ow + c) * 16u;
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) {
+          v4i cell;
+#pragma unroll
+          for (int qq = 0; qq < 4; ++qq) {
+            const float sc[4] = {lsc[mt][qq].x, lsc[mt][qq].y, lsc[mt][qq].z, lsc[mt][qq].w};
+            const float sh[4] = {lsh[mt][qq].x, lsh[mt][qq].y, lsh[mt][qq].z, lsh[mt][qq].w};
+            unsigned pk = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              float f = __builtin_fmaf((float)acc[mt][nt][4 * qq + j], sc[j], sh[j]);
+              if (CLAMP) f = __builtin_amdgcn_fmed3f(f, a.ep.lo, hi);
+              pk = __builtin_amdgcn_cvt_pk_u8_f32(f, j, pk);
+            }
+            cell[qq] = (int)pk;
+          }
+          if (pv && (int)cidx + 32 * mt < oc_real)
+            *reinterpret_cast<v4i *>(outb + (size_t)(2 * mt) * ohw * 16 + off) = cell;
+        }
+      }
+    };
+    // lean == 2: the bounds are the u8 code range, which the byte pack saturates to by itself
+    if (a.lean == 2) lean_store(std::false_type());
+    else lean_store(std::true_type());
+    TRACE_POINT(15);
+    return;
+  }
   size_t pix[TN];
   bool pvalid[TN];
 #pragma unroll
   for (int nt = 0; nt < TN; ++nt) {
-    const int v = v0 + pw0 + nt * 32 + l32;
+    const int v = SP ? v0 + pw0 + TN * l32 + nt : v0 + pw0 + nt * 32 + l32;
     const int r = fastdiv(v, VW, a.vw_magic);
     const int c = v - r * VW;
     pvalid[nt] = r < a.oh && c < a.ow;
@@ -244,38 +430,57 @@ __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(Conv3x3Args a)
   TRACE_POINT(14);
   const size_t pixT[TN][2] = {};
   const bool validT[TN][2] = {};
-  epilogue_wave<TM, TN>(a.ep, acc, k0, cidx, (int)cidx, pix, pvalid, oc_real, (size_t)ohw * 16, a.out, nullptr, pixT,
-                        validT);
+  epilogue_wave<TM, TN, false, true>(a.ep, acc, k0, cidx, (int)cidx, pix, pvalid, oc_real, (size_t)ohw * 16, a.out, nullptr,
+                                     pixT, validT);
   TRACE_POINT(15);
 }
 
 namespace {
 struct Variant {
   const char *name;
-  int oc_t, p_t, cells;
+  int oc_t, p_t, cells;   // cells: staged cells per unit a tile may span
+  int ustride;            // LDS cells between units
   void (*kernel)(Conv3x3Args);
+  void (*unrolled[3])(Conv3x3Args);   // straight-line K loop for layers of exactly 2, 4, 8 unit pairs, or null
 };
 #define V(WM, WN, TM, TN, CT, NPASS)                                                              \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
-    CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS> }
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>, {nullptr, nullptr, nullptr} }
+#define VU(WM, WN, TM, TN, CT, NPASS)                                                             \
+  { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4>,  \
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>} }
+#define VS(WM, WN, TM, TN, CT, NPASS)                                                             \
+  { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ",sp>", WM * TM * 32, WN * TN * 32, \
+    CT * NPASS, conv3x3v_unit_stride(CT * NPASS, TN, true), k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 0, true>, \
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, true>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, true>, \
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>} }
 const Variant kVariants[] = {
     V(2, 2, 2, 1, 128, 1),  // 0: 128 oc x  64 px, rows up to  31 cells
     V(2, 2, 2, 1, 256, 1),  // 1: 128 oc x  64 px, rows up to  95 cells
-    V(2, 2, 2, 2, 256, 1),  // 2: 128 oc x 128 px, rows up to  63 cells
+    VU(2, 2, 2, 2, 256, 1), // 2: 128 oc x 128 px, rows up to  63 cells
     V(2, 2, 2, 2, 256, 3),  // 3: 128 oc x 128 px, rows up to 319 cells
-    V(1, 4, 2, 1, 256, 1),  // 4:  64 oc x 128 px, rows up to  63 cells
+    VU(1, 4, 2, 1, 256, 1), // 4:  64 oc x 128 px, rows up to  63 cells
     V(1, 4, 2, 1, 256, 3),  // 5:  64 oc x 128 px, rows up to 319 cells
     V(1, 4, 1, 1, 256, 1),  // 6:  32 oc x 128 px, rows up to  63 cells
     V(1, 4, 1, 1, 256, 3),  // 7:  32 oc x 128 px, rows up to 319 cells
-    V(4, 1, 1, 1, 128, 1),  // 8: 128 oc x  32 px, rows up to  47 cells
-    V(4, 1, 1, 4, 256, 1),  // 9: 128 oc x 128 px, rows up to  63 cells, every wave all pixels
-    V(4, 1, 1, 2, 128, 1),  // 10: 128 oc x 64 px, rows up to  31 cells, every wave all pixels
+    VU(4, 1, 1, 1, 128, 1), // 8: 128 oc x  32 px, rows up to  47 cells
+    VU(4, 1, 1, 4, 256, 1), // 9: 128 oc x 128 px, rows up to  63 cells, every wave all pixels
+    VU(4, 1, 1, 2, 128, 1), // 10: 128 oc x 64 px, rows up to  31 cells, every wave all pixels
     V(1, 4, 2, 2, 256, 3),  // 11:  64 oc x 256 px, rows up to 255 cells
     V(2, 2, 1, 4, 256, 3),  // 12:  64 oc x 256 px, rows up to 255 cells, a wave = 32 oc x 128 px
-    V(4, 1, 1, 4, 256, 2),  // 13: 128 oc x 128 px, rows up to 191 cells, every wave all pixels
+    VU(4, 1, 1, 4, 256, 2), // 13: 128 oc x 128 px, rows up to 191 cells, every wave all pixels
     V(4, 1, 1, 4, 256, 4),  // 14: 128 oc x 128 px, rows up to 447 cells, every wave all pixels
+    VS(4, 1, 1, 4, 256, 1), // 15: as 9, strided pixels
+    VS(4, 1, 1, 2, 128, 1), // 16: as 10, strided pixels
+    VS(2, 2, 2, 2, 256, 1), // 17: as 2, strided pixels
+    VS(4, 1, 1, 4, 256, 2), // 18: as 13, strided pixels
+    VS(2, 2, 2, 4, 256, 2), // 19: 128 oc x 256 px, rows up to 127 cells, a wave = 64 oc x 128 px, strided pixels
 };
 #undef V
+#undef VU
+#undef VS
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLdsBudget = 64 * 1024;
 }  // namespace
@@ -287,7 +492,7 @@ bool conv3x3v_fits(int v, int ow) { return kVariants[v].p_t + 2 * (ow + 2) + 2 <
 // units of 16 input channels staged per LDS fill: all of them if they fit the budget
 int conv3x3v_chunk_units(int v, int ic2)
 {
-  int cu = (kLdsBudget / (kVariants[v].cells * 16)) & ~1;
+  int cu = (kLdsBudget / (kVariants[v].ustride * 16)) & ~1;
   const int all = up(ic2, 2);
   return cu < all ? cu : all;
 }
@@ -309,7 +514,8 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
   // there the 256-pixel tiles (11, 12) and the two-pass 128-channel tile (13) are 1.3-1.8 x faster
   // than the 128-pixel tiles with three passes.
   const int oc = oc2 * 16, vpx = oh * (ow + 2);
-  static const double pref[] = {0.80, 0.78, 0.92, 0.90, 1.0, 0.95, 1.0, 0.95, 0.85, 0.97, 1.0, 0.97, 1.10, 0.93, 0.85};
+  static const double pref[] = {0.80, 0.78, 0.92, 0.90, 1.0, 0.95, 1.0, 0.95, 0.85, 0.97, 1.0, 0.97, 1.10, 0.93, 0.85,
+                                0.0, 0.0, 0.0, 0.0, 0.0};
   int best = -1;
   double best_score = -1;
   for (int pass = 0; pass < 2 && best < 0; ++pass)   // second pass: any channel tile that fits the rows
@@ -336,7 +542,7 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
 {
   const Variant &k = kVariants[variant];
   Conv3x3Args a = a0;
-  const size_t lds_bytes = (size_t)a.chunk_units * k.cells * 16;
+  const size_t lds_bytes = (size_t)a.chunk_units * k.ustride * 16;
   a.gx = (a.oh * a.vw + k.p_t - 1) / k.p_t;
   a.gy = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   const long long tiles = (long long)a.gx * a.gy * n;
@@ -346,13 +552,28 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
   }
   a.tiles = (int)tiles;
   a.tiles_per_xcd = (a.tiles + 7) / 8;
+  {
+    const Epilogue &e = a.ep;
+    const bool q = e.out_type == EHIP_U8 || e.out_type == EHIP_S8;
+    const bool fast = q && e.with_relu && !e.with_sum && !e.shift_tab && e.lo >= 0.0f && e.hi >= e.lo &&
+        (e.out_type != EHIP_S8 || e.lo <= 127.0f);
+    a.lean = !fast ? 0 : ((e.out_type == EHIP_U8 && e.lo == 0.0f && e.hi >= 255.0f) ? 2 : 1);
+    if (const char *env = getenv("EHIP_CONV3X3V_LEAN")) if (env[0] == '0') a.lean = 0;
+  }
   dim3 grid(8 * a.tiles_per_xcd, 1, 1);
+  void (*kernel)(Conv3x3Args) = k.kernel;
+  if (a.units_pad == a.chunk_units) {   // one fill holds every unit
+    const int pairs = a.units_pad / 2;
+    const int slot = pairs == 2 ? 0 : (pairs == 4 ? 1 : (pairs == 8 ? 2 : -1));
+    const char *env = getenv("EHIP_CONV3X3V_UNROLL");
+    if (slot >= 0 && k.unrolled[slot] && !(env && env[0] == '0')) kernel = k.unrolled[slot];
+  }
   if (lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k.kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(k.kernel, grid, dim3(kBlock), lds_bytes, s, a);
+  hipLaunchKernelGGL(kernel, grid, dim3(kBlock), lds_bytes, s, a);
   return hipGetLastError();
 }
 

@@ -76,6 +76,8 @@ struct Conv3x3Args {
   unsigned vw_magic;    // div_magic(vw)
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
   int gx, gy, tiles, tiles_per_xcd;   // set by the launcher: pixel tiles per image, channel tiles, all tiles, ceil(tiles / 8)
+  int lean;             // set by the launcher: 0 = general epilogue, 1 = u8 / s8 with ReLU bounds 0 <= lo <= hi and no
+                        // sum, 2 = u8 whose bounds are the code range 0 .. 255 (no clamp needed)
 };
 
 struct DepthwiseArgs {

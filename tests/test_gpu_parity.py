@@ -162,11 +162,23 @@ def test_conv3x3_no_padding():
     run_and_compare(Layer(2, 32, 32, 12, k=3, pad=0, out_type=ol.U8, seed=3))
 
 
-@pytest.mark.parametrize("variant", range(15))
-def test_conv3x3_every_virtual_row_kernel_variant(variant, monkeypatch):
+@pytest.mark.parametrize("variant", range(20))
+@pytest.mark.parametrize("ic", [64, 96, 128, 256])
+def test_conv3x3_every_virtual_row_kernel_variant(variant, ic, monkeypatch):
+    """every tile shape, with the K loop as a loop (96 channels: 3 unit pairs) and as straight-line code
+    (2, 4, 8 pairs); variants 15 and up deal a wave's pixels to its lanes with a stride"""
     monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", str(variant))
-    res = run_and_compare(Layer(2, 64, 144, 13, k=3, pad=1, out_type=ol.U8, seed=80 + variant))
+    res = run_and_compare(Layer(2, ic, 144, 13, k=3, pad=1, out_type=ol.U8, seed=80 + variant + ic))
     assert res["conv"].kernel_name.startswith("k_conv3x3v_u8s8")
+
+
+@pytest.mark.parametrize("variant", [15, 16, 17, 18, 19])
+@pytest.mark.parametrize("out_type", [ol.S32, ol.S8, ol.F32])
+def test_conv3x3_strided_pixels_output_types(variant, out_type, monkeypatch):
+    monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", str(variant))
+    run_and_compare(Layer(3, 128, 80, 28, k=3, pad=1, out_type=out_type, seed=60 + variant + out_type))
+    monkeypatch.setenv("EHIP_CONV3X3V_UNROLL", "0")
+    run_and_compare(Layer(1, 128, 80, 9, k=3, pad=0, out_type=out_type, seed=61 + variant + out_type))
 
 
 def test_conv3x3_virtual_rows_many_channels_restage():
