@@ -15,6 +15,7 @@ LIB = os.path.join(HERE, "libeuler_hip.so")
 
 SOURCES = [
     "ehip_gemm.hip",
+    "ehip_gemm1x1.hip",
     "ehip_conv3x3v.hip",
     "ehip_fewch.hip",
     "ehip_depthwise.hip",

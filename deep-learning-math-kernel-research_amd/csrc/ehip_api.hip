@@ -305,6 +305,16 @@ int setup_workspace(ehip_conv *c)
     c->units_pad = c->taps > 1 ? c->ic2 : up(c->ic2, gemm_variant_chunk(c->variant));
     c->kernel_name = gemm_smallk_applies(c->ic2, c->taps, 1) ? "k_gemm_smallk_u8s8" : gemm_variant_name(c->variant);
     if (c->family == FAM_CONV_FEWCH) c->kernel_name = "k_conv_fewch_u8s8";
+    if (c->family == FAM_GEMM_1X1 && c->taps == 1 && !gemm_smallk_applies(c->ic2, c->taps, 1)) {
+      // many input channels, blocked activations: the kernel that keeps its pixel tile resident
+      GemmArgs g;
+      memset(&g, 0, sizeof(g));
+      g.kh = g.kw = 1;
+      g.in_nhwc = d.input_fmt == EHIP_NHWC; g.out_nhwc = d.output_fmt == EHIP_NHWC;
+      g.ic2 = c->ic2; g.units_pad = c->units_pad; g.oc2 = c->oc2; g.p_total = d.n * d.oh * d.ow;
+      const int rv = gemm1x1_res_pick(g, 1);
+      if (rv >= 0) c->kernel_name = gemm1x1_res_name(rv);
+    }
     if (c->taps > 1 && d.input_z != 0.0f) {
       // classes of output rows / columns by their range of valid kernel rows / columns
       auto classes = [](int on, int in, int k, int stride, int pad, std::vector<int> &cls, std::vector<std::pair<int, int>> &rng) {

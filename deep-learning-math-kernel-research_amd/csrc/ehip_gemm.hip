@@ -33,7 +33,7 @@
 #define TRACE_POINT(i)                                                                             \
   do {                                                                                             \
     if (a.trace && lane == 0)                                                                      \
-      a.trace[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = clock64(); \
+      a.trace[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave) * 16 + (i)] = wall_clock64(); \
   } while (0)
 #else
 #define TRACE_POINT(i) do { } while (0)
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   // Workgroups go to the 8 XCDs round-robin by their linear index.  The channel blocks of one pixel
@@ -197,13 +197,20 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     }
   };
 
+  // The accumulators start from the compensation 128 * sum(weights) of their channel instead of zero
+  // (requested before the first fill's loads, so it costs the epilogue nothing).
+  const long long cidx = (long long)b * a.ocpp + oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
   v16i acc[TM][TN];
 #pragma unroll
-  for (int mt = 0; mt < TM; ++mt)
+  for (int mt = 0; mt < TM; ++mt) {
+    v4i c4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c4[q] = *reinterpret_cast<const v4i *>(a.ep.comp + cidx + 32 * mt + 4 * q);
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = c4[v >> 2][v & 3];
+  }
 
   // ---- main loop ------------------------------------------------------------------------------
   v4i opa[2][TM], opb[2][TN];
@@ -255,18 +262,43 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     }
   }
   TRACE_POINT(5);
-  const long long cidx = (long long)b * a.ocpp + oc0 + mw0 + 16 * lh;   // the lane's 16 channels of tile 0
   OcConsts k0;
+  LeanConsts lk[TM];
 #pragma unroll
   for (int d = 0; d < D; ++d) {
     store_stage(buf, d);
     __syncthreads();
     // the epilogue's per-channel constants travel while the last fill is multiplied
-    if (d == D - 1) load_consts(k0, a.ep, cidx);
+    if (d == D - 1) {
+      if (a.lean) {
+#pragma unroll
+        for (int mt = 0; mt < TM; ++mt) load_lean_consts(lk[mt], a.ep, cidx + 32 * mt);
+      } else {
+        load_consts(k0, a.ep, cidx);
+      }
+    }
     multiply(buf);
     buf ^= 1;
   }
   TRACE_POINT(6);
+
+  if (a.lean) {   // u8 / s8 with ReLU bounds, blocked output, per-channel shift: no output-type switch
+    uint8_t *cell[TN];
+    bool pv[TN];
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) {
+      const int gp = pix0 + pw0 + nt * 32 + l32;
+      pv[nt] = gp < a.p_total;
+      const int gpc = pv[nt] ? gp : 0;
+      const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
+      const int r = gpc - n * a.ohw;
+      cell[nt] = static_cast<uint8_t *>(a.out) + (size_t)b * a.out_batch_stride +
+          (((size_t)n * a.oc2 + ((oc0 + mw0) >> 4) + lh) * a.ohw + r) * 16;
+    }
+    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + mw0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
+    TRACE_POINT(15);
+    return;
+  }
 
   // ---- epilogue ------------------------------------------------------------------------------
   // element offset of output pixel gp's cell in 16-channel block 0 (nhwc: its channel vector)
@@ -302,8 +334,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
     xlds = lds + wave * 256;
   }
   TRACE_POINT(14);
-  epilogue_wave<TM, TN, CONV != 0>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real,
-                        a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT, cls);
+  epilogue_wave<TM, TN, CONV != 0, true>(a.ep, acc, k0, cidx, oc0 + mw0 + 16 * lh, pix, pvalid, oc_real,
+                                         a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT, cls);
   TRACE_POINT(15);
 }
 
@@ -532,8 +564,14 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s)
 hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s)
 {
   if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s);
+  {
+    const int rv = gemm1x1_res_pick(a0, nbatch);
+    if (rv >= 0) return launch_gemm1x1_res(a0, rv, s);
+  }
   const Variant &k = kVariants[variant];
   GemmArgs a = a0;
+  a.lean = lean_mode(a.ep, a.out_nhwc != 0);
+  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8), nbatch);

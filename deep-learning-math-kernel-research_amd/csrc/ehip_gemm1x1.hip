@@ -1,0 +1,337 @@
+// 1x1 u8 x s8 -> s32 convolution with MANY input channels on gfx950 matrix cores: the pixel tile is
+// resident, the weights stream.
+//
+// Replaces, for blocked activations, elx_int8_conv_direct_1x1_t::__execute_a160_s1 / _s2 + gemm_a160_s1 / _s2
+// (src/elx_int8_conv_direct_1x1_xopt.hpp:20-195, src/elx_int8_conv_direct_1x1.cpp:357-480) and the u8s8 GEMM
+// micro-kernel with its epilogue (src/kernel/elk_u8s8_gemm.hxx:168-406).
+//
+// Why a second 1x1 kernel.  A layer like 1024 -> 256 at 14 x 14 is a short, wide GEMM whose activations
+// come from HBM exactly once.  The general kernel (ehip_gemm.hip) walks K in fills of 128 channels with two
+// fills in flight: every fill waits a full trip to HBM, eight times in a row.  Here a workgroup asks for
+// its WHOLE pixel tile -- P_T pixels x all input channels -- in one go, with loads that write LDS
+// directly (global_load_lds_dwordx4: no registers held while they fly, so all of them can be in flight
+// at once), pays the trip to HBM once, and then only streams weights, which sit in L2, through a register
+// ring straight into the MFMA A operand.  Every wave owns its own TM x 32 output channels (no weight row is
+// loaded twice by a workgroup) and all of the tile's TN x 32 pixels.
+//
+// The u8 -> s8 remap (top bit of every activation byte flipped, 128 * sum(w) added back through the
+// accumulators' start value) happens when an operand is read from LDS, since the loads bypass registers.
+#include <type_traits>
+
+#include "ehip_internal.hpp"
+
+// Development aid (compile with -DEHIP_TRACE): lane 0 of every wave records the wall clock at phase boundaries.
+#ifdef EHIP_TRACE
+#define TRACE_POINT(i)                                                                             \
+  do {                                                                                             \
+    if (a.trace && lane == 0) a.trace[((size_t)blockIdx.x * 4 + wave) * 16 + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define TRACE_POINT(i) do { } while (0)
+#endif
+
+namespace ehip {
+
+// 16 bytes per lane from global memory straight into LDS: lane i's piece lands at lds_dst + 16 i
+// (lds_dst is wave-uniform).  The builtin exists in the device pass only.
+__device__ __forceinline__ void load_to_lds_16(const void *gsrc, void *lds_dst)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_global_load_lds(gsrc, (__attribute__((address_space(3))) void *)lds_dst, 16, 0, 0);
+#else
+  (void)gsrc;
+  (void)lds_dst;
+#endif
+}
+__device__ __forceinline__ void wait_all_loads()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0), the other counters untouched
+#endif
+}
+
+// NKS > 0: the layer has exactly NKS k-steps (pairs of 16-channel units): the K loop is straight-line code
+// and every wait names the load it needs.  NKS == 0: a loop over blocks of eight k-steps.
+template <int TM, int TN, int NKS>
+__global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
+{
+  constexpr int OC_T = 4 * TM * 32;
+  constexpr int P_T = TN * 32;
+  // Weight ring: k-steps requested ahead.  A kernel launch starts with cold L2s, and in a layer of ONE
+  // generation of workgroups every workgroup asks for the same weight lines at the same time: each request
+  // then takes a trip to the memory-side cache, not to L2, and a ring of eight k-steps is four such trips
+  // in a row.  Where the wave's whole weight slice fits in registers (NKS x TM <= 32 operands) it is
+  // requested up front, next to the pixel tile: one trip.
+  constexpr int R = (NKS > 0 && NKS * TM <= 32) ? NKS : 8;
+  extern __shared__ v4i lds[];         // [units][P_T]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  // channel blocks of one pixel tile follow each other on ONE XCD (the first pulls the pixels into that
+  // XCD's L2, the others find them there); an XCD takes a contiguous eighth of the pixel tiles
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int by = seq % a.ny;
+  const int bx = xcd * ((a.nx + 7) >> 3) + seq / a.ny;
+  if (bx >= a.nx) return;   // whole workgroup
+  const int pix0 = bx * P_T;
+  const int oc0 = by * OC_T + wave * TM * 32;   // the wave's first channel
+  const int oc_real = a.oc2 * 16;
+  const int nks = a.units_pad >> 1;
+  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  TRACE_POINT(0);
+
+  // ---- the accumulators start from the compensation ------------------------------------------------
+  const long long cidx = oc0 + 16 * lh;   // the lane's 16 channels of tile 0
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt) {
+    v4i c4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c4[q] = *reinterpret_cast<const v4i *>(a.ep.comp + cidx + 32 * mt + 4 * q);
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = c4[v >> 2][v & 3];
+  }
+
+  // ---- the whole pixel tile, all units, straight into LDS -----------------------------------------------
+  // A wave-load moves 64 consecutive pixels of one unit (1 KB): lane i's 16 bytes land at the wave-uniform
+  // LDS address + 16 i.  Pixel halves of 64 (P_T / 64) x units are dealt to the four waves round-robin.
+  constexpr int HALVES = P_T / 64 > 0 ? P_T / 64 : 1;
+  constexpr int LPW = P_T >= 64 ? 64 : P_T;   // pixels per wave-load (32-pixel tiles: the upper lanes repeat)
+  const uint8_t *src[HALVES];
+#pragma unroll
+  for (int h = 0; h < HALVES; ++h) {
+    int gp = pix0 + h * 64 + (lane % LPW);
+    gp = gp < a.p_total ? gp : a.p_total - 1;   // pixels behind the end are computed and not stored
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic);
+    const int r = gp - n * a.ohw;
+    long long sp = r;
+    if (!dense) {
+      const int oh = fastdiv(r, a.ow, a.ow_magic);
+      sp = (long long)oh * a.stride_h * a.iw + (long long)(r - oh * a.ow) * a.stride_w;
+    }
+    src[h] = a.in + ((long long)n * a.ic2 * a.ihw + sp) * 16;
+  }
+  const long long unit_stride = (long long)a.ihw * 16;
+  {
+    const int items = a.units_pad * HALVES;
+    for (int it = wave; it < items; it += 4) {
+      const int u = it / HALVES, h = it - u * HALVES;
+      const int uc = u < a.ic2 ? u : a.ic2 - 1;   // the padded unit multiplies zero weights: any data will do
+#pragma unroll
+      for (int hh = 0; hh < HALVES; ++hh)
+        if (hh == h)
+          load_to_lds_16(src[hh] + (long long)uc * unit_stride, lds + (size_t)u * P_T + h * 64);
+    }
+  }
+
+  TRACE_POINT(1);
+  // ---- weights [units_pad][ocpp][16]: lane = packed row l32 of unit 2 ks + lh, tile mt 32 rows on --------
+  const int8_t *wb = a.w + ((long long)lh * a.ocpp + oc0 + l32) * 16;
+  const long long w_step = (long long)a.ocpp * 32;   // two units
+  v4i a_reg[R][TM];
+  auto load_a = [&](int slot, int ks) {
+    const int8_t *p = wb + (long long)ks * w_step;
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) a_reg[slot][mt] = *reinterpret_cast<const v4i *>(p + mt * 512);
+  };
+#pragma unroll
+  for (int k = 0; k < R; ++k) load_a(k, k < nks ? k : nks - 1);
+
+  // the in-place sum's operand is requested now, with everything else, and used in the epilogue
+  uint8_t *cell[TN];
+  bool pv[TN];
+  v4i old[TM][TN];
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) {
+    const int gp = pix0 + nt * 32 + l32;
+    pv[nt] = gp < a.p_total;
+    const int gpc = pv[nt] ? gp : 0;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
+    const int r = gpc - n * a.ohw;
+    cell[nt] = static_cast<uint8_t *>(a.out) + (((size_t)n * a.oc2 + (oc0 >> 4) + lh) * a.ohw + r) * 16;
+    if (a.lean & 4) {
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        const bool ok = pv[nt] && oc0 + 16 * lh + 32 * mt < oc_real;
+        old[mt][nt] = *reinterpret_cast<const v4i *>(ok ? cell[nt] + (size_t)mt * 2 * a.ohw * 16 : cell[nt]);
+      }
+    }
+  }
+
+  LeanConsts lk[TM];
+  OcConsts k0;
+  auto load_epilogue_consts = [&]() {
+    if (a.lean) {
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) load_lean_consts(lk[mt], a.ep, cidx + 32 * mt);
+    } else {
+      load_consts(k0, a.ep, cidx);
+    }
+  };
+
+  // the tile has landed (every wave waits for its own loads, the barrier for everybody else's)
+  wait_all_loads();
+  TRACE_POINT(2);
+  __syncthreads();
+  TRACE_POINT(3);
+
+  // ---- K loop: one memory instruction behind each MFMA ---------------------------------------------------
+  v4i bq[2][TN];
+  const v4i *tile = lds + lh * P_T + l32;
+  // (raw bytes: the u8 -> s8 flip of the top bits happens right before the operand's first use.  Next to the
+  // read it would make the wave wait for the read it has just issued; as a pass over the whole tile in LDS it
+  // was measured to cost more than it saves.  With one wave per SIMD the flip still sits between a read and
+  // the MFMA that waits for it -- 51 instead of 34 clocks per MFMA -- which a second workgroup on the CU
+  // hides: the 64-pixel tiles, two workgroups per CU, are the fast ones.)
+  auto read_b = [&](int par, int ks, int nt) { bq[par][nt] = tile[(size_t)ks * 2 * P_T + nt * 32]; };
+  // k-step ks out of operand buffer par; the operands of k-step ks + 1 are read on the way, the ring slot
+  // is refilled with the weights of k-step ks + R behind the last MFMA
+  auto kstep = [&](int par, int slot, int ks, bool read_next, bool load_next) {
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < TN; ++nt) {
+        if (mt == 0) bq[par][nt] ^= (int)0x80808080;
+        acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[slot][mt], bq[par][nt], acc[mt][nt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (mt == 0 && read_next) read_b(par ^ 1, ks + 1, nt);
+        if (mt == TM - 1 && nt == TN - 1 && load_next) load_a(slot, ks + R);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  };
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) read_b(0, 0, nt);
+  if (NKS > 0) {
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (ks == (NKS > R ? NKS - R : 0)) load_epilogue_consts();
+      kstep(ks & 1, ks % R, ks, ks + 1 < NKS, ks + R < NKS);
+    }
+  } else {
+    // blocks of R k-steps (nks is a multiple of R or the tail is peeled below)
+    int ks0 = 0;
+    for (; ks0 + 2 * R <= nks; ks0 += R) {
+#pragma unroll
+      for (int k = 0; k < R; ++k) kstep(k & 1, k, ks0 + k, true, true);
+    }
+    load_epilogue_consts();
+    // last one or two blocks: requests stop at the end of K
+    for (; ks0 < nks; ks0 += R) {
+#pragma unroll
+      for (int k = 0; k < R; ++k)
+        if (ks0 + k < nks) kstep(k & 1, k, ks0 + k, ks0 + k + 1 < nks, ks0 + k + R < nks);
+    }
+  }
+
+  TRACE_POINT(5);
+  // ---- epilogue ---------------------------------------------------------------------------------------
+  if (a.lean) {
+    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16, old);
+    TRACE_POINT(15);
+    return;
+  }
+  size_t pix[TN];
+  bool pvalid[TN];
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) {
+    const int gp = pix0 + nt * 32 + l32;
+    pvalid[nt] = gp < a.p_total;
+    const int gpc = pvalid[nt] ? gp : 0;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
+    pix[nt] = ((size_t)n * a.oc2 * a.ohw + (gpc - n * a.ohw)) * 16;
+  }
+  const size_t pixT[TN][2] = {};
+  const bool validT[TN][2] = {};
+  epilogue_wave<TM, TN, false, true>(a.ep, acc, k0, cidx, oc0 + 16 * lh, pix, pvalid, oc_real, (size_t)a.ohw * 16, a.out,
+                                     nullptr, pixT, validT);
+}
+
+namespace {
+struct ResVariant {
+  const char *name;
+  int oc_t, p_t;
+  void (*generic)(GemmArgs);
+  void (*unrolled[3])(GemmArgs);   // exactly 8, 16, 32 k-steps
+};
+#define RV(TM, TN)                                                                                           \
+  { "k_gemm1x1_res<" #TM "," #TN ">", 4 * TM * 32, TN * 32, k_gemm1x1_res<TM, TN, 0>,                        \
+    {k_gemm1x1_res<TM, TN, 8>, k_gemm1x1_res<TM, TN, 16>, k_gemm1x1_res<TM, TN, 32>} }
+const ResVariant kRes[] = {
+    RV(1, 4),   // 0: 128 oc x 128 px
+    RV(1, 2),   // 1: 128 oc x  64 px
+    RV(2, 4),   // 2: 256 oc x 128 px
+    RV(2, 2),   // 3: 256 oc x  64 px
+};
+#undef RV
+constexpr int kNumRes = sizeof(kRes) / sizeof(kRes[0]);
+constexpr size_t kResLds = 160 * 1024;
+
+}  // namespace
+
+// -1: the layer is not one for this kernel
+int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
+{
+  const char *env = getenv("EHIP_GEMM1X1_RES");
+  if (env && env[0] == '0') return -1;
+  if (nbatch != 1 || a.kh * a.kw > 1 || a.in_nhwc || a.out_nhwc || a.ep.shift_tab) return -1;
+  if (a.ic2 <= 8 || (a.units_pad & 1)) return -1;   // few channels: the weights-in-registers kernel
+  if (env && env[0] >= '1' && env[0] <= '4') {
+    const int v = env[0] - '1';
+    return (size_t)a.units_pad * kRes[v].p_t * 16 <= kResLds ? v : -1;
+  }
+  const int oc = a.oc2 * 16;
+  int best = -1;
+  double best_score = 0;
+  for (int v = 0; v < kNumRes; ++v) {
+    const ResVariant &k = kRes[v];
+    if ((size_t)a.units_pad * k.p_t * 16 > kResLds) continue;
+    const int gx = (a.p_total + k.p_t - 1) / k.p_t, gy = (oc + k.oc_t - 1) / k.oc_t;
+    const long long wgs = (long long)gx * gy;
+    const int per_cu = (int)(kResLds / ((size_t)a.units_pad * k.p_t * 16));   // resident workgroups
+    const long long slots = 256ll * (per_cu > 2 ? 2 : per_cu);
+    const long long rounds = (wgs + slots - 1) / slots;
+    const double util = ((double)oc / ((double)gy * k.oc_t)) * ((double)a.p_total / ((double)gx * k.p_t));
+    const double fill = (double)wgs / (double)(rounds * slots);
+    // Measured (1024 -> 256 at 14 x 14 and 512 -> 1024 stride 2, N = 64): the 128 x 64 tile, two workgroups
+    // per CU that hide each other's load, flip and epilogue phases, 8.6 / 17.5 us; 128 x 128 10.8 / 19.4 us;
+    // the 256-channel tiles (a wave owns 64 channels, twice the registers) 9.0-14.4 / 22.5-25.9 us.
+    static const double pref[] = {0.95, 1.10, 0.70, 0.85};
+    const double score = util * (0.5 + 0.5 * fill) * pref[v] * (per_cu >= 2 ? 1.0 : 0.9);
+    if (score > best_score) { best_score = score; best = v; }
+  }
+  return best;
+}
+
+const char *gemm1x1_res_name(int v) { return kRes[v].name; }
+
+hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s)
+{
+  const ResVariant &k = kRes[v];
+  GemmArgs a = a0;
+  a.lean = lean_mode(a.ep, false);
+  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
+  a.nx = (a.p_total + k.p_t - 1) / k.p_t;
+  a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
+  const int nks = a.units_pad / 2;
+  void (*kernel)(GemmArgs) = k.generic;
+  const char *env = getenv("EHIP_GEMM1X1_UNROLL");
+  if (!(env && env[0] == '0')) {
+    if (nks == 8) kernel = k.unrolled[0];
+    else if (nks == 16) kernel = k.unrolled[1];
+    else if (nks == 32) kernel = k.unrolled[2];
+  }
+  const size_t lds_bytes = (size_t)a.units_pad * k.p_t * 16;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds_bytes);
+  if (e != hipSuccess) return e;
+  dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
+  hipLaunchKernelGGL(kernel, grid, dim3(kBlock), lds_bytes, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace ehip

@@ -61,6 +61,7 @@ struct GemmArgs {
   unsigned ic2_magic, kw_magic;
   int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
+  int lean;                    // set by the launcher: lean_mode() of the epilogue (0 = general epilogue)
 };
 
 struct Conv3x3Args {
@@ -76,8 +77,7 @@ struct Conv3x3Args {
   unsigned vw_magic;    // div_magic(vw)
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
   int gx, gy, tiles, tiles_per_xcd;   // set by the launcher: pixel tiles per image, channel tiles, all tiles, ceil(tiles / 8)
-  int lean;             // set by the launcher: 0 = general epilogue, 1 = u8 / s8 with ReLU bounds 0 <= lo <= hi and no
-                        // sum, 2 = u8 whose bounds are the code range 0 .. 255 (no clamp needed)
+  int lean;             // set by the launcher: lean_mode() of the epilogue (0 = general epilogue)
 };
 
 struct DepthwiseArgs {
@@ -136,6 +136,11 @@ int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride);
 int gemm_variant_chunk(int variant);
 int gemm_num_variants();
 const char *gemm_variant_name(int variant);
+
+// 1x1 layers with many input channels, blocked activations: pixel tile resident in LDS, weights streamed
+int gemm1x1_res_pick(const GemmArgs &a, int nbatch);   // variant, or -1 when the layer is not one for it
+const char *gemm1x1_res_name(int variant);
+hipError_t launch_gemm1x1_res(const GemmArgs &a, int variant, hipStream_t s);
 
 hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s);
 int conv3x3v_pick_variant(int n, int oh, int ow, int oc2);   // -1: rows too wide for every variant
@@ -513,6 +518,97 @@ __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&a
     epilogue_wave_tab<TM, TN, false, NOCOMP>(ep, acc, k0, cidx, oc_first, pix, pvalid, oc_real, block_stride, out, xlds, pixT, validT, cls);
 }
 
+
+// ---- lean epilogue -------------------------------------------------------------------------------
+// u8 / s8 output, ReLU with bounds 0 <= lo <= hi (lo <= 127 for s8), with or without the in-place sum,
+// per-channel shift only: the case of nearly every layer of the tuned networks.  The launcher decides
+// (lean_mode) so that the kernel carries no output-type switch on this path; the accumulators already hold
+// the u8 -> s8 compensation.  A value costs a convert, a multiply-add, (a second one for the sum,) a
+// clamp -- none when the bounds are exactly the u8 code range, which v_cvt_pk_u8_f32 saturates to by
+// itself -- and a byte pack.  Arithmetic and rounding are those of quant4<.., FAST = true>.
+struct LeanConsts {   // scale and shift of the lane's 16 channels of each 32-channel tile
+  float4 sc[4], sh[4];
+};
+__device__ __forceinline__ void load_lean_consts(LeanConsts &k, const Epilogue &ep, long long idx)
+{
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    k.sc[q] = *reinterpret_cast<const float4 *>(ep.scale + idx + 4 * q);
+    k.sh[q] = *reinterpret_cast<const float4 *>(ep.shift + idx + 4 * q);
+  }
+}
+// 0 = general epilogue; else bit 0 set, bit 1 = no clamp needed, bit 2 = with sum
+inline int lean_mode(const Epilogue &e, bool out_nhwc)
+{
+  const bool q = e.out_type == EHIP_U8 || e.out_type == EHIP_S8;
+  const bool fast = q && e.with_relu && !e.shift_tab && !out_nhwc && e.lo >= 0.0f && e.hi >= e.lo &&
+      (e.out_type != EHIP_S8 || e.lo <= 127.0f);
+  if (!fast) return 0;
+  return 1 | ((e.out_type == EHIP_U8 && e.lo == 0.0f && e.hi >= 255.0f) ? 2 : 0) | (e.with_sum ? 4 : 0);
+}
+// cell[nt]: byte address of the lane's 16-byte cell of pixel tile nt in the wave's FIRST 16-channel block pair
+// member (block lh of tile 0); tile_stride: bytes between the cells of consecutive 32-channel tiles.
+// old_in: the sum operands if the caller has fetched them already (else null: they are read here).
+template <int TM, int TN, bool SUM, bool CLAMP>
+__device__ __forceinline__ void lean_store_typed(const Epilogue &ep, const v16i (&acc)[TM][TN], const LeanConsts (&k)[TM],
+                                                 uint8_t *const (&cell)[TN], const bool (&pvalid)[TN], int oc_first,
+                                                 int oc_real, size_t tile_stride, const v4i (*old_in)[TN])
+{
+  const bool s8 = ep.out_type == EHIP_S8;
+  const float hi = s8 ? __builtin_fminf(ep.hi, 127.0f) : ep.hi;
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) {
+    v4i old[TM];
+    if (SUM) {
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        if (old_in) {
+          old[mt] = old_in[mt][nt];
+        } else {
+          const bool ok = pvalid[nt] && oc_first + 32 * mt < oc_real;
+          old[mt] = *reinterpret_cast<const v4i *>(ok ? cell[nt] + mt * tile_stride : cell[nt]);
+        }
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) {
+      v4i out;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float sc[4] = {k[mt].sc[q].x, k[mt].sc[q].y, k[mt].sc[q].z, k[mt].sc[q].w};
+        const float sh[4] = {k[mt].sh[q].x, k[mt].sh[q].y, k[mt].sh[q].z, k[mt].sh[q].w};
+        unsigned pk = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float f = __builtin_fmaf((float)acc[mt][nt][4 * q + j], sc[j], sh[j]);
+          if (SUM) {
+            const unsigned b = ((unsigned)old[mt][q] >> (8 * j)) & 0xffu;
+            const int o = s8 ? (int)(signed char)b : (int)b;
+            f = __builtin_fmaf((float)o, ep.sum_scale, f);
+          }
+          if (CLAMP) f = __builtin_amdgcn_fmed3f(f, ep.lo, hi);
+          pk = __builtin_amdgcn_cvt_pk_u8_f32(f, j, pk);
+        }
+        out[q] = (int)pk;
+      }
+      if (pvalid[nt] && oc_first + 32 * mt < oc_real) *reinterpret_cast<v4i *>(cell[nt] + mt * tile_stride) = out;
+    }
+  }
+}
+template <int TM, int TN>
+__device__ __forceinline__ void lean_store(int mode, const Epilogue &ep, const v16i (&acc)[TM][TN], const LeanConsts (&k)[TM],
+                                           uint8_t *const (&cell)[TN], const bool (&pvalid)[TN], int oc_first, int oc_real,
+                                           size_t tile_stride, const v4i (*old_in)[TN] = nullptr)
+{
+  // one uniform branch, four straight copies
+  if (mode & 4) {
+    if (mode & 2) lean_store_typed<TM, TN, true, false>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+    else lean_store_typed<TM, TN, true, true>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+  } else {
+    if (mode & 2) lean_store_typed<TM, TN, false, false>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+    else lean_store_typed<TM, TN, false, true>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+  }
+}
 
 }  // namespace ehip
 #endif

@@ -65,6 +65,25 @@ def test_conv1x1_stride2(out_type):
     run_and_compare(Layer(2, 64, 96, 14, stride=2, out_type=out_type, with_sum=(out_type == ol.S8), seed=6))
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+@pytest.mark.parametrize("n,ic,oc,hw,stride", [(2, 256, 256, 14, 1), (3, 144, 80, 9, 1), (1, 512, 272, 14, 2), (2, 1024, 128, 7, 1),
+                                               (1, 272, 48, 5, 1)])
+def test_conv1x1_resident_pixel_tile_kernel(variant, n, ic, oc, hw, stride, monkeypatch):
+    """the 1x1 kernel for many input channels (pixel tile resident in LDS, weights streamed): every tile shape;
+    K loop unrolled (8, 16, 32 k-steps) and as a loop; ragged channel and pixel counts; stride 2; with the sum"""
+    monkeypatch.setenv("EHIP_GEMM1X1_RES", str(variant))
+    for out_type, with_sum in ((ol.U8, False), (ol.S8, True), (ol.F32, False), (ol.S32, False)):
+        res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, with_sum=with_sum,
+                                    seed=300 + variant + ic + out_type))
+    monkeypatch.setenv("EHIP_GEMM1X1_UNROLL", "0")
+    run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=ol.U8, seed=301 + variant + ic, relu_hi=200.0))
+
+
+def test_conv1x1_resident_pixel_tile_kernel_can_be_switched_off(monkeypatch):
+    monkeypatch.setenv("EHIP_GEMM1X1_RES", "0")
+    run_and_compare(Layer(2, 256, 256, 14, out_type=ol.S8, with_sum=True, seed=302))
+
+
 def test_conv1x1_lazy_first_run_and_no_bias():
     run_and_compare(Layer(1, 64, 32, 6, out_type=ol.U8, with_bias=False, seed=8), lazy=True)
 
@@ -72,6 +91,7 @@ def test_conv1x1_lazy_first_run_and_no_bias():
 @pytest.mark.parametrize("variant", range(7))
 def test_conv1x1_every_kernel_variant(variant, monkeypatch):
     monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
+    monkeypatch.setenv("EHIP_GEMM1X1_RES", "0")   # the general kernel, not the one with the resident pixel tile
     res = run_and_compare(Layer(2, 144, 80, 11, out_type=ol.S8, with_sum=True, seed=40 + variant))
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
