@@ -61,6 +61,15 @@ struct ehip_conv {
   uint8_t *tin = nullptr;
   float *tout = nullptr;
   size_t tin_bytes = 0, tout_bytes = 0;
+
+  // launch plans of the steady state (filled by the first execute, see LaunchPlan); the Winograd ones are
+  // used only when the layer runs in one pass (no chunking)
+  LaunchPlan<GemmArgs> plan_gemm;
+  LaunchPlan<Conv3x3Args> plan_3x3;
+  LaunchPlan<FewChArgs> plan_fewch;
+  LaunchPlan<DepthwiseArgs> plan_dw;
+  LaunchPlan<WinoArgs> plan_wino_in, plan_wino_out;
+  LaunchPlan<WinoFusedArgs> plan_wino_fused;
 };
 
 namespace {
@@ -597,7 +606,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       a.cls_h = c->cls_h; a.cls_w = c->cls_w; a.ncls_w = c->ncls_w;
     }
     a.trace = trace_buffer();
-    HIP_TRY(launch_gemm(a, 1, c->variant, s));
+    HIP_TRY(launch_gemm(a, 1, c->variant, s, &c->plan_gemm));
     break;
   }
   case FAM_CONV_FEWCH: {
@@ -617,7 +626,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     }
     if (a.in_nhwc && (reinterpret_cast<uintptr_t>(input_dev) & 3))
       return fail(EHIP_GENERAL_ERROR, "nhwc input of a few-channel layer must be 4-byte aligned");
-    HIP_TRY(launch_conv_fewch(a, s));
+    HIP_TRY(launch_conv_fewch(a, s, &c->plan_fewch));
     break;
   }
   case FAM_CONV_3X3: {
@@ -634,7 +643,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.vw = d.ow + 2;
     a.vw_magic = div_magic(a.vw);
     a.trace = trace_buffer();
-    HIP_TRY(launch_conv3x3v(a, d.n, c->variant, s));
+    HIP_TRY(launch_conv3x3v(a, d.n, c->variant, s, &c->plan_3x3));
     break;
   }
   case FAM_DEPTHWISE: {
@@ -650,11 +659,12 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.T = c->T; a.Tr = c->Tr; a.wt = c->wtb;
     a.out_type = d.output_type; a.with_relu = d.with_relu;
     a.lo = d.relu_lower; a.hi = d.relu_upper;
-    HIP_TRY(launch_depthwise(a, s));
+    HIP_TRY(launch_depthwise(a, s, &c->plan_dw));
     break;
   }
   case FAM_WINOGRAD: {
     if (d.with_bias && !bias_dev) return fail(EHIP_GENERAL_ERROR, "Parameter error. Invalid input data!");
+    const bool one_pass = c->chunk_n >= d.n;   // the launch plans hold ONE pass's arguments
     for (int n0 = 0; n0 < d.n; n0 += c->chunk_n) {
       ehip_conv_desc_t dc = d;
       dc.n = d.n - n0 < c->chunk_n ? d.n - n0 : c->chunk_n;
@@ -670,7 +680,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       const float tin_repS = 1.0f / d.tinput_scale;
       w.mrepS = d.input_scale * tin_repS;
       w.mz = ceilf(d.tinput_z);
-      HIP_TRY(launch_wino_trans_input(w, s));
+      HIP_TRY(launch_wino_trans_input(w, s, one_pass ? &c->plan_wino_in : nullptr));
       if (c->fused) {
         WinoFusedArgs f;
         memset(&f, 0, sizeof(f));
@@ -682,7 +692,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.out_type = w.out_type; f.out_repS = w.out_repS; f.out_z = w.out_z;
         f.out_nhwc = w.out_nhwc;
         f.trace = trace_buffer();
-        HIP_TRY(launch_wino_gemm_output(f, s));
+        HIP_TRY(launch_wino_gemm_output(f, s, one_pass ? &c->plan_wino_fused : nullptr));
         continue;
       }
       GemmArgs a;
@@ -698,8 +708,8 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
       a.in_batch_stride = (long long)c->ic2 * w.t * 16;
       a.out_batch_stride = (long long)c->oc2 * w.t * 16;
-      HIP_TRY(launch_gemm(a, c->nbatch, c->variant, s));
-      HIP_TRY(launch_wino_trans_output(w, s));
+      HIP_TRY(launch_gemm(a, c->nbatch, c->variant, s, one_pass ? &c->plan_gemm : nullptr));
+      HIP_TRY(launch_wino_trans_output(w, s, one_pass ? &c->plan_wino_out : nullptr));
     }
     break;
   }

@@ -188,23 +188,26 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 }
 
 namespace {
+typedef void (*dw_kernel_t)(DepthwiseArgs);
 template <int RB, int S>
-void launch_rbs(const DepthwiseArgs &a, int mode, dim3 grid, dim3 block, hipStream_t s)
+dw_kernel_t kernel_rbs(int mode)
 {
-  if (mode == 2) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 2, S>), grid, block, 0, s, a);
-  else if (mode == 1) hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 1, S>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((k_depthwise3x3_u8s8<RB, 0, S>), grid, block, 0, s, a);
+  return mode == 2 ? k_depthwise3x3_u8s8<RB, 2, S> : (mode == 1 ? k_depthwise3x3_u8s8<RB, 1, S> : k_depthwise3x3_u8s8<RB, 0, S>);
 }
 template <int RB>
-void launch_rb(const DepthwiseArgs &a, int mode, dim3 grid, dim3 block, hipStream_t s)
+dw_kernel_t kernel_rb(int stride, int mode)
 {
-  if (a.stride == 2) launch_rbs<RB, 2>(a, mode, grid, block, s);
-  else launch_rbs<RB, 1>(a, mode, grid, block, s);
+  return stride == 2 ? kernel_rbs<RB, 2>(mode) : kernel_rbs<RB, 1>(mode);
 }
 }  // namespace
 
-hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s)
+hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<DepthwiseArgs> *plan)
 {
+  if (plan && plan->valid) {   // everything but the tensors is as on the first launch
+    plan->args.in = a0.in;
+    plan->args.out = a0.out;
+    return plan_relaunch(*plan, s);
+  }
   DepthwiseArgs a = a0;
   if (a.stride != 1 && a.stride != 2) {
     set_error("depthwise: stride must be 1 or 2");
@@ -230,11 +233,9 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s)
   a.blocks_per_plane = (a.lanes_per_plane + block - 1) / block;
   const long long planes = (long long)a.n * a.g2;
   dim3 grid((unsigned)(8 * ((planes + 7) / 8) * a.blocks_per_plane), 1, 1);
-  if (rb == 7) launch_rb<7>(a, mode, grid, dim3(block), s);
-  else if (rb == 4) launch_rb<4>(a, mode, grid, dim3(block), s);
-  else if (rb == 2) launch_rb<2>(a, mode, grid, dim3(block), s);
-  else launch_rb<1>(a, mode, grid, dim3(block), s);
-  return hipGetLastError();
+  const dw_kernel_t kernel = rb == 7 ? kernel_rb<7>(a.stride, mode)
+      : (rb == 4 ? kernel_rb<4>(a.stride, mode) : (rb == 2 ? kernel_rb<2>(a.stride, mode) : kernel_rb<1>(a.stride, mode)));
+  return plan_launch(plan, kernel, grid, dim3(block), 0, a, s);
 }
 
 }  // namespace ehip

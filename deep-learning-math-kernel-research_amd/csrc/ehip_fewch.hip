@@ -239,8 +239,14 @@ int conv_fewch_row_pitch(int ic, int kw, int iw, int ow, int stride_w, int pad_l
 
 // Fills the derived fields (cells, strip height, LDS row pitch, wave split) and launches.
 // Expects in a: tensors, epilogue, n, ih, iw, oh, ow, ic, kh, kw, strides, pads, oc2, ocpp, formats, classes.
-hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s)
+hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> *plan)
 {
+  if (plan && plan->valid) {   // everything but the tensors is as on the first launch
+    if (a.in_nhwc && (reinterpret_cast<uintptr_t>(a.in) & 3)) return hipErrorInvalidValue;   // aligned dword loads
+    plan->args.in = a.in;
+    plan->args.out = a.out;
+    return plan_relaunch(*plan, s);
+  }
   a.ppc = 16 / a.ic;
   a.nu = (a.kw + a.ppc - 1) / a.ppc;
   a.cells = a.kh * a.nu;
@@ -313,8 +319,7 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s)
   const int ks = (a.cells + 1) / 2;
   void (*kern)(FewChArgs) = ks <= 2 ? k_conv_fewch_u8s8<2> : ks == 3 ? k_conv_fewch_u8s8<3> : ks == 4 ? k_conv_fewch_u8s8<4>
       : ks == 5 ? k_conv_fewch_u8s8<5> : k_conv_fewch_u8s8<7>;
-  hipLaunchKernelGGL(kern, dim3(a.n * a.strips, gy), dim3(kBlock), lds, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, kern, dim3(a.n * a.strips, gy), dim3(kBlock), lds, a, s);
 }
 
 }  // namespace ehip

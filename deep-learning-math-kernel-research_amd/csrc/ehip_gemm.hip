@@ -537,7 +537,7 @@ bool gemm_smallk_applies(int ic2, int taps, int nbatch)
   return nbatch == 1 && taps <= 1 && ic2 <= 8;
 }
 
-hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s)
+hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr)
 {
   GemmArgs a = a0;
   const int ks = a.ic2 <= 2 ? 1 : (a.ic2 <= 4 ? 2 : 4);
@@ -557,16 +557,20 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s)
   const int cap = (wgs + ny - 1) / ny;
   if (nx > cap) nx = cap;
   void (*kernel)(GemmArgs) = ks == 1 ? smallk_kernel<1>(tnw) : (ks == 2 ? smallk_kernel<2>(tnw) : smallk_kernel<4>(tnw));
-  hipLaunchKernelGGL(kernel, dim3(nx, ny), dim3(kBlock), 0, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, kernel, dim3(nx, ny), dim3(kBlock), 0, a, s);
 }
 
-hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s)
+hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s, LaunchPlan<GemmArgs> *plan)
 {
-  if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s);
+  if (plan && plan->valid) {   // everything but the tensors is as on the first launch
+    plan->args.in = a0.in;
+    plan->args.out = a0.out;
+    return plan_relaunch(*plan, s);
+  }
+  if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s, plan);
   {
     const int rv = gemm1x1_res_pick(a0, nbatch);
-    if (rv >= 0) return launch_gemm1x1_res(a0, rv, s);
+    if (rv >= 0) return launch_gemm1x1_res(a0, rv, s, plan);
   }
   const Variant &k = kVariants[variant];
   GemmArgs a = a0;
@@ -589,8 +593,7 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   if (taps > 1 && (taps > 64 || nbatch != 1)) return hipErrorInvalidValue;
   const int fmt = taps > 1 ? (a.in_nhwc ? 4 : (a.ic2 % k.kc == 0 ? 2 : 3)) : (a.in_nhwc ? 1 : 0);
   while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[fmt][dl])) --dl;
-  hipLaunchKernelGGL(k.kernel[fmt][dl], grid, dim3(kBlock), 0, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, k.kernel[fmt][dl], grid, dim3(kBlock), 0, a, s);
 }
 
 }  // namespace ehip

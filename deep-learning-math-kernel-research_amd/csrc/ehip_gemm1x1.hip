@@ -309,7 +309,7 @@ int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
 
 const char *gemm1x1_res_name(int v) { return kRes[v].name; }
 
-hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s)
+hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPlan<GemmArgs> *plan)
 {
   const ResVariant &k = kRes[v];
   GemmArgs a = a0;
@@ -330,8 +330,7 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s)
                                      (int)lds_bytes);
   if (e != hipSuccess) return e;
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
-  hipLaunchKernelGGL(kernel, grid, dim3(kBlock), lds_bytes, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, kernel, grid, dim3(kBlock), lds_bytes, a, s);
 }
 
 }  // namespace ehip

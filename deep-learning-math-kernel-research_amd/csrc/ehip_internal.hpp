@@ -129,8 +129,42 @@ struct WinoFusedArgs {
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
 };
 
+// ---- launch plans -------------------------------------------------------------------------------
+// What a launcher works out from the layer -- kernel, grid, LDS size, derived arguments, the EHIP_* knobs
+// read from the environment, the one-off hipFuncSetAttribute -- is kept in the handle after the first
+// launch: later executes of the handle patch the tensor pointers into the kept argument block and launch.
+template <typename Args>
+struct LaunchPlan {
+  bool valid = false;
+  void (*kernel)(Args) = nullptr;
+  dim3 grid, block;
+  unsigned lds = 0;
+  Args args;
+};
+template <typename Args>
+inline hipError_t plan_launch(LaunchPlan<Args> *plan, void (*kernel)(Args), dim3 grid, dim3 block, size_t lds, const Args &a,
+                              hipStream_t s)
+{
+  if (plan) {
+    plan->valid = true;
+    plan->kernel = kernel;
+    plan->grid = grid;
+    plan->block = block;
+    plan->lds = (unsigned)lds;
+    plan->args = a;
+  }
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, a);
+  return hipGetLastError();
+}
+template <typename Args>
+inline hipError_t plan_relaunch(LaunchPlan<Args> &plan, hipStream_t s)
+{
+  hipLaunchKernelGGL(plan.kernel, plan.grid, plan.block, plan.lds, s, plan.args);
+  return hipGetLastError();
+}
+
 // ---- launchers (implemented next to their kernels) ------------------------------------------
-hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s);
+hipError_t launch_gemm(const GemmArgs &a, int nbatch, int variant, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr);
 bool gemm_smallk_applies(int ic2, int taps, int nbatch);
 int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride);
 int gemm_variant_chunk(int variant);
@@ -140,18 +174,18 @@ const char *gemm_variant_name(int variant);
 // 1x1 layers with many input channels, blocked activations: pixel tile resident in LDS, weights streamed
 int gemm1x1_res_pick(const GemmArgs &a, int nbatch);   // variant, or -1 when the layer is not one for it
 const char *gemm1x1_res_name(int variant);
-hipError_t launch_gemm1x1_res(const GemmArgs &a, int variant, hipStream_t s);
+hipError_t launch_gemm1x1_res(const GemmArgs &a, int variant, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr);
 
-hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s);
+hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s, LaunchPlan<Conv3x3Args> *plan = nullptr);
 int conv3x3v_pick_variant(int n, int oh, int ow, int oc2);   // -1: rows too wide for every variant
 int conv3x3v_chunk_units(int variant, int ic2);
 int conv3x3v_num_variants();
 const char *conv3x3v_variant_name(int variant);
 
-hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s);
-hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s);
-hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s);
-hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s);
+hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s, LaunchPlan<DepthwiseArgs> *plan = nullptr);
+hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
+hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
+hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);
 // min / max of the transformed input: partials = 2 * a.ic2 dwords of device scratch, result = two floats
 // of device memory (min, max); three launches on `s`, nothing else
 hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *partials, float *minmax_out_dev, hipStream_t s);
@@ -187,7 +221,7 @@ struct FewChArgs {
 };
 bool conv_fewch_applies(int ic, int kh, int kw);
 int conv_fewch_row_pitch(int ic, int kw, int iw, int ow, int stride_w, int pad_l);
-hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s);
+hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> *plan = nullptr);
 hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int kh, int kw, int ppc, int nu,
                                     int ocpp, const ehip_conv_desc_t &d, float *absmax, int8_t *wpacked, float *scale,
                                     float *shift, int *wsum, int *comp, hipStream_t s);

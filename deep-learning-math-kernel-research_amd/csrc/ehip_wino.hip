@@ -532,8 +532,12 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   }
 }
 
-hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s)
+hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s, LaunchPlan<WinoArgs> *plan)
 {
+  if (plan && plan->valid) {   // everything but the tensors is as on the first launch
+    plan->args.in = a0.in;
+    return plan_relaunch(*plan, s);
+  }
   WinoArgs a = a0;
   a.nblocks = (a.t + 63) / 64;
   a.items_per_xcd = (int)(((long long)a.nblocks * a.ic2 + 7) / 8);
@@ -542,12 +546,16 @@ hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s)
   if (a.tile == 4) kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 4> : k_wino_trans_input_u8<float4, 4>;
   else if (a.tile == 5) kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 5> : k_wino_trans_input_u8<float4, 5>;
   else kern = a.in_u8 ? k_wino_trans_input_u8<unsigned, 6> : k_wino_trans_input_u8<float4, 6>;
-  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, kern, grid, dim3(kBlock), 0, a, s);
 }
 
-hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s)
+hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan)
 {
+  if (plan && plan->valid) {   // everything but the tensors is as on the first launch
+    plan->args.out = a.out;
+    plan->args.bias = a.bias;
+    return plan_relaunch(*plan, s);
+  }
   dim3 grid((a.t + 63) / 64, a.oc2);
   void (*kern)(WinoArgs) = nullptr;
 #define EHIP_WO(A)                                                                                         \
@@ -557,13 +565,17 @@ hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s)
   else if (a.tile == 5) EHIP_WO(5);
   else EHIP_WO(6);
 #undef EHIP_WO
-  hipLaunchKernelGGL(kern, grid, dim3(kBlock), 0, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, kern, grid, dim3(kBlock), 0, a, s);
 }
 
 // k-steps per ring block: the largest of 8, 4, 2 that divides the k-steps of a position
-hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s)
+hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan)
 {
+  if (plan && plan->valid) {   // everything but the tensors is as on the first launch
+    plan->args.out = a0.out;
+    plan->args.bias = a0.bias;
+    return plan_relaunch(*plan, s);
+  }
   WinoFusedArgs a = a0;
   a.nx = (a.t + 31) / 32;
   a.ny = (a.oc2 * 16 + 63) / 64;
@@ -577,8 +589,7 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s)
   if (nks % 2 != 0) return hipErrorInvalidValue;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, grid, dim3(kBlock), lds, s, a);
-  return hipGetLastError();
+  return plan_launch(plan, kernel, grid, dim3(kBlock), lds, a, s);
 }
 
 // partials: 2 * a.ic2 dwords of device memory; minmax_out_dev: two floats of device memory
