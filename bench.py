@@ -6,8 +6,9 @@
 A step is one pass of the hot path (one elx_conv-equivalent execute) over one batch of synthetic,
 device-resident tensors of the named layer.  The headline workload is C2 (int8 3x3 direct conv,
 ResNet-50 res3 shape, N=32).  Prints ONE JSON line: effective INT8 TOPS (2 x direct-conv MACs /
-time, the reference's accounting), the roofline of the dominant kernel from HIP-event timing, the
-host-CPU baseline of the same layer, and -- under "layers" -- the other configured layers.
+time, the reference's accounting), the roofline of the dominant kernel (from the same interval as
+ms_per_step, with the HIP-event figure of the same steps beside it), the host-CPU baseline of the
+same layer, and -- under "layers" -- the other configured layers, each with its own CPU baseline.
 """
 import argparse
 import ctypes
@@ -60,70 +61,144 @@ def single_launch_latency(layer, reps=20):
     return best
 
 
-def roofline_of(wl, sec_per_launch, traffic):
+def roofline_of(wl, sec_per_step, sec_per_step_events, traffic):
+    """`achieved` and `frac` come from the same interval as ms_per_step (host clock around the timed
+    steps, synchronised on both sides); `frac_event` is the same figure from the HIP events recorded
+    on the kernels' stream around the same steps, which leaves out the host's share of the first
+    enqueue and of the final synchronisation."""
     from importlib import import_module
     W = import_module(PKG + ".workloads")
     kind, _ = wl.bound()
     if kind == "mfma":
-        achieved = wl.ops() / sec_per_launch / 1e12
+        work, scale = wl.ops(), 1e12
         peak, unit = W.PEAK_INT8_TOPS, "TFLOP/s"
     else:
-        achieved = wl.algorithmic_bytes() / sec_per_launch / 1e9
+        work, scale = wl.algorithmic_bytes(), 1e9
         peak, unit = W.PEAK_HBM_GBS, "GB/s"
+    achieved = work / sec_per_step / scale
     return {"bound": kind, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 5), "traffic": traffic}
+            "frac": round(achieved / peak, 5), "traffic": traffic,
+            "achieved_event": round(work / sec_per_step_events / scale, 3),
+            "frac_event": round(work / sec_per_step_events / scale / peak, 5)}
 
 
-def cpu_model():
+def host_cpus():
+    """(model name, logical CPUs visible, physical cores, threads per core) from /proc/cpuinfo"""
+    model, cores, logical = "unknown", set(), 0
+    phys = core = None
     try:
         with open("/proc/cpuinfo") as f:
             for line in f:
-                if line.startswith("model name"):
-                    return line.split(":", 1)[1].strip()
+                key, _, val = line.partition(":")
+                key, val = key.strip(), val.strip()
+                if key == "model name":
+                    model = val
+                elif key == "processor":
+                    logical += 1
+                elif key == "physical id":
+                    phys = val
+                elif key == "core id":
+                    core = val
+                    cores.add((phys, core))
     except OSError:
         pass
-    return "unknown"
+    physical = len(cores) or logical
+    return model, logical, physical, (logical // physical if physical else 1)
+
+
+def reference_iterations(ops):
+    """the repeat count of the reference's benchmark loop (tests/elt_conv_utils.cpp:661-664)"""
+    return min(1024, max(int(5e12 / ops), 64))
 
 
 def cpu_baseline(wl, budget_s=12.0):
-    """The CPU oracle (a port of the reference's loop nest; AVX-512-VNNI inner loop when the host
-    has it) timed on this host's cores on the same layer.  Bounded: as many passes as fit ~budget."""
+    """The CPU oracle (a port of the reference's loop nests; AVX-512-VNNI inner loops when the host
+    has them) timed on this host's cores on the same layer: the direct 1x1 / k x k nest, the depthwise
+    nest or the three Winograd stages (input transform, u8 x s8 GEMM, output transform), steady state
+    (weight preparation excluded).  The reference's benchmark repeats a layer
+    clamp(5e12 / ops, 64, 1024) times (tests/elt_conv_utils.cpp:661-664); here the same count is the
+    upper limit and `budget_s` seconds end the loop earlier, and a layer whose single pass would not fit
+    the budget runs on a slice of its batch (every image is independent, so the rate carries over)."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import numpy as np
     import oracle_lib as ol
+    E = importlib.import_module(PKG)
     rng = np.random.default_rng(7)
-    n = wl.n
-    # keep one pass in the low seconds even on a scalar host: sample a slice of the batch
     lib = ol.oracle()
     vnni = bool(lib.orc_has_vnni())
     threads = int(lib.orc_num_threads())
-    if wl.algorithm != 2 or wl.depthwise or wl.k not in (1, 3):
-        return None
-    if not vnni:
-        n = max(1, n // 8)
-    x = rng.integers(0, 256, (n, ol.up16(wl.ic) // 16, wl.hw, wl.hw, 16)).astype(np.uint8)
-    w = rng.normal(0, wl.w_sigma, (wl.oc, wl.ic, wl.k, wl.k)).astype(np.float32)
+    model, logical, physical, smt = host_cpus()
+    wino = wl.algorithm == E.CONV_WINOGRAD
+    if wl.in_z != 0.0 or (wl.nhwc_in and wl.ic <= 4):
+        return None   # the oracle's border-shift path is a per-case checker, not a timed loop nest
+    # a first guess of one pass: ~1 TOPS per 8 VNNI threads for the direct nests, far less for the others
+    n = wl.n
+    rate = (0.12 if vnni else 0.004) * threads * (0.05 if wl.depthwise else (0.3 if wino else 1.0)) * 1e12
+    while n > 1 and wl.ops() * n / wl.n / rate > budget_s / 4:
+        n = (n + 1) // 2
+    ic2, oc2 = ol.up16(wl.ic) // 16, ol.up16(wl.oc) // 16
+    g = wl.ic if wl.depthwise else 1
+    relu_hi = 255.0 if wl.relu6 else ol.FLT_MAX
+    p = ol.make_params(n, wl.ic, wl.oc, wl.hw, wl.hw, wl.k, wl.k, wl.pad, wl.stride, g=g, out_type=wl.out_type,
+                       with_sum=wl.with_sum, out_scale=0.02, sum_scale=0.7 if wl.with_sum else 0.0, relu_hi=relu_hi,
+                       T=wl.T, out_hw=(wl.oh, wl.oh), pad_tl=wl.pad, wino_tile=wl.tile if wino else 0,
+                       in_scale=1.0 if wl.in_type == E.F32 else 1.0 / 255.0)
     b = rng.normal(0, 0.01, ol.up16(wl.oc)).astype(np.float32)
-    p = ol.make_params(n, wl.ic, wl.oc, wl.hw, wl.hw, wl.k, wl.k, wl.pad, wl.stride, out_type=wl.out_type,
-                       out_scale=0.02)
-    wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(w), b)   # first run, excluded from timing
-    out = np.zeros((n, ol.up16(wl.oc) // 16, wl.oh, wl.oh, 16), ol.NP_OF[wl.out_type])
-    args = (ctypes.byref(p), ol.ptr(x), ol.ptr(wq), ol.ptr(scale), ol.ptr(shift), ol.ptr(out), None)
-    lib.orc_direct_execute(*args)  # warm-up
+    out = np.zeros((n, oc2, wl.oh, wl.oh, 16), ol.NP_OF[wl.out_type])
+    if wl.with_sum:
+        out[...] = rng.integers(-127, 128, out.shape)
+    if wino:
+        x = rng.random((n, ic2, wl.hw, wl.hw, 16), dtype=np.float32)   # u8 input enters dequantized
+        w = rng.normal(0, wl.w_sigma, (wl.oc, wl.ic, 3, 3)).astype(np.float32)
+        mn, mx = ol.wino_tinput_range(p, x)
+        p.tin_scale = (mx - mn + 1e-6) / 255.0
+        p.tin_z = -mn * 255.0 / (mx - mn + 1e-6)
+        twq, tscale, tshift = ol.wino_prepare(p, ol.weights_to_blocked(w))
+        t, pos = ol.wino_tiles(p), ol.wino_positions(p)
+        tin = np.zeros((pos, ic2, t, 16), np.uint8)
+        tout = np.zeros((pos, oc2, t, 16), np.float32)
+        pp = ctypes.byref(p)
+
+        def one_pass():
+            lib.orc_wino_trans_input(pp, ol.ptr(x), ol.ptr(tin))
+            lib.orc_wino_gemm(pp, ol.ptr(tin), ol.ptr(twq), ol.ptr(tscale), ol.ptr(tshift), ol.ptr(tout), None)
+            lib.orc_wino_trans_output(pp, ol.ptr(tout), ol.ptr(b), ol.ptr(out))
+        nest = "Winograd input transform + u8 x s8 GEMM + output transform"
+    elif wl.depthwise:
+        x = rng.integers(0, 256, (n, ic2, wl.hw, wl.hw, 16)).astype(np.uint8)
+        w = rng.normal(0, wl.w_sigma, (wl.ic, 1, 3, 3)).astype(np.float32)
+        wq, scale, shift, _ = ol.depthwise_prepare(p, w, b)
+        args = (ctypes.byref(p), ol.ptr(x), ol.ptr(wq), ol.ptr(scale), ol.ptr(shift), ol.ptr(out), None)
+
+        def one_pass():
+            lib.orc_depthwise_execute(*args)
+        nest = "depthwise nest"
+    else:
+        x = rng.integers(0, 256, (n, ic2, wl.hw, wl.hw, 16)).astype(np.uint8)
+        w = rng.normal(0, wl.w_sigma, (wl.oc, wl.ic, wl.k, wl.k)).astype(np.float32)
+        wq, scale, shift, _ = ol.direct_prepare(p, ol.weights_to_blocked(w), b)
+        args = (ctypes.byref(p), ol.ptr(x), ol.ptr(wq), ol.ptr(scale), ol.ptr(shift), ol.ptr(out), None)
+
+        def one_pass():
+            lib.orc_direct_execute(*args)
+        nest = "direct %dx%d nest" % (wl.k, wl.k)
+    one_pass()  # warm-up
+    limit = reference_iterations(wl.ops())
     passes, t0 = 0, time.perf_counter()
     while True:
-        lib.orc_direct_execute(*args)
+        one_pass()
         passes += 1
         el = time.perf_counter() - t0
-        if el > budget_s or passes >= 20000:
+        if el > budget_s or passes >= limit:
             break
     sec = el / passes
     ops = wl.ops() * n / wl.n
     return {"value": round(ops / sec / 1e12, 4), "unit": "TOPS", "cores": threads, "kind": "port",
             "isa": "avx512-vnni" if vnni else "scalar/auto-vectorised",
-            "sample": "%d passes of %s with N=%d of %d in %.1f s (weight preparation excluded)" % (
-                passes, wl.key, n, wl.n, el),
-            "ms_per_pass": round(sec * 1e3, 3), "images_per_s": round(n / sec, 1), "cpu_model": cpu_model()}
+            "sample": "%d passes (the reference's loop would run %d) of the %s of %s with N=%d of %d in %.1f s on %d "
+                      "OpenMP threads; weight preparation excluded" % (passes, limit, nest, wl.key, n, wl.n, el, threads),
+            "ms_per_pass": round(sec * 1e3, 3), "images_per_s": round(n / sec, 1), "cpu_model": model,
+            "host_logical_cpus": logical, "host_physical_cores": physical, "host_threads_per_core": smt}
 
 
 def load_traffic():
@@ -141,7 +216,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--layers", default="all", help="other layers to report: all, none or a comma list")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baselines")
+    ap.add_argument("--cpu-budget", type=float, default=12.0, help="seconds of CPU work for the headline layer's baseline")
+    ap.add_argument("--cpu-budget-layer", type=float, default=2.5,
+                    help="seconds of CPU work for the baseline of each layer under \"layers\"")
     ap.add_argument("--batch", type=int, default=0, help="override the workload's batch size N (scaling studies; "
                                                          "the headline figure uses the configured N)")
     ap.add_argument("--network", default="", help="instead of one layer: every convolution layer of one of the reference's "
@@ -277,7 +355,7 @@ def main():
         "images_per_s": round(wl.n / wall, 1),
         "single_launch_latency_us": round(lat * 1e6, 2),
         "event_ms_per_step": round(ev * 1e3, 6),
-        "roofline": roofline_of(wl, ev, traffic.get(wl.key)),
+        "roofline": roofline_of(wl, wall, ev, traffic.get(wl.key)),
     }
     del layer
     torch.cuda.empty_cache()
@@ -293,18 +371,21 @@ def main():
         layers[k] = {"title": w2.title, "tops": round(w2.ops() / wall2 / 1e12, 3),
                      "images_per_s": round(w2.n / wall2, 1), "ms_per_step": round(wall2 * 1e3, 5),
                      "event_ms_per_step": round(ev2 * 1e3, 5), "kernel": l2.conv.kernel_name,
-                     "roofline": roofline_of(w2, ev2, traffic.get(k))}
+                     "roofline": roofline_of(w2, wall2, ev2, traffic.get(k))}
         del l2
         torch.cuda.empty_cache()
     if layers:
         result["layers"] = layers
 
     if not args.no_cpu:
-        try:
-            result["cpu_baseline"] = cpu_baseline(wl)
-        except Exception as exc:  # the baseline is a report, never a reason to lose the GPU number
-            result["cpu_baseline"] = {"value": None, "unit": "TOPS", "cores": 0, "kind": "port",
-                                      "sample": "failed: %r" % (exc,)}
+        def baseline(w2, budget_s):
+            try:
+                return cpu_baseline(w2, budget_s)
+            except Exception as exc:  # the baseline is a report, never a reason to lose the GPU number
+                return {"value": None, "unit": "TOPS", "cores": 0, "kind": "port", "sample": "failed: %r" % (exc,)}
+        result["cpu_baseline"] = baseline(wl, args.cpu_budget)
+        for k in layers:
+            layers[k]["cpu_baseline"] = baseline(W.WORKLOADS[k], args.cpu_budget_layer)
     print(json.dumps(result))
 
 
