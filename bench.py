@@ -293,16 +293,26 @@ def main():
         return
 
     if args.mfma_probe:
+        probe = ctypes.CDLL(os.path.join(ROOT, PKG, "build", "libehip_probe.so"))
+        probe.ehip_bench_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                   ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+
+        def probe_mfma_i8(workgroups, iters, out, stream):
+            ops = ctypes.c_double()
+            rc = probe.ehip_bench_probe_mfma_i8(workgroups, iters, ctypes.c_void_p(out.data_ptr()), ctypes.byref(ops),
+                                                ctypes.c_void_p(stream))
+            assert rc == 0
+            return ops.value
         out = torch.empty(4096 * 256, dtype=torch.int32, device="cuda")
         res = {}
         stream = torch.cuda.current_stream().cuda_stream
         for wgs in (256, 512, 1024, 2048, 4096):   # 1, 2, 4, 8, 16 waves per SIMD's worth of workgroups
-            ops = E.probe_mfma_i8(wgs, 2000, out, stream)
+            ops = probe_mfma_i8(wgs, 2000, out, stream)
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(5):
-                E.probe_mfma_i8(wgs, 2000, out, stream)
+                probe_mfma_i8(wgs, 2000, out, stream)
             e1.record()
             torch.cuda.synchronize()
             res["wgs_%d" % wgs] = round(ops / (e0.elapsed_time(e1) * 1e-3 / 5) / 1e12, 1)

@@ -79,7 +79,6 @@ def _load():
     lib.ehip_reorder_nchw_to_blocked.argtypes = [vp, vp, ci, ci, ci, ci, ci, vp]
     lib.ehip_reorder_blocked_to_nchw.argtypes = [vp, vp, ci, ci, ci, ci, ci, vp]
     lib.ehip_reorder_oihw_to_blocked.argtypes = [vp, vp, ci, ci, ci, ci, vp]
-    lib.ehip_probe_mfma_i8.argtypes = [ci, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
     return lib
 
 
@@ -89,7 +88,7 @@ EXPORTED_SYMBOLS = (
     "ehip_init", "ehip_last_error", "ehip_conv_create", "ehip_conv_destroy", "ehip_conv_prepare",
     "ehip_conv_execute", "ehip_conv_execute_repeat", "ehip_conv_query", "ehip_conv_kernel_name", "ehip_quantize_input_u8",
     "ehip_wino_tinput_range", "ehip_wino_tinput_range_noalloc", "ehip_reorder_nchw_to_blocked", "ehip_reorder_blocked_to_nchw",
-    "ehip_reorder_oihw_to_blocked", "ehip_probe_mfma_i8",
+    "ehip_reorder_oihw_to_blocked",
 )
 
 
@@ -196,13 +195,6 @@ def wino_tinput_range(desc, input):
 def wino_tinput_range_noalloc(desc, input, minmax_out, stream=0):
     """min / max into two floats of device memory (minmax_out), asynchronous, no device allocation"""
     _check(lib.ehip_wino_tinput_range_noalloc(ctypes.byref(desc), _ptr(input), _ptr(minmax_out), ctypes.c_void_p(stream)))
-
-
-def probe_mfma_i8(workgroups, iters, out, stream=0):
-    """Launches the MFMA rate probe; returns the integer operations it issues (the caller times it)."""
-    ops = ctypes.c_double()
-    _check(lib.ehip_probe_mfma_i8(workgroups, iters, _ptr(out), ctypes.byref(ops), ctypes.c_void_p(stream)))
-    return ops.value
 
 
 def reorder_nchw_to_blocked(dst, src, elem_size, n, c, h, w, stream=0):

@@ -21,7 +21,6 @@ SOURCES = [
     "ehip_depthwise.hip",
     "ehip_wino.hip",
     "ehip_prepare.hip",
-    "ehip_probe.hip",
     "ehip_api.hip",
     "euler_api.hip",
 ]
@@ -69,10 +68,23 @@ def build(verbose=True, jobs=8, incremental=False):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    # the MFMA rate probe of the benchmark: a library of its own, not part of the product's C-ABI
+    cmd = [hipcc] + FLAGS + ["-shared", os.path.join(CSRC, "ehip_probe.hip"), "-o", os.path.join(objdir, "libehip_probe.so")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    procs.append(("ehip_probe.hip", subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+    _wait(procs)
     # a small client of the C++ API (include/euler.hpp), used by the GPU tests
     check = os.path.join(objdir, "euler_api_check")
     cmd = [hipcc, "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"),
            os.path.join(ROOT, "tests", "cxx", "euler_api_check.cpp"), "-o", check,
+           "-L" + HERE, "-leuler_hip", "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/.."]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    # every reorder<> instantiation behind one C entry point, used by the CPU tests (host code only)
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-I" + os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cxx", "reorder_check.cpp"), "-o", os.path.join(objdir, "libreorder_check.so"),
            "-L" + HERE, "-leuler_hip", "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/.."]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -8,8 +8,12 @@
 // ELD_GENERAL_ERROR with the same code values; the message is available from ehip_last_error().
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <thread>
+#include <vector>
 
 #include "euler.hpp"
 #include "euler_reorder.hpp"
@@ -236,102 +240,156 @@ int elx_conv(eld_conv_t &desc, void *output, void *input, void *weights, void *b
   }
   if (!out_on_device) {
     if (hipMemcpy(output, dout, desc.byte_sizes.output, hipMemcpyDeviceToHost) != hipSuccess) return ELX_GENERAL_ERROR;
-  } else if (desc.eager_mode || desc.stream_sync) {
+  } else if (desc.stream_sync) {
+    // Device tensors: the layer is ordered on the NULL stream like every later kernel or copy that touches
+    // them, so eager mode needs no host wait (a chain of layers stays asynchronous).  stream_sync asks for
+    // the wait, as it does for the reference's stream (src/elx_conv.cpp:233-236).
     if (hipStreamSynchronize(nullptr) != hipSuccess) return ELX_GENERAL_ERROR;
   }
   return ELX_OK;
 }
 
 // ---- reorders (host memory) --------------------------------------------------------------------
-#define IDX4(a, A, b, B, c, C, d, D) ((((size_t)(a) * (B) + (b)) * (C) + (c)) * (D) + (d))
+// The reference spreads every reorder over its thread pool (src/elx_reorder.cpp:35-93, estl::parallel_for
+// over the outer dimensions).  Here the outermost loop of each reorder is cut into contiguous ranges, one
+// per host thread; OMP_NUM_THREADS caps the thread count as it does the reference's, and a tensor of a few
+// thousand elements stays on the calling thread.
+namespace {
+int reorder_threads(size_t rows, size_t elements)
+{
+  size_t t = std::thread::hardware_concurrency();
+  if (const char *e = getenv("OMP_NUM_THREADS")) {
+    const long v = strtol(e, nullptr, 10);
+    if (v > 0) t = (size_t)v;
+  }
+  t = std::min(t, rows);
+  t = std::min(t, elements / 32768 + 1);
+  return (int)std::max<size_t>(t, 1);
+}
+
+// fn(first_row, last_row) over [0, rows), ranges of nearly equal length on separate threads
+template <typename F> void parallel_rows(size_t rows, size_t elements, F fn)
+{
+  const int nt = reorder_threads(rows, elements);
+  if (nt <= 1) {
+    fn((size_t)0, rows);
+    return;
+  }
+  std::vector<std::thread> pool;
+  pool.reserve(nt - 1);
+  for (int t = 1; t < nt; ++t) pool.emplace_back(fn, rows * t / nt, rows * (t + 1) / nt);
+  fn((size_t)0, rows / nt);
+  for (auto &th : pool) th.join();
+}
+}  // namespace
 
 template <typename Type> reorder<Type, nchw, nhwc>::reorder(Type *dst, Type *src, int n, int c, int h, int w)
 {
-  for (int _n = 0; _n < n; ++_n)
-    for (int _c = 0; _c < c; ++_c)
-      for (int _h = 0; _h < h; ++_h)
-        for (int _w = 0; _w < w; ++_w)
-          dst[IDX4(_n, n, _c, c, _h, h, _w, w)] = src[IDX4(_n, n, _h, h, _w, w, _c, c)];
+  const size_t hw = (size_t)h * w;
+  parallel_rows((size_t)n * c, (size_t)n * c * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _n = r / c, _c = r % c;
+      Type *d = dst + r * hw;
+      const Type *s = src + _n * hw * c + _c;
+      for (size_t p = 0; p < hw; ++p) d[p] = s[p * c];
+    }
+  });
 }
 
 template <typename Type> reorder<Type, nhwc, nchw>::reorder(Type *dst, Type *src, int n, int c, int h, int w)
 {
-  for (int _n = 0; _n < n; ++_n)
-    for (int _h = 0; _h < h; ++_h)
-      for (int _w = 0; _w < w; ++_w)
-        for (int _c = 0; _c < c; ++_c)
-          dst[IDX4(_n, n, _h, h, _w, w, _c, c)] = src[IDX4(_n, n, _c, c, _h, h, _w, w)];
+  const size_t hw = (size_t)h * w;
+  parallel_rows((size_t)n * h, (size_t)n * c * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _n = r / h, _h = r % h;
+      for (int _w = 0; _w < w; ++_w) {
+        Type *d = dst + (r * w + _w) * c;
+        const Type *s = src + _n * c * hw + _h * w + _w;
+        for (int _c = 0; _c < c; ++_c) d[_c] = s[_c * hw];
+      }
+    }
+  });
 }
 
 template <typename Type> reorder<Type, nchw, nChw16c>::reorder(Type *dst, Type *src, int n, int c, int h, int w)
 {
-  const int C2 = (c + 15) / 16;
-  for (int _n = 0; _n < n; ++_n)
-    for (int ch = 0; ch < c; ++ch)
-      for (int _h = 0; _h < h; ++_h)
-        for (int _w = 0; _w < w; ++_w)
-          dst[IDX4(_n, n, ch, c, _h, h, _w, w)] = src[IDX4(_n * C2 + ch / 16, 0, _h, h, _w, w, ch % 16, 16)];
+  const size_t hw = (size_t)h * w, C2 = ((size_t)c + 15) / 16;
+  parallel_rows((size_t)n * c, (size_t)n * c * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _n = r / c, ch = r % c;
+      Type *d = dst + r * hw;
+      const Type *s = src + (_n * C2 + ch / 16) * hw * 16 + ch % 16;
+      for (size_t p = 0; p < hw; ++p) d[p] = s[p * 16];
+    }
+  });
 }
 
 template <typename Type> reorder<Type, nChw16c, nchw>::reorder(Type *dst, Type *src, int n, int c, int h, int w)
 {
-  const int C2 = (c + 15) / 16;
-  for (int _n = 0; _n < n; ++_n)
-    for (int c2 = 0; c2 < C2; ++c2)
-      for (int _h = 0; _h < h; ++_h)
-        for (int _w = 0; _w < w; ++_w)
-          for (int v = 0; v < 16; ++v) {
-            const int ch = c2 * 16 + v;
-            dst[IDX4(_n * C2 + c2, 0, _h, h, _w, w, v, 16)] = ch < c ? src[IDX4(_n, n, ch, c, _h, h, _w, w)] : (Type)0;
-          }
+  const size_t hw = (size_t)h * w, C2 = ((size_t)c + 15) / 16;
+  parallel_rows((size_t)n * C2, (size_t)n * C2 * 16 * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _n = r / C2, c2 = r % C2;
+      const int real = (int)std::min<size_t>(16, c - c2 * 16);   // the last unit's tail is zero-filled
+      Type *d = dst + r * hw * 16;
+      const Type *s = src + (_n * c + c2 * 16) * hw;
+      for (size_t p = 0; p < hw; ++p)
+        for (int v = 0; v < 16; ++v) d[p * 16 + v] = v < real ? s[v * hw + p] : (Type)0;
+    }
+  });
 }
 
 namespace {
 template <typename Type> void plain_to_blocked_weights(Type *dst, Type *src, int g, int o, int i, int h, int w)
 {
-  const int O2 = (o + 15) / 16, I2 = (i + 15) / 16;
-  for (int _g = 0; _g < g; ++_g)
-    for (int o2 = 0; o2 < O2; ++o2)
-      for (int i2 = 0; i2 < I2; ++i2)
-        for (int _h = 0; _h < h; ++_h)
-          for (int _w = 0; _w < w; ++_w)
-            for (int iv = 0; iv < 16; ++iv)
-              for (int ov = 0; ov < 16; ++ov) {
-                const int oc = o2 * 16 + ov, ic = i2 * 16 + iv;
-                dst[((((((size_t)_g * O2 + o2) * I2 + i2) * h + _h) * w + _w) * 16 + iv) * 16 + ov] =
-                    (oc < o && ic < i) ? src[((((size_t)_g * o + oc) * i + ic) * h + _h) * w + _w] : (Type)0;
-              }
+  const size_t O2 = ((size_t)o + 15) / 16, I2 = ((size_t)i + 15) / 16, hw = (size_t)h * w;
+  parallel_rows((size_t)g * O2 * I2, (size_t)g * O2 * I2 * hw * 256, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _g = r / (O2 * I2), o2 = r / I2 % O2, i2 = r % I2;
+      for (size_t p = 0; p < hw; ++p)
+        for (int iv = 0; iv < 16; ++iv)
+          for (int ov = 0; ov < 16; ++ov) {
+            const size_t oc = o2 * 16 + ov, ic = i2 * 16 + iv;
+            dst[((r * hw + p) * 16 + iv) * 16 + ov] =
+                (oc < (size_t)o && ic < (size_t)i) ? src[((_g * o + oc) * i + ic) * hw + p] : (Type)0;
+          }
+    }
+  });
 }
 template <typename Type> void blocked_to_plain_weights(Type *dst, Type *src, int g, int o, int i, int h, int w)
 {
-  const int O2 = (o + 15) / 16, I2 = (i + 15) / 16;
-  for (int _g = 0; _g < g; ++_g)
-    for (int oc = 0; oc < o; ++oc)
-      for (int ic = 0; ic < i; ++ic)
-        for (int _h = 0; _h < h; ++_h)
-          for (int _w = 0; _w < w; ++_w)
-            dst[((((size_t)_g * o + oc) * i + ic) * h + _h) * w + _w] =
-                src[((((((size_t)_g * O2 + oc / 16) * I2 + ic / 16) * h + _h) * w + _w) * 16 + ic % 16) * 16 + oc % 16];
+  const size_t O2 = ((size_t)o + 15) / 16, I2 = ((size_t)i + 15) / 16, hw = (size_t)h * w;
+  parallel_rows((size_t)g * o, (size_t)g * o * i * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _g = r / o, oc = r % o;
+      for (size_t ic = 0; ic < (size_t)i; ++ic)
+        for (size_t p = 0; p < hw; ++p)
+          dst[(r * i + ic) * hw + p] =
+              src[((((_g * O2 + oc / 16) * I2 + ic / 16) * hw + p) * 16 + ic % 16) * 16 + oc % 16];
+    }
+  });
 }
 template <typename Type> void hwio_to_oihw(Type *dst, Type *src, int g, int o, int i, int h, int w)
 {
-  for (int _g = 0; _g < g; ++_g)
-    for (int oc = 0; oc < o; ++oc)
-      for (int ic = 0; ic < i; ++ic)
-        for (int _h = 0; _h < h; ++_h)
-          for (int _w = 0; _w < w; ++_w)
-            dst[((((size_t)_g * o + oc) * i + ic) * h + _h) * w + _w] =
-                src[((((size_t)_g * h + _h) * w + _w) * i + ic) * o + oc];
+  const size_t hw = (size_t)h * w;
+  parallel_rows((size_t)g * o, (size_t)g * o * i * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _g = r / o, oc = r % o;
+      for (size_t ic = 0; ic < (size_t)i; ++ic)
+        for (size_t p = 0; p < hw; ++p) dst[(r * i + ic) * hw + p] = src[((_g * hw + p) * i + ic) * o + oc];
+    }
+  });
 }
 template <typename Type> void oihw_to_hwio(Type *dst, Type *src, int g, int o, int i, int h, int w)
 {
-  for (int _g = 0; _g < g; ++_g)
-    for (int _h = 0; _h < h; ++_h)
-      for (int _w = 0; _w < w; ++_w)
-        for (int ic = 0; ic < i; ++ic)
-          for (int oc = 0; oc < o; ++oc)
-            dst[((((size_t)_g * h + _h) * w + _w) * i + ic) * o + oc] =
-                src[((((size_t)_g * o + oc) * i + ic) * h + _h) * w + _w];
+  const size_t hw = (size_t)h * w;
+  parallel_rows((size_t)g * hw, (size_t)g * o * i * hw, [=](size_t r0, size_t r1) {
+    for (size_t r = r0; r < r1; ++r) {
+      const size_t _g = r / hw, p = r % hw;
+      for (size_t ic = 0; ic < (size_t)i; ++ic)
+        for (size_t oc = 0; oc < (size_t)o; ++oc) dst[(r * i + ic) * o + oc] = src[((_g * o + oc) * i + ic) * hw + p];
+    }
+  });
 }
 }  // namespace
 

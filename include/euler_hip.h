@@ -169,13 +169,6 @@ EHIP_API int ehip_reorder_blocked_to_nchw(void *dst_dev, const void *src_dev, in
 EHIP_API int ehip_reorder_oihw_to_blocked(void *dst_dev, const void *src_dev, int o, int i, int h,
                                           int w, void *hip_stream);
 
-/* No counterpart in the reference: a measuring stick for the benchmark.  Launches `workgroups` x 4 waves
- * that each retire 8 x iters v_mfma_i32_32x32x32_i8 from registers (no memory traffic in the loop)
- * and writes one int per thread (workgroups x 256) to out_dev; *ops_out = the integer operations
- * issued.  The caller times it; the result is what the instruction reaches on this chip, to set
- * beside the published int8 peak the rooflines are quoted against. */
-EHIP_API int ehip_probe_mfma_i8(int workgroups, int iters, void *out_dev, double *ops_out, void *hip_stream);
-
 #ifdef __cplusplus
 }
 #endif
