@@ -361,7 +361,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "%s: %s" % (wl.key, wl.title), "ops_per_step": wl.ops(),
                    "algorithmic_bytes_per_step": wl.algorithmic_bytes(), "kernel": layer.conv.kernel_name,
-                   "untimed_preheat_ms": PREHEAT_S * 1e3},
+                   "untimed_preheat_ms": PREHEAT_S * 1e3, "seed": W.seed_of(wl.key), "calibration": layer.calibration},
         "images_per_s": round(wl.n / wall, 1),
         "single_launch_latency_us": round(lat * 1e6, 2),
         "event_ms_per_step": round(ev * 1e3, 6),

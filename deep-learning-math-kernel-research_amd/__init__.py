@@ -76,6 +76,8 @@ def _load():
     lib.ehip_quantize_input_u8.argtypes = [vp, vp, sz, fl, fl, vp]
     lib.ehip_wino_tinput_range.argtypes = [ctypes.POINTER(ConvDesc), vp, ctypes.POINTER(fl), ctypes.POINTER(fl)]
     lib.ehip_wino_tinput_range_noalloc.argtypes = [ctypes.POINTER(ConvDesc), vp, vp, vp]
+    lib.ehip_ref_conv_f32_range.argtypes = [ctypes.POINTER(ConvDesc), vp, vp, vp, vp, ctypes.POINTER(fl), ctypes.POINTER(fl)]
+    lib.ehip_calibrate_output_quant.argtypes = [ctypes.POINTER(ConvDesc), fl, fl, fl, fl] + [ctypes.POINTER(fl)] * 3
     lib.ehip_reorder_nchw_to_blocked.argtypes = [vp, vp, ci, ci, ci, ci, ci, vp]
     lib.ehip_reorder_blocked_to_nchw.argtypes = [vp, vp, ci, ci, ci, ci, ci, vp]
     lib.ehip_reorder_oihw_to_blocked.argtypes = [vp, vp, ci, ci, ci, ci, vp]
@@ -88,7 +90,7 @@ EXPORTED_SYMBOLS = (
     "ehip_init", "ehip_last_error", "ehip_conv_create", "ehip_conv_destroy", "ehip_conv_prepare",
     "ehip_conv_execute", "ehip_conv_execute_repeat", "ehip_conv_query", "ehip_conv_kernel_name", "ehip_quantize_input_u8",
     "ehip_wino_tinput_range", "ehip_wino_tinput_range_noalloc", "ehip_reorder_nchw_to_blocked", "ehip_reorder_blocked_to_nchw",
-    "ehip_reorder_oihw_to_blocked",
+    "ehip_reorder_oihw_to_blocked", "ehip_ref_conv_f32_range", "ehip_calibrate_output_quant",
 )
 
 
@@ -195,6 +197,23 @@ def wino_tinput_range(desc, input):
 def wino_tinput_range_noalloc(desc, input, minmax_out, stream=0):
     """min / max into two floats of device memory (minmax_out), asynchronous, no device allocation"""
     _check(lib.ehip_wino_tinput_range_noalloc(ctypes.byref(desc), _ptr(input), _ptr(minmax_out), ctypes.c_void_p(stream)))
+
+
+def ref_conv_f32_range(desc, input_f32, weights, bias, output_f32=None):
+    """The harness's fp32 reference convolution on the device: (min, max) of its result; output_f32 (optional,
+    required with with_ip_sum: it holds the sum operand) receives the result itself."""
+    mn, mx = ctypes.c_float(), ctypes.c_float()
+    _check(lib.ehip_ref_conv_f32_range(ctypes.byref(desc), _ptr(output_f32), _ptr(input_f32), _ptr(weights), _ptr(bias),
+                                       ctypes.byref(mn), ctypes.byref(mx)))
+    return mn.value, mx.value
+
+
+def calibrate_output_quant(desc, out_min, out_max, sum_absmax=0.0, representation=127.0):
+    """(output scale, output z, sum scale) from the range of the fp32 reference output, by the harness's rule"""
+    s, z, ss = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
+    _check(lib.ehip_calibrate_output_quant(ctypes.byref(desc), out_min, out_max, sum_absmax, representation,
+                                           ctypes.byref(s), ctypes.byref(z), ctypes.byref(ss)))
+    return s.value, z.value, ss.value
 
 
 def reorder_nchw_to_blocked(dst, src, elem_size, n, c, h, w, stream=0):

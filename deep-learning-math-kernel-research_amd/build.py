@@ -21,6 +21,7 @@ SOURCES = [
     "ehip_depthwise.hip",
     "ehip_wino.hip",
     "ehip_prepare.hip",
+    "ehip_harness.hip",
     "ehip_api.hip",
     "euler_api.hip",
 ]

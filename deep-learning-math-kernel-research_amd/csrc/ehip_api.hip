@@ -898,3 +898,78 @@ EHIP_API int ehip_reorder_oihw_to_blocked(void *dst_dev, const void *src_dev, in
 }
 
 }  // extern "C"
+
+// ---- harness calibration (tests/elt_conv_utils.cpp:290-352) ------------------------------------
+EHIP_API int ehip_ref_conv_f32_range(const ehip_conv_desc_t *desc, void *output_f32_dev, const void *input_f32_dev,
+                                     const void *weights_dev, const void *bias_dev, float *min_out, float *max_out)
+{
+  if (!desc || !input_f32_dev || !weights_dev || !min_out || !max_out) return fail(EHIP_GENERAL_ERROR, "null argument");
+  const ehip_conv_desc_t &d = *desc;
+  if (d.with_bias && !bias_dev) return fail(EHIP_GENERAL_ERROR, "null argument");
+  if (d.with_ip_sum && !output_f32_dev)
+    return fail(EHIP_GENERAL_ERROR, "reference convolution: with_ip_sum needs the output buffer (it holds the sum operand)");
+  if (d.n < 1 || d.g < 1 || d.ic < 1 || d.oc < 1 || d.ic % d.g || d.oc % d.g || d.oh < 1 || d.ow < 1 || d.kh < 1 || d.kw < 1)
+    return fail(EHIP_GENERAL_ERROR, "reference convolution: bad dims");
+  if (d.dilation_h != 1 || d.dilation_w != 1) return fail(EHIP_UNIMPLEMENTED, "reference convolution: dilation");
+  const bool in_ok = d.input_fmt == EHIP_NCHW16C || d.input_fmt == EHIP_NHWC;
+  const bool out_ok = d.output_fmt == EHIP_NCHW16C || d.output_fmt == EHIP_NHWC;
+  const bool w_ok = (d.weights_fmt == EHIP_OIHW16I16O && d.g == 1) || d.weights_fmt == EHIP_GOIHW || d.weights_fmt == EHIP_OIHW;
+  if (!in_ok || !out_ok || !w_ok)
+    return fail(EHIP_UNIMPLEMENTED, "reference convolution: activations nChw16c or nhwc; weights OIhw16i16o (g = 1), oihw or goihw");
+  RefConvArgs a = {};
+  a.in = static_cast<const float *>(input_f32_dev);
+  a.w = static_cast<const float *>(weights_dev);
+  a.bias = static_cast<const float *>(bias_dev);
+  a.out = static_cast<float *>(output_f32_dev);
+  a.n = d.n; a.g = d.g; a.ic = d.ic; a.oc = d.oc; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
+  a.kh = d.kh; a.kw = d.kw; a.pad_t = d.pad_t; a.pad_l = d.pad_l; a.sh = d.stride_h; a.sw = d.stride_w;
+  a.in_nhwc = d.input_fmt == EHIP_NHWC;
+  a.out_nhwc = d.output_fmt == EHIP_NHWC;
+  a.w_goihw = d.weights_fmt != EHIP_OIHW16I16O;
+  a.with_relu = d.with_relu; a.with_sum = d.with_ip_sum; a.with_bias = d.with_bias;
+  a.ic2 = up(d.ic, 16) / 16;
+  a.oc2 = up(d.oc, 16) / 16;
+  const long long blocks = (long long)d.n * a.oc2 * (((long long)d.oh * d.ow + 15) / 16);
+  if (blocks >= (1ll << 31)) return fail(EHIP_UNIMPLEMENTED, "reference convolution: too many outputs");
+  HIP_TRY(hipMalloc(reinterpret_cast<void **>(&a.partials), 2 * (size_t)blocks * sizeof(float)));
+  hipError_t e = launch_ref_conv_f32(a, (unsigned)blocks);
+  std::vector<float> part(2 * (size_t)blocks);
+  if (e == hipSuccess) e = hipMemcpy(part.data(), a.partials, part.size() * sizeof(float), hipMemcpyDeviceToHost);
+  (void)hipFree(a.partials);
+  HIP_TRY(e);
+  float lo = part[0], hi = part[1];
+  for (size_t b = 1; b < (size_t)blocks; ++b) {
+    lo = std::min(lo, part[2 * b]);
+    hi = std::max(hi, part[2 * b + 1]);
+  }
+  *min_out = lo;
+  *max_out = hi;
+  return EHIP_OK;
+}
+
+EHIP_API int ehip_calibrate_output_quant(const ehip_conv_desc_t *desc, float out_min, float out_max, float sum_absmax,
+                                         float representation, float *output_scale, float *output_z, float *sum_scale)
+{
+  if (!desc || !output_scale || !output_z) return fail(EHIP_GENERAL_ERROR, "null argument");
+  if (!(representation > 0.0f)) return fail(EHIP_GENERAL_ERROR, "calibration: representation must be positive");
+  const float abs_min = out_min > 0 ? out_min : -out_min;
+  const float abs_max = out_max > abs_min ? out_max : abs_min;
+  if (desc->with_relu || desc->output_type == EHIP_S8) {
+    // ReLU output, or a signed code: symmetric scale, zero point 0 (tests/elt_conv_utils.cpp:313-323)
+    *output_scale = abs_max / representation;
+    *output_z = 0.0f;
+  } else {
+    // the full range mapped onto the code range (tests/elt_conv_utils.cpp:324-328; the harness adds its
+    // 0.000001 as a double, so the two quotients are formed in double and then narrowed)
+    const double diff = (double)(out_max - out_min) + 0.000001;
+    *output_scale = (float)(diff / representation);
+    *output_z = (float)((double)(-out_min * representation) / diff);
+  }
+  if (desc->with_ip_sum) {
+    if (!sum_scale) return fail(EHIP_GENERAL_ERROR, "null argument");
+    // the sum operand's own scale over the output scale (tests/elt_conv_utils.cpp:333-345)
+    const float sum_operand_scale = sum_absmax / representation;
+    *sum_scale = sum_operand_scale / *output_scale;
+  }
+  return EHIP_OK;
+}

@@ -644,5 +644,17 @@ __device__ __forceinline__ void lean_store(int mode, const Epilogue &ep, const v
   }
 }
 
+// the harness's fp32 reference convolution (calibration), ehip_harness.hip
+struct RefConvArgs {
+  const float *in, *w, *bias;
+  float *out;        // nullable unless with_sum
+  float *partials;   // [blocks][2]
+  int n, g, ic, oc, ih, iw, oh, ow, kh, kw, pad_t, pad_l, sh, sw;
+  int in_nhwc, out_nhwc, w_goihw, with_relu, with_sum, with_bias;
+  int ic2, oc2;
+};
+
+hipError_t launch_ref_conv_f32(const RefConvArgs &a, unsigned blocks);
+
 }  // namespace ehip
 #endif

@@ -9,7 +9,7 @@ algorithmic.
 """
 import math
 
-from . import (CONV_DIRECT, CONV_DIRECT_1X1, CONV_WINOGRAD, EL_NO_CALI, F32, FLT_MAX, NHWC, S8, U8, Conv,
+from . import (CONV_DIRECT, CONV_DIRECT_1X1, CONV_WINOGRAD, EL_NO_CALI, F32, FLT_MAX, NCHW16C, NHWC, S8, U8, Conv,
                make_desc, up16, wino_tinput_range)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
@@ -68,11 +68,16 @@ class Workload:
         t_hbm = self.algorithmic_bytes() / (PEAK_HBM_GBS * 1e9)
         return ("mfma", t_mfma) if t_mfma >= t_hbm else ("hbm", t_hbm)
 
-    def descriptor(self, out_scale=None, tinput_quant=(EL_NO_CALI, EL_NO_CALI)):
+    def descriptor(self, out_quant=None, sum_scale=None, tinput_quant=(EL_NO_CALI, EL_NO_CALI)):
+        """out_quant = (scale, z) and sum_scale as calibrated (DeviceLayer); left out, an analytic estimate
+        stands in: four sigmas of the pre-activation over the code range, and 0.7 for the sum operand."""
         fan = self.k * self.k * (1 if self.depthwise else self.ic)
-        if out_scale is None:
-            # u8 in [0,255]/255 ~ U[0,1): E[x^2] = 1/3; four sigmas of the pre-activation over the code range
-            out_scale = 4.0 * self.w_sigma * math.sqrt(fan / 3.0) / (127.0 if self.out_type == S8 else 255.0)
+        if out_quant is None:
+            # u8 in [0,255]/255 ~ U[0,1): E[x^2] = 1/3
+            out_quant = (4.0 * self.w_sigma * math.sqrt(fan / 3.0) / (127.0 if self.out_type == S8 else 255.0), 0.0)
+        out_scale, out_z = out_quant
+        if sum_scale is None:
+            sum_scale = 0.7
         relu = (0.0, FLT_MAX)
         if self.relu6:
             out_scale = 6.0 / 255.0
@@ -84,7 +89,7 @@ class Workload:
                       algorithm=self.algorithm, input_type=self.in_type, output_type=self.out_type,
                       with_bias=True, with_relu=True, with_ip_sum=self.with_sum,
                       input_quant=(1.0, 0.0) if self.in_type == F32 else (1.0 / 255.0, self.in_z),
-                      output_quant=(out_scale, 0.0), sum_quant=(0.7, 0.0) if self.with_sum else (0.0, 0.0),
+                      output_quant=(out_scale, out_z), sum_quant=(sum_scale, 0.0) if self.with_sum else (0.0, 0.0),
                       wino_tinput_quant=tinput_quant, relu_bound=relu, flatting_t=self.T,
                       tile_size=self.tile if self.algorithm == CONV_WINOGRAD else 0,
                       execution_mode=0xa161 if self.algorithm == CONV_WINOGRAD else 0)
@@ -219,44 +224,172 @@ NETWORKS = {
 }
 
 
+# ---- synthetic tensors: a self-contained generator, so that a seed gives the same bytes on every host -------
+_GAMMA = 0x9E3779B97F4A7C15
+
+
+def splitmix64(seed, count, offset=0):
+    """outputs offset .. offset+count-1 of the splitmix64 sequence started at `seed` (uint64 array).  The
+    state of step k is seed + (k + 1) * GAMMA, so the sequence is evaluated as a vector."""
+    import numpy as np
+    with np.errstate(over="ignore"):
+        z = np.arange(offset + 1, offset + count + 1, dtype=np.uint64)
+        z *= np.uint64(_GAMMA)
+        z += np.uint64(seed)
+        z ^= z >> np.uint64(30)
+        z *= np.uint64(0xBF58476D1CE4E5B9)
+        z ^= z >> np.uint64(27)
+        z *= np.uint64(0x94D049BB133111EB)
+        z ^= z >> np.uint64(31)
+        return z
+
+
+_last_uniform = {}
+
+
+def uniform01(seed, count, offset=0):
+    """U[0,1) as float32: the top 24 bits of each splitmix64 output over 2^24 (exact in float32); evaluated
+    in blocks that stay in the host's cache.  The last array is kept: variants of one layer share its tensors."""
+    import numpy as np
+    if (seed, count, offset) in _last_uniform:
+        return _last_uniform[(seed, count, offset)]
+    out = np.empty(count, np.float32)
+    step = 1 << 18
+    for lo in range(0, count, step):
+        m = min(step, count - lo)
+        out[lo:lo + m] = splitmix64(seed, m, offset + lo) >> np.uint64(40)
+    out *= np.float32(2.0 ** -24)
+    _last_uniform.clear()
+    _last_uniform[(seed, count, offset)] = out
+    return out
+
+
+def normal(seed, count, sigma):
+    """N(0, sigma) as float32 by Box-Muller on pairs of the uniform stream (both branches used)"""
+    import numpy as np
+    half = (count + 1) // 2
+    out = np.empty(2 * half, np.float32)
+    step = 1 << 17
+    for lo in range(0, half, step):
+        m = min(step, half - lo)
+        u = (splitmix64(seed, 2 * m, 2 * lo) >> np.uint64(11)).astype(np.float64) * 2.0 ** -53
+        r = np.sqrt(-2.0 * np.log1p(-u[0::2])) * sigma          # 1 - u is in (0, 1]
+        t = 2.0 * np.pi * u[1::2]
+        out[2 * lo:2 * (lo + m):2] = r * np.cos(t)
+        out[2 * lo + 1:2 * (lo + m):2] = r * np.sin(t)
+    return out[:count]
+
+
+# frozen seeds of the configured layers; every tensor of a layer takes its own stream (seed + 2^32 * index)
+SEEDS = {"C1": 1001, "C2": 1002, "C3a": 1003, "C3b": 1004, "C4a": 1005, "C4b": 1006, "C5a": 1007, "C5b": 1008}
+
+
+def seed_of(key):
+    base = key.split("@")[0].split("_")[0]   # C3a_nhwc, C4b_i8_t4, C2@N=512 share their layer's tensors
+    if base in SEEDS:
+        return SEEDS[base]
+    return 2000 + sum((i + 1) * ord(ch) for i, ch in enumerate(key)) % 100000
+
+
 class DeviceLayer:
     """Synthetic device-resident tensors of one workload (torch owns the memory) and its prepared
-    convolution handle."""
+    convolution handle, set up the way the reference's harness sets up a layer (tests/elt_conv_utils.cpp:
+    87-463): fp32 tensors are drawn (here: seeded, U[0,1) activations, N(0, sigma) weights, N(0, 0.01)
+    bias, N(0, 1) sum operand), the quantization scales are calibrated from them -- output_quant and
+    sum_quant from the fp32 reference convolution (ehip_ref_conv_f32_range + ehip_calibrate_output_quant),
+    wino_tinput_quant from the transformed-input range (ehip_wino_tinput_range) -- and the input and the sum
+    operand are quantized with the harness's helper (ehip_quantize_input_u8).  Differences from the harness:
+    the input scale is the fixed 1/255 of a U[0,1) image, u8 tensors are calibrated onto 255 codes rather
+    than the harness's 127, and a ReLU6 layer keeps its 6/255 output scale."""
 
-    def __init__(self, wl, seed=1234):
+    def __init__(self, wl, seed=None, calibrate=True):
+        import numpy as np
         import torch
+        from . import (quantize_input_u8, ref_conv_f32_range, calibrate_output_quant, reorder_nchw_to_blocked,
+                       reorder_oihw_to_blocked)
         self.wl = wl
-        gen = torch.Generator(device="cuda")
-        gen.manual_seed(seed)
+        seed = seed_of(wl.key) if seed is None else seed
         ic2, oc2 = up16(wl.ic) // 16, up16(wl.oc) // 16
-        if wl.in_type == U8:
-            # fp32 U[0,1) activations quantized with scale 1/255 are uniform codes 0..255
-            # (random codes: the nhwc tensor has the same number of bytes, only their meaning differs;
-            # nhwc with at most four channels is compact, [n][h][w][ic])
-            shape = (wl.n, wl.hw, wl.hw, wl.ic) if wl.nhwc_in and wl.ic <= 4 else (wl.n, ic2, wl.hw, wl.hw, 16)
-            self.x = torch.randint(0, 256, shape, dtype=torch.uint8, device="cuda", generator=gen)
-        else:
-            self.x = torch.rand((wl.n, ic2, wl.hw, wl.hw, 16), dtype=torch.float32, device="cuda", generator=gen)
+        few = wl.nhwc_in and wl.ic <= 4    # a first layer's compact image [n][h][w][ic]
+
+        def stream(index):
+            return seed + (index << 32)
+
+        def blocked(t_nchw, c):            # nchw -> nChw16c on the device
+            n, _, h, w = t_nchw.shape
+            out = torch.empty((n, up16(c) // 16, h, w, 16), dtype=t_nchw.dtype, device="cuda")
+            reorder_nchw_to_blocked(out, t_nchw, t_nchw.element_size(), n, c, h, w)
+            return out
+
+        def nhwc(t_blocked, c):            # nChw16c -> [n][h][w][c]
+            n, c2, h, w, _ = t_blocked.shape
+            return t_blocked.permute(0, 2, 3, 1, 4).reshape(n, h, w, c2 * 16)[..., :c].contiguous()
+
+        # fp32 tensors; a zero point moves the image to U[0,1) - z / 255, so that its codes still cover 0..255
+        in_scale = 1.0 if wl.in_type == F32 else 1.0 / 255.0
+        x = torch.from_numpy(uniform01(stream(0), wl.n * wl.ic * wl.hw * wl.hw)).cuda().reshape(wl.n, wl.ic, wl.hw, wl.hw)
+        if wl.in_z:
+            x -= wl.in_z / 255.0
+        x_f32 = blocked(x, wl.ic)
+        kshape = (wl.ic, 1, wl.k, wl.k) if wl.depthwise else (wl.oc, wl.ic, wl.k, wl.k)
+        w = torch.from_numpy(normal(stream(1), int(np.prod(kshape)), wl.w_sigma)).cuda().reshape(kshape)
         if wl.depthwise:
-            self.w = torch.randn((wl.ic, 3, 3), dtype=torch.float32, device="cuda", generator=gen) * wl.w_sigma
+            self.w = w.reshape(wl.ic, wl.k, wl.k).contiguous()
         else:
-            self.w = torch.randn((oc2, ic2, wl.k, wl.k, 16, 16), dtype=torch.float32, device="cuda",
-                                 generator=gen) * wl.w_sigma
-        self.bias = torch.randn(oc2 * 16, dtype=torch.float32, device="cuda", generator=gen) * 0.01
-        tdt = {U8: torch.uint8, S8: torch.int8, F32: torch.float32}[wl.out_type]
-        shape = (wl.n, oc2, wl.oh, wl.oh, 16)
+            self.w = torch.empty((oc2, ic2, wl.k, wl.k, 16, 16), dtype=torch.float32, device="cuda")
+            reorder_oihw_to_blocked(self.w, w, wl.oc, wl.ic, wl.k, wl.k)
+        bias = np.zeros(oc2 * 16, np.float32)
+        bias[:wl.oc] = normal(stream(2), wl.oc, 0.01)
+        self.bias = torch.from_numpy(bias).cuda()
+        r_f32 = None
         if wl.with_sum:
-            self.out = torch.randint(-127, 128, shape, dtype=torch.int8, device="cuda", generator=gen).to(tdt)
+            r = torch.from_numpy(normal(stream(3), wl.n * wl.oc * wl.oh * wl.oh, 1.0)).cuda()
+            r_f32 = blocked(r.reshape(wl.n, wl.oc, wl.oh, wl.oh), wl.oc)
+        torch.cuda.synchronize()
+
+        # calibration
+        out_quant, sum_scale = None, 0.0
+        self.calibration = {}
+        if calibrate and wl.out_type != F32 and not wl.relu6:
+            d32 = wl.descriptor(out_quant=(1.0, 0.0))
+            d32.input_type, d32.input_fmt, d32.output_fmt = F32, NCHW16C, NCHW16C
+            scratch = r_f32.clone() if wl.with_sum else None
+            mn, mx = ref_conv_f32_range(d32, x_f32, self.w, self.bias, scratch)
+            sum_absmax = float(r_f32.abs().max()) if wl.with_sum else 0.0
+            rep = 127.0 if wl.out_type == S8 else 255.0
+            s_o, z_o, sum_scale = calibrate_output_quant(d32, mn, mx, sum_absmax, rep)
+            out_quant = (s_o, z_o)
+            self.calibration = {"ref_out_min": mn, "ref_out_max": mx, "output_scale": s_o, "output_z": z_o,
+                                "sum_scale": sum_scale if wl.with_sum else None}
+            del scratch
+
+        # user tensors
+        if wl.in_type == U8:
+            xq = torch.empty(x_f32.shape, dtype=torch.uint8, device="cuda")
+            quantize_input_u8(xq, x_f32, x_f32.numel(), in_scale, wl.in_z)
+            self.x = nhwc(xq, wl.ic) if wl.nhwc_in else xq
         else:
-            self.out = torch.zeros(shape, dtype=tdt, device="cuda")
+            self.x = nhwc(x_f32, wl.ic) if wl.nhwc_in else x_f32
+        tdt = {U8: torch.uint8, S8: torch.int8, F32: torch.float32}[wl.out_type]
+        oshape = (wl.n, wl.oh, wl.oh, wl.oc) if wl.nhwc_out else (wl.n, oc2, wl.oh, wl.oh, 16)
+        if wl.with_sum:
+            # the sum operand in the output's own type: its codes at scale max|r| / 127 (s8) or 255 (u8)
+            rq = torch.empty(r_f32.shape, dtype=torch.uint8, device="cuda")
+            rep = 127.0 if wl.out_type == S8 else 255.0
+            quantize_input_u8(rq, r_f32, r_f32.numel(), float(r_f32.abs().max()) / rep, 0.0)
+            rq = rq.view(tdt) if wl.out_type != F32 else r_f32
+            self.out = nhwc(rq, wl.oc) if wl.nhwc_out else rq
+        else:
+            self.out = torch.zeros(oshape, dtype=tdt, device="cuda")
+        del x, x_f32, w, r_f32
         tq = (EL_NO_CALI, EL_NO_CALI)
         if wl.algorithm == CONV_WINOGRAD:
             mn, mx = wino_tinput_range(wl.descriptor(tinput_quant=(1.0, 0.0)), self.x)
-            in_s = 1.0 / 255.0 if wl.in_type == U8 else 1.0   # u8 input: the range comes back in code units
-            mn, mx = mn * in_s, mx * in_s
+            mn, mx = mn * in_scale, mx * in_scale   # u8 input: the range comes back in code units
             diff = mx - mn + 1e-6
             tq = (diff / 255.0, -mn * 255.0 / diff)
-        self.desc = wl.descriptor(tinput_quant=tq)
+            self.calibration.update({"tinput_min": mn, "tinput_max": mx})
+        self.desc = wl.descriptor(out_quant=out_quant, sum_scale=sum_scale, tinput_quant=tq)
         self.conv = Conv(self.desc)
         self.conv.prepare(self.w, self.bias)
         torch.cuda.synchronize()

@@ -147,6 +147,27 @@ EHIP_API int ehip_quantize_input_u8(void *dst_dev, const void *src_dev, size_t c
 EHIP_API int ehip_wino_tinput_range(const ehip_conv_desc_t *desc, const void *input_dev,
                                     float *min_out, float *max_out);
 
+/* Replaces the harness's fp32 reference convolution where it serves calibration (ref_convolution2d,
+ * tests/elt_conv_utils.cpp:666-750, called from :300-304): every output starts from the bias (plus the old
+ * output with with_ip_sum), takes the products in the order (ic, kh, kw) with padded taps skipped, one
+ * fused multiply-add each, and is clamped at zero with with_relu.  All tensors fp32: input and output in
+ * the descriptor's activation formats (nChw16c or nhwc), weights OIhw16i16o (g = 1), oihw or goihw.
+ * output_f32_dev may be NULL when only the range is wanted (it must be given with with_ip_sum: it holds
+ * the sum operand on entry).  *min_out / *max_out: range of the result, over real channels only.
+ * Synchronous, allocates a temporary. */
+EHIP_API int ehip_ref_conv_f32_range(const ehip_conv_desc_t *desc, void *output_f32_dev, const void *input_f32_dev,
+                                     const void *weights_dev, const void *bias_dev, float *min_out, float *max_out);
+
+/* Replaces the harness's rule for output_quant and sum_quant (tests/elt_conv_utils.cpp:306-346), host
+ * arithmetic only.  out_min / out_max: range of the fp32 reference output; sum_absmax: largest magnitude
+ * of the fp32 sum operand (read only with with_ip_sum).  With ReLU or an s8 output:
+ * scale = max(|min|, |max|) / representation, z = 0; otherwise scale = (max - min + 1e-6) / representation,
+ * z = -min * representation / (max - min + 1e-6).  sum_scale = (sum_absmax / representation) / scale.
+ * `representation` is the code range the scales map onto: the harness uses 127 for every type
+ * (PRECISION_REPRESENTATION_7B); 255 uses the whole range of a u8 tensor. */
+EHIP_API int ehip_calibrate_output_quant(const ehip_conv_desc_t *desc, float out_min, float out_max, float sum_absmax,
+                                         float representation, float *output_scale, float *output_z, float *sum_scale);
+
 /* No counterpart in the reference.  ehip_wino_tinput_range for callers that cannot allocate device
  * memory (a stream under HIP graph capture, a serving loop or a harness that forbids hipMalloc): the
  * per-unit partial minima / maxima go to a static device array of the library (32 KB on every GPU the

@@ -489,6 +489,61 @@ void orc_quantize_input_u8(uint8_t *dst, const float *src, size_t count, float s
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// harness fp32 reference convolution -- tests/elt_conv_utils.cpp:666-750.  The accumulation
+// `out[...] += in[...] * w[...]` is one vfmadd in the compiled harness (g++ -O2 contracts it).
+// ---------------------------------------------------------------------------------------
+int orc_ref_conv_f32(const orc_conv_params *p, float *output, const float *input, const float *weights, const float *bias)
+{
+  if (p->g < 1 || p->ic % p->g || p->oc % p->g) return -1;
+  const int icg = p->ic / p->g, ocg = p->oc / p->g;
+#pragma omp parallel for collapse(2)
+  for (int n = 0; n < p->n; ++n)
+    for (int oc = 0; oc < p->oc; ++oc) {
+      const int grp = oc / ocg;
+      for (int oh = 0; oh < p->oh; ++oh)
+        for (int ow = 0; ow < p->ow; ++ow) {
+          float *o = &output[(((size_t)n * p->oc + oc) * p->oh + oh) * p->ow + ow];
+          const float b = p->with_bias ? bias[oc] : 0.0f;
+          float acc = p->with_sum ? *o + b : b;
+          for (int i = 0; i < icg; ++i)
+            for (int kh = 0; kh < p->kh; ++kh) {
+              const int ih = oh * p->stride_h - p->pad_t + kh;
+              if (ih < 0 || ih >= p->ih) continue;
+              for (int kw = 0; kw < p->kw; ++kw) {
+                const int iw = ow * p->stride_w - p->pad_l + kw;
+                if (iw < 0 || iw >= p->iw) continue;
+                acc = fmaf(input[(((size_t)n * p->ic + grp * icg + i) * p->ih + ih) * p->iw + iw],
+                           weights[(((size_t)oc * icg + i) * p->kh + kh) * p->kw + kw], acc);
+              }
+            }
+          *o = (p->with_relu && acc < 0.0f) ? 0.0f : acc;
+        }
+    }
+  return 0;
+}
+
+// tests/elt_conv_utils.cpp:306-346; `diff` is a double there (the 0.000001 literal promotes it), so the
+// asymmetric scale and zero point are double quotients narrowed on assignment
+void orc_calibrate_output_quant(int with_relu, int out_type, int with_sum, float out_min, float out_max, float sum_absmax,
+                                float representation, float *output_scale, float *output_z, float *sum_scale)
+{
+  const float abs_cur = out_min > 0 ? out_min : -out_min;
+  const float abs_max = out_max > abs_cur ? out_max : abs_cur;
+  if (with_relu || out_type == ORC_S8) {
+    *output_scale = abs_max / representation;
+    *output_z = 0.0f;
+  } else {
+    const double diff = (double)(out_max - out_min) + 0.000001;
+    *output_scale = (float)(diff / representation);
+    *output_z = (float)((double)(-out_min * representation) / diff);
+  }
+  if (with_sum) {
+    const float sum_operand_scale = sum_absmax / representation;
+    *sum_scale = sum_operand_scale / *output_scale;
+  }
+}
+
 int orc_epilogue(int out_kind, int32_t acc, float scale, float shift, int with_sum, int old_q,
                  float sum_scale, int with_relu, float lo, float hi, float *fout)
 {

@@ -31,6 +31,8 @@
  *     objects hold (vfmadd bias*repS+z, vfnmadd of the zero-point term, unfused sum_z*sum_S), on data
  *     checked to tell that pattern from its neighbours.
  *   - reorders: closed-form index maps, pinned by numpy transposes.
+ *   - harness (fp32 reference convolution, output / sum scale calibration, input quantization): pinned against
+ *     the reference's own harness translation unit compiled from /root/reference (oracle/ref_harness.cpp).
  *   - not pinned by anything but the source: the ORDER of exact integer additions in the executors.
  */
 #ifndef EULER_ORACLE_H
@@ -70,6 +72,18 @@ void orc_reorder_blocked_to_oihw_f32(float *dst, const float *src, int o, int i,
 
 /* ---- harness-side input quantization: tests/elt_conv_utils.cpp:354-401 ---- */
 void orc_quantize_input_u8(uint8_t *dst, const float *src, size_t count, float scale, float z);
+
+/* ---- harness: fp32 reference convolution and the calibration rule built on it ----
+ * orc_ref_conv_f32: tests/elt_conv_utils.cpp:666-750 on plain tensors (input / output nchw, weights oihw, or
+ * goihw [g][oc/g][ic/g][kh][kw] for g > 1): out = (old out +) bias, then += x * w over (ic, kh, kw) with
+ * padded taps skipped, each step one fused multiply-add as the compiled harness has it, then ReLU.
+ * `output` holds the sum operand on entry when p->with_sum.
+ * orc_calibrate_output_quant: tests/elt_conv_utils.cpp:306-346 (see ehip_calibrate_output_quant). */
+int orc_ref_conv_f32(const orc_conv_params *p, float *output, const float *input, const float *weights,
+                     const float *bias);
+void orc_calibrate_output_quant(int with_relu, int out_type, int with_sum, float out_min, float out_max,
+                                float sum_absmax, float representation, float *output_scale, float *output_z,
+                                float *sum_scale);
 
 /* ---- direct 1x1 / KxK ----
  * weight quantization + scale/shift folding:

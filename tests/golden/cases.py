@@ -836,3 +836,81 @@ for _A in (6, 4, 5):
                                          glue_w_reference, glue_w_oracle)
     CASES["wino_glue_weights%d_negz" % _A] = (lambda A=_A: glue_w_inputs(A, 48, 16, 0.4071, -12.6, 950 + A),
                                               glue_w_reference, glue_w_oracle)
+
+
+# ---- the test harness: fp32 reference convolution, scale calibration, quantization of the input and of the
+# sum operand (tests/elt_conv_utils.cpp:87-463, :666-750) -------------------------------------------------------
+# The harness draws its own tensors (a default-seeded std::normal_distribution for input and weights, rand_r
+# seeded from the clock for bias and sum operand), so the stored inputs of these cases are what the compiled
+# harness produced, not something this file can regenerate: make_inputs() holds the layer only and the
+# reference run adds the tensors before the fixture is written.
+HARNESS_REPRESENTATION = 127.0   # PRECISION_REPRESENTATION_7B, used by the harness for every type
+
+
+def harness_config(out_s8, zero_point, n, g, ic, oc, hw, k, pad, stride, with_relu, with_sum):
+    oh = (hw + 2 * pad - k) // stride + 1
+    return dict(out_s8=np.int32(out_s8), zero_point=np.int32(zero_point), n=np.int32(n), g=np.int32(g), ic=np.int32(ic),
+                oc=np.int32(oc), hw=np.int32(hw), k=np.int32(k), pad=np.int32(pad), stride=np.int32(stride), oh=np.int32(oh),
+                with_relu=np.int32(with_relu), with_sum=np.int32(with_sum))
+
+
+def _harness_pack(quant, input_q, sum_q, conv_out):
+    return np.concatenate([np.ascontiguousarray(quant, np.float32).view(np.uint8).ravel(), input_q.ravel(), sum_q.ravel(),
+                           np.ascontiguousarray(conv_out, np.float32).view(np.uint8).ravel()])
+
+
+def harness_reference(d, _ref):
+    lib = ol.ref_harness()
+    assert lib is not None, "oracle/_ref/libeuler_ref_harness.so is not built"
+    n, g, ic, oc, hw, k, pad, stride, oh = (int(d[key]) for key in ("n", "g", "ic", "oc", "hw", "k", "pad", "stride", "oh"))
+    x = np.zeros((n, ic, hw, hw), np.float32)
+    w = np.zeros((oc, ic // g, k, k), np.float32)
+    out = np.zeros((n, oc, oh, oh), np.float32)
+    bias = np.zeros(oc, np.float32)
+    xq = np.zeros(x.shape, np.uint8)
+    sq = np.zeros(out.shape, np.uint8)
+    quant = np.zeros(5, np.float32)
+    lib.ref_harness_prepare(int(d["out_s8"]), int(d["zero_point"]), n, g, ic, oc, hw, hw, oh, oh, k, k, pad, pad, stride, stride,
+                            int(d["with_relu"]), int(d["with_sum"]), ol.ptr(x), ol.ptr(w), ol.ptr(out), ol.ptr(bias),
+                            ol.ptr(xq), ol.ptr(sq), ol.ptr(quant))
+    if int(d["with_sum"]):
+        sum_operand = out.copy()
+    else:
+        sum_operand = np.zeros_like(out)   # without a sum the harness leaves the convolution result there
+    conv = sum_operand.copy()
+    lib.ref_harness_conv2d(n, g, ic, oc, hw, hw, oh, oh, k, k, pad, pad, stride, stride, 1, int(d["with_relu"]),
+                           int(d["with_sum"]), ol.ptr(conv), ol.ptr(x), ol.ptr(w), ol.ptr(bias))
+    d.update(x=x, w=w, bias=bias, sum_operand=sum_operand)
+    return _harness_pack(quant, xq, sq, conv)
+
+
+def harness_oracle(d):
+    f32 = np.float32
+    n, g, ic, oc, hw, k, pad, stride, oh = (int(d[key]) for key in ("n", "g", "ic", "oc", "hw", "k", "pad", "stride", "oh"))
+    with_relu, with_sum = int(d["with_relu"]), int(d["with_sum"])
+    out_type = ol.S8 if int(d["out_s8"]) else ol.U8
+    x, w, bias, sum_operand = d["x"], d["w"], d["bias"], d["sum_operand"]
+    # input_quant: abs-max over 127, zero point 128 for the "...z" configurations (tests/elt_conv_utils.cpp:264-289)
+    in_scale = f32(np.abs(x).max()) / f32(HARNESS_REPRESENTATION)
+    in_z = f32(128.0 if int(d["zero_point"]) else 0.0)
+    xq = ol.quantize_input_u8(x, float(in_scale), float(in_z))
+    p = ol.make_params(n, ic, oc, hw, hw, k, k, pad, stride, g=g, with_relu=bool(with_relu), with_sum=bool(with_sum),
+                       out_type=out_type)
+    conv = ol.ref_conv_f32(p, x, w, bias, out_init=sum_operand if with_sum else None)
+    sum_absmax = float(np.abs(sum_operand).max()) if with_sum else 0.0
+    s_o, z_o, s_sum = ol.calibrate_output_quant(with_relu, out_type, with_sum, conv.min(), conv.max(), sum_absmax,
+                                                HARNESS_REPRESENTATION)
+    sq = np.zeros(conv.shape, np.uint8)
+    if with_sum:
+        # the sum operand is quantized with its own scale and the harness's rounding helper, then narrowed
+        # to a byte (tests/elt_conv_utils.cpp:444-462)
+        sq = ol.quantize_input_u8(sum_operand, float(f32(sum_absmax) / f32(HARNESS_REPRESENTATION)), 0.0)
+    return _harness_pack(np.array([in_scale, in_z, s_o, z_o, s_sum if with_sum else 0.0], f32), xq, sq, conv)
+
+
+CASES["harness_u8_relu_3x3"] = (lambda: harness_config(0, 0, 2, 1, 20, 24, 9, 3, 1, 1, 1, 0), harness_reference, harness_oracle)
+CASES["harness_s8_relu_sum_1x1"] = (lambda: harness_config(1, 0, 2, 1, 32, 16, 7, 1, 0, 1, 1, 1), harness_reference, harness_oracle)
+CASES["harness_u8_norelu_3x3_s2"] = (lambda: harness_config(0, 0, 1, 1, 16, 32, 11, 3, 1, 2, 0, 0), harness_reference, harness_oracle)
+CASES["harness_s8_norelu_z128_1x1"] = (lambda: harness_config(1, 1, 2, 1, 48, 16, 6, 1, 0, 1, 0, 0), harness_reference, harness_oracle)
+CASES["harness_u8_norelu_sum_1x1"] = (lambda: harness_config(0, 0, 1, 1, 16, 16, 8, 1, 0, 1, 0, 1), harness_reference, harness_oracle)
+CASES["harness_u8_relu_depthwise"] = (lambda: harness_config(0, 0, 2, 16, 16, 16, 10, 3, 1, 1, 1, 0), harness_reference, harness_oracle)

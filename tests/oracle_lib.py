@@ -14,6 +14,7 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 ORACLE_SO = os.path.join(ORACLE_DIR, "libeuler_oracle.so")
 REF_SO = os.path.join(ORACLE_DIR, "_ref", "libeuler_ref_kernels.so")
 REF_GLUE_SO = os.path.join(ORACLE_DIR, "_ref", "libeuler_ref_wino_glue.so")
+REF_HARNESS_SO = os.path.join(ORACLE_DIR, "_ref", "libeuler_ref_harness.so")
 
 F32, U8, S8, S32 = 1, 3, 4, 5
 NP_OF = {F32: np.float32, U8: np.uint8, S8: np.int8, S32: np.int32}
@@ -94,6 +95,8 @@ def oracle():
         lib.orc_epilogue.argtypes = [ctypes.c_int, ctypes.c_int32, ctypes.c_float, ctypes.c_float, ctypes.c_int,
                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_float,
                                      ctypes.POINTER(ctypes.c_float)]
+        lib.orc_calibrate_output_quant.argtypes = [ctypes.c_int] * 3 + [ctypes.c_float] * 4 + [ctypes.POINTER(ctypes.c_float)] * 3
+        lib.orc_calibrate_output_quant.restype = None
         _oracle = lib
     return _oracle
 
@@ -161,9 +164,62 @@ def ref_wino_glue():
     return _ref_glue
 
 
+def ref_harness():
+    """The reference's test harness (tests/elt_conv_utils.cpp: fp32 reference convolution, scale calibration,
+    input quantization) compiled from the reference tree by oracle/Makefile, or None where oracle/_ref was
+    not built or the host lacks AVX-512."""
+    global _ref_harness
+    if _ref_harness is None:
+        if not os.path.exists(REF_HARNESS_SO):
+            return None
+        try:
+            flags = open("/proc/cpuinfo").read()
+        except OSError:
+            flags = ""
+        if "avx512_vnni" not in flags or "avx512bw" not in flags:
+            return None
+        # The harness unit calls the executor library in one place (elx_conv, for Winograd calibration), which
+        # is not built here and which nothing below reaches: bind lazily, so that the unresolved function
+        # does not stop the load (ctypes itself always asks for immediate binding).
+        dl = ctypes.CDLL(None)
+        dl.dlopen.restype = ctypes.c_void_p
+        dl.dlopen.argtypes = [ctypes.c_char_p, ctypes.c_int]
+        handle = dl.dlopen(REF_HARNESS_SO.encode(), os.RTLD_LAZY | os.RTLD_LOCAL)
+        if not handle:
+            return None
+        lib = ctypes.CDLL(REF_HARNESS_SO, handle=handle)
+        ci, vp = ctypes.c_int, ctypes.c_void_p
+        lib.ref_harness_conv2d.argtypes = [ci] * 17 + [vp] * 4
+        lib.ref_harness_prepare.argtypes = [ci] * 18 + [vp] * 7
+        _ref_harness = lib
+    return _ref_harness
+
+
+_ref_harness = None
+
+
 # --------------------------------------------------------------------------------------------
 # numpy-level wrappers
 # --------------------------------------------------------------------------------------------
+def ref_conv_f32(p, x_nchw, w_goihw, bias, out_init=None):
+    """the harness's fp32 reference convolution on plain tensors (out_init: the sum operand)"""
+    out = np.zeros((p.n, p.oc, p.oh, p.ow), np.float32)
+    if out_init is not None:
+        out[...] = out_init
+    x_nchw, w_goihw, bias = (np.ascontiguousarray(a, np.float32) for a in (x_nchw, w_goihw, bias))
+    assert oracle().orc_ref_conv_f32(ctypes.byref(p), ptr(out), ptr(x_nchw), ptr(w_goihw), ptr(bias)) == 0
+    return out
+
+
+def calibrate_output_quant(with_relu, out_type, with_sum, out_min, out_max, sum_absmax, representation):
+    """(output scale, output z, sum scale) by the harness's rule"""
+    s, z, ss = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
+    oracle().orc_calibrate_output_quant(int(with_relu), int(out_type), int(with_sum), float(out_min), float(out_max),
+                                        float(sum_absmax), float(representation), ctypes.byref(s), ctypes.byref(z),
+                                        ctypes.byref(ss))
+    return s.value, z.value, ss.value
+
+
 def up16(x):
     return (x + 15) // 16 * 16
 

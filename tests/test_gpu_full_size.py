@@ -107,3 +107,41 @@ def test_configured_winograd_layer_u8_in_s8_out(key, check_images, nhwc):
     assert np.array_equal(got[:k], exp), "%d values differ" % int((got[:k] != exp).sum())
     assert not (got == -7).any()          # ReLU output: every cell was written
     assert len(np.unique(got)) > 60       # and the s8 codes use their range
+
+
+@pytest.mark.parametrize("key", ["C2", "C3a", "C3b", "C1", "C5a"])
+def test_benchmark_layer_with_calibrated_scales(key):
+    """The benchmark's own tensors (workloads.DeviceLayer: seeded fp32 tensors, output / sum scales calibrated
+    from the fp32 reference convolution as the reference's harness does) through the oracle: same bytes, and
+    the calibrated codes reach the top of their range."""
+    import torch
+    wl = W.WORKLOADS[key]
+    layer = W.DeviceLayer(wl)
+    d = layer.desc
+    old = host(layer.out).copy()
+    layer.run(1)
+    torch.cuda.synchronize()
+    got = host(layer.out)
+    g = wl.ic if wl.depthwise else 1
+    p = ol.make_params(wl.n, wl.ic, wl.oc, wl.hw, wl.hw, wl.k, wl.k, wl.pad, wl.stride, g=g, out_type=wl.out_type,
+                       with_sum=wl.with_sum, T=wl.T, in_scale=d.input_scale, out_scale=d.output_scale, out_z=d.output_z,
+                       sum_scale=d.sum_scale, relu_lo=d.relu_lower, relu_hi=d.relu_upper)
+    x, w, bias = host(layer.x), host(layer.w), host(layer.bias)
+    if wl.depthwise:
+        wq, scale, shift, _ = ol.depthwise_prepare(p, w.reshape(wl.ic, 1, 3, 3), bias)
+        exp, _ = ol.depthwise_execute(p, x, wq, scale, shift)
+    else:
+        wq, scale, shift, _ = ol.direct_prepare(p, w, bias)
+        exp, _ = ol.direct_execute(p, x, wq, scale, shift, out_init=old if wl.with_sum else None)
+    assert np.array_equal(bits(got), bits(exp)), "%d of %d values differ" % (int((got != exp).sum()), got.size)
+    if wl.relu6:
+        assert layer.calibration == {}   # a ReLU6 layer keeps its fixed 6/255 output scale
+    elif wl.out_type == ol.U8:
+        assert got.max() >= 250
+    elif wl.out_type == ol.S8:
+        assert got.max() >= 120
+        assert layer.calibration["sum_scale"] > 0
+    # seeded: a second layer holds the same bytes
+    again = W.DeviceLayer(wl)
+    assert torch.equal(again.x, layer.x) and torch.equal(again.w, layer.w)
+    assert again.desc.output_scale == d.output_scale
