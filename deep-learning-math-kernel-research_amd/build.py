@@ -37,6 +37,13 @@ FLAGS = [
 ]
 
 
+# per-source additions.  The depthwise matrix-core kernel has one accumulator tile per wave and turns it
+# straight into bytes: in the accumulation registers every value would be moved in and out once.
+EXTRA_FLAGS = {
+    "ehip_depthwise.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def _stale(obj, src):
     """an object is reused only when it is newer than its source and every header"""
     if not os.path.exists(obj):
@@ -58,7 +65,7 @@ def build(verbose=True, jobs=8, incremental=False):
         objs.append(obj)
         if incremental and not _stale(obj, os.path.join(CSRC, src)):
             continue
-        cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))

@@ -367,7 +367,8 @@ int setup_workspace(ehip_conv *c)
     c->T = d.flatting_t > 0 ? (d.flatting_t > d.ow ? d.ow : d.flatting_t) : 1;
     c->wtb = (d.ow + c->T - 1) / c->T;
     c->Tr = d.ow % c->T ? d.ow % c->T : c->T;
-    c->kernel_name = "k_depthwise3x3_u8s8";
+    c->kernel_name = depthwise_mfma_applies(d.stride_h, d.oh, d.ow, d.pad_t, d.pad_l, d.output_type, d.with_relu, d.relu_lower,
+                                            d.relu_upper) ? "k_depthwise3x3_mfma" : "k_depthwise3x3_u8s8";
     break;
   }
   case FAM_WINOGRAD: {
@@ -413,7 +414,8 @@ int setup_workspace(ehip_conv *c)
 
   if (c->family == FAM_DEPTHWISE) {
     c->ocpp = c->oc2 * 16;
-    c->wpacked_bytes = (size_t)c->oc2 * 3 * 16 * 4;
+    // [g2][kh][16][4] s8, then the matrix-core kernel's diagonal A operands [g2][6][64][16 bytes]
+    c->wpacked_bytes = (size_t)c->oc2 * 3 * 16 * 4 + (size_t)c->oc2 * 6 * 64 * 16;
   } else {
     c->ocpp = up(c->oc2 * 16, kOcTile);
     // (the K loop may run up to one chunk of 8 units past the last real one: zero rows)
@@ -543,6 +545,7 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const vo
     break;
   case FAM_DEPTHWISE:
     HIP_TRY(launch_prepare_depthwise(w, b, d.g, d, c->wpacked, c->scale, c->shift, c->wsum, s));
+    HIP_TRY(launch_depthwise_diag(c->wpacked, c->oc2, c->wpacked + (size_t)c->oc2 * 192, s));
     break;
   case FAM_WINOGRAD: {
     float *u_tmp = nullptr;
@@ -653,6 +656,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.w = c->wpacked;
     a.out = output_dev;
     a.scale = c->scale; a.shift = c->shift; a.wsum = c->wsum;
+    a.wdiag = reinterpret_cast<const uint4 *>(c->wpacked + (size_t)c->oc2 * 192);
     a.n = d.n; a.g2 = c->oc2; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow;
     a.stride = d.stride_h;
     a.pad_t = d.pad_t; a.pad_l = d.pad_l;

@@ -86,10 +86,12 @@ struct DepthwiseArgs {
   void *out;            // [n][g2][oh][ow][16]
   const float *scale, *shift;  // [G]
   const int *wsum;      // [G] sum of the packed weights per channel
+  const uint4 *wdiag;   // [g2][6][64] A operands of the matrix-core kernel (launch_depthwise_diag)
   int n, g2, ih, iw, oh, ow, pad_t, pad_l;
   int stride;           // 1 or 2, both directions
   int T, Tr, wt;        // width blocking of the reference kernel (decides floor vs round per column)
   int lanes_per_plane;  // set by the launcher: row blocks x column pairs x 4
+  int strips_per_wg;    // set by the launcher (matrix-core kernel): consecutive strips a workgroup walks
   int blocks_per_plane; // set by the launcher: workgroups per plane
   unsigned wp_magic, T_magic;  // div_magic of the column pairs per row and of T
   int out_type, with_relu;
@@ -183,6 +185,8 @@ int conv3x3v_num_variants();
 const char *conv3x3v_variant_name(int variant);
 
 hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s, LaunchPlan<DepthwiseArgs> *plan = nullptr);
+hipError_t launch_depthwise_diag(const int8_t *wpacked, int g2n, void *diag, hipStream_t s);
+bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, int out_type, int with_relu, float lo, float hi);
 hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
 hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);

@@ -329,6 +329,36 @@ def test_depthwise_u8_other_bounds(relu_hi, with_relu):
                           relu_hi=relu_hi, with_relu=with_relu))
 
 
+@pytest.mark.parametrize("g,hw,pad,T,relu_hi,in_z", [
+    (32, 28, 1, 14, 255.0, 0.0), (144, 56, 1, 14, 255.0, 0.0), (16, 70, 1, 7, 255.0, 0.0), (16, 112, 1, 28, 255.0, 0.0),
+    (32, 30, 1, 11, 255.0, 0.0), (48, 9, 1, 4, 255.0, 0.0), (32, 13, 0, 0, 255.0, 0.0), (16, 37, 0, 5, 200.0, 0.0),
+    (32, 28, 1, 7, 100.0, 0.0), (48, 14, 1, 14, 255.0, 37.0), (16, 128, 1, 16, 255.0, 0.0), (32, 5, 1, 5, 255.0, 0.0),
+])
+def test_depthwise_on_the_matrix_cores(g, hw, pad, T, relu_hi, in_z, monkeypatch):
+    """k_depthwise3x3_mfma (stride 1, u8 output, ReLU inside the code range) forced onto every shape it accepts:
+    1 to 4 chunks of 32 columns, widths and heights that fill neither the last chunk nor the last strip of
+    8 rows, no padding, both clamp forms, width-block sizes that split lanes into floor and round columns."""
+    monkeypatch.setenv("EHIP_DW_MFMA", "1")
+    n = 2 if hw < 56 else 1
+    layer = Layer(n, g, g, hw, k=3, pad=pad, out_type=ol.U8, depthwise=True, seed=g + hw + T + 11, w_sigma=0.1, T=T,
+                  relu_hi=relu_hi, in_z=in_z)
+    res = run_and_compare(layer)
+    if res is not None:
+        assert res["conv"].kernel_name == "k_depthwise3x3_mfma"
+
+
+def test_depthwise_matrix_core_kernel_is_the_default_where_it_fits(monkeypatch):
+    monkeypatch.delenv("EHIP_DW_MFMA", raising=False)
+    E = pkg()
+    names = {}
+    for hw in (7, 14, 28, 56, 112):
+        d = E.make_desc(1, 32, 32, hw, hw, 3, 3, pad=1, g=32, output_type=E.U8, relu_bound=(0.0, 255.0), flatting_t=7,
+                        output_quant=(0.02, 0.0))
+        names[hw] = E.Conv(d).kernel_name
+    assert names[56] == names[28] == "k_depthwise3x3_mfma"
+    assert names[7] == names[14] == names[112] == "k_depthwise3x3_u8s8"   # half-empty chunks, or too wide: the dot4 kernel
+
+
 # stride 2 (MobileNet's down-sampling layers, scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh:48:
 # pad 0 with the output size asking for one pad row / column at the bottom / right)
 @pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
