@@ -50,6 +50,39 @@ __device__ __forceinline__ void wait_all_loads()
 #endif
 }
 
+// The same load written as assembly.  The compiler cannot tell which part of LDS an LDS-writing load
+// touches, and makes the first LDS read behind such loads wait for ALL of them; this form it does not see as
+// a memory instruction at all.  The caller waits for these loads itself (wait_loads_but) and must not rely
+// on the compiler's own waits to cover them: those then wait for a few older loads more than they need,
+// never for fewer, because the wave's loads complete in issue order.
+__device__ __forceinline__ void load_to_lds_16_unseen(const void *gsrc, void *lds_dst)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  const unsigned m = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m), "v"(gsrc) : "memory", "m0");
+#else
+  (void)gsrc;
+  (void)lds_dst;
+#endif
+}
+// vmcnt(n): at most n of the wave's vector-memory loads still in flight.  n is a constant after unrolling.
+__device__ __forceinline__ void wait_loads_but(int n)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+#define EHIP_W(N) case N: __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14)); break;
+  switch (n) {
+    EHIP_W(0) EHIP_W(1) EHIP_W(2) EHIP_W(3) EHIP_W(4) EHIP_W(5) EHIP_W(6) EHIP_W(7) EHIP_W(8) EHIP_W(9) EHIP_W(10)
+    EHIP_W(11) EHIP_W(12) EHIP_W(13) EHIP_W(14) EHIP_W(15) EHIP_W(16) EHIP_W(17) EHIP_W(18) EHIP_W(19) EHIP_W(20)
+    EHIP_W(21) EHIP_W(22) EHIP_W(23) EHIP_W(24) EHIP_W(25) EHIP_W(26) EHIP_W(27) EHIP_W(28) EHIP_W(29) EHIP_W(30)
+    EHIP_W(31) EHIP_W(32)
+    default: __builtin_amdgcn_s_waitcnt(0x0f70); break;
+  }
+#undef EHIP_W
+#else
+  (void)n;
+#endif
+}
+
 // NKS > 0: the layer has exactly NKS k-steps (pairs of 16-channel units): the K loop is straight-line code
 // and every wait names the load it needs.  NKS == 0: a loop over blocks of eight k-steps.
 template <int TM, int TN, int NKS>
@@ -117,7 +150,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
     src[h] = a.in + ((long long)n * a.ic2 * a.ihw + sp) * 16;
   }
   const long long unit_stride = (long long)a.ihw * 16;
-  {
+  auto request_tile = [&]() {   // in unit order: what lands first is what the K loop needs first
     const int items = a.units_pad * HALVES;
     for (int it = wave; it < items; it += 4) {
       const int u = it / HALVES, h = it - u * HALVES;
@@ -127,7 +160,28 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
         if (hh == h)
           load_to_lds_16(src[hh] + (long long)uc * unit_stride, lds + (size_t)u * P_T + h * 64);
     }
-  }
+  };
+  // PIPE (the wave's whole weight slice fits in registers and is requested up front, BEFORE the tile, and
+  // nothing else is loaded until the K loop is over): the tile is consumed as it arrives.  Loads complete in
+  // issue order, so the weights (from L2) are there first; the K loop then waits for eight units (four
+  // k-steps) of the tile at a time -- its own share by count, everybody else's by a barrier -- instead of
+  // for all 64 KB before its first MFMA.
+  constexpr bool PIPE = NKS > 0 && R == NKS && NKS % 4 == 0;
+  constexpr int LPC = 2 * HALVES;            // loads of one wave per chunk: 8 units x HALVES dealt to four waves
+  constexpr int TILE_LOADS = NKS * HALVES / 2;   // of one wave, all chunks (PIPE)
+  auto request_tile_unseen = [&]() {
+#pragma unroll
+    for (int j = 0; j < TILE_LOADS; ++j) {
+      const int it = wave + 4 * j;
+      const int u = it / HALVES, h = it - u * HALVES;
+      const int uc = u < a.ic2 ? u : a.ic2 - 1;
+      const uint8_t *p = src[0];
+#pragma unroll
+      for (int hh = 1; hh < HALVES; ++hh) p = hh == h ? src[hh] : p;
+      load_to_lds_16_unseen(p + (long long)uc * unit_stride, lds + (size_t)u * P_T + h * 64);
+    }
+  };
+  if (!PIPE) request_tile();
 
   TRACE_POINT(1);
   // ---- weights [units_pad][ocpp][16]: lane = packed row l32 of unit 2 ks + lh, tile mt 32 rows on --------
@@ -174,10 +228,21 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
     }
   };
 
-  // the tile has landed (every wave waits for its own loads, the barrier for everybody else's)
-  wait_all_loads();
-  TRACE_POINT(2);
-  __syncthreads();
+  auto next_chunk = [&](int c) {   // units 8 c .. 8 c + 7 of the tile are in LDS, everybody's share
+    wait_loads_but(TILE_LOADS - (c + 1) * LPC);
+    __syncthreads();
+  };
+  if (PIPE) {
+    load_epilogue_consts();   // nothing may be requested behind the tile
+    request_tile_unseen();
+    TRACE_POINT(2);
+    next_chunk(0);
+  } else {
+    // the tile has landed (every wave waits for its own loads, the barrier for everybody else's)
+    wait_all_loads();
+    TRACE_POINT(2);
+    __syncthreads();
+  }
   TRACE_POINT(3);
 
   // ---- K loop: one memory instruction behind each MFMA ---------------------------------------------------
@@ -209,7 +274,8 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
   if (NKS > 0) {
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      if (ks == (NKS > R ? NKS - R : 0)) load_epilogue_consts();
+      if (!PIPE && ks == (NKS > R ? NKS - R : 0)) load_epilogue_consts();
+      if (PIPE && (ks + 1) % 4 == 0 && ks + 1 < NKS) next_chunk((ks + 1) / 4);   // k-step ks reads the operands of ks + 1
       kstep(ks & 1, ks % R, ks, ks + 1 < NKS, ks + R < NKS);
     }
   } else {
