@@ -37,16 +37,23 @@ def measure(layer, steps, warmup):
     while time.perf_counter() - t0 < PREHEAT_S:
         layer.run(200)
         torch.cuda.synchronize()
-    layer.run(warmup)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    layer.run(steps)
-    e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    return (t1 - t0) / steps, e0.elapsed_time(e1) * 1e-3 / steps
+    def region(count):
+        # exactly `count` steps between two synchronisations, on the host clock and on HIP events
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        layer.run(count)
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) / count, e0.elapsed_time(e1) * 1e-3 / count
+
+    # the warmup steps take the same path as the timed ones (event creation and recording included): what a
+    # first call costs the host once -- lazy initialisation behind the first event, cold code -- stays out
+    if warmup > 0:
+        region(warmup)
+    return region(steps)
 
 
 def single_launch_latency(layer, reps=20):

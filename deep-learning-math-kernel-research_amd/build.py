@@ -41,6 +41,8 @@ FLAGS = [
 # straight into bytes: in the accumulation registers every value would be moved in and out once.
 EXTRA_FLAGS = {
     "ehip_depthwise.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    # the 3x3 kernel takes what its first instructions need as leading scalar arguments: preloaded with the wave
+    "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 
