@@ -59,6 +59,7 @@ struct ehip_conv {
   int chunk_n = 0;   // images per pass of the three-stage pipeline (intermediates sized for it)
   bool fused = true; // GEMM and output transform in one kernel (no f32 GEMM result in memory)
   uint8_t *tin = nullptr;
+  bool tin_blocked = false;   // Winograd, fused schedule: tin as [t / 32][36][ic2][32][16]
   float *tout = nullptr;
   size_t tin_bytes = 0, tout_bytes = 0;
 
@@ -402,7 +403,12 @@ int setup_workspace(ehip_conv *c)
     }
     c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
                               : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output";
-    c->tin_bytes = (size_t)c->nbatch * c->ic2 * c->t * 16;   // allocated with one pad unit behind it
+    {
+      const char *env = getenv("EHIP_WINO_TIN_BLOCKED");
+      c->tin_blocked = c->fused && !(env && env[0] == '0');
+    }
+    // (blocked: whole blocks of 32 tiles)  allocated with one pad unit behind it
+    c->tin_bytes = (size_t)c->nbatch * c->ic2 * (c->tin_blocked ? up(c->t, 32) : c->t) * 16;
     c->tout_bytes = c->fused ? 16 : (size_t)c->nbatch * c->oc2 * c->t * 16 * sizeof(float);
     if ((rc = dev_alloc(&c->tin, c->tin_bytes + (size_t)c->t * 16, true)) != EHIP_OK) return rc;
     if ((rc = dev_alloc(reinterpret_cast<uint8_t **>(&c->tout), c->tout_bytes, false)) != EHIP_OK) return rc;
@@ -676,6 +682,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       const size_t in_esz = d.input_type == EHIP_U8 ? 1 : 4, out_esz = d.output_type == EHIP_F32 ? 4 : 1;
       w.in = static_cast<const uint8_t *>(input_dev) + (size_t)n0 * c->ic2 * d.ih * d.iw * 16 * in_esz;
       w.tin = c->tin;
+      w.tin_blocked = c->tin_blocked;
       w.tout = c->tout;
       w.out = static_cast<uint8_t *>(output_dev) + (size_t)n0 * c->oc2 * d.oh * d.ow * 16 * out_esz;
       w.bias = static_cast<const float *>(bias_dev);
@@ -688,7 +695,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       if (c->fused) {
         WinoFusedArgs f;
         memset(&f, 0, sizeof(f));
-        f.tin = c->tin; f.w = c->wpacked; f.out = w.out; f.bias = w.bias;
+        f.tin = c->tin; f.tin_blocked = c->tin_blocked; f.w = c->wpacked; f.out = w.out; f.bias = w.bias;
         f.scale = c->scale; f.shift = c->shift; f.comp = c->comp;
         f.n = w.n; f.ic2 = c->ic2; f.units_pad = c->units_pad; f.oc2 = c->oc2; f.ocpp = c->ocpp;
         f.oh = d.oh; f.ow = d.ow; f.ht = w.ht; f.wt = w.wt; f.nt = w.nt; f.t = w.t;
@@ -795,6 +802,19 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
   case EHIP_Q_TINPUT_U8:
     if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "not a Winograd handle");
     if (c->chunk_n < d.n) return fail(EHIP_UNIMPLEMENTED, "the intermediates of a multi-pass layer hold its last pass only");
+    if (c->tin_blocked) {   // back to the canonical [pos][ic2][t][16]
+      const size_t canon = (size_t)c->nbatch * c->ic2 * c->t * 16;
+      if (!want(canon)) return EHIP_OK;
+      std::vector<uint8_t> raw(c->tin_bytes);
+      HIP_TRY(hipMemcpy(raw.data(), c->tin, c->tin_bytes, hipMemcpyDeviceToHost));
+      uint8_t *dst = static_cast<uint8_t *>(host_dst);
+      for (int p = 0; p < c->nbatch; ++p)
+        for (int u = 0; u < c->ic2; ++u)
+          for (int t = 0; t < c->t; ++t)
+            memcpy(dst + (((size_t)p * c->ic2 + u) * c->t + t) * 16,
+                   raw.data() + ((((size_t)(t >> 5) * c->nbatch + p) * c->ic2 + u) * 32 + (t & 31)) * 16, 16);
+      return EHIP_OK;
+    }
     if (!want(c->tin_bytes)) return EHIP_OK;
     HIP_TRY(hipMemcpy(host_dst, c->tin, c->tin_bytes, hipMemcpyDeviceToHost));
     return EHIP_OK;

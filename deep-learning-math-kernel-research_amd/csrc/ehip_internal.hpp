@@ -100,7 +100,8 @@ struct DepthwiseArgs {
 
 struct WinoArgs {
   const void *in;       // [n][ic2][ih][iw][16] f32, or u8 codes (in_u8)
-  uint8_t *tin;         // [36][ic2][t][16]
+  uint8_t *tin;         // [36][ic2][t][16], or (tin_blocked) [t / 32][36][ic2][32][16]
+  int tin_blocked;      // the fused schedule's layout: everything a block of 32 tiles needs is one contiguous run
   const float *tout;    // [36][oc2][t][16]
   void *out;            // [n][oc2][oh][ow][16] f32 / u8 / s8 (out_type)
   const float *bias;
@@ -116,7 +117,8 @@ struct WinoArgs {
 };
 
 struct WinoFusedArgs {
-  const uint8_t *tin;   // [36][ic2][t][16] u8
+  const uint8_t *tin;   // [36][ic2][t][16] u8, or (tin_blocked) [t / 32][36][ic2][32][16]
+  int tin_blocked;
   const int8_t *w;      // [36][units_pad][OCpp][16] s8
   void *out;            // [n][oc2][oh][ow][16] f32 / u8 / s8 (out_type)
   const float *bias;

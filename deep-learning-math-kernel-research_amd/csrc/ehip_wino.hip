@@ -126,8 +126,10 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   const int q = threadIdx.x & 3;
   const int item = (blockIdx.x & 7) * a.items_per_xcd + (blockIdx.x >> 3);
   if (item >= a.nblocks * a.ic2) return;   // whole workgroup
-  const int c2 = item / a.nblocks;
-  const int t = (item - c2 * a.nblocks) * 64 + (threadIdx.x >> 2);
+  // plain layout: an XCD walks the tile blocks of one unit after the other (neighbours share input rows in
+  // its L2); blocked layout: the units of one tile block after the other, whose pieces are neighbours in tin
+  const int c2 = a.tin_blocked ? item % a.ic2 : item / a.nblocks;
+  const int t = (a.tin_blocked ? item / a.ic2 : item - c2 * a.nblocks) * 64 + (threadIdx.x >> 2);
   if (t >= a.t) return;
   const TileCoord c = tile_coord<A>(a, t);
   Cell d[AA];
@@ -156,8 +158,9 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   };
   if (__ballot(c.border) != 0) channels(true);   // wave-uniform
   else channels(false);
-  unsigned *dst = reinterpret_cast<unsigned *>(a.tin) + ((size_t)c2 * a.t + t) * 4 + q;
-  const size_t pos_stride = (size_t)a.ic2 * a.t * 4;
+  unsigned *dst = reinterpret_cast<unsigned *>(a.tin) +
+      (a.tin_blocked ? (((size_t)(t >> 5) * AA * a.ic2 + c2) * 32 + (t & 31)) * 4 + q : ((size_t)c2 * a.t + t) * 4 + q);
+  const size_t pos_stride = a.tin_blocked ? (size_t)a.ic2 * 32 * 4 : (size_t)a.ic2 * a.t * 4;
 #pragma unroll
   for (int e = 0; e < AA; ++e) dst[e * pos_stride] = packed[e];
 }
@@ -391,7 +394,9 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   // never changes: lane = packed row / tile l32 of unit 2 * ks + lh
   const unsigned a_lane = (unsigned)(lh * a.ocpp + l32) * 16u;
   const int tile = t0 + l32 < a.t ? t0 + l32 : a.t - 1;
-  const unsigned b_lane = (unsigned)(lh * a.t + tile) * 16u;
+  // plain layout: tile `tile` of unit lh; blocked: cell l32 of unit lh inside the block's own run (cells of
+  // tiles past the end hold nothing and are never stored)
+  const unsigned b_lane = a.tin_blocked ? (unsigned)(lh * 32 + l32) * 16u : (unsigned)(lh * a.t + tile) * 16u;
   const int ks_last = ((a.ic2 + 1) >> 1) - 1;   // last k-step that holds real channels
 
   TRACE_POINT(0);
@@ -403,7 +408,8 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     // padded k-steps multiply zero weights: any valid cell will do (an odd unit count reads one
     // unit past the position, which is the next position or the pad unit behind the buffer)
     const int ksc = ks < ks_last ? ks : ks_last;
-    const uint8_t *pb = a.tin + ((long long)p * a.ic2 + 2 * ksc) * a.t * 16;
+    const uint8_t *pb = a.tin_blocked ? a.tin + (((long long)bx * 36 + p) * a.ic2 + 2 * ksc) * 512
+                                      : a.tin + ((long long)p * a.ic2 + 2 * ksc) * a.t * 16;
     rb[slot] = *reinterpret_cast<const v4i *>(pb + b_lane);
   };
 
