@@ -133,9 +133,6 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
   const long long w_tap = (long long)a.units_pad * w_unit;
   v4i a_reg[9][TM];
   auto load_a = [&](int tap, int pair) {
-#if defined(EHIP_KO) && (EHIP_KO & 1)
-    if (pair > 0) return;   // knock-out (development): the weight operands of pair 0 are used throughout
-#endif
     const int8_t *p = wb + tap * w_tap + (long long)(2 * pair) * w_unit;
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) a_reg[tap][mt] = *reinterpret_cast<const v4i *>(p + mt * 512);

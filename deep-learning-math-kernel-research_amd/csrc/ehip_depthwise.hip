@@ -88,12 +88,16 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
   // column pair, then row block).  Workgroups go round the eight XCDs (block b runs on XCD b % 8), each
   // with an L2 of its own, and neighbouring row blocks share two input rows: so all blocks of a plane
   // are given to ONE XCD, one after the other -- plane = 8 * (seq / blocks_per_plane) + xcd.
+  // Small planes (7 x 7: 64 lanes) share a workgroup, planes_per_block of them, each on whole waves of its
+  // own: one-wave workgroups by the ten thousand are bound by the rate at which workgroups are dispatched.
   const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
   const int pgrp = seq / a.blocks_per_plane;
-  const int plane_id = pgrp * 8 + xcd;
-  if (plane_id >= a.n * a.g2) return;   // whole workgroup
+  const int sub = a.planes_per_block > 1 ? (int)threadIdx.x / a.lanes_padded : 0;   // wave-uniform
+  const int plane_id = (pgrp * 8 + xcd) * a.planes_per_block + sub;
+  if (plane_id >= a.n * a.g2) return;   // whole waves
   const int wp = (a.ow + 1) >> 1;
-  const int local = (seq - pgrp * a.blocks_per_plane) * blockDim.x + threadIdx.x;
+  const int local = a.planes_per_block > 1 ? (int)threadIdx.x - sub * a.lanes_padded
+                                           : (seq - pgrp * a.blocks_per_plane) * (int)blockDim.x + (int)threadIdx.x;
   if (local >= a.lanes_per_plane) return;
   const int q = local & 3;
   const int hb = fastdiv(local >> 2, wp, a.wp_magic);
@@ -512,10 +516,17 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<D
   int mode = 0;
   if (a.out_type == EHIP_U8 && a.with_relu && a.lo >= 0.0f && a.hi <= 255.0f && a.hi >= a.lo)
     mode = (a.lo == 0.0f && a.hi == 255.0f) ? 2 : 1;
-  const int block = a.lanes_per_plane >= kBlock ? kBlock : up(a.lanes_per_plane, kWave);
+  int block = a.lanes_per_plane >= kBlock ? kBlock : up(a.lanes_per_plane, kWave);
   a.blocks_per_plane = (a.lanes_per_plane + block - 1) / block;
   const long long planes = (long long)a.n * a.g2;
-  dim3 grid((unsigned)(8 * ((planes + 7) / 8) * a.blocks_per_plane), 1, 1);
+  a.planes_per_block = 1;
+  a.lanes_padded = block;
+  if (block <= kBlock / 2) {   // a plane fits one or two waves: several planes per workgroup
+    a.planes_per_block = kBlock / block;
+    block *= a.planes_per_block;
+  }
+  const long long groups = (planes + a.planes_per_block - 1) / a.planes_per_block;
+  dim3 grid((unsigned)(8 * ((groups + 7) / 8) * a.blocks_per_plane), 1, 1);
   const dw_kernel_t kernel = rb == 7 ? kernel_rb<7>(a.stride, mode)
       : (rb == 4 ? kernel_rb<4>(a.stride, mode) : (rb == 2 ? kernel_rb<2>(a.stride, mode) : kernel_rb<1>(a.stride, mode)));
   return plan_launch(plan, kernel, grid, dim3(block), 0, a, s);

@@ -92,6 +92,7 @@ struct DepthwiseArgs {
   int T, Tr, wt;        // width blocking of the reference kernel (decides floor vs round per column)
   int lanes_per_plane;  // set by the launcher: row blocks x column pairs x 4
   int strips_per_wg;    // set by the launcher (matrix-core kernel): consecutive strips a workgroup walks
+  int planes_per_block, lanes_padded;   // set by the launcher (dot4 kernel): small planes sharing a workgroup, lanes per plane rounded up to waves
   int blocks_per_plane; // set by the launcher: workgroups per plane
   unsigned wp_magic, T_magic;  // div_magic of the column pairs per row and of T
   int out_type, with_relu;
