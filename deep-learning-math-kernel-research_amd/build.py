@@ -42,7 +42,9 @@ FLAGS = [
 EXTRA_FLAGS = {
     "ehip_depthwise.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     # the 3x3 kernel takes what its first instructions need as leading scalar arguments: preloaded with the wave
-    "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    # (and its straight-line K loops are 72 steps of ~250 instructions: beyond the default budget of
+    # `#pragma unroll`, which then leaves a loop whose weight registers are indexed at run time, i.e. in scratch)
+    "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-pragma-unroll-threshold=1000000"],
 }
 
 

@@ -506,7 +506,7 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
   // there the 256-pixel tiles (11, 12) and the two-pass 128-channel tile (13) are 1.3-1.8 x faster
   // than the 128-pixel tiles with three passes.
   const int oc = oc2 * 16, vpx = oh * (ow + 2);
-  static const double pref[] = {0.80, 0.78, 0.92, 0.90, 1.0, 0.95, 1.0, 0.95, 0.85, 1.12, 0.95, 0.97, 1.10, 0.93, 0.85,
+  static const double pref[] = {0.80, 0.78, 0.92, 0.90, 1.0, 0.95, 1.0, 0.95, 0.85, 1.12, 0.95, 0.97, 1.14, 0.93, 0.85,
                                 0.0, 0.0, 0.0, 0.0, 0.0};
   int best = -1;
   double best_score = -1;
@@ -516,8 +516,9 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
     const Variant &k = kVariants[v];
     if (pass == 0) {
       if (oc > 64 && k.oc_t < 128) continue;
-      // (64 channels: the 128-channel tile whose waves own 32 channels each, half of them idle, still beats
-      // the 64-channel tiles on narrow rows -- measured 16.9 against 19.3 us for 64 -> 64 at 56 x 56, N = 64)
+      // (64 channels: the 128-channel tile whose waves own 32 channels each, half of them idle, is within a
+      // few percent of the best 64-channel tile -- 64 -> 64 at 56 x 56, N = 64: 19.1 us against 16.8 us for
+      // variant 12 and 19.4 us for variant 4 -- and wins where 256-pixel tiles waste too many pixels)
       if (oc <= 64 && oc > 32 && k.oc_t != 64 && v != 9) continue;
       if (oc <= 32 && k.oc_t != 32) continue;
     }
