@@ -41,6 +41,31 @@ namespace ehip {
 
 namespace {
 
+// Buffer addressing (a load whose offset lies outside the buffer returns zero and touches no memory).  The
+// builtins exist in the device pass only.
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+__device__ __forceinline__ BufferRsrc make_rsrc(const void *base, unsigned bytes)
+{
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), (short)0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ void buffer_load_cell(BufferRsrc r, unsigned off, float4 &v)
+{
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  const v4f x = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
+  v = make_float4(x.x, x.y, x.z, x.w);
+}
+__device__ __forceinline__ void buffer_load_cell(BufferRsrc r, unsigned off, unsigned &v)
+{
+  v = __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
+}
+#else
+typedef int BufferRsrc;
+__device__ inline BufferRsrc make_rsrc(const void *, unsigned) { return 0; }
+__device__ inline void buffer_load_cell(BufferRsrc, unsigned, float4 &v) { v = float4(); }
+__device__ inline void buffer_load_cell(BufferRsrc, unsigned, unsigned &v) { v = 0u; }
+#endif
+
 __device__ __forceinline__ float comp_of(const float4 &v, int k)
 {
   return k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w));
@@ -110,6 +135,36 @@ __device__ __forceinline__ void gather_tile(const WinoArgs &a, const TileCoord &
     }
 }
 
+// The same gather through buffer addressing, for tensors below 4 GB (WinoArgs::buf_gather).  A cell's byte
+// offset is the lane's first cell's (32 bits, possibly "negative" for a tile that starts in the frame) plus
+// a scalar; rows and columns are tested once each, a cell's test is the AND of two lane masks (scalar
+// instructions), and a cell of the frame is sent to an offset outside the buffer, where the load returns
+// the frame's zero.  Two vector instructions per cell instead of a bounds test, a 64-bit multiply-add and
+// a branch.
+template <int A, typename Cell>
+__device__ __forceinline__ void gather_tile_buf(const WinoArgs &a, const TileCoord &c, int c2, int q, Cell *d)
+{
+  const unsigned pq = a.in_nhwc ? (unsigned)a.ic2 * 4u : 4u;   // cells between neighbouring pixels
+  const unsigned cells = (unsigned)a.n * a.ic2 * a.ih * a.iw * 4u;
+  const BufferRsrc rin = make_rsrc(a.in, cells * (unsigned)sizeof(Cell));
+  const unsigned plane = a.in_nhwc ? (unsigned)c.n * a.ih * a.iw * pq + c2 * 4u
+                                   : ((unsigned)c.n * a.ic2 + c2) * a.ih * a.iw * 4u;
+  const unsigned voff = (plane + (unsigned)(c.h0 * a.iw + c.w0) * pq + q) * (unsigned)sizeof(Cell);
+  bool rv[A], cv[A];
+#pragma unroll
+  for (int i = 0; i < A; ++i) {
+    rv[i] = (unsigned)(c.h0 + i) < (unsigned)a.ih;
+    cv[i] = (unsigned)(c.w0 + i) < (unsigned)a.iw;
+  }
+#pragma unroll
+  for (int i = 0; i < A; ++i)
+#pragma unroll
+    for (int j = 0; j < A; ++j) {
+      const unsigned so = (unsigned)(i * a.iw + j) * pq * (unsigned)sizeof(Cell);   // scalar
+      buffer_load_cell(rin, (rv[i] && cv[j]) ? voff + so : 0xffffff00u, d[A * i + j]);
+    }
+}
+
 }  // namespace
 
 // block: 64 consecutive tiles x 4 channel quads of one 16-channel unit.  Work items are numbered tile
@@ -133,12 +188,21 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   if (t >= a.t) return;
   const TileCoord c = tile_coord<A>(a, t);
   Cell d[AA];
-  gather_tile<A>(a, c, c2, q, d);
+  if (a.buf_gather) gather_tile_buf<A>(a, c, c2, q, d);
+  else gather_tile<A>(a, c, c2, q, d);
   unsigned packed[AA];
+  // mixed: the wave holds interior and rim tiles -- the per-lane, branch-free form of the transform.
+  // Quantization: sat_u8(rne_to_u32(V * (in_S / tin_S) + tin_z)), one rounding in the multiply-add.  The
+  // reference's float -> u32 conversion turns everything below -0.5 (and NaN) into 0xffffffff, which then
+  // saturates to 255; v_cvt_pk_u8_f32 rounds to nearest even and saturates the rest.  watch: the plain
+  // conversion, with the quirk's cases only looked for -- two running integer maxima over the values' bit
+  // patterns, one instruction per value instead of a compare and a select -- and the result says whether
+  // one was seen (never, with a calibrated tinput_quant); the caller then runs the exact form again.
+  auto channels = [&](bool mixed, bool watch) {
+    unsigned seen_u = 0u;
+    int seen_s = 0;
 #pragma unroll
-  for (int k = 0; k < AA; ++k) packed[k] = 0u;
-  // mixed: the wave holds interior and rim tiles -- the per-lane, branch-free form of the transform
-  auto channels = [&](bool mixed) {
+    for (int k = 0; k < AA; ++k) packed[k] = 0u;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       float f[AA], v[AA];
@@ -146,18 +210,44 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
       for (int e = 0; e < AA; ++e) f[e] = comp_of(d[e], k);
       if (mixed) wino::tile_input_lanes<A>(f, v, c.border);
       else wino::tile_input<A>(f, v, false);
+      if (watch) {
+        float y[AA];
 #pragma unroll
-      for (int e = 0; e < AA; ++e) {
-        // sat_u8(rne_to_u32(V * (in_S / tin_S) + tin_z)), one rounding in the multiply-add.  The
-        // reference's float -> u32 conversion turns everything below -0.5 (and NaN) into 0xffffffff,
-        // which then saturates to 255; v_cvt_pk_u8_f32 rounds to nearest even and saturates the rest.
-        const float y = __builtin_fmaf(v[e], a.mrepS, a.mz);
-        packed[e] = __builtin_amdgcn_cvt_pk_u8_f32(y >= -0.5f ? y : 300.0f, k, packed[e]);
+        for (int e = 0; e < AA; ++e) {
+          y[e] = __builtin_fmaf(v[e], a.mrepS, a.mz);
+          packed[e] = __builtin_amdgcn_cvt_pk_u8_f32(y[e], k, packed[e]);
+        }
+        // bit patterns above 0xbf000000 unsigned: below -0.5, or a negative NaN; above 0x7f800000 signed: a
+        // positive NaN
+#pragma unroll
+        for (int e = 0; e + 1 < AA; e += 2) {
+          const unsigned b0 = __float_as_uint(y[e]), b1 = __float_as_uint(y[e + 1]);
+          seen_u = max(seen_u, max(b0, b1));
+          seen_s = max(seen_s, max((int)b0, (int)b1));
+        }
+        if (AA & 1) {
+          const unsigned b = __float_as_uint(y[AA - 1]);
+          seen_u = max(seen_u, b);
+          seen_s = max(seen_s, (int)b);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < AA; ++e) {
+          const float y = __builtin_fmaf(v[e], a.mrepS, a.mz);
+          packed[e] = __builtin_amdgcn_cvt_pk_u8_f32(y >= -0.5f ? y : 300.0f, k, packed[e]);
+        }
       }
     }
+    return seen_u > 0xbf000000u || seen_s > 0x7f800000;
   };
-  if (__ballot(c.border) != 0) channels(true);   // wave-uniform
-  else channels(false);
+  const bool mixed = __ballot(c.border) != 0;   // wave-uniform
+  bool again;
+  if (mixed) again = channels(true, true);
+  else again = channels(false, true);
+  if (__ballot(again) != 0) {
+    if (mixed) channels(true, false);
+    else channels(false, false);
+  }
   unsigned *dst = reinterpret_cast<unsigned *>(a.tin) +
       (a.tin_blocked ? (((size_t)(t >> 5) * AA * a.ic2 + c2) * 32 + (t & 31)) * 4 + q : ((size_t)c2 * a.t + t) * 4 + q);
   const size_t pos_stride = a.tin_blocked ? (size_t)a.ic2 * 32 * 4 : (size_t)a.ic2 * a.t * 4;
@@ -545,6 +635,11 @@ hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s, LaunchPlan
     return plan_relaunch(*plan, s);
   }
   WinoArgs a = a0;
+  {
+    const unsigned long long bytes = (unsigned long long)a.n * a.ic2 * a.ih * a.iw * 16 * (a.in_u8 ? 1 : 4);
+    const char *env = getenv("EHIP_WINO_BUF_GATHER");
+    a.buf_gather = bytes <= 0xffffff00ull && !(env && env[0] == '0');
+  }
   a.nblocks = (a.t + 63) / 64;
   a.items_per_xcd = (int)(((long long)a.nblocks * a.ic2 + 7) / 8);
   dim3 grid(8 * a.items_per_xcd, 1);

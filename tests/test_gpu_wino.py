@@ -66,6 +66,33 @@ def test_wino_pipeline(n, ic, oc, hw, tile, monkeypatch):
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d" % int((got != exp).sum())
 
 
+@pytest.mark.parametrize("tile", [6, 4, 5])
+@pytest.mark.parametrize("buf_gather", ["0", "1"])
+def test_wino_tinput_under_range_and_both_gathers(tile, buf_gather, monkeypatch):
+    """A tinput zero point too small for the data: transformed values below -0.5 end as code 255
+    (src/elx_conv_wino_trans_input.cpp:643-650 converts through an unsigned integer), which the input
+    transform handles in a second pass of the wave; and the gather with plain loads (what a tensor of 4 GB
+    or more takes) next to the one with buffer loads."""
+    import torch
+    monkeypatch.setenv("EHIP_WINO_FUSED", "0")
+    monkeypatch.setenv("EHIP_WINO_BUF_GATHER", buf_gather)
+    E, p, d, xb, wb, bias = make_wino(2, 32, 32, 13, seed=77 + tile, tile=tile)
+    mn, mx = ol.wino_tinput_range(p, xb)
+    s_t = float((f32(mx) - f32(mn)) / f32(255.0))
+    z_t = float(-f32(mn) / f32(s_t)) * 0.5      # half of what the range needs
+    p.tin_scale, p.tin_z = s_t, z_t
+    d.tinput_scale, d.tinput_z = s_t, z_t
+    tin = ol.wino_trans_input(p, xb)
+    assert (tin == 255).sum() > 300 and (tin == 0).sum() < tin.size // 2
+    conv = E.Conv(d)
+    d_b = dev(bias)
+    d_out = torch.zeros((2, 2, 13, 13, 16), dtype=torch.float32, device="cuda")
+    conv.execute(d_out, dev(xb), dev(wb), d_b)
+    torch.cuda.synchronize()
+    g_tin = conv.query(E.Q_TINPUT_U8).reshape(tin.shape)
+    assert np.array_equal(g_tin, tin), "u8 transformed input differs at %d cells" % int((g_tin != tin).sum())
+
+
 @pytest.mark.parametrize("n,ic,oc,hw", [(2, 32, 32, 10), (1, 64, 48, 12), (3, 16, 80, 7), (1, 32, 144, 28),
                                         (2, 256, 64, 9), (1, 272, 32, 6)])
 def test_wino_fused_gemm_and_output_transform(n, ic, oc, hw):
