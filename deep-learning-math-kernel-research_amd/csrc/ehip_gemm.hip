@@ -416,13 +416,24 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
   // per tile they would cost the vector-memory path more than the activations do)
   OcConsts k0;
   load_consts(k0, a.ep, cidx);
+  // Lean epilogue (a.lean, decided by the launcher: u8 / s8 blocked output, ReLU, per-channel shift): these
+  // layers produce an output value per 32-128 multiply-adds, so the epilogue's instructions per value, not
+  // the multiplies, are what a tile costs; the lean form takes 3-4 of them where the general one takes ~10.
+  // Its accumulators start from the compensation instead of zero.
+  LeanConsts lk[1];
+  v16i acc0;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc0[v] = 0;
+  if (a.lean) {
+    load_lean_consts(lk[0], a.ep, cidx);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc0[v] = k0.comp[v >> 2][v & 3];
+  }
   v4i *xlds = ((a.ep.out_type == EHIP_F32 || a.ep.out_type == EHIP_S32) && !a.out_nhwc) ? xpatch + wave * 256 : nullptr;
   for (; tile < ntiles; tile += tstep) {
     v16i acc[1][TNW];
 #pragma unroll
-    for (int nt = 0; nt < TNW; ++nt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[0][nt][v] = 0;
+    for (int nt = 0; nt < TNW; ++nt) acc[0][nt] = acc0;
     v4i bcur[TNW][KS];
 #pragma unroll
     for (int nt = 0; nt < TNW; ++nt)
@@ -438,6 +449,16 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
         acc[0][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ks], bcur[nt][ks], acc[0][nt], 0, 0, 0);
     size_t pix[TNW], pixT[TNW][2];
     bool pvalid[TNW], validT[TNW][2];
+    if (a.lean) {   // blocked output: the lane's cell = its pixel in 16-channel block (oc0 / 16) + lh
+      uint8_t *cell[TNW];
+#pragma unroll
+      for (int nt = 0; nt < TNW; ++nt) {
+        const size_t px = pixel_offset((tile * TNW + nt) * 32 + l32, pvalid[nt]);
+        cell[nt] = static_cast<uint8_t *>(a.out) + px + ((size_t)(oc0 >> 4) + lh) * a.ohw * 16;
+      }
+      lean_store<1, TNW>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
+      continue;
+    }
 #pragma unroll
     for (int nt = 0; nt < TNW; ++nt) {
       const int p0 = (tile * TNW + nt) * 32;
@@ -447,6 +468,123 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
     }
     epilogue_wave<1, TNW>(a.ep, acc, k0, cidx, oc0 + 16 * lh, pix, pvalid, oc_real,
                           a.out_nhwc ? (size_t)16 : (size_t)a.ohw * 16, a.out, xlds, pixT, validT);
+  }
+}
+
+// The same walk for the lean epilogue's cases (u8 / s8 blocked output, ReLU, per-channel shift), with OCW
+// tiles of 32 output channels per wave instead of one.  A layer like 64 -> 256 at 56 x 56 writes four
+// times the bytes it reads; with one channel tile per wave every activation cell is pulled from L2 once
+// per channel tile (eight times), which then outweighs the output.  Here a wave keeps the weights of all
+// its OCW tiles in registers (OCW x KS <= 8 operands), reads a pixel tile once and produces OCW x 32
+// channels from it.  Scale, shift and the accumulators' start values (the u8 -> s8 compensation) of the
+// wave's channels sit in a wave-private piece of LDS -- in registers they would take 48 per tile -- and every
+// lane of a half-wave reads the same 16 bytes of them (a broadcast).
+template <int KS, int OCW>
+__global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(GemmArgs a)
+{
+  __shared__ float4 cst_lds[4 * OCW * 24];   // [wave][tile][scale | shift | compensation][8 cells of 4 channels]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int wo = wave % a.sk_wo, wp = wave / a.sk_wo, wpn = 4 / a.sk_wo;
+  const int oc0 = (blockIdx.y * a.sk_wo + wo) * OCW * 32;
+  const int oc_real = a.oc2 * 16;
+  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  const long long unit_stride = (long long)a.ihw * 16;
+
+  v4i wreg[OCW][KS];
+#pragma unroll
+  for (int ot = 0; ot < OCW; ++ot)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      wreg[ot][ks] = *reinterpret_cast<const v4i *>(a.w + ((long long)(2 * ks + lh) * a.ocpp + oc0 + 32 * ot + l32) * 16);
+  float4 *cst = cst_lds + wave * (OCW * 24);
+  for (int i = lane; i < OCW * 24; i += 64) {
+    const int ot = i / 24, r = i - 24 * ot, arr = r >> 3, c = r & 7;
+    const float *src = arr == 0 ? a.ep.scale : (arr == 1 ? a.ep.shift : reinterpret_cast<const float *>(a.ep.comp));
+    cst[i] = *reinterpret_cast<const float4 *>(src + oc0 + 32 * ot + 4 * c);
+  }
+
+  auto input_pixel = [&](int gp) -> long long {
+    gp = gp < a.p_total ? gp : a.p_total - 1;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic);
+    const int r = gp - n * a.ohw;
+    long long sp;
+    if (dense) {
+      sp = r;
+    } else {
+      const int oh = fastdiv(r, a.ow, a.ow_magic);
+      sp = (long long)(oh * a.stride_h) * a.iw + (r - oh * a.ow) * a.stride_w;
+    }
+    return a.in_nhwc ? ((long long)n * a.ihw + sp) * a.ic2 * 16 : ((long long)n * a.ic2 * a.ihw + sp) * 16;
+  };
+  int ucl[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ucl[ks] = 2 * ks + lh < a.ic2 ? 2 * ks + lh : a.ic2 - 1;
+  const long long ustride = a.in_nhwc ? 16 : unit_stride;
+
+  const int ntiles = (a.p_total + 31) / 32;
+  const int tstep = wpn * gridDim.x;
+  int tile = wpn * blockIdx.x + wp;
+  v4i breg[KS];
+  auto load_b = [&](int t) {
+    const uint8_t *src = a.in + input_pixel(t * 32 + l32);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) breg[ks] = *reinterpret_cast<const v4i *>(src + (long long)ucl[ks] * ustride);
+  };
+  if (tile < ntiles) load_b(tile);
+  __builtin_amdgcn_wave_barrier();   // the constants are the wave's own: its LDS writes are done before its reads
+  for (; tile < ntiles; tile += tstep) {
+    v4i bcur[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) bcur[ks] = breg[ks] ^ (int)0x80808080;
+    load_b(tile + tstep < ntiles ? tile + tstep : tile);
+    // the lane's cell of 16-channel block (oc0 / 16) + lh
+    const int gp = tile * 32 + l32;
+    bool pvalid[1] = {gp < a.p_total};
+    const int gpc = pvalid[0] ? gp : 0;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
+    uint8_t *const cell0 = static_cast<uint8_t *>(a.out) +
+        (((size_t)n * a.oc2 + (oc0 >> 4) + lh) * a.ohw + (gpc - n * a.ohw)) * 16;
+    // The multiplies of tile ot + 1 are issued before the epilogue of tile ot and run behind it; the
+    // scheduling barriers keep the compiler from pulling all OCW tiles' constants and accumulators up front
+    // (it then runs out of registers).
+    v16i acc2[2];
+    auto multiply = [&](int ot) {
+      const float4 *k = cst + ot * 24 + 4 * lh;
+      v16i x;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 c = k[16 + q];
+        x[4 * q + 0] = __float_as_int(c.x);
+        x[4 * q + 1] = __float_as_int(c.y);
+        x[4 * q + 2] = __float_as_int(c.z);
+        x[4 * q + 3] = __float_as_int(c.w);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) x = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ot][ks], bcur[ks], x, 0, 0, 0);
+      acc2[ot & 1] = x;
+    };
+    multiply(0);
+#pragma unroll
+    for (int ot = 0; ot < OCW; ++ot) {
+      if (ot + 1 < OCW) multiply(ot + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      const float4 *k = cst + ot * 24 + 4 * lh;
+      LeanConsts lk[1];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        lk[0].sc[q] = k[q];
+        lk[0].sh[q] = k[8 + q];
+      }
+      v16i acc[1][1];
+      acc[0][0] = acc2[ot & 1];
+      uint8_t *cell[1] = {cell0 + (size_t)ot * 2 * a.ohw * 16};
+      lean_store<1, 1>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 32 * ot + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 }
 
@@ -540,6 +678,8 @@ bool gemm_smallk_applies(int ic2, int taps, int nbatch)
 hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr)
 {
   GemmArgs a = a0;
+  a.lean = lean_mode(a.ep, a.out_nhwc != 0);
+  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   const int ks = a.ic2 <= 2 ? 1 : (a.ic2 <= 4 ? 2 : 4);
   const int oc_tiles = (a.oc2 * 16 + 31) / 32;
   // one tile of 32 channels per wave (its constants then stay in registers) x two tiles of 32 pixels
@@ -557,6 +697,31 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
   const int cap = (wgs + ny - 1) / ny;
   if (nx > cap) nx = cap;
   void (*kernel)(GemmArgs) = ks == 1 ? smallk_kernel<1>(tnw) : (ks == 2 ? smallk_kernel<2>(tnw) : smallk_kernel<4>(tnw));
+  // lean epilogue and blocked activations: several channel tiles per wave.  Measured at N = 64 (64 -> 256 and
+  // 64 -> 128 at 56 x 56, 128 -> 512 at 28 x 28, 128 -> 128 at 56 x 56, 32 -> 64 at 112 x 112): four tiles per
+  // wave up to 64 input channels, two above (more weights in registers cost a resident workgroup), 20-25 %
+  // faster than one; eight tiles lose again.
+  int ocw = ks == 4 ? 2 : 4;
+  while (ocw > 1 && ocw > oc_tiles) ocw >>= 1;
+  if (const char *env = getenv("EHIP_SMALLK_OCW")) { const int e = atoi(env); if (e == 1 || e == 2 || (e == 4 && ks < 4)) ocw = e; }
+  if (a.lean && !a.in_nhwc && ocw > 1) {
+    const int groups2 = (oc_tiles + ocw - 1) / ocw;
+    a.sk_wo = groups2 >= 4 ? 4 : (groups2 >= 2 ? 2 : 1);
+    const int ny2 = (groups2 + a.sk_wo - 1) / a.sk_wo;
+    const int wpn2 = 4 / a.sk_wo;
+    const int ntiles2 = (a.p_total + 31) / 32;
+    int nx2 = (ntiles2 + wpn2 - 1) / wpn2;
+    // one resident set: four workgroups per CU with the weights of up to 32 channels per lane, else three
+    int wgs2 = ks == 1 ? 1024 : 768;
+    if (const char *env = getenv("EHIP_SMALLK_WGS")) wgs2 = atoi(env) > 0 ? atoi(env) : wgs2;
+    const int cap2 = (wgs2 + ny2 - 1) / ny2;
+    if (nx2 > cap2) nx2 = cap2;
+    void (*lk)(GemmArgs) = nullptr;
+    if (ks == 1) lk = ocw == 4 ? k_gemm_smallk_lean<1, 4> : k_gemm_smallk_lean<1, 2>;
+    else if (ks == 2) lk = ocw == 4 ? k_gemm_smallk_lean<2, 4> : k_gemm_smallk_lean<2, 2>;
+    else lk = k_gemm_smallk_lean<4, 2>;
+    return plan_launch(plan, lk, dim3(nx2, ny2), dim3(kBlock), 0, a, s);
+  }
   return plan_launch(plan, kernel, dim3(nx, ny), dim3(kBlock), 0, a, s);
 }
 

@@ -109,6 +109,18 @@ def test_conv1x1_few_input_channels(out_type, n, ic, oc, hw, stride, nhwc):
     assert res["conv"].kernel_name == "k_gemm_smallk_u8s8"
 
 
+@pytest.mark.parametrize("out_type,with_sum", [(ol.U8, False), (ol.S8, True), (ol.S8, False)])
+@pytest.mark.parametrize("n,ic,oc,hw,stride", [(2, 32, 256, 12, 1), (1, 32, 128, 17, 1), (2, 64, 128, 11, 1), (2, 64, 256, 14, 1),
+                                               (1, 128, 144, 13, 1), (3, 128, 64, 9, 1), (2, 64, 80, 10, 1), (2, 128, 512, 12, 2),
+                                               (1, 48, 272, 15, 1)])
+def test_conv1x1_few_input_channels_several_channel_tiles_per_wave(out_type, with_sum, n, ic, oc, hw, stride):
+    """u8 / s8 blocked output with ReLU: a wave keeps the weights of 2 or 4 tiles of 32 output channels and
+    reads every pixel tile once; channel counts that leave the last wave group partly or wholly past the real
+    channels included"""
+    res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, seed=510 + ic + oc, with_sum=with_sum))
+    assert res["conv"].kernel_name == "k_gemm_smallk_u8s8"
+
+
 def test_conv1x1_few_input_channels_can_be_switched_off(monkeypatch):
     monkeypatch.setenv("EHIP_GEMM_SMALLK", "0")
     res = run_and_compare(Layer(2, 64, 96, 9, out_type=ol.U8, seed=177))
