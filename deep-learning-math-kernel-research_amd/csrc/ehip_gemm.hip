@@ -282,7 +282,9 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
   }
   TRACE_POINT(6);
 
-  if (a.lean) {   // u8 / s8 with ReLU bounds, blocked output, per-channel shift: no output-type switch
+  if (a.lean) {   // u8 / s8 with ReLU bounds, per-channel shift: no output-type switch
+    // the lane's 16 bytes: its pixel's cell in 16-channel block (oc0 + mw0) / 16 + lh, or (nhwc) channels
+    // oc0 + mw0 + 16 lh .. + 15 of its pixel's vector; the next 32-channel tile is two blocks / 32 bytes on
     uint8_t *cell[TN];
     bool pv[TN];
 #pragma unroll
@@ -290,12 +292,17 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
       const int gp = pix0 + pw0 + nt * 32 + l32;
       pv[nt] = gp < a.p_total;
       const int gpc = pv[nt] ? gp : 0;
-      const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
-      const int r = gpc - n * a.ohw;
-      cell[nt] = static_cast<uint8_t *>(a.out) + (size_t)b * a.out_batch_stride +
-          (((size_t)n * a.oc2 + ((oc0 + mw0) >> 4) + lh) * a.ohw + r) * 16;
+      if (a.out_nhwc) {
+        cell[nt] = static_cast<uint8_t *>(a.out) + (size_t)gpc * oc_real + (oc0 + mw0 + 16 * lh);
+      } else {
+        const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
+        const int r = gpc - n * a.ohw;
+        cell[nt] = static_cast<uint8_t *>(a.out) + (size_t)b * a.out_batch_stride +
+            (((size_t)n * a.oc2 + ((oc0 + mw0) >> 4) + lh) * a.ohw + r) * 16;
+      }
     }
-    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + mw0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
+    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + mw0 + 16 * lh, oc_real,
+                       a.out_nhwc ? (size_t)32 : (size_t)2 * a.ohw * 16);
     TRACE_POINT(15);
     return;
   }
@@ -416,7 +423,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
   // per tile they would cost the vector-memory path more than the activations do)
   OcConsts k0;
   load_consts(k0, a.ep, cidx);
-  // Lean epilogue (a.lean, decided by the launcher: u8 / s8 blocked output, ReLU, per-channel shift): these
+  // Lean epilogue (a.lean, decided by the launcher: u8 / s8 output, ReLU, per-channel shift): these
   // layers produce an output value per 32-128 multiply-adds, so the epilogue's instructions per value, not
   // the multiplies, are what a tile costs; the lean form takes 3-4 of them where the general one takes ~10.
   // Its accumulators start from the compensation instead of zero.
@@ -449,14 +456,16 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
         acc[0][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ks], bcur[nt][ks], acc[0][nt], 0, 0, 0);
     size_t pix[TNW], pixT[TNW][2];
     bool pvalid[TNW], validT[TNW][2];
-    if (a.lean) {   // blocked output: the lane's cell = its pixel in 16-channel block (oc0 / 16) + lh
+    if (a.lean) {   // the lane's 16 bytes: its pixel in 16-channel block (oc0 / 16) + lh, or of its nhwc vector
       uint8_t *cell[TNW];
 #pragma unroll
       for (int nt = 0; nt < TNW; ++nt) {
         const size_t px = pixel_offset((tile * TNW + nt) * 32 + l32, pvalid[nt]);
-        cell[nt] = static_cast<uint8_t *>(a.out) + px + ((size_t)(oc0 >> 4) + lh) * a.ohw * 16;
+        cell[nt] = static_cast<uint8_t *>(a.out) + px +
+            (a.out_nhwc ? (size_t)(oc0 + 16 * lh) : ((size_t)(oc0 >> 4) + lh) * a.ohw * 16);
       }
-      lean_store<1, TNW>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
+      lean_store<1, TNW>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real,
+                         a.out_nhwc ? (size_t)32 : (size_t)2 * a.ohw * 16);
       continue;
     }
 #pragma unroll
@@ -471,7 +480,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
   }
 }
 
-// The same walk for the lean epilogue's cases (u8 / s8 blocked output, ReLU, per-channel shift), with OCW
+// The same walk for the lean epilogue's cases (u8 / s8 output, ReLU, per-channel shift), with OCW
 // tiles of 32 output channels per wave instead of one.  A layer like 64 -> 256 at 56 x 56 writes four
 // times the bytes it reads; with one channel tile per wave every activation cell is pulled from L2 once
 // per channel tile (eight times), which then outweighs the output.  Here a wave keeps the weights of all
@@ -547,7 +556,9 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(GemmArgs a)
     const int gpc = pvalid[0] ? gp : 0;
     const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
     uint8_t *const cell0 = static_cast<uint8_t *>(a.out) +
-        (((size_t)n * a.oc2 + (oc0 >> 4) + lh) * a.ohw + (gpc - n * a.ohw)) * 16;
+        (a.out_nhwc ? (size_t)gpc * oc_real + (oc0 + 16 * lh)
+                    : (((size_t)n * a.oc2 + (oc0 >> 4) + lh) * a.ohw + (gpc - n * a.ohw)) * 16);
+    const size_t tile_stride = a.out_nhwc ? (size_t)32 : (size_t)2 * a.ohw * 16;
     // The multiplies of tile ot + 1 are issued before the epilogue of tile ot and run behind it; the
     // scheduling barriers keep the compiler from pulling all OCW tiles' constants and accumulators up front
     // (it then runs out of registers).
@@ -581,8 +592,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(GemmArgs a)
       }
       v16i acc[1][1];
       acc[0][0] = acc2[ot & 1];
-      uint8_t *cell[1] = {cell0 + (size_t)ot * 2 * a.ohw * 16};
-      lean_store<1, 1>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 32 * ot + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
+      uint8_t *cell[1] = {cell0 + (size_t)ot * tile_stride};
+      lean_store<1, 1>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 32 * ot + 16 * lh, oc_real, tile_stride);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -678,7 +689,7 @@ bool gemm_smallk_applies(int ic2, int taps, int nbatch)
 hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr)
 {
   GemmArgs a = a0;
-  a.lean = lean_mode(a.ep, a.out_nhwc != 0);
+  a.lean = lean_mode(a.ep, false);   // blocked and nhwc output alike
   if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   const int ks = a.ic2 <= 2 ? 1 : (a.ic2 <= 4 ? 2 : 4);
   const int oc_tiles = (a.oc2 * 16 + 31) / 32;
@@ -704,7 +715,7 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
   int ocw = ks == 4 ? 2 : 4;
   while (ocw > 1 && ocw > oc_tiles) ocw >>= 1;
   if (const char *env = getenv("EHIP_SMALLK_OCW")) { const int e = atoi(env); if (e == 1 || e == 2 || (e == 4 && ks < 4)) ocw = e; }
-  if (a.lean && !a.in_nhwc && ocw > 1) {
+  if (a.lean && ocw > 1) {
     const int groups2 = (oc_tiles + ocw - 1) / ocw;
     a.sk_wo = groups2 >= 4 ? 4 : (groups2 >= 2 ? 2 : 1);
     const int ny2 = (groups2 + a.sk_wo - 1) / a.sk_wo;
@@ -739,7 +750,7 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   }
   const Variant &k = kVariants[variant];
   GemmArgs a = a0;
-  a.lean = lean_mode(a.ep, a.out_nhwc != 0);
+  a.lean = lean_mode(a.ep, false);   // blocked and nhwc output alike
   if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
