@@ -367,7 +367,15 @@ int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
     // per CU that hide each other's load, flip and epilogue phases, 8.6 / 17.5 us; 128 x 128 10.8 / 19.4 us;
     // the 256-channel tiles (a wave owns 64 channels, twice the registers) 9.0-14.4 / 22.5-25.9 us.
     static const double pref[] = {0.95, 1.10, 0.70, 0.85};
-    const double score = util * (0.5 + 0.5 * fill) * pref[v] * (per_cu >= 2 ? 1.0 : 0.9);
+    double score = util * (0.5 + 0.5 * fill) * pref[v] * (per_cu >= 2 ? 1.0 : 0.9);
+    // 1024 input channels, whole 256-channel tiles, enough of them for three quarters of the CUs: the
+    // 256 x 64 tile pulls every pixel tile through L2 half as often (1024 -> 256 at 14 x 14, N = 64: 8.1 against
+    // 9.0 us, 1024 -> 512: 12.2 against 15.4 us); with 512 channels its weights-in-registers form needs too
+    // many registers and loses (512 -> 1024 stride 2: 23.9 against 15.2 us)
+    if (v == 3 && a.units_pad == 64 && oc % 256 == 0 && wgs >= 192) score = 2.0;
+    // fewer than 3/4 of the tile's channels real (64 output channels): the general kernel's 64-channel tiles
+    // win (256 -> 64 at 56 x 56, N = 64: 13.4 against 17.1 us)
+    if (util < 0.75) continue;
     if (score > best_score) { best_score = score; best = v; }
   }
   return best;
