@@ -207,6 +207,30 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
     validT[0][1] = p0 + (lane >> 2) + 16 < npix;
     pixT[0][0] = out0 + (size_t)(p0 + (lane >> 2)) * px_stride;
     pixT[0][1] = pixT[0][0] + 16 * px_stride;
+    if (a.lean) {
+      // Lean epilogue (u8 / s8 output, ReLU: 3-4 instructions per value instead of ~10 -- with 16-112
+      // multiply-adds per output value the epilogue is most of a tile's instructions).  The scale is the
+      // lane's channels'; the shift row is the one of the pixel's border class where the layer has classes.
+      LeanConsts lk[1];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        lk[0].sc[q] = k0.sc[q];
+        lk[0].sh[q] = k0.sh[q];
+      }
+      if (a.tab_lds) {
+        const float *row = lds_shift + (lds_cls_h[ro] + lds_cls_w[ox]) * (a.wo * 32) + wo * 32 + 16 * lh;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) lk[0].sh[q] = *reinterpret_cast<const float4 *>(row + 4 * q);
+      } else if (a.ep.shift_tab) {
+        const float *row = a.ep.shift_tab + (size_t)(a.cls_h[oh0 + ro] * a.ncls_w + a.cls_w[ox]) * a.ep.tab_stride + cidx;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) lk[0].sh[q] = *reinterpret_cast<const float4 *>(row + 4 * q);
+      }
+      uint8_t *cell[1] = {static_cast<uint8_t *>(a.out) + pix[0] +
+                          (a.out_nhwc ? (size_t)(oc0 + 16 * lh) : (size_t)((oc0 >> 4) + lh) * block_stride)};
+      lean_store<1, 1>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, 0);
+      continue;
+    }
     if (a.tab_lds) {
       cls[0] = lds_cls_h[ro] + lds_cls_w[ox];
       epilogue_wave<1, 1, true, true>(ep_lds, acc, k0, wo * 32 + 16 * lh, oc0 + 16 * lh, pix, pvalid, oc_real,
@@ -246,6 +270,14 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
     plan->args.in = a.in;
     plan->args.out = a.out;
     return plan_relaunch(*plan, s);
+  }
+  {
+    // lean_mode() but for the per-pixel shift rows, which this kernel's lean path reads itself
+    Epilogue e = a.ep;
+    e.shift_tab = nullptr;
+    a.lean = lean_mode(e, false);
+    if (a.ep.with_sum) a.lean = 0;
+    if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   }
   a.ppc = 16 / a.ic;
   a.nu = (a.kw + a.ppc - 1) / a.ppc;

@@ -225,6 +225,7 @@ struct FewChArgs {
   int rows, strips;     // output rows per workgroup, workgroups per image
   int nrows_in, lrow;   // staged input rows and their pitch in bytes (a multiple of 4)
   int wo;               // waves of a workgroup along the channels (1, 2, 4)
+  int lean;             // lean_mode() of the epilogue, per-pixel shift rows allowed (0 = general epilogue)
   unsigned ow_magic, iw_magic, lrow4_magic;
 };
 bool conv_fewch_applies(int ic, int kh, int kw);
