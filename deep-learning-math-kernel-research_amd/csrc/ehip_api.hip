@@ -616,6 +616,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     }
     a.trace = trace_buffer();
     HIP_TRY(launch_gemm(a, 1, c->variant, s, &c->plan_gemm));
+    if (c->plan_gemm.name) c->kernel_name = c->plan_gemm.name;   // the launcher's choice depends on the epilogue
     break;
   }
   case FAM_CONV_FEWCH: {

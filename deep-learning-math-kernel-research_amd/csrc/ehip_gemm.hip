@@ -731,6 +731,12 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
     if (ks == 1) lk = ocw == 4 ? k_gemm_smallk_lean<1, 4> : k_gemm_smallk_lean<1, 2>;
     else if (ks == 2) lk = ocw == 4 ? k_gemm_smallk_lean<2, 4> : k_gemm_smallk_lean<2, 2>;
     else lk = k_gemm_smallk_lean<4, 2>;
+    if (plan) {
+      static const char *const names[3][2] = {{"k_gemm_smallk_lean<1,2>", "k_gemm_smallk_lean<1,4>"},
+                                              {"k_gemm_smallk_lean<2,2>", "k_gemm_smallk_lean<2,4>"},
+                                              {"k_gemm_smallk_lean<4,2>", "k_gemm_smallk_lean<4,2>"}};
+      plan->name = names[ks == 1 ? 0 : (ks == 2 ? 1 : 2)][ocw == 4 ? 1 : 0];
+    }
     return plan_launch(plan, lk, dim3(nx2, ny2), dim3(kBlock), 0, a, s);
   }
   return plan_launch(plan, kernel, dim3(nx, ny), dim3(kBlock), 0, a, s);

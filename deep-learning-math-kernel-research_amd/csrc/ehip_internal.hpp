@@ -146,6 +146,7 @@ struct LaunchPlan {
   dim3 grid, block;
   unsigned lds = 0;
   Args args;
+  const char *name = nullptr;   // set by a launcher whose choice of kernel the handle cannot know beforehand
 };
 template <typename Args>
 inline hipError_t plan_launch(LaunchPlan<Args> *plan, void (*kernel)(Args), dim3 grid, dim3 block, size_t lds, const Args &a,

@@ -106,7 +106,7 @@ def test_conv1x1_few_input_channels(out_type, n, ic, oc, hw, stride, nhwc):
         pytest.skip("nhwc needs whole channel blocks")
     res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, seed=170 + ic + oc,
                                 with_sum=out_type in (ol.U8, ol.S8), in_nhwc=nhwc, out_nhwc=nhwc))
-    assert res["conv"].kernel_name == "k_gemm_smallk_u8s8"
+    assert res["conv"].kernel_name.startswith("k_gemm_smallk")
 
 
 @pytest.mark.parametrize("out_type,with_sum", [(ol.U8, False), (ol.S8, True), (ol.S8, False)])
@@ -118,7 +118,7 @@ def test_conv1x1_few_input_channels_several_channel_tiles_per_wave(out_type, wit
     reads every pixel tile once; channel counts that leave the last wave group partly or wholly past the real
     channels included"""
     res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, seed=510 + ic + oc, with_sum=with_sum))
-    assert res["conv"].kernel_name == "k_gemm_smallk_u8s8"
+    assert res["conv"].kernel_name.startswith("k_gemm_smallk_lean")
 
 
 def test_conv1x1_few_input_channels_can_be_switched_off(monkeypatch):
