@@ -63,9 +63,10 @@ constexpr int conv3x3v_unit_stride(int cells, int tn, bool sp)
   return r * tn;
 }
 
-template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS, bool SP>
+template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS, bool SP, bool SL>
 __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
 {
+  static_assert(!SL || (PAIRS > 0 && !SP && TM == 1 && TN == 4), "split last pair: straight-line form, 32 channels x 4 tiles");
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
   constexpr int STRIDE = conv3x3v_unit_stride(CT * NPASS, TN, SP);   // LDS cells per unit
@@ -338,11 +339,90 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
     // straight line over the 9 * PAIRS taps, each one's pixel operands read during the tap before
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt) read_b(0, 0, 0, nt);
+    constexpr int LAST0 = 9 * (PAIRS - 1);   // first tap of the last channel pair
 #pragma unroll
-    for (int st = 0; st < 9 * PAIRS; ++st) {
-      const int pl = st / 9, tap = st % 9;
-      if (st == 9 * (PAIRS - 1)) load_epilogue_consts();
-      tap_mfmas(st & 1, tap, pl, pl == PAIRS - 1, st + 1 < 9 * PAIRS ? (st + 1) / 9 : -1, (st + 1) % 9);
+    for (int st = 0; st < LAST0; ++st) tap_mfmas(st & 1, st % 9, st / 9, false, (st + 1) / 9, (st + 1) % 9);
+    load_epilogue_consts();
+    // Split last pair (a wave of 32 channels x four pixel tiles, lean epilogue without the sum): with one
+    // workgroup per CU nothing hides the epilogue -- a convert, a multiply-add and a byte pack per value, a
+    // sixth of the kernel's time for 128 input channels.  So the last channel pair is multiplied tile pair by
+    // tile pair instead of tap by tap: tiles 0 and 1 through all nine taps (their accumulators alternate, so
+    // no MFMA waits for the one before), then tiles 2 and 3, and behind each of THEIR eighteen MFMAs goes a
+    // piece of the epilogue of tiles 0 and 1.  All nine weight operands of the last pair are in registers by then.
+    // (SL: a kernel of its own, launched only for such epilogues.)
+    if constexpr (SL) {
+      constexpr int P0 = LAST0 & 1;   // operand buffer of the last pair's first tap
+      uint8_t *outb = static_cast<uint8_t *>(a.out) + ((size_t)n * a.oc2 + ((oc0 + mw0) >> 4)) * ohw * 16;
+      uint8_t *cell[TN];
+      bool pv[TN];
+      auto locate = [&](int nt) {
+        const int v = v0 + pw0 + nt * 32 + l32;
+        const int r = fastdiv(v, VW, a.vw_magic);
+        const int c = v - r * VW;
+        pv[nt] = r < a.oh && c < a.ow && (int)cidx < oc_real;
+        cell[nt] = outb + (unsigned)(lh * ohw + (pv[nt] ? r * a.ow + c : 0)) * 16u;
+      };
+      const bool s8 = a.ep.out_type == EHIP_S8;
+      const float hi = s8 ? __builtin_fminf(a.ep.hi, 127.0f) : a.ep.hi;
+      auto last_pair = [&](auto clampc) {
+        constexpr bool CLAMP = decltype(clampc)::value;
+        auto pack = [&](int tile, int q) -> int {   // four values of tile `tile`: arithmetic of lean_store_typed
+          const float sc[4] = {lk[0].sc[q].x, lk[0].sc[q].y, lk[0].sc[q].z, lk[0].sc[q].w};
+          const float sh[4] = {lk[0].sh[q].x, lk[0].sh[q].y, lk[0].sh[q].z, lk[0].sh[q].w};
+          unsigned pk = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float f = __builtin_fmaf((float)acc[0][tile][4 * q + j], sc[j], sh[j]);
+            if (CLAMP) f = __builtin_amdgcn_fmed3f(f, a.ep.lo, hi);
+            pk = __builtin_amdgcn_cvt_pk_u8_f32(f, j, pk);
+          }
+          return (int)pk;
+        };
+        // tiles 0 and 1; where they go is worked out behind the first MFMAs
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap)
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            const int par = (P0 + tap) & 1;
+            acc[0][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[tap][0], bq[par][nt], acc[0][nt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (tap < 8) read_b(par ^ 1, PAIRS - 1, tap + 1, nt);
+            if (2 * tap + nt < TN) locate(2 * tap + nt);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        // tiles 2 and 3, with the epilogue of tiles 0 and 1 in their shadow
+        v4i outv[2];
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap)
+#pragma unroll
+          for (int nt = 2; nt < 4; ++nt) {
+            const int par = (P0 + tap) & 1;
+            acc[0][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_reg[tap][0], bq[par][nt], acc[0][nt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (tap < 8) read_b(par ^ 1, PAIRS - 1, tap + 1, nt);
+            const int k = 2 * tap + (nt - 2);   // 0 .. 17
+            if (k < 8) outv[k >> 2][k & 3] = pack(k >> 2, k & 3);
+            if (k == 8 && pv[0]) *reinterpret_cast<v4i *>(cell[0]) = outv[0];
+            if (k == 9 && pv[1]) *reinterpret_cast<v4i *>(cell[1]) = outv[1];
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        TRACE_POINT(5);
+#pragma unroll
+        for (int tile = 2; tile < 4; ++tile) {
+          v4i o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = pack(tile, q);
+          if (pv[tile]) *reinterpret_cast<v4i *>(cell[tile]) = o;
+        }
+      };
+      if (a.lean & 2) last_pair(std::false_type());
+      else last_pair(std::true_type());
+      TRACE_POINT(15);
+      return;
+    } else {
+#pragma unroll
+      for (int st = LAST0; st < 9 * PAIRS; ++st)
+        tap_mfmas(st & 1, st % 9, PAIRS - 1, true, st + 1 < 9 * PAIRS ? PAIRS - 1 : -1, (st + 1) % 9);
     }
   } else
   for (int chunk = 0; chunk < nchunks; ++chunk) {
@@ -410,14 +490,14 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
 #define EHIP_CONV3X3V_HEAD                                                                                            \
   const uint8_t *in, int ih, int iw, int oh, int ow, int pad_t, int pad_l, int ic2, int chunk_units, int vw,         \
       unsigned vw_magic, int gx, int gy, int tiles, int tiles_per_xcd
-template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS = 0, bool SP = false>
+template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS = 0, bool SP = false, bool SL = false>
 __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(EHIP_CONV3X3V_HEAD, Conv3x3Args rest)
 {
   Conv3x3Args a = rest;
   a.in = in; a.ih = ih; a.iw = iw; a.oh = oh; a.ow = ow; a.pad_t = pad_t; a.pad_l = pad_l; a.ic2 = ic2;
   a.chunk_units = chunk_units; a.vw = vw; a.vw_magic = vw_magic; a.gx = gx; a.gy = gy; a.tiles = tiles;
   a.tiles_per_xcd = tiles_per_xcd;
-  conv3x3v_body<WM, WN, TM, TN, CT, NPASS, PAIRS, SP>(a);
+  conv3x3v_body<WM, WN, TM, TN, CT, NPASS, PAIRS, SP, SL>(a);
 }
 
 namespace {
@@ -434,20 +514,28 @@ struct Variant {
   int ustride;            // LDS cells between units
   conv3x3v_kernel_t kernel;
   conv3x3v_kernel_t unrolled[3];   // straight-line K loop for layers of exactly 2, 4, 8 unit pairs, or null
+  conv3x3v_kernel_t split[3];      // the same with the last pair split (lean epilogue without the sum), or null
 };
 #define V(WM, WN, TM, TN, CT, NPASS)                                                              \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
-    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>, {nullptr, nullptr, nullptr} }
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>, {nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr} }
 #define VU(WM, WN, TM, TN, CT, NPASS)                                                             \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4>,  \
-     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>} }
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>}, {nullptr, nullptr, nullptr} }
+#define VK(WM, WN, TM, TN, CT, NPASS)                                                             \
+  { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4>,  \
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>},                                               \
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, false, true>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, false, true>, \
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, false, true>} }
 #define VS(WM, WN, TM, TN, CT, NPASS)                                                             \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ",sp>", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, conv3x3v_unit_stride(CT * NPASS, TN, true), k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 0, true>, \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, true>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, true>, \
-     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>} }
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>}, {nullptr, nullptr, nullptr} }
 const Variant kVariants[] = {
     V(2, 2, 2, 1, 128, 1),  // 0: 128 oc x  64 px, rows up to  31 cells
     V(2, 2, 2, 1, 256, 1),  // 1: 128 oc x  64 px, rows up to  95 cells
@@ -458,11 +546,11 @@ const Variant kVariants[] = {
     V(1, 4, 1, 1, 256, 1),  // 6:  32 oc x 128 px, rows up to  63 cells
     V(1, 4, 1, 1, 256, 3),  // 7:  32 oc x 128 px, rows up to 319 cells
     VU(4, 1, 1, 1, 128, 1), // 8: 128 oc x  32 px, rows up to  47 cells
-    VU(4, 1, 1, 4, 256, 1), // 9: 128 oc x 128 px, rows up to  63 cells, every wave all pixels
+    VK(4, 1, 1, 4, 256, 1), // 9: 128 oc x 128 px, rows up to  63 cells, every wave all pixels
     VU(4, 1, 1, 2, 128, 1), // 10: 128 oc x 64 px, rows up to  31 cells, every wave all pixels
     V(1, 4, 2, 2, 256, 3),  // 11:  64 oc x 256 px, rows up to 255 cells
     V(2, 2, 1, 4, 256, 3),  // 12:  64 oc x 256 px, rows up to 255 cells, a wave = 32 oc x 128 px
-    VU(4, 1, 1, 4, 256, 2), // 13: 128 oc x 128 px, rows up to 191 cells, every wave all pixels
+    VK(4, 1, 1, 4, 256, 2), // 13: 128 oc x 128 px, rows up to 191 cells, every wave all pixels
     V(4, 1, 1, 4, 256, 4),  // 14: 128 oc x 128 px, rows up to 447 cells, every wave all pixels
     VS(4, 1, 1, 4, 256, 1), // 15: as 9, strided pixels
     VS(4, 1, 1, 2, 128, 1), // 16: as 10, strided pixels
@@ -472,6 +560,7 @@ const Variant kVariants[] = {
 };
 #undef V
 #undef VU
+#undef VK
 #undef VS
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLdsBudget = 64 * 1024;
@@ -561,7 +650,15 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
     const int pairs = a.units_pad / 2;
     const int slot = pairs == 2 ? 0 : (pairs == 4 ? 1 : (pairs == 8 ? 2 : -1));
     const char *env = getenv("EHIP_CONV3X3V_UNROLL");
-    if (slot >= 0 && k.unrolled[slot] && !(env && env[0] == '0')) kernel = k.unrolled[slot];
+    if (slot >= 0 && k.unrolled[slot] && !(env && env[0] == '0')) {
+      kernel = k.unrolled[slot];
+      // (the split form needs 238 registers against 164: two workgroups per CU instead of three, which costs
+      // more than the split gains once a CU gets more than two -- C2 at N = 512: 63.7 against 61.1 us; at its
+      // own N = 32, one workgroup per CU: 6.12 against 6.54 us)
+      const char *sl = getenv("EHIP_CONV3X3V_SPLIT_LAST");
+      const bool want = sl && sl[0] ? sl[0] != '0' : a.tiles <= 512;
+      if (k.split[slot] && (a.lean & 1) && !(a.lean & 4) && want) kernel = k.split[slot];
+    }
   }
   if (lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),

@@ -204,6 +204,20 @@ def test_conv3x3_every_virtual_row_kernel_variant(variant, ic, monkeypatch):
     assert res["conv"].kernel_name.startswith("k_conv3x3v_u8s8")
 
 
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("variant", [9, 13])
+@pytest.mark.parametrize("out_type,relu_hi", [(ol.U8, None), (ol.U8, 200.0), (ol.S8, None)])
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 64, 144, 13), (3, 128, 128, 28), (1, 256, 80, 14)])
+def test_conv3x3_split_last_pair(split, variant, out_type, relu_hi, n, ic, oc, hw, monkeypatch):
+    """u8 / s8 output with ReLU: the last channel pair multiplied tile pair by tile pair with half of the
+    epilogue behind its MFMAs (2, 4, 8 unit pairs; with and without a clamp), and the same layers in tap order"""
+    monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", str(variant))
+    monkeypatch.setenv("EHIP_CONV3X3V_SPLIT_LAST", split)
+    kw = {} if relu_hi is None else {"relu_hi": relu_hi}
+    res = run_and_compare(Layer(n, ic, oc, hw, k=3, pad=1, out_type=out_type, seed=640 + ic + out_type, **kw))
+    assert res["conv"].kernel_name.startswith("k_conv3x3v_u8s8")
+
+
 @pytest.mark.parametrize("variant", [15, 16, 17, 18, 19])
 @pytest.mark.parametrize("out_type", [ol.S32, ol.S8, ol.F32])
 def test_conv3x3_strided_pixels_output_types(variant, out_type, monkeypatch):
