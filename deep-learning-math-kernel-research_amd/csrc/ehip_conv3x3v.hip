@@ -402,8 +402,8 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
             if (tap < 8) read_b(par ^ 1, PAIRS - 1, tap + 1, nt);
             const int k = 2 * tap + (nt - 2);   // 0 .. 17
             if (k < 8) outv[k >> 2][k & 3] = pack(k >> 2, k & 3);
-            if (k == 8 && pv[0]) *reinterpret_cast<v4i *>(cell[0]) = outv[0];
-            if (k == 9 && pv[1]) *reinterpret_cast<v4i *>(cell[1]) = outv[1];
+            if (k == 8 && pv[0]) store_out16<false>(cell[0], outv[0]);
+            if (k == 9 && pv[1]) store_out16<false>(cell[1], outv[1]);
             __builtin_amdgcn_sched_barrier(0);
           }
         TRACE_POINT(5);
@@ -412,7 +412,7 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
           v4i o;
 #pragma unroll
           for (int q = 0; q < 4; ++q) o[q] = pack(tile, q);
-          if (pv[tile]) *reinterpret_cast<v4i *>(cell[tile]) = o;
+          if (pv[tile]) store_out16<false>(cell[tile], o);
         }
       };
       if (a.lean & 2) last_pair(std::false_type());

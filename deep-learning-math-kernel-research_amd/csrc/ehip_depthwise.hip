@@ -52,7 +52,8 @@ __device__ __forceinline__ void buffer_store_8(BufferRsrc r, unsigned off, uint2
 {
   typedef unsigned v2u __attribute__((ext_vector_type(2)));
   const v2u d = {v.x, v.y};
-  __builtin_amdgcn_raw_buffer_store_b64(d, r, (int)off, 0, 0);
+  // non-temporal (the line is not kept in L2): C5a 13.6 -> 12.3 us
+  __builtin_amdgcn_raw_buffer_store_b64(d, r, (int)off, 0, 2);
 }
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0f70); }   // vmcnt(0)
 #else   // the host pass only needs the names

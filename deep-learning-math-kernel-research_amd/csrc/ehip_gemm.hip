@@ -301,8 +301,9 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
             (((size_t)n * a.oc2 + ((oc0 + mw0) >> 4) + lh) * a.ohw + r) * 16;
       }
     }
-    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + mw0 + 16 * lh, oc_real,
-                       a.out_nhwc ? (size_t)32 : (size_t)2 * a.ohw * 16);
+    // (non-temporal stores for blocked output only: in nhwc a line's pieces come from several waves)
+    if (a.out_nhwc) lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + mw0 + 16 * lh, oc_real, (size_t)32);
+    else lean_store<TM, TN, true>(a.lean, a.ep, acc, lk, cell, pv, oc0 + mw0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
     TRACE_POINT(15);
     return;
   }
@@ -464,8 +465,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
         cell[nt] = static_cast<uint8_t *>(a.out) + px +
             (a.out_nhwc ? (size_t)(oc0 + 16 * lh) : ((size_t)(oc0 >> 4) + lh) * a.ohw * 16);
       }
-      lean_store<1, TNW>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real,
-                         a.out_nhwc ? (size_t)32 : (size_t)2 * a.ohw * 16);
+      if (a.out_nhwc) lean_store<1, TNW>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, (size_t)32);
+      else lean_store<1, TNW, true>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16);
       continue;
     }
 #pragma unroll
@@ -593,7 +594,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(GemmArgs a)
       v16i acc[1][1];
       acc[0][0] = acc2[ot & 1];
       uint8_t *cell[1] = {cell0 + (size_t)ot * tile_stride};
-      lean_store<1, 1>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 32 * ot + 16 * lh, oc_real, tile_stride);
+      if (a.out_nhwc) lean_store<1, 1>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 32 * ot + 16 * lh, oc_real, tile_stride);
+      else lean_store<1, 1, true>(a.lean, a.ep, acc, lk, cell, pvalid, oc0 + 32 * ot + 16 * lh, oc_real, tile_stride);
       __builtin_amdgcn_sched_barrier(0);
     }
   }

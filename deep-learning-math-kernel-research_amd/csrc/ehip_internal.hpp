@@ -570,6 +570,15 @@ __device__ __forceinline__ void epilogue_wave(const Epilogue &ep, const v16i (&a
 // the u8 -> s8 compensation.  A value costs a convert, a multiply-add, (a second one for the sum,) a
 // clamp -- none when the bounds are exactly the u8 code range, which v_cvt_pk_u8_f32 saturates to by
 // itself -- and a byte pack.  Arithmetic and rounding are those of quant4<.., FAST = true>.
+// A lane's 16 output bytes.  NT: a non-temporal store -- the line is not kept in L2.  Measured: kernels that
+// write several times what they read (1x1 layers with few input channels: 8-10 % faster, the strided 3x3
+// GEMM 4 %) gain, the 3x3 and the resident-tile 1x1 kernel do not (0 to -1 %), so the caller chooses.
+template <bool NT>
+__device__ __forceinline__ void store_out16(uint8_t *p, const v4i &v)
+{
+  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(p));
+  else *reinterpret_cast<v4i *>(p) = v;
+}
 struct LeanConsts {   // scale and shift of the lane's 16 channels of each 32-channel tile
   float4 sc[4], sh[4];
 };
@@ -593,7 +602,7 @@ inline int lean_mode(const Epilogue &e, bool out_nhwc)
 // cell[nt]: byte address of the lane's 16-byte cell of pixel tile nt in the wave's FIRST 16-channel block pair
 // member (block lh of tile 0); tile_stride: bytes between the cells of consecutive 32-channel tiles.
 // old_in: the sum operands if the caller has fetched them already (else null: they are read here).
-template <int TM, int TN, bool SUM, bool CLAMP>
+template <int TM, int TN, bool SUM, bool CLAMP, bool NT>
 __device__ __forceinline__ void lean_store_typed(const Epilogue &ep, const v16i (&acc)[TM][TN], const LeanConsts (&k)[TM],
                                                  uint8_t *const (&cell)[TN], const bool (&pvalid)[TN], int oc_first,
                                                  int oc_real, size_t tile_stride, const v4i (*old_in)[TN])
@@ -635,22 +644,22 @@ __device__ __forceinline__ void lean_store_typed(const Epilogue &ep, const v16i 
         }
         out[q] = (int)pk;
       }
-      if (pvalid[nt] && oc_first + 32 * mt < oc_real) *reinterpret_cast<v4i *>(cell[nt] + mt * tile_stride) = out;
+      if (pvalid[nt] && oc_first + 32 * mt < oc_real) store_out16<NT>(cell[nt] + mt * tile_stride, out);
     }
   }
 }
-template <int TM, int TN>
+template <int TM, int TN, bool NT = false>
 __device__ __forceinline__ void lean_store(int mode, const Epilogue &ep, const v16i (&acc)[TM][TN], const LeanConsts (&k)[TM],
                                            uint8_t *const (&cell)[TN], const bool (&pvalid)[TN], int oc_first, int oc_real,
                                            size_t tile_stride, const v4i (*old_in)[TN] = nullptr)
 {
   // one uniform branch, four straight copies
   if (mode & 4) {
-    if (mode & 2) lean_store_typed<TM, TN, true, false>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
-    else lean_store_typed<TM, TN, true, true>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+    if (mode & 2) lean_store_typed<TM, TN, true, false, NT>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+    else lean_store_typed<TM, TN, true, true, NT>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
   } else {
-    if (mode & 2) lean_store_typed<TM, TN, false, false>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
-    else lean_store_typed<TM, TN, false, true>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+    if (mode & 2) lean_store_typed<TM, TN, false, false, NT>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
+    else lean_store_typed<TM, TN, false, true, NT>(ep, acc, k, cell, pvalid, oc_first, oc_real, tile_stride, old_in);
   }
 }
 

@@ -392,7 +392,12 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
       const int e = M * i + j;
       const size_t cell = ((size_t)oh * ow_n + ow) * px + 4 * q;   // element index inside the plane
       if (OUT == EHIP_F32) {
-        *reinterpret_cast<float4 *>(static_cast<float *>(plane) + cell) = make_float4(y[0][e], y[1][e], y[2][e], y[3][e]);
+        {   // non-temporal: 200 MB of f32 output that nothing reads back soon (C4a 287 -> 261 us); the 4-byte
+            // stores of u8 / s8 output, and the transformed input (read right after), lose with it
+          typedef float v4f __attribute__((ext_vector_type(4)));
+          const v4f vv = {y[0][e], y[1][e], y[2][e], y[3][e]};
+          __builtin_nontemporal_store(vv, reinterpret_cast<v4f *>(static_cast<float *>(plane) + cell));
+        }
       } else {
         unsigned o = 0u;
 #pragma unroll
