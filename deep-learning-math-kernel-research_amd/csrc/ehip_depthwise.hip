@@ -450,16 +450,18 @@ dw_kernel_t kernel_rb(int stride, int mode)
 }  // namespace
 
 // The matrix-core kernel: stride 1, u8 output with a ReLU inside the code range, pads 0 / 1, and a plane
-// of one or two 32-column chunks whose chunks and 8-row strips are mostly real pixels (EHIP_DW_MFMA=0 / 1
-// overrides the last two conditions).
+// of up to four 32-column chunks whose chunks and 8-row strips are mostly real pixels (EHIP_DW_MFMA=0 / 1
+// overrides the last condition).
 bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, int out_type, int with_relu, float lo, float hi)
 {
   if (stride != 1 || out_type != EHIP_U8 || !with_relu || !(lo >= 0.0f && hi <= 255.0f && hi >= lo)) return false;
   if (pad_t < 0 || pad_t > 1 || pad_l < 0 || pad_l > 1 || ow > 128) return false;
   if (const char *env = getenv("EHIP_DW_MFMA")) return atoi(env) != 0;
-  // measured: ahead of the dot4 kernel on planes up to two chunks wide (28, 56 columns), behind it at 112
+  // measured (N = 64, with non-temporal output stores): ahead of the dot4 kernel at 28, 56 and 112 columns
+  // (8.8 / 13.1 / 14.2 us against 10.2 / 16.7 / 16.4 us for 256 / 128 / 32 channels), behind it on the half-empty
+  // chunks and strips of 14 x 14 and 7 x 7 planes (9.8 / 11.8 us against 7.9 / 5.0 us)
   const int nc = (ow + 31) / 32, strips = (oh + 7) / 8;
-  return nc <= 2 && 32.0 * nc * 8.0 * strips <= 1.35 * ow * oh;
+  return 32.0 * nc * 8.0 * strips <= 1.35 * ow * oh;
 }
 
 hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<DepthwiseArgs> *plan)

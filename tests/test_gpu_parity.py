@@ -381,8 +381,8 @@ def test_depthwise_matrix_core_kernel_is_the_default_where_it_fits(monkeypatch):
         d = E.make_desc(1, 32, 32, hw, hw, 3, 3, pad=1, g=32, output_type=E.U8, relu_bound=(0.0, 255.0), flatting_t=7,
                         output_quant=(0.02, 0.0))
         names[hw] = E.Conv(d).kernel_name
-    assert names[56] == names[28] == "k_depthwise3x3_mfma"
-    assert names[7] == names[14] == names[112] == "k_depthwise3x3_u8s8"   # half-empty chunks, or too wide: the dot4 kernel
+    assert names[112] == names[56] == names[28] == "k_depthwise3x3_mfma"
+    assert names[7] == names[14] == "k_depthwise3x3_u8s8"   # half-empty chunks and strips: the dot4 kernel
 
 
 # stride 2 (MobileNet's down-sampling layers, scripts/best_configs/mobilenetv1-n64-clx-1s-int8.sh:48:
