@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
   __shared__ v4i xpatch[4 * 256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   const int img = blockIdx.x / a.strips, strip = blockIdx.x - img * a.strips;

@@ -364,7 +364,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
   __shared__ v4i xpatch[4 * 256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   const int wo = wave % a.sk_wo, wp = wave / a.sk_wo, wpn = 4 / a.sk_wo;
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(GemmArgs a)
   __shared__ float4 cst_lds[4 * OCW * 24];   // [wave][tile][scale | shift | compensation][8 cells of 4 channels]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   const int wo = wave % a.sk_wo, wp = wave / a.sk_wo, wpn = 4 / a.sk_wo;
