@@ -690,7 +690,9 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   const int nks = a.units_pad / 2;
   const size_t lds = (size_t)36 * 32 * 32 * sizeof(float) + 4 * 216 * sizeof(float4);   // exchange + constants
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
-  int ks_max = 8;
+  // operand ring depth in k-steps.  Measured (C4a / C4b / C4a_i8 / C4b_i8, us): 8 deep 261.7 / 177.3 / 247.6 /
+  // 178.6, 4 deep 250.4 / 172.8 / 241.2 / 176.5, 2 deep 286.8 / 215.6 (f32 layers)
+  int ks_max = 4;
   if (const char *env = getenv("EHIP_WINO_KS")) ks_max = atoi(env);
   void (*kernel)(WinoFusedArgs) = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8>
       : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4> : k_wino_gemm_output<2>);

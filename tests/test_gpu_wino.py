@@ -97,6 +97,18 @@ def test_wino_tinput_under_range_and_both_gathers(tile, buf_gather, monkeypatch)
                                         (2, 256, 64, 9), (1, 272, 32, 6)])
 def test_wino_fused_gemm_and_output_transform(n, ic, oc, hw):
     """Default schedule: GEMM + output transform in one kernel; final output bit for bit."""
+    _fused(n, ic, oc, hw)
+
+
+@pytest.mark.parametrize("ring", ["2", "4", "8"])
+def test_wino_fused_every_operand_ring_depth(ring, monkeypatch):
+    """256 input channels = 8 k-steps per position: the fused kernel with its operands requested 2, 4 and 8
+    k-steps ahead (three instantiations; 4 is the default where it divides the k-steps)"""
+    monkeypatch.setenv("EHIP_WINO_KS", ring)
+    _fused(2, 256, 80, 9)
+
+
+def _fused(n, ic, oc, hw):
     import torch
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
     s_t, z_t = 22.0 / 255.0, 104.0
