@@ -200,6 +200,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
   uint8_t *cell[TN];
   bool pv[TN];
   v4i old[TM][TN];
+  const size_t tile_stride = a.out_nhwc ? (size_t)32 : (size_t)2 * a.ohw * 16;   // to the next 32 channels' cell
 #pragma unroll
   for (int nt = 0; nt < TN; ++nt) {
     const int gp = pix0 + nt * 32 + l32;
@@ -207,12 +208,13 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
     const int gpc = pv[nt] ? gp : 0;
     const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gpc, a.ohw, a.ohw_magic);
     const int r = gpc - n * a.ohw;
-    cell[nt] = static_cast<uint8_t *>(a.out) + (((size_t)n * a.oc2 + (oc0 >> 4) + lh) * a.ohw + r) * 16;
+    cell[nt] = static_cast<uint8_t *>(a.out) +
+        (a.out_nhwc ? (size_t)gpc * oc_real + (oc0 + 16 * lh) : (((size_t)n * a.oc2 + (oc0 >> 4) + lh) * a.ohw + r) * 16);
     if (a.lean & 4) {
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) {
         const bool ok = pv[nt] && oc0 + 16 * lh + 32 * mt < oc_real;
-        old[mt][nt] = *reinterpret_cast<const v4i *>(ok ? cell[nt] + (size_t)mt * 2 * a.ohw * 16 : cell[nt]);
+        old[mt][nt] = *reinterpret_cast<const v4i *>(ok ? cell[nt] + (size_t)mt * tile_stride : cell[nt]);
       }
     }
   }
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
   TRACE_POINT(5);
   // ---- epilogue ---------------------------------------------------------------------------------------
   if (a.lean) {
-    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + 16 * lh, oc_real, (size_t)2 * a.ohw * 16, old);
+    lean_store<TM, TN>(a.lean, a.ep, acc, lk, cell, pv, oc0 + 16 * lh, oc_real, tile_stride, old);
     TRACE_POINT(15);
     return;
   }
@@ -344,7 +346,10 @@ int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
 {
   const char *env = getenv("EHIP_GEMM1X1_RES");
   if (env && env[0] == '0') return -1;
-  if (nbatch != 1 || a.kh * a.kw > 1 || a.in_nhwc || a.out_nhwc || a.ep.shift_tab) return -1;
+  if (nbatch != 1 || a.kh * a.kw > 1 || a.in_nhwc || a.ep.shift_tab) return -1;
+  // nhwc output: through the lean epilogue only (a lane's 16 bytes are contiguous there as well; the general
+  // epilogue of this kernel addresses blocked cells)
+  if (a.out_nhwc && !lean_mode(a.ep, false)) return -1;
   if (a.ic2 <= 8 || (a.units_pad & 1)) return -1;   // few channels: the weights-in-registers kernel
   if (env && env[0] >= '1' && env[0] <= '4') {
     const int v = env[0] - '1';
@@ -404,6 +409,7 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
                                      (int)lds_bytes);
   if (e != hipSuccess) return e;
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
+  if (plan) plan->name = k.name;   // (nhwc output: the handle could not tell at creation whether the lean epilogue applies)
   return plan_launch(plan, kernel, grid, dim3(kBlock), lds_bytes, a, s);
 }
 

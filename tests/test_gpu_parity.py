@@ -79,6 +79,23 @@ def test_conv1x1_resident_pixel_tile_kernel(variant, n, ic, oc, hw, stride, monk
     run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=ol.U8, seed=301 + variant + ic, relu_hi=200.0))
 
 
+@pytest.mark.parametrize("variant", ["", "1", "2", "3", "4"])
+@pytest.mark.parametrize("n,ic,oc,hw,stride", [(2, 256, 272, 14, 1), (3, 144, 80, 9, 1), (1, 512, 176, 14, 2), (2, 1024, 256, 7, 1)])
+def test_conv1x1_resident_pixel_tile_kernel_nhwc_output(variant, n, ic, oc, hw, stride, monkeypatch):
+    """blocked input, nhwc output, u8 / s8 with ReLU (the lean epilogue's cases): a lane's 16 channels are 16
+    contiguous bytes of its pixel's vector; with the sum the old output is read from the same place"""
+    if variant:
+        monkeypatch.setenv("EHIP_GEMM1X1_RES", variant)
+    for out_type, with_sum, kw in ((ol.U8, False, {}), (ol.S8, True, {}), (ol.U8, True, {"relu_hi": 200.0})):
+        res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, with_sum=with_sum, out_nhwc=True,
+                                    seed=330 + ic + out_type, **kw))
+        if variant:
+            assert res["conv"].kernel_name.startswith("k_gemm1x1_res")
+    # what the lean epilogue does not cover goes through the general kernel
+    res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=ol.F32, out_nhwc=True, seed=331 + ic))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+
+
 def test_conv1x1_resident_pixel_tile_kernel_can_be_switched_off(monkeypatch):
     monkeypatch.setenv("EHIP_GEMM1X1_RES", "0")
     run_and_compare(Layer(2, 256, 256, 14, out_type=ol.S8, with_sum=True, seed=302))
