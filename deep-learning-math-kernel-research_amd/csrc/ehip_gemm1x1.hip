@@ -85,7 +85,12 @@ __device__ __forceinline__ void wait_loads_but(int n)
 
 // NKS > 0: the layer has exactly NKS k-steps (pairs of 16-channel units): the K loop is straight-line code
 // and every wait names the load it needs.  NKS == 0: a loop over blocks of eight k-steps.
-template <int TM, int TN, int NKS>
+// NHWC: nhwc input.  A pixel's channel vector is contiguous in memory, so the tile is kept pixel-major in LDS,
+// [P_T pixels][units_pad + 1 cells]: the odd row length spreads the 16 pixels a 16-byte operand read serves per
+// clock over all banks.  A wave-load still fills 64 consecutive LDS cells; its lane i fetches whatever cell
+// 64 j + i of that layout is (the pad cell and padded units repeat a real unit: they multiply zero weights or
+// nothing).  The whole tile is waited for before the K loop (no unit order to consume it in).
+template <int TM, int TN, int NKS, bool NHWC = false>
 __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
 {
   constexpr int OC_T = 4 * TM * 32;
@@ -135,6 +140,30 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
   // LDS address + 16 i.  Pixel halves of 64 (P_T / 64) x units are dealt to the four waves round-robin.
   constexpr int HALVES = P_T / 64 > 0 ? P_T / 64 : 1;
   constexpr int LPW = P_T >= 64 ? 64 : P_T;   // pixels per wave-load (32-pixel tiles: the upper lanes repeat)
+  const int U1 = a.units_pad + 1;   // nhwc: cells per staged pixel
+  // byte offset of output pixel gp's first input cell in an nhwc tensor (clamped past the end)
+  auto nhwc_pixel = [&](int gp) -> long long {
+    gp = gp < a.p_total ? gp : a.p_total - 1;
+    const int n = a.ohw == a.p_total ? 0 : fastdiv_any(gp, a.ohw, a.ohw_magic);
+    const int r = gp - n * a.ohw;
+    long long sp = r;
+    if (!dense) {
+      const int oh = fastdiv(r, a.ow, a.ow_magic);
+      sp = (long long)oh * a.stride_h * a.iw + (long long)(r - oh * a.ow) * a.stride_w;
+    }
+    return ((long long)n * a.ihw + sp) * a.ic2 * 16;
+  };
+  auto request_tile_nhwc = [&]() {
+    const int cells = P_T * U1;
+    for (int c0 = wave * 64; c0 < cells; c0 += 256) {   // wave-uniform
+      const int c = c0 + lane;
+      int p = fastdiv(c, U1, a.u1_magic);
+      int u = c - p * U1;
+      p = p < P_T ? p : P_T - 1;            // the last load runs past the tile: into the allocation's slack
+      u = u < a.ic2 ? u : a.ic2 - 1;
+      load_to_lds_16(a.in + nhwc_pixel(pix0 + p) + u * 16, lds + c0);
+    }
+  };
   const uint8_t *src[HALVES];
 #pragma unroll
   for (int h = 0; h < HALVES; ++h) {
@@ -166,7 +195,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
   // issue order, so the weights (from L2) are there first; the K loop then waits for eight units (four
   // k-steps) of the tile at a time -- its own share by count, everybody else's by a barrier -- instead of
   // for all 64 KB before its first MFMA.
-  constexpr bool PIPE = NKS > 0 && R == NKS && NKS % 4 == 0;
+  constexpr bool PIPE = !NHWC && NKS > 0 && R == NKS && NKS % 4 == 0;
   constexpr int LPC = 2 * HALVES;            // loads of one wave per chunk: 8 units x HALVES dealt to four waves
   constexpr int TILE_LOADS = NKS * HALVES / 2;   // of one wave, all chunks (PIPE)
   auto request_tile_unseen = [&]() {
@@ -181,7 +210,8 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
       load_to_lds_16_unseen(p + (long long)uc * unit_stride, lds + (size_t)u * P_T + h * 64);
     }
   };
-  if (!PIPE) request_tile();
+  if (NHWC) request_tile_nhwc();
+  else if (!PIPE) request_tile();
 
   TRACE_POINT(1);
   // ---- weights [units_pad][ocpp][16]: lane = packed row l32 of unit 2 ks + lh, tile mt 32 rows on --------
@@ -249,13 +279,15 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
 
   // ---- K loop: one memory instruction behind each MFMA ---------------------------------------------------
   v4i bq[2][TN];
-  const v4i *tile = lds + lh * P_T + l32;
+  const v4i *tile = NHWC ? lds + l32 * U1 + lh : lds + lh * P_T + l32;
   // (raw bytes: the u8 -> s8 flip of the top bits happens right before the operand's first use.  Next to the
   // read it would make the wave wait for the read it has just issued; as a pass over the whole tile in LDS it
   // was measured to cost more than it saves.  With one wave per SIMD the flip still sits between a read and
   // the MFMA that waits for it -- 51 instead of 34 clocks per MFMA -- which a second workgroup on the CU
   // hides: the 64-pixel tiles, two workgroups per CU, are the fast ones.)
-  auto read_b = [&](int par, int ks, int nt) { bq[par][nt] = tile[(size_t)ks * 2 * P_T + nt * 32]; };
+  auto read_b = [&](int par, int ks, int nt) {
+    bq[par][nt] = NHWC ? tile[nt * 32 * U1 + 2 * ks] : tile[(size_t)ks * 2 * P_T + nt * 32];
+  };
   // k-step ks out of operand buffer par; the operands of k-step ks + 1 are read on the way, the ring slot
   // is refilled with the weights of k-step ks + R behind the last MFMA
   auto kstep = [&](int par, int slot, int ks, bool read_next, bool load_next) {
@@ -325,20 +357,35 @@ struct ResVariant {
   int oc_t, p_t;
   void (*generic)(GemmArgs);
   void (*unrolled[3])(GemmArgs);   // exactly 8, 16, 32 k-steps
+  void (*generic_nhwc)(GemmArgs);  // nhwc input (64-pixel tiles only), or null
+  void (*unrolled_nhwc[3])(GemmArgs);
 };
 #define RV(TM, TN)                                                                                           \
   { "k_gemm1x1_res<" #TM "," #TN ">", 4 * TM * 32, TN * 32, k_gemm1x1_res<TM, TN, 0>,                        \
-    {k_gemm1x1_res<TM, TN, 8>, k_gemm1x1_res<TM, TN, 16>, k_gemm1x1_res<TM, TN, 32>} }
+    {k_gemm1x1_res<TM, TN, 8>, k_gemm1x1_res<TM, TN, 16>, k_gemm1x1_res<TM, TN, 32>}, nullptr, {nullptr, nullptr, nullptr} }
+#define RVN(TM, TN)                                                                                          \
+  { "k_gemm1x1_res<" #TM "," #TN ">", 4 * TM * 32, TN * 32, k_gemm1x1_res<TM, TN, 0>,                        \
+    {k_gemm1x1_res<TM, TN, 8>, k_gemm1x1_res<TM, TN, 16>, k_gemm1x1_res<TM, TN, 32>}, k_gemm1x1_res<TM, TN, 0, true>, \
+    {k_gemm1x1_res<TM, TN, 8, true>, k_gemm1x1_res<TM, TN, 16, true>, k_gemm1x1_res<TM, TN, 32, true>} }
 const ResVariant kRes[] = {
-    RV(1, 4),   // 0: 128 oc x 128 px
-    RV(1, 2),   // 1: 128 oc x  64 px
-    RV(2, 4),   // 2: 256 oc x 128 px
-    RV(2, 2),   // 3: 256 oc x  64 px
+    RV(1, 4),    // 0: 128 oc x 128 px
+    RVN(1, 2),   // 1: 128 oc x  64 px
+    RV(2, 4),    // 2: 256 oc x 128 px
+    RVN(2, 2),   // 3: 256 oc x  64 px
 };
 #undef RV
+#undef RVN
 constexpr int kNumRes = sizeof(kRes) / sizeof(kRes[0]);
 constexpr size_t kResLds = 160 * 1024;
 
+}  // namespace
+
+namespace {
+// LDS of a workgroup: [units][P_T] cells, or (nhwc input) [P_T][units + 1] rounded up to whole wave-loads
+size_t res_lds_bytes(const GemmArgs &a, int p_t)
+{
+  return a.in_nhwc ? (size_t)up((a.units_pad + 1) * p_t, 64) * 16 : (size_t)a.units_pad * p_t * 16;
+}
 }  // namespace
 
 // -1: the layer is not one for this kernel
@@ -346,24 +393,25 @@ int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
 {
   const char *env = getenv("EHIP_GEMM1X1_RES");
   if (env && env[0] == '0') return -1;
-  if (nbatch != 1 || a.kh * a.kw > 1 || a.in_nhwc || a.ep.shift_tab) return -1;
+  if (nbatch != 1 || a.kh * a.kw > 1 || a.ep.shift_tab) return -1;
   // nhwc output: through the lean epilogue only (a lane's 16 bytes are contiguous there as well; the general
   // epilogue of this kernel addresses blocked cells)
   if (a.out_nhwc && !lean_mode(a.ep, false)) return -1;
   if (a.ic2 <= 8 || (a.units_pad & 1)) return -1;   // few channels: the weights-in-registers kernel
   if (env && env[0] >= '1' && env[0] <= '4') {
     const int v = env[0] - '1';
-    return (size_t)a.units_pad * kRes[v].p_t * 16 <= kResLds ? v : -1;
+    if (a.in_nhwc && !kRes[v].generic_nhwc) return -1;
+    return res_lds_bytes(a, kRes[v].p_t) <= kResLds ? v : -1;
   }
   const int oc = a.oc2 * 16;
   int best = -1;
   double best_score = 0;
   for (int v = 0; v < kNumRes; ++v) {
     const ResVariant &k = kRes[v];
-    if ((size_t)a.units_pad * k.p_t * 16 > kResLds) continue;
+    if (res_lds_bytes(a, k.p_t) > kResLds || (a.in_nhwc && !k.generic_nhwc)) continue;
     const int gx = (a.p_total + k.p_t - 1) / k.p_t, gy = (oc + k.oc_t - 1) / k.oc_t;
     const long long wgs = (long long)gx * gy;
-    const int per_cu = (int)(kResLds / ((size_t)a.units_pad * k.p_t * 16));   // resident workgroups
+    const int per_cu = (int)(kResLds / res_lds_bytes(a, k.p_t));   // resident workgroups
     const long long slots = 256ll * (per_cu > 2 ? 2 : per_cu);
     const long long rounds = (wgs + slots - 1) / slots;
     const double util = ((double)oc / ((double)gy * k.oc_t)) * ((double)a.p_total / ((double)gx * k.p_t));
@@ -397,14 +445,17 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   const int nks = a.units_pad / 2;
-  void (*kernel)(GemmArgs) = k.generic;
+  void (*kernel)(GemmArgs) = a.in_nhwc ? k.generic_nhwc : k.generic;
   const char *env = getenv("EHIP_GEMM1X1_UNROLL");
   if (!(env && env[0] == '0')) {
-    if (nks == 8) kernel = k.unrolled[0];
-    else if (nks == 16) kernel = k.unrolled[1];
-    else if (nks == 32) kernel = k.unrolled[2];
+    void (*const *un)(GemmArgs) = a.in_nhwc ? k.unrolled_nhwc : k.unrolled;
+    if (nks == 8) kernel = un[0];
+    else if (nks == 16) kernel = un[1];
+    else if (nks == 32) kernel = un[2];
   }
-  const size_t lds_bytes = (size_t)a.units_pad * k.p_t * 16;
+  if (!kernel) return hipErrorInvalidValue;
+  a.u1_magic = div_magic(a.units_pad + 1);
+  const size_t lds_bytes = res_lds_bytes(a, k.p_t);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds_bytes);
   if (e != hipSuccess) return e;

@@ -62,6 +62,7 @@ struct GemmArgs {
   int nx, ny;                  // set by the launcher: pixel blocks, channel blocks
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
   int lean;                    // set by the launcher: lean_mode() of the epilogue (0 = general epilogue)
+  unsigned u1_magic;           // set by the resident-tile launcher: div_magic(units_pad + 1)
 };
 
 struct Conv3x3Args {

@@ -96,6 +96,28 @@ def test_conv1x1_resident_pixel_tile_kernel_nhwc_output(variant, n, ic, oc, hw, 
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
+@pytest.mark.parametrize("variant", ["", "2", "4"])
+@pytest.mark.parametrize("n,ic,oc,hw,stride", [(2, 256, 272, 14, 1), (3, 144, 80, 9, 1), (1, 512, 176, 14, 2), (2, 1024, 256, 7, 1),
+                                               (1, 2048, 64, 5, 1)])
+def test_conv1x1_resident_pixel_tile_kernel_nhwc_input(variant, n, ic, oc, hw, stride, monkeypatch):
+    """nhwc input: the tile pixel-major in LDS (one pad cell per pixel); blocked output with every output
+    type, nhwc output with the lean epilogue's cases; generic and unrolled K loops, stride 2, ragged tiles"""
+    if variant:
+        monkeypatch.setenv("EHIP_GEMM1X1_RES", variant)
+    for out_type, with_sum in ((ol.U8, False), (ol.S8, True), (ol.F32, False), (ol.S32, False)):
+        res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, with_sum=with_sum, in_nhwc=True,
+                                    seed=350 + ic + out_type))
+        if variant:
+            assert res["conv"].kernel_name.startswith("k_gemm1x1_res")
+    for out_type, with_sum in ((ol.U8, True), (ol.S8, False)):
+        res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=out_type, with_sum=with_sum, in_nhwc=True,
+                                    out_nhwc=True, seed=351 + ic + out_type))
+        if variant:
+            assert res["conv"].kernel_name.startswith("k_gemm1x1_res")
+    monkeypatch.setenv("EHIP_GEMM1X1_UNROLL", "0")
+    run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=ol.U8, seed=352 + ic, in_nhwc=True))
+
+
 def test_conv1x1_resident_pixel_tile_kernel_can_be_switched_off(monkeypatch):
     monkeypatch.setenv("EHIP_GEMM1X1_RES", "0")
     run_and_compare(Layer(2, 256, 256, 14, out_type=ol.S8, with_sum=True, seed=302))
