@@ -49,7 +49,7 @@ struct ehip_conv {
   float *shift_tab = nullptr;
   // k x k direct with at most four input channels: ppc = 16 / ic pixels per 16-byte cell, nu cells per
   // kernel row; gtaps = taps of the K axis of the packed weights (kh * nu there, kh * kw otherwise)
-  int ppc = 0, nu = 0, gtaps = 1;
+  int ppc = 0, nu = 0, gtaps = 1, icl = 0;   // icl: bytes per pixel in a cell (conv_fewch_icl)
   // 3x3
   int chunk_units = 2;
   // depthwise
@@ -299,14 +299,15 @@ int setup_workspace(ehip_conv *c)
     if (c->taps > 1 && (long long)d.n * c->ic2 * d.ih * d.iw * 16 >= (1ll << 40))
       return fail(EHIP_UNIMPLEMENTED, "direct: input too large");
     c->gtaps = c->taps;
+    c->icl = conv_fewch_icl(d.ic, d.kw);
     if (c->family == FAM_CONV_FEWCH &&
-        (size_t)d.kh * conv_fewch_row_pitch(d.ic, d.kw, d.iw, d.ow, d.stride_w, d.pad_l) > 48 * 1024) {
+        (size_t)d.kh * conv_fewch_row_pitch(c->icl, d.kw, d.iw, d.ow, d.stride_w, d.pad_l) > 48 * 1024) {
       // one strip's input rows do not fit in LDS
       if (d.input_fmt == EHIP_NHWC) return fail(EHIP_UNIMPLEMENTED, "direct: few-channel nhwc input: rows too wide");
       c->family = FAM_GEMM_1X1;
     }
     if (c->family == FAM_CONV_FEWCH) {
-      c->ppc = 16 / d.ic;
+      c->ppc = 16 / c->icl;
       c->nu = (d.kw + c->ppc - 1) / c->ppc;
       c->gtaps = d.kh * c->nu;
     }
@@ -536,10 +537,10 @@ EHIP_API int ehip_conv_prepare(ehip_conv_t *c, const void *weights_dev, const vo
   case FAM_GEMM_1X1:
   case FAM_CONV_3X3:
     if (c->family == FAM_CONV_FEWCH) {
-      HIP_TRY(launch_prepare_direct_px(w, b, d.oc, d.ic, d.kh, d.kw, c->ppc, c->nu, c->ocpp, d, c->absmax, c->wpacked,
+      HIP_TRY(launch_prepare_direct_px(w, b, d.oc, d.ic, c->icl, d.kh, d.kw, c->ppc, c->nu, c->ocpp, d, c->absmax, c->wpacked,
                                        c->scale, c->shift, c->wsum, c->comp, s));
       if (c->nclass > 1)
-        HIP_TRY(launch_fold_direct_border_px(c->wpacked, c->absmax, b, d.oc, d.ic, c->ppc, c->nu, c->ocpp, d, c->rects,
+        HIP_TRY(launch_fold_direct_border_px(c->wpacked, c->absmax, b, d.oc, c->icl, c->ppc, c->nu, c->ocpp, d, c->rects,
                                              c->nclass, c->shift_tab, s));
       break;
     }
@@ -628,7 +629,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.ep = make_epilogue(c, d.output_type, false, d.with_relu);
     a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.oh = d.oh; a.ow = d.ow; a.ic = d.ic; a.kh = d.kh; a.kw = d.kw;
     a.stride_h = d.stride_h; a.stride_w = d.stride_w; a.pad_t = d.pad_t; a.pad_l = d.pad_l;
-    a.oc2 = c->oc2; a.ocpp = c->ocpp;
+    a.oc2 = c->oc2; a.ocpp = c->ocpp; a.icl = c->icl;
     a.in_nhwc = d.input_fmt == EHIP_NHWC; a.out_nhwc = d.output_fmt == EHIP_NHWC;
     if (c->nclass > 1) {
       a.ep.shift_tab = c->shift_tab; a.ep.tab_stride = c->ocpp;
@@ -772,7 +773,7 @@ EHIP_API int ehip_conv_query(ehip_conv_t *c, int what, void *host_dst, size_t *b
       for (int oc = 0; oc < ocp; ++oc)
         for (int ic = 0; ic < icp; ++ic)
           for (int tap = 0; tap < taps; ++tap) {
-            const int kh = tap / d.kw, kw = tap % d.kw, j = kw / c->ppc, byte = (kw % c->ppc) * d.ic + ic;
+            const int kh = tap / d.kw, kw = tap % d.kw, j = kw / c->ppc, byte = (kw % c->ppc) * c->icl + ic;
             dst[((size_t)oc * icp + ic) * taps + tap] =
                 ic < d.ic ? packed[((size_t)(kh * c->nu + j) * c->ocpp + packed_row_of_oc(oc)) * 16 + byte] : 0;
           }

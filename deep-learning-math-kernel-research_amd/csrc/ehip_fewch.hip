@@ -87,11 +87,20 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
         const int r = fastdiv(idx, lrow4, a.lrow4_magic);
         const int d = idx - r * lrow4;
         const int h = ihb + r;
-        const int g = g00 + r * rowbytes + 4 * d;   // first byte of the staged dword
-        const int rs = g00 + r * rowbytes + a.pad_l * a.ic;   // first byte of the input row
-        const int lo = rs - g, hi = rs + rowbytes - g;        // bytes lo .. hi - 1 of the dword belong to the row
         const bool inside = (unsigned)h < (unsigned)a.ih;
-        m[u] = inside ? low_bytes(hi) & ~low_bytes(lo) : 0u;
+        int g;
+        if (a.icl != a.ic) {
+          // three channels staged as four bytes: dword d of a staged row is pixel d - pad_l, its three bytes
+          // wherever they lie in memory, and a pad byte
+          const int x = d - a.pad_l;
+          g = e0 + (h * a.iw + x) * 3;
+          m[u] = inside && (unsigned)x < (unsigned)a.iw ? 0x00ffffffu : 0u;
+        } else {
+          g = g00 + r * rowbytes + 4 * d;   // first byte of the staged dword
+          const int rs = g00 + r * rowbytes + a.pad_l * a.ic;   // first byte of the input row
+          const int lo = rs - g, hi = rs + rowbytes - g;        // bytes lo .. hi - 1 of the dword belong to the row
+          m[u] = inside ? low_bytes(hi) & ~low_bytes(lo) : 0u;
+        }
         // dwords outside the image hold nothing of the row: any address inside will do for them
         int ga = g & ~3, gb = ga + 4;
         ga = ga < 0 ? 0 : ga > last_dw ? last_dw : ga;
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
         const int x = idx - r * a.iw;
         const int h = ihb + r;
         const bool inside = in_range && h >= 0 && h < a.ih;
-        at[u] = inside ? r * a.lrow + (x + a.pad_l) * a.ic : -1;
+        at[u] = inside ? r * a.lrow + (x + a.pad_l) * a.icl : -1;
         v[u] = *reinterpret_cast<const unsigned *>(a.in + (inside ? ((long long)(img * a.ih + h) * a.iw + x) * 16 : 0));
       }
 #pragma unroll
@@ -155,7 +164,7 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
     int tc = 2 * ks + lh;
     tc = tc < a.cells ? tc : a.cells - 1;
     const int kr = tc / a.nu;
-    cell_at[ks] = kr * a.lrow + (tc - kr * a.nu) * a.ppc * a.ic;
+    cell_at[ks] = kr * a.lrow + (tc - kr * a.nu) * a.ppc * a.icl;
   }
 
   const long long cidx = oc0 + 16 * lh;
@@ -175,7 +184,7 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
   const size_t out0 = a.out_nhwc ? ((size_t)img * ohw + (size_t)oh0 * a.ow) * oc_real
                                  : ((size_t)img * a.oc2 * ohw + (size_t)oh0 * a.ow) * 16;
   const size_t block_stride = a.out_nhwc ? (size_t)16 : (size_t)ohw * 16;
-  const int row_step = a.stride_h * a.lrow, px_step = a.stride_w * a.ic;
+  const int row_step = a.stride_h * a.lrow, px_step = a.stride_w * a.icl;
   const int ntiles = (npix + 31) >> 5;
   for (int tile = wp; tile < ntiles; tile += wpn) {
     int p = tile * 32 + l32;
@@ -184,14 +193,22 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
     const int ox = p - ro * a.ow;
     const int at0 = ro * row_step + ox * px_step;
     v4i b[KS];
+    if (a.icl == 4) {   // every cell starts on a dword: four reads, nothing to shift
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int A = at0 + cell_at[ks];
-      const unsigned *src = rows_lds + (A >> 2);
-      const unsigned sh = A & 3;
-      const unsigned d0 = src[0], d1 = src[1], d2 = src[2], d3 = src[3], d4 = src[4];
-      b[ks] = v4i{(int)__builtin_amdgcn_alignbyte(d1, d0, sh), (int)__builtin_amdgcn_alignbyte(d2, d1, sh),
-                  (int)__builtin_amdgcn_alignbyte(d3, d2, sh), (int)__builtin_amdgcn_alignbyte(d4, d3, sh)};
+      for (int ks = 0; ks < KS; ++ks) {
+        const unsigned *src = rows_lds + ((at0 + cell_at[ks]) >> 2);
+        b[ks] = v4i{(int)src[0], (int)src[1], (int)src[2], (int)src[3]};
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int A = at0 + cell_at[ks];
+        const unsigned *src = rows_lds + (A >> 2);
+        const unsigned sh = A & 3;
+        const unsigned d0 = src[0], d1 = src[1], d2 = src[2], d3 = src[3], d4 = src[4];
+        b[ks] = v4i{(int)__builtin_amdgcn_alignbyte(d1, d0, sh), (int)__builtin_amdgcn_alignbyte(d2, d1, sh),
+                    (int)__builtin_amdgcn_alignbyte(d3, d2, sh), (int)__builtin_amdgcn_alignbyte(d4, d3, sh)};
+      }
     }
     v16i acc[1][1];
     acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[0], b[0], comp0, 0, 0, 0);
@@ -246,20 +263,31 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
   }
 }
 
+int conv_fewch_icl(int ic, int kw)
+{
+  if (ic != 3 || (kw + 3) / 4 != (kw + 4) / 5) return ic;
+  // 7x7, stride 2 at 224 x 224, N = 64: 33.6 -> 29.1 us (a cell is four dword reads instead of five and four
+  // byte shifts); 3x3, stride 2: 16.0 -> 16.8 us -- with one cell per kernel row the third more dwords to
+  // stage cost more than the cells save.  So by default only kernels at least five wide.
+  const char *env = getenv("EHIP_FEWCH_PAD_PIXEL");
+  if (env && env[0]) return env[0] == '0' ? 3 : 4;
+  return kw >= 5 ? 4 : 3;
+}
+
 bool conv_fewch_applies(int ic, int kh, int kw)
 {
   if (ic < 1 || ic > 4 || kh * kw <= 1 || kw < 2) return false;
-  const int ppc = 16 / ic, nu = (kw + ppc - 1) / ppc;
+  const int ppc = 16 / ic, nu = (kw + ppc - 1) / ppc;   // the same nu with padded pixels
   return kh * nu <= 14;
 }
 
 // pitch in bytes of a staged input row: pad_l + iw pixels or the last output pixel's last cell
 // (16 bytes), whichever ends later, + 4 for the fifth dword of a shifted cell
-int conv_fewch_row_pitch(int ic, int kw, int iw, int ow, int stride_w, int pad_l)
+int conv_fewch_row_pitch(int icl, int kw, int iw, int ow, int stride_w, int pad_l)
 {
-  const int ppc = 16 / ic, nu = (kw + ppc - 1) / ppc;
-  int need = (pad_l + iw) * ic;
-  const int last = ((ow - 1) * stride_w + (nu - 1) * ppc) * ic + 16;
+  const int ppc = 16 / icl, nu = (kw + ppc - 1) / ppc;
+  int need = (pad_l + iw) * icl;
+  const int last = ((ow - 1) * stride_w + (nu - 1) * ppc) * icl + 16;
   if (last > need) need = last;
   return up(need + 4, 4) + 4;
 }
@@ -282,12 +310,13 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
     if (a.ep.with_sum) a.lean = 0;
     if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   }
-  a.ppc = 16 / a.ic;
+  if (a.icl != a.ic && !(a.ic == 3 && a.icl == 4)) return hipErrorInvalidValue;
+  a.ppc = 16 / a.icl;
   a.nu = (a.kw + a.ppc - 1) / a.ppc;
   a.cells = a.kh * a.nu;
   if (!conv_fewch_applies(a.ic, a.kh, a.kw)) return hipErrorInvalidValue;
   if (a.in_nhwc && (reinterpret_cast<uintptr_t>(a.in) & 3)) return hipErrorInvalidValue;   // aligned dword loads
-  a.lrow = conv_fewch_row_pitch(a.ic, a.kw, a.iw, a.ow, a.stride_w, a.pad_l);
+  a.lrow = conv_fewch_row_pitch(a.icl, a.kw, a.iw, a.ow, a.stride_w, a.pad_l);
   const int octiles = up(a.oc2 * 16, 32) / 32;   // <= ocpp / 32
   a.wo = octiles % 4 == 0 ? 4 : octiles % 2 == 0 ? 2 : 1;
   const int gy = octiles / a.wo, wpn = 4 / a.wo;

@@ -227,13 +227,20 @@ struct FewChArgs {
   int rows, strips;     // output rows per workgroup, workgroups per image
   int nrows_in, lrow;   // staged input rows and their pitch in bytes (a multiple of 4)
   int wo;               // waves of a workgroup along the channels (1, 2, 4)
+  int icl;              // bytes per pixel in a staged row and in an operand cell (conv_fewch_icl); set by the caller
   int lean;             // lean_mode() of the epilogue, per-pixel shift rows allowed (0 = general epilogue)
   unsigned ow_magic, iw_magic, lrow4_magic;
 };
+// Bytes a pixel takes in the staged rows and operand cells of the few-channel kernel: its ic channels, except
+// that three channels are padded to four (the fourth multiplies a zero weight) where that costs no extra cell
+// per kernel row (3x3 and 7x7 kernels: ceil(kw / 4) == ceil(kw / 5)) -- every cell then starts on a dword.
+// By default only for kernels at least five wide; EHIP_FEWCH_PAD_PIXEL=0 never, =1 wherever it can.  A handle
+// asks once and keeps the answer.
+int conv_fewch_icl(int ic, int kw);
 bool conv_fewch_applies(int ic, int kh, int kw);
-int conv_fewch_row_pitch(int ic, int kw, int iw, int ow, int stride_w, int pad_l);
+int conv_fewch_row_pitch(int icl, int kw, int iw, int ow, int stride_w, int pad_l);   // icl: conv_fewch_icl()
 hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> *plan = nullptr);
-hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int kh, int kw, int ppc, int nu,
+hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int icl, int kh, int kw, int ppc, int nu,
                                     int ocpp, const ehip_conv_desc_t &d, float *absmax, int8_t *wpacked, float *scale,
                                     float *shift, int *wsum, int *comp, hipStream_t s);
 hipError_t launch_fold_direct_border_px(const int8_t *wpacked, const float *absmax, const float *bias, int oc, int ic,

@@ -118,13 +118,13 @@ __global__ __launch_bounds__(kBlock) void k_quant_pack_direct(const float *w, co
 }
 
 // Layers with at most four input channels (first layers, k_conv_fewch_u8s8): a 16-byte cell
-// holds ppc = 16 / ic horizontally adjacent pixels x ic channels, so one kernel row is
-// nu = ceil(kw / ppc) cells instead of kw.  Packed weights: [kh * nu + j][OCpp rows][16], byte b of
-// unit j = tap kw = j * ppc + b / ic, channel b % ic (zero where kw >= KW or b >= ppc * ic).
-// One thread per packed dword.
+// holds ppc = 16 / icl horizontally adjacent pixels of icl bytes each (icl = ic, or 4 for three channels: see
+// conv_fewch_icl), so one kernel row is nu = ceil(kw / ppc) cells instead of kw.  Packed weights:
+// [kh * nu + j][OCpp rows][16], byte b of unit j = tap kw = j * ppc + b / icl, channel b % icl (zero where
+// kw >= KW, b >= ppc * icl or the channel is the pad byte).  One thread per packed dword.
 __global__ __launch_bounds__(kBlock) void k_quant_pack_direct_px(const float *w, const float *absmax, int oc2n,
-                                                                 int ic, int KH, int KW, int ppc, int nu, int ocpp,
-                                                                 unsigned *wpacked)
+                                                                 int ic, int icl, int KH, int KW, int ppc, int nu,
+                                                                 int ocpp, unsigned *wpacked)
 {
   const long long total = (long long)KH * nu * ocpp * 4;
   const long long idx = (long long)blockIdx.x * kBlock + threadIdx.x;
@@ -140,16 +140,17 @@ __global__ __launch_bounds__(kBlock) void k_quant_pack_direct_px(const float *w,
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int b = 4 * q + k;
-      const int jj = b / ic, c = b - jj * ic, kw = j * ppc + jj;
+      const int jj = b / icl, c = b - jj * icl, kw = j * ppc + jj;
       int v = 0;
-      if (jj < ppc && kw < KW) v = quant_w(w[((size_t)(oc >> 4) * KH * KW + kh * KW + kw) * 256 + c * 16 + (oc & 15)], am);
+      if (jj < ppc && kw < KW && c < ic) v = quant_w(w[((size_t)(oc >> 4) * KH * KW + kh * KW + kw) * 256 + c * 16 + (oc & 15)], am);
       packed |= ((unsigned)v & 0xffu) << (8 * k);
     }
   }
   wpacked[idx] = packed;
 }
 
-// pixel-packed counterpart of k_fold_direct_border: one thread per (class, channel)
+// pixel-packed counterpart of k_fold_direct_border: one thread per (class, channel); ic = bytes per pixel of a
+// cell (pad bytes hold zero weights)
 __global__ __launch_bounds__(kBlock) void k_fold_direct_border_px(const unsigned *wpacked, const float *absmax,
                                                                   const float *bias, int oc_rows, int ic, int ppc,
                                                                   int nu, int ocpp, FoldParams p, const int4 *rects,
@@ -412,15 +413,15 @@ hipError_t launch_prepare_direct(const float *w, const float *bias, int oc, int 
 }
 
 // weight side of the pixel-packed form (see k_quant_pack_direct_px): taps = kh * nu units of one cell
-hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int kh, int kw, int ppc, int nu,
+hipError_t launch_prepare_direct_px(const float *w, const float *bias, int oc, int ic, int icl, int kh, int kw, int ppc, int nu,
                                     int ocpp, const ehip_conv_desc_t &d, float *absmax, int8_t *wpacked, float *scale,
                                     float *shift, int *wsum, int *comp, hipStream_t s)
 {
   const int oc2 = up(oc, 16) / 16;
   hipLaunchKernelGGL(k_absmax_direct, dim3(oc2), dim3(kBlock), 0, s, w, 1, kh * kw, absmax);
   const size_t dwords = (size_t)kh * nu * ocpp * 4;
-  hipLaunchKernelGGL(k_quant_pack_direct_px, grid_for(dwords), dim3(kBlock), 0, s, w, absmax, oc2, ic, kh, kw, ppc, nu,
-                     ocpp, reinterpret_cast<unsigned *>(wpacked));
+  hipLaunchKernelGGL(k_quant_pack_direct_px, grid_for(dwords), dim3(kBlock), 0, s, w, absmax, oc2, ic, icl, kh, kw, ppc,
+                     nu, ocpp, reinterpret_cast<unsigned *>(wpacked));
   const FoldParams fp = make_fold(d, false);
   hipLaunchKernelGGL(k_fold_direct, grid_for(ocpp), dim3(kBlock), 0, s, reinterpret_cast<const unsigned *>(wpacked),
                      absmax, bias, oc2 * 16, kh * nu, 1, ocpp, fp, scale, shift, wsum, comp);

@@ -347,6 +347,20 @@ def test_direct_few_input_channels_output_types(out_type, out_nhwc):
                           in_nhwc=False, out_nhwc=out_nhwc))
 
 
+@pytest.mark.parametrize("pad_pixel", ["0", "1"])
+@pytest.mark.parametrize("in_nhwc", [False, True])
+def test_direct_three_channels_padded_to_four_or_not(pad_pixel, in_nhwc, monkeypatch):
+    # three channels take four bytes per pixel in the staged rows and the cells (every cell starts on a dword),
+    # or three: by default the first for kernels at least five wide only; both forms of every width give the
+    # same bytes
+    monkeypatch.setenv("EHIP_FEWCH_PAD_PIXEL", pad_pixel)
+    for n, hw, k, pad, stride, oc, in_z in [(3, 37, 7, 3, 2, 64, 128.0), (2, 23, 3, 1, 2, 32, 128.0), (3, 9, 3, 1, 1, 16, 0.0),
+                                            (1, 29, 7, 2, 2, 32, 0.0), (2, 16, 5, 2, 1, 16, 0.0)]:
+        res = run_and_compare(Layer(n, 3, oc, hw, k=k, pad=pad, stride=stride, out_type=ol.U8, seed=197 + k + hw,
+                                    in_z=in_z, in_nhwc=in_nhwc))
+        assert res["conv"].kernel_name == "k_conv_fewch_u8s8"
+
+
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 16])
 def test_direct_few_input_channels_strip_heights(rows, monkeypatch):
     # output rows per workgroup, including strips that end below the image
