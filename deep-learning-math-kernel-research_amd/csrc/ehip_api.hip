@@ -638,6 +638,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     if (a.in_nhwc && (reinterpret_cast<uintptr_t>(input_dev) & 3))
       return fail(EHIP_GENERAL_ERROR, "nhwc input of a few-channel layer must be 4-byte aligned");
     HIP_TRY(launch_conv_fewch(a, s, &c->plan_fewch));
+    if (c->plan_fewch.name) c->kernel_name = c->plan_fewch.name;
     break;
   }
   case FAM_CONV_3X3: {

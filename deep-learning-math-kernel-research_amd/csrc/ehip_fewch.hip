@@ -27,24 +27,15 @@ __device__ __forceinline__ unsigned low_bytes(int k)   // mask of the k lowest b
 }
 }  // namespace
 
-template <int KS>
-__global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
+// Section 1 of both kernels: the input rows under the strip (and, with a.tab_lds, the border-class tables and
+// the shift rows of the workgroup's channels) go to LDS.  The caller synchronises.
+struct FewChTables {
+  float *shift;      // [class][wo * 32]
+  int *cls_h, *cls_w;   // class of each of the strip's output rows (times ncls_w) / of each output column
+};
+__device__ __forceinline__ FewChTables fewch_stage(const FewChArgs &a, unsigned *rows_lds, int tid, int img, int ihb,
+                                                   int oh0, int rows_valid)
 {
-  // [nrows_in][lrow / 4] staged rows; with border classes kept on chip (a.tab_lds): the shift rows of
-  // the workgroup's channels [class][wo * 32], then the class of each of the strip's output rows
-  // (times ncls_w) and of each output column
-  extern __shared__ unsigned rows_lds[];
-  __shared__ v4i xpatch[4 * 256];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
-  const int l32 = lane & 31;
-  const int lh = lane >> 5;
-  const int img = blockIdx.x / a.strips, strip = blockIdx.x - img * a.strips;
-  const int oh0 = strip * a.rows;
-  const int rows_valid = a.oh - oh0 < a.rows ? a.oh - oh0 : a.rows;
-  const int npix = rows_valid * a.ow;
-  const int ihb = oh0 * a.stride_h - a.pad_t;   // input row of staged row 0
   const int lrow4 = a.lrow >> 2;
   const int rowbytes = a.iw * a.ic;
 
@@ -145,6 +136,30 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
         }
     }
   }
+  return FewChTables{lds_shift, lds_cls_h, lds_cls_w};
+}
+
+template <int KS>
+__global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
+{
+  // [nrows_in][lrow / 4] staged rows; with border classes kept on chip (a.tab_lds): the shift rows of
+  // the workgroup's channels [class][wo * 32], then the class of each of the strip's output rows
+  // (times ncls_w) and of each output column
+  extern __shared__ unsigned rows_lds[];
+  __shared__ v4i xpatch[4 * 256];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: what depends on it stays scalar
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int img = blockIdx.x / a.strips, strip = blockIdx.x - img * a.strips;
+  const int oh0 = strip * a.rows;
+  const int rows_valid = a.oh - oh0 < a.rows ? a.oh - oh0 : a.rows;
+  const int npix = rows_valid * a.ow;
+  const int ihb = oh0 * a.stride_h - a.pad_t;   // input row of staged row 0
+  const FewChTables tabs = fewch_stage(a, rows_lds, tid, img, ihb, oh0, rows_valid);
+  float *const lds_shift = tabs.shift;
+  int *const lds_cls_h = tabs.cls_h, *const lds_cls_w = tabs.cls_w;
   __syncthreads();
 
   // ---- 2. / 3. tiles --------------------------------------------------------------------------
@@ -260,6 +275,113 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_u8s8(FewChArgs a)
       epilogue_wave<1, 1, true, true>(a.ep, acc, k0, cidx, oc0 + 16 * lh, pix, pvalid, oc_real, block_stride, a.out,
                                       xlds, pixT, validT, cls);
     }
+  }
+}
+
+// The same tiles for u8 / s8 output with ReLU (FewChArgs::lean; TAB: the shift row of the pixel's border class
+// comes from LDS): nothing but that epilogue, so the tile loop is straight-line code with 32-bit output offsets,
+// and the cells of a wave's next tile are read while the present one is scaled and stored.
+template <int KS, bool CLAMP, bool TAB>
+__global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_lean(FewChArgs a)
+{
+  extern __shared__ unsigned rows_lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int img = blockIdx.x / a.strips, strip = blockIdx.x - img * a.strips;
+  const int oh0 = strip * a.rows;
+  const int rows_valid = a.oh - oh0 < a.rows ? a.oh - oh0 : a.rows;
+  const int npix = rows_valid * a.ow;
+  const int ihb = oh0 * a.stride_h - a.pad_t;
+  const FewChTables tabs = fewch_stage(a, rows_lds, tid, img, ihb, oh0, rows_valid);
+  __syncthreads();
+
+  const int wo = wave % a.wo, wp = wave / a.wo, wpn = 4 / a.wo;
+  const int oc0 = (blockIdx.y * a.wo + wo) * 32;
+  const int oc_real = a.oc2 * 16;
+  const int ohw = a.oh * a.ow;
+  v4i wreg[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    wreg[ks] = *reinterpret_cast<const v4i *>(a.w + ((long long)(2 * ks + lh) * a.ocpp + oc0 + l32) * 16);
+  int cell_at[KS];   // as in k_conv_fewch_u8s8
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    int tc = 2 * ks + lh;
+    tc = tc < a.cells ? tc : a.cells - 1;
+    const int kr = tc / a.nu;
+    cell_at[ks] = kr * a.lrow + (tc - kr * a.nu) * a.ppc * a.icl;
+  }
+  const long long cidx = oc0 + 16 * lh;
+  LeanConsts lk[1];
+  load_lean_consts(lk[0], a.ep, cidx);
+  v16i comp0;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const v4i c = *reinterpret_cast<const v4i *>(a.ep.comp + cidx + 4 * q);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) comp0[4 * q + j] = c[j];
+  }
+  // output: a uniform base (the strip's first pixel) and a byte offset per lane that fits 32 bits (the launcher checks)
+  const unsigned px_stride = a.out_nhwc ? (unsigned)oc_real : 16u;
+  uint8_t *const out_base = static_cast<uint8_t *>(a.out) +
+      (a.out_nhwc ? ((size_t)img * ohw + (size_t)oh0 * a.ow) * oc_real : ((size_t)img * a.oc2 * ohw + (size_t)oh0 * a.ow) * 16);
+  const unsigned lane_off = (a.out_nhwc ? (unsigned)(oc0 + 16 * lh) : (unsigned)((oc0 >> 4) + lh) * (unsigned)ohw * 16u) +
+      (unsigned)l32 * px_stride;
+  const float *const shift_rows = TAB ? tabs.shift + wo * 32 + 16 * lh : nullptr;
+  const int tab_width = a.wo * 32;
+  const int row_step = a.stride_h * a.lrow, px_step = a.stride_w * a.icl;
+  const int ntiles = (npix + 31) >> 5;
+
+  int ro, ox;   // output row (in the strip) and column of the lane's pixel of the tile whose cells were read last
+  v4i b[KS];
+  auto read_cells = [&](int tile) {
+    int p = tile * 32 + l32;
+    p = p < npix ? p : npix - 1;   // also beyond the wave's last tile: some cell of the strip
+    ro = fastdiv(p, a.ow, a.ow_magic);
+    ox = p - ro * a.ow;
+    const int at0 = ro * row_step + ox * px_step;
+    if (a.icl == 4) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const unsigned *src = rows_lds + ((at0 + cell_at[ks]) >> 2);
+        b[ks] = v4i{(int)src[0], (int)src[1], (int)src[2], (int)src[3]};
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int A = at0 + cell_at[ks];
+        const unsigned *src = rows_lds + (A >> 2);
+        const unsigned sh = A & 3;
+        const unsigned d0 = src[0], d1 = src[1], d2 = src[2], d3 = src[3], d4 = src[4];
+        b[ks] = v4i{(int)__builtin_amdgcn_alignbyte(d1, d0, sh), (int)__builtin_amdgcn_alignbyte(d2, d1, sh),
+                    (int)__builtin_amdgcn_alignbyte(d3, d2, sh), (int)__builtin_amdgcn_alignbyte(d4, d3, sh)};
+      }
+    }
+  };
+  read_cells(wp);
+  for (int tile = wp; tile < ntiles; tile += wpn) {
+    v16i acc[1][1];
+    acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[0], b[0], comp0, 0, 0, 0);
+#pragma unroll
+    for (int ks = 1; ks < KS; ++ks) acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[ks], b[ks], acc[0][0], 0, 0, 0);
+    if (TAB) {
+      const float *row = shift_rows + (tabs.cls_h[ro] + tabs.cls_w[ox]) * tab_width;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) lk[0].sh[q] = *reinterpret_cast<const float4 *>(row + 4 * q);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    read_cells(tile + wpn);   // the MFMAs above have taken their operands
+    __builtin_amdgcn_sched_barrier(0);
+    const int p0 = tile * 32;
+    const bool pvalid[1] = {p0 + l32 < npix};
+    uint8_t *const cell[1] = {out_base + ((unsigned)p0 * px_stride + lane_off)};
+    // blocked output: non-temporal stores (3x3 s2 3 -> 32 at 224 x 224, N = 64: 15.9 -> 14.3 us); in nhwc a line's
+    // 16-byte pieces come from several waves and should meet in L2 (7x7 s2 3 -> 64: 32.9 -> 37.6 us with them)
+    if (a.out_nhwc) lean_store_typed<1, 1, false, CLAMP, false>(a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, 0, nullptr);
+    else lean_store_typed<1, 1, false, CLAMP, true>(a.ep, acc, lk, cell, pvalid, oc0 + 16 * lh, oc_real, 0, nullptr);
   }
 }
 
@@ -383,7 +505,21 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
   const int ks = (a.cells + 1) / 2;
   void (*kern)(FewChArgs) = ks <= 2 ? k_conv_fewch_u8s8<2> : ks == 3 ? k_conv_fewch_u8s8<3> : ks == 4 ? k_conv_fewch_u8s8<4>
       : ks == 5 ? k_conv_fewch_u8s8<5> : k_conv_fewch_u8s8<7>;
-  return plan_launch(plan, kern, dim3(a.n * a.strips, gy), dim3(kBlock), lds, a, s);
+  const char *name = "k_conv_fewch_u8s8";
+  // the kernel of the lean epilogue alone: shift rows per channel or on chip, an image's output below 2 GB
+  const char *env_lean = getenv("EHIP_FEWCH_LEAN_KERNEL");
+  if (a.lean && !(env_lean && env_lean[0] == '0') && (!a.ep.shift_tab || a.tab_lds) &&
+      (long long)a.oc2 * 16 * a.oh * a.ow < (1ll << 31)) {
+    const bool clamp = !(a.lean & 2), tab = a.tab_lds != 0;
+#define FL(K) (clamp ? (tab ? k_conv_fewch_lean<K, true, true> : k_conv_fewch_lean<K, true, false>) \
+                     : (tab ? k_conv_fewch_lean<K, false, true> : k_conv_fewch_lean<K, false, false>))
+    kern = ks <= 2 ? FL(2) : ks == 3 ? FL(3) : ks == 4 ? FL(4) : ks == 5 ? FL(5) : FL(7);
+#undef FL
+    name = "k_conv_fewch_lean";
+  }
+  const hipError_t e = plan_launch(plan, kern, dim3(a.n * a.strips, gy), dim3(kBlock), lds, a, s);
+  if (plan) plan->name = name;
+  return e;
 }
 
 }  // namespace ehip

@@ -307,7 +307,7 @@ def test_direct_zero_point_with_padding(out_type, n, ic, oc, hw, k, pad, stride,
     res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=140 + k + stride,
                                 out_hw=out_hw, in_z=128.0, with_relu=(out_type != ol.F32)))
     if pad or out_hw:
-        assert res["conv"].kernel_name.startswith("k_conv_fewch_u8s8" if ic <= 4 else "k_gemm_u8s8")
+        assert res["conv"].kernel_name.startswith("k_conv_fewch" if ic <= 4 else "k_gemm_u8s8")
 
 
 # at most four input channels (first layers; the reference feeds them 3-channel nhwc,
@@ -331,11 +331,11 @@ FEWCH_SHAPES = [
 def test_direct_few_input_channels(in_z, in_nhwc, n, ic, oc, hw, k, pad, stride, out_hw, monkeypatch):
     layer = dict(k=k, pad=pad, stride=stride, out_type=ol.U8, seed=170 + k + ic, out_hw=out_hw, in_z=in_z)
     res = run_and_compare(Layer(n, ic, oc, hw, in_nhwc=in_nhwc, **layer))
-    assert res["conv"].kernel_name == "k_conv_fewch_u8s8"
+    assert res["conv"].kernel_name.startswith("k_conv_fewch")
     if not in_nhwc:
         monkeypatch.setenv("EHIP_FEWCH", "0")     # the general kernels give the same bytes
         res2 = run_and_compare(Layer(n, ic, oc, hw, **layer))
-        assert res2["conv"].kernel_name != "k_conv_fewch_u8s8"
+        assert not res2["conv"].kernel_name.startswith("k_conv_fewch")
 
 
 @pytest.mark.parametrize("out_type,out_nhwc", [(ol.S32, False), (ol.F32, False), (ol.S8, False), (ol.S8, True),
@@ -358,7 +358,24 @@ def test_direct_three_channels_padded_to_four_or_not(pad_pixel, in_nhwc, monkeyp
                                             (1, 29, 7, 2, 2, 32, 0.0), (2, 16, 5, 2, 1, 16, 0.0)]:
         res = run_and_compare(Layer(n, 3, oc, hw, k=k, pad=pad, stride=stride, out_type=ol.U8, seed=197 + k + hw,
                                     in_z=in_z, in_nhwc=in_nhwc))
-        assert res["conv"].kernel_name == "k_conv_fewch_u8s8"
+        assert res["conv"].kernel_name.startswith("k_conv_fewch")
+
+
+@pytest.mark.parametrize("lean_kernel", ["0", "1"])
+@pytest.mark.parametrize("out_type,out_nhwc,with_relu", [(ol.U8, False, True), (ol.S8, True, True), (ol.U8, True, True),
+                                                         (ol.S8, False, True), (ol.S8, False, False)])
+def test_direct_few_input_channels_lean_kernel(lean_kernel, out_type, out_nhwc, with_relu, monkeypatch):
+    # u8 / s8 output with ReLU has a kernel of its own (straight-line tile loop, the next tile's cells read during
+    # the epilogue); EHIP_FEWCH_LEAN_KERNEL=0 sends those layers through the general one: the same bytes.  With and
+    # without border classes (input zero point), every number of cells per tile, channel tiles over several waves.
+    monkeypatch.setenv("EHIP_FEWCH_LEAN_KERNEL", lean_kernel)
+    want = "k_conv_fewch_lean" if (lean_kernel == "1" and with_relu) else "k_conv_fewch_u8s8"
+    for n, ic, oc, hw, k, pad, stride, in_z, in_nhwc in [(2, 3, 64, 37, 7, 3, 2, 128.0, True), (2, 3, 32, 23, 3, 1, 2, 128.0, True),
+                                                         (1, 4, 16, 13, 5, 2, 1, 0.0, False), (2, 1, 96, 17, 3, 1, 1, 3.0, True),
+                                                         (1, 2, 128, 21, 7, 3, 2, 0.0, True), (3, 3, 16, 9, 5, 2, 1, 128.0, False)]:
+        res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=230 + k + ic,
+                                    in_z=in_z, in_nhwc=in_nhwc, out_nhwc=out_nhwc, with_relu=with_relu))
+        assert res["conv"].kernel_name == want
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 16])

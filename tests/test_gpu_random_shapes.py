@@ -80,7 +80,7 @@ def test_random_first_layer(seed):
     res = run_and_compare(Layer(int(r.integers(1, 4)), ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type,
                                 seed=seed, out_hw=out_hw, in_z=in_z, in_nhwc=bool(r.integers(0, 2)),
                                 out_nhwc=bool(r.integers(0, 2)), with_relu=(out_type != ol.F32 or in_z == 0.0)))
-    assert res["conv"].kernel_name == "k_conv_fewch_u8s8"
+    assert res["conv"].kernel_name.startswith("k_conv_fewch")
 
 
 @pytest.mark.parametrize("seed", range(16))
