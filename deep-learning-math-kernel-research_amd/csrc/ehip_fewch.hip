@@ -67,7 +67,54 @@ __device__ __forceinline__ FewChTables fewch_stage(const FewChArgs &a, unsigned 
       lds_shift[idx] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - c * width)];
     }
   }
-  if (a.in_nhwc) {
+  if (a.in_nhwc && a.icl != a.ic) {
+    // Three channels staged as four bytes.  A thread takes four pixels: their twelve bytes, wherever they lie, come
+    // out of four aligned dwords shifted together, and go to LDS as the four staged dwords at once (a staged row is
+    // a whole number of such groups; group q of a row = pixels 4 q - pad_l ...).  Dwords outside the image hold
+    // nothing of these pixels: any address inside will do for them.
+    constexpr int kGroupDepth = 2;
+    const int lrow16 = a.lrow >> 4;
+    const int total = a.nrows_in * lrow16;
+    for (int base = 0; base < total; base += kBlock * kGroupDepth) {
+      unsigned v[kGroupDepth][4];
+      int x0[kGroupDepth], sft[kGroupDepth];
+      bool inside[kGroupDepth];
+#pragma unroll
+      for (int u = 0; u < kGroupDepth; ++u) {
+        int idx = base + u * kBlock + tid;
+        idx = idx < total ? idx : total - 1;
+        const int r = fastdiv(idx, lrow16, a.lrow16_magic);
+        const int h = ihb + r;
+        x0[u] = 4 * (idx - r * lrow16) - a.pad_l;
+        inside[u] = (unsigned)h < (unsigned)a.ih;
+        const int g = e0 + (h * a.iw + x0[u]) * 3;
+        sft[u] = g & 3;
+        const int ga = g & ~3;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          int at = ga + 4 * k;
+          at = at < 0 ? 0 : at > last_dw ? last_dw : at;
+          v[u][k] = *reinterpret_cast<const unsigned *>(in_al + (unsigned)at);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kGroupDepth; ++u) {
+        const int idx = base + u * kBlock + tid;
+        const unsigned p0 = __builtin_amdgcn_alignbyte(v[u][1], v[u][0], sft[u]);
+        const unsigned p1 = __builtin_amdgcn_alignbyte(v[u][2], v[u][1], sft[u]);
+        const unsigned p2 = __builtin_amdgcn_alignbyte(v[u][3], v[u][2], sft[u]);
+        const unsigned px[4] = {p0, __builtin_amdgcn_alignbyte(p1, p0, 3), __builtin_amdgcn_alignbyte(p2, p1, 2), p2 >> 8};
+        uint4 o;
+        unsigned *const ov = reinterpret_cast<unsigned *>(&o);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool ok = inside[u] && (unsigned)(x0[u] + j) < (unsigned)a.iw;
+          ov[j] = (px[j] & (ok ? 0x00ffffffu : 0u)) ^ 0x80808080u;
+        }
+        if (idx < total) *reinterpret_cast<uint4 *>(rows_lds + 4 * idx) = o;
+      }
+    }
+  } else if (a.in_nhwc) {
     const int total = a.nrows_in * lrow4;
     for (int base = 0; base < total; base += kBlock * kStageDepth) {
       unsigned v[kStageDepth], v2[kStageDepth], m[kStageDepth], sft[kStageDepth];
@@ -79,19 +126,10 @@ __device__ __forceinline__ FewChTables fewch_stage(const FewChArgs &a, unsigned 
         const int d = idx - r * lrow4;
         const int h = ihb + r;
         const bool inside = (unsigned)h < (unsigned)a.ih;
-        int g;
-        if (a.icl != a.ic) {
-          // three channels staged as four bytes: dword d of a staged row is pixel d - pad_l, its three bytes
-          // wherever they lie in memory, and a pad byte
-          const int x = d - a.pad_l;
-          g = e0 + (h * a.iw + x) * 3;
-          m[u] = inside && (unsigned)x < (unsigned)a.iw ? 0x00ffffffu : 0u;
-        } else {
-          g = g00 + r * rowbytes + 4 * d;   // first byte of the staged dword
-          const int rs = g00 + r * rowbytes + a.pad_l * a.ic;   // first byte of the input row
-          const int lo = rs - g, hi = rs + rowbytes - g;        // bytes lo .. hi - 1 of the dword belong to the row
-          m[u] = inside ? low_bytes(hi) & ~low_bytes(lo) : 0u;
-        }
+        const int g = g00 + r * rowbytes + 4 * d;   // first byte of the staged dword
+        const int rs = g00 + r * rowbytes + a.pad_l * a.ic;   // first byte of the input row
+        const int lo = rs - g, hi = rs + rowbytes - g;        // bytes lo .. hi - 1 of the dword belong to the row
+        m[u] = inside ? low_bytes(hi) & ~low_bytes(lo) : 0u;
         // dwords outside the image hold nothing of the row: any address inside will do for them
         int ga = g & ~3, gb = ga + 4;
         ga = ga < 0 ? 0 : ga > last_dw ? last_dw : ga;
@@ -388,12 +426,10 @@ __global__ __launch_bounds__(kBlock, 3) void k_conv_fewch_lean(FewChArgs a)
 int conv_fewch_icl(int ic, int kw)
 {
   if (ic != 3 || (kw + 3) / 4 != (kw + 4) / 5) return ic;
-  // 7x7, stride 2 at 224 x 224, N = 64: 33.6 -> 29.1 us (a cell is four dword reads instead of five and four
-  // byte shifts); 3x3, stride 2: 16.0 -> 16.8 us -- with one cell per kernel row the third more dwords to
-  // stage cost more than the cells save.  So by default only kernels at least five wide.
+  // A cell is four dword reads instead of five and four byte shifts, and nhwc input is staged four pixels per
+  // thread: 7x7, stride 2 at 224 x 224, N = 64: 31.9 -> 26.4 us; 3x3, stride 2: 13.9 -> 12.6 us.
   const char *env = getenv("EHIP_FEWCH_PAD_PIXEL");
-  if (env && env[0]) return env[0] == '0' ? 3 : 4;
-  return kw >= 5 ? 4 : 3;
+  return env && env[0] == '0' ? 3 : 4;
 }
 
 bool conv_fewch_applies(int ic, int kh, int kw)
@@ -411,7 +447,8 @@ int conv_fewch_row_pitch(int icl, int kw, int iw, int ow, int stride_w, int pad_
   int need = (pad_l + iw) * icl;
   const int last = ((ow - 1) * stride_w + (nu - 1) * ppc) * icl + 16;
   if (last > need) need = last;
-  return up(need + 4, 4) + 4;
+  // four-byte pixels: whole 16-byte groups (the staging writes four pixels at a time); else the cell reads' fifth dword
+  return icl == 4 ? up(need + 4, 16) : up(need + 4, 4) + 4;
 }
 
 // Fills the derived fields (cells, strip height, LDS row pitch, wave split) and launches.
@@ -500,6 +537,7 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
   a.ow_magic = div_magic(a.ow);
   a.iw_magic = div_magic(a.iw);
   a.lrow4_magic = div_magic(a.lrow / 4);
+  a.lrow16_magic = div_magic(a.lrow / 16 > 0 ? a.lrow / 16 : 1);
   if ((long long)a.nrows_in * (a.lrow / 4) * (a.lrow / 4) >= (1ll << 32) || (long long)a.nrows_in * a.iw * a.iw >= (1ll << 32))
     return hipErrorInvalidValue;
   const int ks = (a.cells + 1) / 2;

@@ -229,13 +229,12 @@ struct FewChArgs {
   int wo;               // waves of a workgroup along the channels (1, 2, 4)
   int icl;              // bytes per pixel in a staged row and in an operand cell (conv_fewch_icl); set by the caller
   int lean;             // lean_mode() of the epilogue, per-pixel shift rows allowed (0 = general epilogue)
-  unsigned ow_magic, iw_magic, lrow4_magic;
+  unsigned ow_magic, iw_magic, lrow4_magic, lrow16_magic;
 };
 // Bytes a pixel takes in the staged rows and operand cells of the few-channel kernel: its ic channels, except
 // that three channels are padded to four (the fourth multiplies a zero weight) where that costs no extra cell
 // per kernel row (3x3 and 7x7 kernels: ceil(kw / 4) == ceil(kw / 5)) -- every cell then starts on a dword.
-// By default only for kernels at least five wide; EHIP_FEWCH_PAD_PIXEL=0 never, =1 wherever it can.  A handle
-// asks once and keeps the answer.
+// EHIP_FEWCH_PAD_PIXEL=0 keeps three bytes.  A handle asks once and keeps the answer.
 int conv_fewch_icl(int ic, int kw);
 bool conv_fewch_applies(int ic, int kh, int kw);
 int conv_fewch_row_pitch(int icl, int kw, int iw, int ow, int stride_w, int pad_l);   // icl: conv_fewch_icl()

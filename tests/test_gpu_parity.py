@@ -350,9 +350,8 @@ def test_direct_few_input_channels_output_types(out_type, out_nhwc):
 @pytest.mark.parametrize("pad_pixel", ["0", "1"])
 @pytest.mark.parametrize("in_nhwc", [False, True])
 def test_direct_three_channels_padded_to_four_or_not(pad_pixel, in_nhwc, monkeypatch):
-    # three channels take four bytes per pixel in the staged rows and the cells (every cell starts on a dword),
-    # or three: by default the first for kernels at least five wide only; both forms of every width give the
-    # same bytes
+    # three channels take four bytes per pixel in the staged rows and the cells (every cell starts on a dword;
+    # the default wherever it costs no extra cell per kernel row), or three: the same bytes either way
     monkeypatch.setenv("EHIP_FEWCH_PAD_PIXEL", pad_pixel)
     for n, hw, k, pad, stride, oc, in_z in [(3, 37, 7, 3, 2, 64, 128.0), (2, 23, 3, 1, 2, 32, 128.0), (3, 9, 3, 1, 1, 16, 0.0),
                                             (1, 29, 7, 2, 2, 32, 0.0), (2, 16, 5, 2, 1, 16, 0.0)]:
