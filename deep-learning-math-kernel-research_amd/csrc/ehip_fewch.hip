@@ -501,10 +501,12 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
       const int nrows_in = (r - 1) * a.stride_h + a.kh;
       const size_t dyn = (size_t)nrows_in * a.lrow + 32;
       if (dyn > 40 * 1024) break;
-      // workgroups of 4 waves resident per CU: registers (3 waves per SIMD), LDS (16 KB static
-      // exchange patch + the rows)
-      int resident = 3;
-      const int by_lds = (int)((160 * 1024) / (16 * 1024 + dyn));
+      // workgroups of 4 waves resident per CU: registers (3 waves per SIMD; 4 for the lean kernel with at most
+      // five operands, which stays below 128 registers), LDS (the general kernel's 16 KB static exchange patch +
+      // the rows).  3x3 s2 3 -> 32 at 224 x 224, N = 64: strips of 7 rows (4 workgroups per CU) 12.0 us, of 10 rows
+      // (3 per CU) 12.6 us.
+      int resident = (a.lean && (a.cells + 1) / 2 <= 5) ? 4 : 3;
+      const int by_lds = (int)((160 * 1024) / ((a.lean ? 0 : 16 * 1024) + dyn));
       if (by_lds < resident) resident = by_lds < 1 ? 1 : by_lds;
       const double slots = (double)n_cu * resident;
       const double wgs = (double)a.n * ((a.oh + r - 1) / r) * gy;
