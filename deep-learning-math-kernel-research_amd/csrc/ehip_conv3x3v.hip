@@ -643,7 +643,6 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
   a.tiles = (int)tiles;
   a.tiles_per_xcd = (a.tiles + 7) / 8;
   a.lean = lean_mode(a.ep, false);
-  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   dim3 grid(8 * a.tiles_per_xcd, 1, 1);
   conv3x3v_kernel_t kernel = k.kernel;
   if (a.units_pad == a.chunk_units) {   // one fill holds every unit

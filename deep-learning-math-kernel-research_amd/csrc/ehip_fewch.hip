@@ -467,7 +467,6 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
     e.shift_tab = nullptr;
     a.lean = lean_mode(e, false);
     if (a.ep.with_sum) a.lean = 0;
-    if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   }
   if (a.icl != a.ic && !(a.ic == 3 && a.icl == 4)) return hipErrorInvalidValue;
   a.ppc = 16 / a.icl;

@@ -692,7 +692,6 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
 {
   GemmArgs a = a0;
   a.lean = lean_mode(a.ep, false);   // blocked and nhwc output alike
-  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   const int ks = a.ic2 <= 2 ? 1 : (a.ic2 <= 4 ? 2 : 4);
   const int oc_tiles = (a.oc2 * 16 + 31) / 32;
   // one tile of 32 channels per wave (its constants then stay in registers) x two tiles of 32 pixels
@@ -759,7 +758,6 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   const Variant &k = kVariants[variant];
   GemmArgs a = a0;
   a.lean = lean_mode(a.ep, false);   // blocked and nhwc output alike
-  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8), nbatch);

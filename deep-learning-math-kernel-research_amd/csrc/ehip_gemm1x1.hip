@@ -441,7 +441,6 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
   const ResVariant &k = kRes[v];
   GemmArgs a = a0;
   a.lean = lean_mode(a.ep, false);
-  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') a.lean = 0;
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   const int nks = a.units_pad / 2;

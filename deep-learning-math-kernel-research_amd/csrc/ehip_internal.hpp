@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string>
 
 #include "euler_hip.h"
@@ -597,9 +598,11 @@ __device__ __forceinline__ void load_lean_consts(LeanConsts &k, const Epilogue &
     k.sh[q] = *reinterpret_cast<const float4 *>(ep.shift + idx + 4 * q);
   }
 }
-// 0 = general epilogue; else bit 0 set, bit 1 = no clamp needed, bit 2 = with sum
+// 0 = general epilogue; else bit 0 set, bit 1 = no clamp needed, bit 2 = with sum.  EHIP_LEAN_EPILOGUE=0 switches
+// it off here, in the one place every launcher and every choice of kernel that depends on it asks.
 inline int lean_mode(const Epilogue &e, bool out_nhwc)
 {
+  if (const char *env = getenv("EHIP_LEAN_EPILOGUE")) if (env[0] == '0') return 0;
   const bool q = e.out_type == EHIP_U8 || e.out_type == EHIP_S8;
   const bool fast = q && e.with_relu && !e.shift_tab && !out_nhwc && e.lo >= 0.0f && e.hi >= e.lo &&
       (e.out_type != EHIP_S8 || e.lo <= 127.0f);

@@ -94,6 +94,11 @@ def test_conv1x1_resident_pixel_tile_kernel_nhwc_output(variant, n, ic, oc, hw, 
     # what the lean epilogue does not cover goes through the general kernel
     res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=ol.F32, out_nhwc=True, seed=331 + ic))
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
+    # and so does everything when the lean epilogue is switched off: the switch must reach the choice of kernel, not
+    # only the launcher (this kernel's general epilogue writes blocked output only)
+    monkeypatch.setenv("EHIP_LEAN_EPILOGUE", "0")
+    res = run_and_compare(Layer(n, ic, oc, hw, stride=stride, out_type=ol.S8, with_sum=True, out_nhwc=True, seed=332 + ic))
+    assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
 @pytest.mark.parametrize("variant", ["", "2", "4"])
