@@ -45,6 +45,8 @@ EXTRA_FLAGS = {
     # (and its straight-line K loops are 72 steps of ~250 instructions: beyond the default budget of
     # `#pragma unroll`, which then leaves a loop whose weight registers are indexed at run time, i.e. in scratch)
     "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-pragma-unroll-threshold=1000000"],
+    # the resident-tile 1x1 kernel's leading scalar arguments: preloaded as well
+    "ehip_gemm1x1.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 

@@ -90,9 +90,20 @@ __device__ __forceinline__ void wait_loads_but(int n)
 // clock over all banks.  A wave-load still fills 64 consecutive LDS cells; its lane i fetches whatever cell
 // 64 j + i of that layout is (the pad cell and padded units repeat a real unit: they multiply zero weights or
 // nothing).  The whole tile is waited for before the K loop (no unit order to consume it in).
+// What a wave's first instructions need -- the three pointers its first loads go through and the geometry
+// their addresses are made of -- is passed as leading scalar arguments, which the dispatcher preloads into scalar
+// registers with the wave (the file is compiled with -amdgpu-kernarg-preload-count=16); the rest of the argument
+// block is loaded as usual while those loads fly.  geom = stride_h | stride_w << 8 | dense << 16 | oc2 << 20.
+#define EHIP_RES_HEAD                                                                                                  \
+  const uint8_t *in, const int8_t *w, const int *comp, int nx, int ny, int p_total, int ohw, unsigned ohw_magic, int ihw, \
+      int ic2, int units_pad, int ocpp, unsigned geom
 template <int TM, int TN, int NKS, bool NHWC = false>
-__global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
+__global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(EHIP_RES_HEAD, GemmArgs rest)
 {
+  GemmArgs a = rest;
+  a.in = in; a.w = w; a.ep.comp = comp; a.nx = nx; a.ny = ny; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic;
+  a.ihw = ihw; a.ic2 = ic2; a.units_pad = units_pad; a.ocpp = ocpp;
+  a.stride_h = (int)(geom & 0xffu); a.stride_w = (int)((geom >> 8) & 0xffu); a.oc2 = (int)(geom >> 20);
   constexpr int OC_T = 4 * TM * 32;
   constexpr int P_T = TN * 32;
   // Weight ring: k-steps requested ahead.  A kernel launch starts with cold L2s, and in a layer of ONE
@@ -118,7 +129,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
   const int oc0 = by * OC_T + wave * TM * 32;   // the wave's first channel
   const int oc_real = a.oc2 * 16;
   const int nks = a.units_pad >> 1;
-  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  const bool dense = (geom >> 16) & 1u;   // stride 1 and the output plane is the input plane
   TRACE_POINT(0);
 
   // ---- the accumulators start from the compensation ------------------------------------------------
@@ -352,14 +363,24 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(GemmArgs a)
 }
 
 namespace {
+typedef void (*res_kernel_t)(EHIP_RES_HEAD, GemmArgs);
 struct ResVariant {
   const char *name;
   int oc_t, p_t;
-  void (*generic)(GemmArgs);
-  void (*unrolled[3])(GemmArgs);   // exactly 8, 16, 32 k-steps
-  void (*generic_nhwc)(GemmArgs);  // nhwc input (64-pixel tiles only), or null
-  void (*unrolled_nhwc[3])(GemmArgs);
+  res_kernel_t generic;
+  res_kernel_t unrolled[3];   // exactly 8, 16, 32 k-steps
+  res_kernel_t generic_nhwc;  // nhwc input (64-pixel tiles only), or null
+  res_kernel_t unrolled_nhwc[3];
 };
+hipError_t res_enqueue(const LaunchPlan<GemmArgs> &plan, hipStream_t s)
+{
+  const GemmArgs &a = plan.args;
+  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  const unsigned geom = (unsigned)a.stride_h | (unsigned)a.stride_w << 8 | (dense ? 1u << 16 : 0u) | (unsigned)a.oc2 << 20;
+  hipLaunchKernelGGL(reinterpret_cast<res_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.ep.comp,
+                     a.nx, a.ny, a.p_total, a.ohw, a.ohw_magic, a.ihw, a.ic2, a.units_pad, a.ocpp, geom, a);
+  return hipGetLastError();
+}
 #define RV(TM, TN)                                                                                           \
   { "k_gemm1x1_res<" #TM "," #TN ">", 4 * TM * 32, TN * 32, k_gemm1x1_res<TM, TN, 0>,                        \
     {k_gemm1x1_res<TM, TN, 8>, k_gemm1x1_res<TM, TN, 16>, k_gemm1x1_res<TM, TN, 32>}, nullptr, {nullptr, nullptr, nullptr} }
@@ -444,10 +465,10 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
   a.nx = (a.p_total + k.p_t - 1) / k.p_t;
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   const int nks = a.units_pad / 2;
-  void (*kernel)(GemmArgs) = a.in_nhwc ? k.generic_nhwc : k.generic;
+  res_kernel_t kernel = a.in_nhwc ? k.generic_nhwc : k.generic;
   const char *env = getenv("EHIP_GEMM1X1_UNROLL");
   if (!(env && env[0] == '0')) {
-    void (*const *un)(GemmArgs) = a.in_nhwc ? k.unrolled_nhwc : k.unrolled;
+    const res_kernel_t *un = a.in_nhwc ? k.unrolled_nhwc : k.unrolled;
     if (nks == 8) kernel = un[0];
     else if (nks == 16) kernel = un[1];
     else if (nks == 32) kernel = un[2];
@@ -459,8 +480,18 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
                                      (int)lds_bytes);
   if (e != hipSuccess) return e;
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
-  if (plan) plan->name = k.name;   // (nhwc output: the handle could not tell at creation whether the lean epilogue applies)
-  return plan_launch(plan, kernel, grid, dim3(kBlock), lds_bytes, a, s);
+  if (a.stride_h > 255 || a.stride_w > 255 || a.oc2 >= 4096) return hipErrorInvalidValue;   // geom's fields
+  LaunchPlan<GemmArgs> local;
+  LaunchPlan<GemmArgs> *p = plan ? plan : &local;
+  p->valid = true;
+  p->kernel = reinterpret_cast<void (*)(GemmArgs)>(kernel);
+  p->grid = grid;
+  p->block = dim3(kBlock);
+  p->lds = (unsigned)lds_bytes;
+  p->args = a;
+  p->enqueue = res_enqueue;
+  p->name = k.name;   // (nhwc output: the handle could not tell at creation whether the lean epilogue applies)
+  return res_enqueue(*p, s);
 }
 
 }  // namespace ehip

@@ -149,6 +149,9 @@ struct LaunchPlan {
   unsigned lds = 0;
   Args args;
   const char *name = nullptr;   // set by a launcher whose choice of kernel the handle cannot know beforehand
+  // set by a launcher whose kernel takes leading scalar arguments besides the block (`kernel` is then that
+  // kernel's pointer under the one-argument type): how to launch the plan
+  hipError_t (*enqueue)(const LaunchPlan &, hipStream_t) = nullptr;
 };
 template <typename Args>
 inline hipError_t plan_launch(LaunchPlan<Args> *plan, void (*kernel)(Args), dim3 grid, dim3 block, size_t lds, const Args &a,
@@ -168,6 +171,7 @@ inline hipError_t plan_launch(LaunchPlan<Args> *plan, void (*kernel)(Args), dim3
 template <typename Args>
 inline hipError_t plan_relaunch(LaunchPlan<Args> &plan, hipStream_t s)
 {
+  if (plan.enqueue) return plan.enqueue(plan, s);
   hipLaunchKernelGGL(plan.kernel, plan.grid, plan.block, plan.lds, s, plan.args);
   return hipGetLastError();
 }
