@@ -47,6 +47,8 @@ EXTRA_FLAGS = {
     "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-pragma-unroll-threshold=1000000"],
     # the resident-tile 1x1 kernel's leading scalar arguments: preloaded as well
     "ehip_gemm1x1.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    # and those of the 1x1 kernels with few input channels
+    "ehip_gemm.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 

@@ -358,9 +358,21 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_u8s8(GemmArgs a)
 // The four waves of a workgroup split into a.sk_wo tiles of 32 channels (1, 2 or 4) times
 // 4 / a.sk_wo pixel tiles of TNW x 32 pixels; waves of different channel groups walk the same tiles at the same time,
 // so the activations reach the CU once.  grid: (workgroups over pixel tiles, 4-wave channel blocks).
+// What a wave's first loads need -- the two pointers and the geometry their addresses are made of -- is passed as
+// leading scalar arguments, which the dispatcher preloads into scalar registers with the wave (the file is compiled
+// with -amdgpu-kernarg-preload-count=16); the rest of the argument block is loaded as usual meanwhile.
+// geom = stride_h | stride_w << 8 | dense << 16 | in_nhwc << 17 | out_nhwc << 18 | sk_wo << 20.
+#define EHIP_SMALLK_HEAD                                                                                             \
+  const uint8_t *in, const int8_t *w, int p_total, int ohw, unsigned ohw_magic, int ihw, int ic2, int ocpp, int oc2, \
+      unsigned geom, int iw, int ow, unsigned ow_magic
 template <int TNW, int KS>
-__global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
+__global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(EHIP_SMALLK_HEAD, GemmArgs rest)
 {
+  GemmArgs a = rest;
+  a.in = in; a.w = w; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic; a.ihw = ihw; a.ic2 = ic2; a.ocpp = ocpp;
+  a.oc2 = oc2; a.iw = iw; a.ow = ow; a.ow_magic = ow_magic;
+  a.stride_h = (int)(geom & 0xffu); a.stride_w = (int)((geom >> 8) & 0xffu);
+  a.in_nhwc = (int)((geom >> 17) & 1u); a.out_nhwc = (int)((geom >> 18) & 1u); a.sk_wo = (int)(geom >> 20);
   __shared__ v4i xpatch[4 * 256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -490,8 +502,13 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_u8s8(GemmArgs a)
 // wave's channels sit in a wave-private piece of LDS -- in registers they would take 48 per tile -- and every
 // lane of a half-wave reads the same 16 bytes of them (a broadcast).
 template <int KS, int OCW>
-__global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(GemmArgs a)
+__global__ __launch_bounds__(kBlock, 2) void k_gemm_smallk_lean(EHIP_SMALLK_HEAD, GemmArgs rest)
 {
+  GemmArgs a = rest;
+  a.in = in; a.w = w; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic; a.ihw = ihw; a.ic2 = ic2; a.ocpp = ocpp;
+  a.oc2 = oc2; a.iw = iw; a.ow = ow; a.ow_magic = ow_magic;
+  a.stride_h = (int)(geom & 0xffu); a.stride_w = (int)((geom >> 8) & 0xffu);
+  a.in_nhwc = (int)((geom >> 17) & 1u); a.out_nhwc = (int)((geom >> 18) & 1u); a.sk_wo = (int)(geom >> 20);
   __shared__ float4 cst_lds[4 * OCW * 24];   // [wave][tile][scale | shift | compensation][8 cells of 4 channels]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -672,10 +689,35 @@ int gemm_pick_variant(int p_total, int oc2, int ic2, int nbatch, int stride)
 }
 
 namespace {
+typedef void (*smallk_kernel_t)(EHIP_SMALLK_HEAD, GemmArgs);
 template <int KS>
-void (*smallk_kernel(int tnw))(GemmArgs)
+smallk_kernel_t smallk_kernel(int tnw)
 {
   return tnw == 2 ? k_gemm_smallk_u8s8<2, KS> : k_gemm_smallk_u8s8<1, KS>;
+}
+hipError_t smallk_enqueue(const LaunchPlan<GemmArgs> &plan, hipStream_t s)
+{
+  const GemmArgs &a = plan.args;
+  const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
+  const unsigned geom = (unsigned)a.stride_h | (unsigned)a.stride_w << 8 | (dense ? 1u << 16 : 0u) | (a.in_nhwc ? 1u << 17 : 0u) |
+      (a.out_nhwc ? 1u << 18 : 0u) | (unsigned)a.sk_wo << 20;
+  hipLaunchKernelGGL(reinterpret_cast<smallk_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.p_total,
+                     a.ohw, a.ohw_magic, a.ihw, a.ic2, a.ocpp, a.oc2, geom, a.iw, a.ow, a.ow_magic, a);
+  return hipGetLastError();
+}
+hipError_t smallk_launch(LaunchPlan<GemmArgs> *plan, smallk_kernel_t kernel, dim3 grid, const GemmArgs &a, hipStream_t s)
+{
+  if (a.stride_h > 255 || a.stride_w > 255) return hipErrorInvalidValue;   // geom's fields
+  LaunchPlan<GemmArgs> local;
+  LaunchPlan<GemmArgs> *p = plan ? plan : &local;
+  p->valid = true;
+  p->kernel = reinterpret_cast<void (*)(GemmArgs)>(kernel);
+  p->grid = grid;
+  p->block = dim3(kBlock);
+  p->lds = 0;
+  p->args = a;
+  p->enqueue = smallk_enqueue;
+  return smallk_enqueue(*p, s);
 }
 }  // namespace
 
@@ -708,7 +750,7 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
   if (const char *env = getenv("EHIP_SMALLK_WGS")) wgs = atoi(env) > 0 ? atoi(env) : wgs;
   const int cap = (wgs + ny - 1) / ny;
   if (nx > cap) nx = cap;
-  void (*kernel)(GemmArgs) = ks == 1 ? smallk_kernel<1>(tnw) : (ks == 2 ? smallk_kernel<2>(tnw) : smallk_kernel<4>(tnw));
+  smallk_kernel_t kernel = ks == 1 ? smallk_kernel<1>(tnw) : (ks == 2 ? smallk_kernel<2>(tnw) : smallk_kernel<4>(tnw));
   // lean epilogue and blocked activations: several channel tiles per wave.  Measured at N = 64 (64 -> 256 and
   // 64 -> 128 at 56 x 56, 128 -> 512 at 28 x 28, 128 -> 128 at 56 x 56, 32 -> 64 at 112 x 112): four tiles per
   // wave up to 64 input channels, two above (more weights in registers cost a resident workgroup), 20-25 %
@@ -728,7 +770,7 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
     if (const char *env = getenv("EHIP_SMALLK_WGS")) wgs2 = atoi(env) > 0 ? atoi(env) : wgs2;
     const int cap2 = (wgs2 + ny2 - 1) / ny2;
     if (nx2 > cap2) nx2 = cap2;
-    void (*lk)(GemmArgs) = nullptr;
+    smallk_kernel_t lk = nullptr;
     if (ks == 1) lk = ocw == 4 ? k_gemm_smallk_lean<1, 4> : k_gemm_smallk_lean<1, 2>;
     else if (ks == 2) lk = ocw == 4 ? k_gemm_smallk_lean<2, 4> : k_gemm_smallk_lean<2, 2>;
     else lk = k_gemm_smallk_lean<4, 2>;
@@ -738,9 +780,9 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
                                               {"k_gemm_smallk_lean<4,2>", "k_gemm_smallk_lean<4,2>"}};
       plan->name = names[ks == 1 ? 0 : (ks == 2 ? 1 : 2)][ocw == 4 ? 1 : 0];
     }
-    return plan_launch(plan, lk, dim3(nx2, ny2), dim3(kBlock), 0, a, s);
+    return smallk_launch(plan, lk, dim3(nx2, ny2), a, s);
   }
-  return plan_launch(plan, kernel, dim3(nx, ny), dim3(kBlock), 0, a, s);
+  return smallk_launch(plan, kernel, dim3(nx, ny), a, s);
 }
 
 hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s, LaunchPlan<GemmArgs> *plan)
