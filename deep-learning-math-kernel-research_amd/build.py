@@ -40,7 +40,7 @@ FLAGS = [
 # per-source additions.  The depthwise matrix-core kernel has one accumulator tile per wave and turns it
 # straight into bytes: in the accumulation registers every value would be moved in and out once.
 EXTRA_FLAGS = {
-    "ehip_depthwise.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "ehip_depthwise.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1", "-mllvm", "-amdgpu-kernarg-preload-count=16"],
     # the 3x3 kernel takes what its first instructions need as leading scalar arguments: preloaded with the wave
     # (and its straight-line K loops are 72 steps of ~250 instructions: beyond the default budget of
     # `#pragma unroll`, which then leaves a loop whose weight registers are indexed at run time, i.e. in scratch)

@@ -80,9 +80,25 @@ __device__ __forceinline__ uint2 swap_halves(unsigned x, unsigned y)
 // round-to-nearest both land in the code range, so the pack-with-saturation instruction, which
 // rounds to nearest even itself, finishes either).  MODE 2: as 1 with lo == 0 and hi == 255, where
 // the clamp is the instruction's own saturation.
+// Both kernels take what a wave's first loads need -- three pointers and the geometry the addresses are made of,
+// packed into 16 dwords -- as leading scalar arguments, which the dispatcher preloads into scalar registers with
+// the wave (the file is compiled with -amdgpu-kernarg-preload-count=16); the rest of the argument block is loaded
+// as usual meanwhile.  ihw = ih | iw << 16, ohw = oh | ow << 16, geom = pad_t | pad_l << 8 | stride << 16,
+// ppb_lp = planes_per_block | lanes_padded << 16.
+#define EHIP_DW_HEAD                                                                                                   \
+  const uint8_t *in_, const int8_t *w_, const int *wsum_, int n_, int g2_, unsigned ihw_, unsigned ohw_, unsigned geom_, \
+      int blocks_per_plane_, int lanes_per_plane_, unsigned ppb_lp_, unsigned wp_magic_, int strips_per_wg_
+#define EHIP_DW_UNPACK                                                                                                 \
+  DepthwiseArgs a = rest;                                                                                              \
+  a.in = in_; a.w = w_; a.wsum = wsum_; a.n = n_; a.g2 = g2_; a.ih = (int)(ihw_ & 0xffffu); a.iw = (int)(ihw_ >> 16);  \
+  a.oh = (int)(ohw_ & 0xffffu); a.ow = (int)(ohw_ >> 16); a.pad_t = (int)(geom_ & 0xffu);                              \
+  a.pad_l = (int)((geom_ >> 8) & 0xffu); a.stride = (int)(geom_ >> 16); a.blocks_per_plane = blocks_per_plane_;        \
+  a.lanes_per_plane = lanes_per_plane_; a.planes_per_block = (int)(ppb_lp_ & 0xffffu);                                 \
+  a.lanes_padded = (int)(ppb_lp_ >> 16); a.wp_magic = wp_magic_; a.strips_per_wg = strips_per_wg_
 template <int RB, int MODE, int S>
-__global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
+__global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(EHIP_DW_HEAD, DepthwiseArgs rest)
 {
+  EHIP_DW_UNPACK;
   constexpr int NPX = S == 1 ? 4 : 5;          // input pixels per row a lane touches
   constexpr int NROWS = S * (RB - 1) + 3;      // input rows
   // A plane (one image x one 16-channel block) is split into blocks over its lanes (q fastest, then
@@ -256,8 +272,9 @@ __global__ __launch_bounds__(kBlock) void k_depthwise3x3_u8s8(DepthwiseArgs a)
 // other half of a double LDS buffer once the arithmetic is done (one barrier per strip).  A layer this short (57.8 MB,
 // 9 us for a plain copy) has no time for workgroups that load, compute and store one after the other.
 template <int MODE, int NC>
-__global__ __launch_bounds__(kBlock) void k_depthwise3x3_mfma(DepthwiseArgs a)
+__global__ __launch_bounds__(kBlock) void k_depthwise3x3_mfma(EHIP_DW_HEAD, DepthwiseArgs rest)
 {
+  EHIP_DW_UNPACK;
   constexpr int R = 8, WL = 32 * NC + 2, CELLS = (R + 2) * WL, PER = (CELLS + kBlock - 1) / kBlock;
   constexpr unsigned kNowhere = 0xffffff00u;   // an offset past the end of every tensor: loads give 0, stores vanish
   __shared__ uint4 tile[2][CELLS];
@@ -436,7 +453,35 @@ hipError_t launch_depthwise_diag(const int8_t *wpacked, int g2n, void *diag, hip
 }
 
 namespace {
-typedef void (*dw_kernel_t)(DepthwiseArgs);
+typedef void (*dw_kernel_t)(EHIP_DW_HEAD, DepthwiseArgs);
+hipError_t dw_enqueue(const LaunchPlan<DepthwiseArgs> &plan, hipStream_t s)
+{
+  const DepthwiseArgs &a = plan.args;
+  hipLaunchKernelGGL(reinterpret_cast<dw_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.wsum, a.n, a.g2,
+                     (unsigned)a.ih | (unsigned)a.iw << 16, (unsigned)a.oh | (unsigned)a.ow << 16,
+                     (unsigned)a.pad_t | (unsigned)a.pad_l << 8 | (unsigned)a.stride << 16, a.blocks_per_plane, a.lanes_per_plane,
+                     (unsigned)a.planes_per_block | (unsigned)a.lanes_padded << 16, a.wp_magic, a.strips_per_wg, a);
+  return hipGetLastError();
+}
+hipError_t dw_launch(LaunchPlan<DepthwiseArgs> *plan, dw_kernel_t kernel, dim3 grid, dim3 block, const DepthwiseArgs &a, hipStream_t s)
+{
+  // what the packed leading arguments can hold
+  if (a.ih >= 65536 || a.iw >= 65536 || a.oh >= 65536 || a.ow >= 65536 || a.pad_t < 0 || a.pad_t > 255 || a.pad_l < 0 ||
+      a.pad_l > 255 || a.planes_per_block >= 65536 || a.lanes_padded >= 65536) {
+    set_error("depthwise: plane or padding too large");
+    return hipErrorInvalidValue;
+  }
+  LaunchPlan<DepthwiseArgs> local;
+  LaunchPlan<DepthwiseArgs> *p = plan ? plan : &local;
+  p->valid = true;
+  p->kernel = reinterpret_cast<void (*)(DepthwiseArgs)>(kernel);
+  p->grid = grid;
+  p->block = block;
+  p->lds = 0;
+  p->args = a;
+  p->enqueue = dw_enqueue;
+  return dw_enqueue(*p, s);
+}
 template <int RB, int S>
 dw_kernel_t kernel_rbs(int mode)
 {
@@ -501,7 +546,7 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<D
 #define EHIP_DWM(NC) (full ? k_depthwise3x3_mfma<2, NC> : k_depthwise3x3_mfma<1, NC>)
     kernel = nc == 1 ? EHIP_DWM(1) : (nc == 2 ? EHIP_DWM(2) : (nc == 3 ? EHIP_DWM(3) : EHIP_DWM(4)));
 #undef EHIP_DWM
-    return plan_launch(plan, kernel, dim3((unsigned)wgs), dim3(kBlock), 0, a, s);
+    return dw_launch(plan, kernel, dim3((unsigned)wgs), dim3(kBlock), a, s);
   }
   // four rows per lane on tall planes (seven where that divides the height: 28, 56, 112 -- fewer halo
   // rows re-read, 2-5 % on the MobileNet layers), fewer where that would leave lanes idle
@@ -532,7 +577,7 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<D
   dim3 grid((unsigned)(8 * ((groups + 7) / 8) * a.blocks_per_plane), 1, 1);
   const dw_kernel_t kernel = rb == 7 ? kernel_rb<7>(a.stride, mode)
       : (rb == 4 ? kernel_rb<4>(a.stride, mode) : (rb == 2 ? kernel_rb<2>(a.stride, mode) : kernel_rb<1>(a.stride, mode)));
-  return plan_launch(plan, kernel, grid, dim3(block), 0, a, s);
+  return dw_launch(plan, kernel, grid, dim3(block), a, s);
 }
 
 }  // namespace ehip
