@@ -61,10 +61,33 @@ __device__ __forceinline__ FewChTables fewch_stage(const FewChArgs &a, unsigned 
     // a pixel's shift row is looked up per tile: two dependent trips to memory if the tables stay there
     for (int idx = tid; idx < rows_valid; idx += kBlock) lds_cls_h[idx] = a.cls_h[oh0 + idx] * a.ncls_w;
     for (int idx = tid; idx < a.ow; idx += kBlock) lds_cls_w[idx] = a.cls_w[idx];
-    const int width = a.wo * 32;
-    for (int idx = tid; idx < a.nclass * width; idx += kBlock) {
-      const int c = idx / width;
-      lds_shift[idx] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - c * width)];
+    // (eight loads in flight per thread: one at a time, the up to 49 rows of a 7 x 7 layer were twelve trips to
+    // memory one after the other at the head of every workgroup)
+    const int width = a.wo * 32, wshift = a.wo == 4 ? 7 : (a.wo == 2 ? 6 : 5);   // width = 1 << wshift
+    const int cells = a.nclass * width;
+    constexpr int kTabDepth = 8;
+    int base = 0;
+    if (cells <= 2 * kBlock) {   // a few classes: nothing to batch
+      for (int idx = tid; idx < cells; idx += kBlock) {
+        const int c = idx >> wshift;
+        lds_shift[idx] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - (c << wshift))];
+      }
+      base = cells;
+    }
+    for (; base < cells; base += kBlock * kTabDepth) {
+      float v[kTabDepth];
+#pragma unroll
+      for (int u = 0; u < kTabDepth; ++u) {
+        int idx = base + u * kBlock + tid;
+        idx = idx < cells ? idx : cells - 1;
+        const int c = idx >> wshift;
+        v[u] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - (c << wshift))];
+      }
+#pragma unroll
+      for (int u = 0; u < kTabDepth; ++u) {
+        const int idx = base + u * kBlock + tid;
+        if (idx < cells) lds_shift[idx] = v[u];
+      }
     }
   }
   if (a.in_nhwc && a.icl != a.ic) {
