@@ -627,3 +627,27 @@ def test_setup_rejects_what_the_reference_rejects():
     conv = E.Conv(E.make_desc(1, 64, 64, 8, 8))
     with pytest.raises(E.EulerHipError):
         conv.execute(None, None)
+
+
+@pytest.mark.parametrize("kind", ["1x1 many channels", "1x1 many channels, sum, nhwc", "1x1 few channels", "1x1 few channels f32", "3x3",
+                                  "3x3 stride 2", "depthwise 56", "depthwise 7", "depthwise stride 2", "first layer", "first layer f32"])
+def test_prepared_handle_on_other_buffers(kind):
+    # a handle keeps its launch (kernel, grid, derived and leading scalar arguments) from the first execute; the
+    # next execute must run on the tensors it is given: same bytes into a fresh output at another address
+    layer = {
+        "1x1 many channels": lambda: Layer(2, 256, 144, 14, out_type=ol.U8, seed=501),
+        "1x1 many channels, sum, nhwc": lambda: Layer(2, 512, 256, 14, stride=2, out_type=ol.S8, with_sum=True, in_nhwc=True,
+                                                      out_nhwc=True, seed=502),
+        "1x1 few channels": lambda: Layer(2, 64, 128, 14, out_type=ol.U8, seed=503),
+        "1x1 few channels f32": lambda: Layer(1, 32, 48, 9, out_type=ol.F32, seed=504),
+        "3x3": lambda: Layer(2, 64, 64, 14, k=3, pad=1, out_type=ol.U8, seed=505),
+        "3x3 stride 2": lambda: Layer(2, 32, 32, 15, k=3, pad=1, stride=2, out_type=ol.S8, seed=506),
+        "depthwise 56": lambda: Layer(2, 32, 32, 56, k=3, pad=1, depthwise=True, out_type=ol.U8, seed=507, T=14, relu_hi=255.0),
+        "depthwise 7": lambda: Layer(3, 48, 48, 7, k=3, pad=1, depthwise=True, out_type=ol.U8, seed=508, T=7, relu_hi=255.0),
+        "depthwise stride 2": lambda: Layer(2, 32, 32, 28, k=3, pad=1, stride=2, depthwise=True, out_type=ol.S8, seed=509, T=7),
+        "first layer": lambda: Layer(2, 3, 64, 37, k=7, pad=3, stride=2, out_type=ol.S8, seed=510, in_z=128.0, in_nhwc=True, out_nhwc=True),
+        "first layer f32": lambda: Layer(2, 3, 32, 23, k=3, pad=1, stride=2, out_type=ol.F32, seed=511, in_nhwc=True, with_relu=False),
+    }[kind]()
+    res = run_and_compare(layer)
+    again = layer.rerun_gpu(res["conv"])
+    assert again.shape == res["out"].shape and (again == res["out"]).all(), kind
