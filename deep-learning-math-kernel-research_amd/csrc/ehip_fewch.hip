@@ -57,39 +57,44 @@ __device__ __forceinline__ FewChTables fewch_stage(const FewChArgs &a, unsigned 
   float *const lds_shift = reinterpret_cast<float *>(rows_lds) + a.tab_lds;   // 16-byte aligned
   int *const lds_cls_h = reinterpret_cast<int *>(lds_shift + a.nclass * a.wo * 32);
   int *const lds_cls_w = lds_cls_h + a.rows;
+  // With border classes: the class of each of the strip's rows and of each column, and the shift rows of the
+  // workgroup's channels (a pixel's shift row is looked up per tile: two dependent trips to memory if the tables
+  // stayed there).  Their loads go out HERE, up to sixteen per thread, and are stored behind the staging of the input
+  // rows: one trip to memory for both (one load at a time, the up to 49 rows of a 7 x 7 layer were twelve trips one
+  // after the other at the head of every workgroup).
+  constexpr int kTabHold = 16;
+  const int width = a.wo * 32, wshift = a.wo == 4 ? 7 : (a.wo == 2 ? 6 : 5);   // width = 1 << wshift
+  const int cells = a.tab_lds ? a.nclass * width : 0;
+  auto tab_cell = [&](int idx) -> float {
+    const int c = idx >> wshift;
+    return a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - (c << wshift))];
+  };
+  float tab_held[kTabHold];
+  int cls_h_held = 0, cls_w_held = 0;
   if (a.tab_lds) {
-    // a pixel's shift row is looked up per tile: two dependent trips to memory if the tables stay there
-    for (int idx = tid; idx < rows_valid; idx += kBlock) lds_cls_h[idx] = a.cls_h[oh0 + idx] * a.ncls_w;
-    for (int idx = tid; idx < a.ow; idx += kBlock) lds_cls_w[idx] = a.cls_w[idx];
-    // (eight loads in flight per thread: one at a time, the up to 49 rows of a 7 x 7 layer were twelve trips to
-    // memory one after the other at the head of every workgroup)
-    const int width = a.wo * 32, wshift = a.wo == 4 ? 7 : (a.wo == 2 ? 6 : 5);   // width = 1 << wshift
-    const int cells = a.nclass * width;
-    constexpr int kTabDepth = 8;
-    int base = 0;
-    if (cells <= 2 * kBlock) {   // a few classes: nothing to batch
-      for (int idx = tid; idx < cells; idx += kBlock) {
-        const int c = idx >> wshift;
-        lds_shift[idx] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - (c << wshift))];
-      }
-      base = cells;
-    }
-    for (; base < cells; base += kBlock * kTabDepth) {
-      float v[kTabDepth];
+    cls_h_held = a.cls_h[oh0 + (tid < rows_valid ? tid : 0)] * a.ncls_w;
+    cls_w_held = a.cls_w[tid < a.ow ? tid : 0];
 #pragma unroll
-      for (int u = 0; u < kTabDepth; ++u) {
-        int idx = base + u * kBlock + tid;
-        idx = idx < cells ? idx : cells - 1;
-        const int c = idx >> wshift;
-        v[u] = a.ep.shift_tab[(size_t)c * a.ep.tab_stride + blockIdx.y * width + (idx - (c << wshift))];
-      }
-#pragma unroll
-      for (int u = 0; u < kTabDepth; ++u) {
-        const int idx = base + u * kBlock + tid;
-        if (idx < cells) lds_shift[idx] = v[u];
-      }
+    for (int u = 0; u < kTabHold; ++u) {
+      const int idx = u * kBlock + tid;
+      tab_held[u] = tab_cell(idx < cells ? idx : cells - 1);
+      if ((u + 1) * kBlock >= cells) break;   // uniform
     }
   }
+  auto store_tables = [&]() {
+    if (!a.tab_lds) return;
+    if (tid < rows_valid) lds_cls_h[tid] = cls_h_held;
+    if (tid < a.ow) lds_cls_w[tid] = cls_w_held;
+    for (int idx = tid + kBlock; idx < rows_valid; idx += kBlock) lds_cls_h[idx] = a.cls_h[oh0 + idx] * a.ncls_w;
+    for (int idx = tid + kBlock; idx < a.ow; idx += kBlock) lds_cls_w[idx] = a.cls_w[idx];
+#pragma unroll
+    for (int u = 0; u < kTabHold; ++u) {
+      const int idx = u * kBlock + tid;
+      if (idx < cells) lds_shift[idx] = tab_held[u];
+      if ((u + 1) * kBlock >= cells) break;   // uniform
+    }
+    for (int idx = kTabHold * kBlock + tid; idx < cells; idx += kBlock) lds_shift[idx] = tab_cell(idx);
+  };
   if (a.in_nhwc && a.icl != a.ic) {
     // Three channels staged as four bytes.  A thread takes four pixels: their twelve bytes, wherever they lie, come
     // out of four aligned dwords shifted together, and go to LDS as the four staged dwords at once (a staged row is
@@ -197,6 +202,7 @@ __device__ __forceinline__ FewChTables fewch_stage(const FewChArgs &a, unsigned 
         }
     }
   }
+  store_tables();
   return FewChTables{lds_shift, lds_cls_h, lds_cls_w};
 }
 
