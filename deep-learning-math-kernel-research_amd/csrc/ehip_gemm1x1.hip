@@ -447,6 +447,11 @@ int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
     // 9.0 us, 1024 -> 512: 12.2 against 15.4 us); with 512 channels its weights-in-registers form needs too
     // many registers and loses (512 -> 1024 stride 2: 23.9 against 15.2 us)
     if (v == 3 && a.units_pad == 64 && oc % 256 == 0 && wgs >= 192) score = 2.0;
+    // up to 512 input channels and about one and a half workgroups of the 128 x 128 tile per CU (where the 128 x 64
+    // tile needs twice as many): measured at N = 64 with 392-400 of them, 512 -> 128 at 28 x 28 7.9 against 9.1 us,
+    // 512 -> 512 at 14 x 14 7.5 against 8.4 us, 256 -> 512 at 14 x 14 6.1 against 6.7 us, 512 -> 2048 at 7 x 7 9.3
+    // against 10.0 us; with 196-294 or 784 and more of them the 64-pixel tile stays ahead by 5-30 %
+    if (v == 0 && a.units_pad <= 32 && wgs >= 352 && wgs <= 448 && util >= 0.95) score = 1.9;
     // fewer than 3/4 of the tile's channels real (64 output channels): the general kernel's 64-channel tiles
     // win (256 -> 64 at 56 x 56, N = 64: 13.4 against 17.1 us)
     if (util < 0.75) continue;
