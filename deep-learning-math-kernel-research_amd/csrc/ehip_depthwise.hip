@@ -550,7 +550,13 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<D
   }
   // four rows per lane on tall planes (seven where that divides the height: 28, 56, 112 -- fewer halo
   // rows re-read, 2-5 % on the MobileNet layers), fewer where that would leave lanes idle
-  const int rb = (a.oh >= 28 && a.oh % 7 == 0) ? 7 : (a.oh >= 16 ? 4 : (a.oh >= 7 ? 2 : 1));
+  int rb = (a.oh >= 28 && a.oh % 7 == 0) ? 7 : (a.oh >= 16 ? 4 : (a.oh >= 7 ? 2 : 1));
+  // measured at N = 64: 14 x 14 planes at stride 1 want seven rows as well (512 channels: 6.05 against 7.2 us with
+  // two, 6.3 with four), 56 x 56 outputs of a stride-2 layer two (64 channels 112 -> 56: 13.4 against 15.3 us with
+  // seven: 15 input rows of five pixels per lane are too many loads in flight); EHIP_DW_RB forces 1, 2, 4 or 7
+  if (a.stride == 1 && a.oh == 14) rb = 7;
+  if (a.stride == 2 && a.oh >= 56) rb = 2;
+  if (const char *env = getenv("EHIP_DW_RB")) { const int e = atoi(env); if (e == 1 || e == 2 || e == 4 || e == 7) rb = e; }
   const int ohb = (a.oh + rb - 1) / rb;
   const int wp = (a.ow + 1) / 2;
   a.lanes_per_plane = ohb * wp * 4;
