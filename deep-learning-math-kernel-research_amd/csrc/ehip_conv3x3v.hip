@@ -524,6 +524,10 @@ struct Variant {
     CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4>,  \
      k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>}, {nullptr, nullptr, nullptr} }
+#define VU2(WM, WN, TM, TN, CT, NPASS) /* straight-line form for two unit pairs only (64 input channels) */ \
+  { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, nullptr, nullptr}, {nullptr, nullptr, nullptr} }
 #define VK(WM, WN, TM, TN, CT, NPASS)                                                             \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
@@ -549,7 +553,7 @@ const Variant kVariants[] = {
     VK(4, 1, 1, 4, 256, 1), // 9: 128 oc x 128 px, rows up to  63 cells, every wave all pixels
     VU(4, 1, 1, 2, 128, 1), // 10: 128 oc x 64 px, rows up to  31 cells, every wave all pixels
     V(1, 4, 2, 2, 256, 3),  // 11:  64 oc x 256 px, rows up to 255 cells
-    V(2, 2, 1, 4, 256, 3),  // 12:  64 oc x 256 px, rows up to 255 cells, a wave = 32 oc x 128 px
+    VU2(2, 2, 1, 4, 256, 3), // 12:  64 oc x 256 px, rows up to 255 cells, a wave = 32 oc x 128 px
     VK(4, 1, 1, 4, 256, 2), // 13: 128 oc x 128 px, rows up to 191 cells, every wave all pixels
     V(4, 1, 1, 4, 256, 4),  // 14: 128 oc x 128 px, rows up to 447 cells, every wave all pixels
     VS(4, 1, 1, 4, 256, 1), // 15: as 9, strided pixels
@@ -561,6 +565,7 @@ const Variant kVariants[] = {
 #undef V
 #undef VU
 #undef VK
+#undef VU2
 #undef VS
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLdsBudget = 64 * 1024;
