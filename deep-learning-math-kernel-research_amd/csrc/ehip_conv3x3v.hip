@@ -336,31 +336,12 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
       row_taps(st & 1, kh, pl, pl == PAIRS - 1, st + 1 < 3 * PAIRS ? (st + 1) / 3 : -1, (st + 1) % 3);
     }
   } else if (PAIRS > 0) {
-    // straight line over the 9 * PAIRS taps of a fill, each one's pixel operands read during the tap before;
-    // layers of several fills of PAIRS pairs (512 input channels: two of eight) walk them in a loop
-    constexpr int LAST0 = 9 * (PAIRS - 1);   // first tap of a fill's last channel pair
-    for (int chunk = 0; chunk + 1 < nchunks; ++chunk) {   // every fill but the last
-      if (chunk) {
-        __syncthreads();
-        stage(chunk, false);
-        __syncthreads();
-      }
-#pragma unroll
-      for (int nt = 0; nt < TN; ++nt) read_b(0, 0, 0, nt);
-#pragma unroll
-      for (int st = 0; st < 9 * PAIRS; ++st)
-        tap_mfmas(st & 1, st % 9, chunk * PAIRS + st / 9, false, st + 1 < 9 * PAIRS ? (st + 1) / 9 : -1, (st + 1) % 9);
-    }
-    const int pair0 = (nchunks - 1) * PAIRS;   // the last fill's first pair
-    if (nchunks > 1) {
-      __syncthreads();
-      stage(nchunks - 1, false);
-      __syncthreads();
-    }
+    // straight line over the 9 * PAIRS taps, each one's pixel operands read during the tap before
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt) read_b(0, 0, 0, nt);
+    constexpr int LAST0 = 9 * (PAIRS - 1);   // first tap of the last channel pair
 #pragma unroll
-    for (int st = 0; st < LAST0; ++st) tap_mfmas(st & 1, st % 9, pair0 + st / 9, false, (st + 1) / 9, (st + 1) % 9);
+    for (int st = 0; st < LAST0; ++st) tap_mfmas(st & 1, st % 9, st / 9, false, (st + 1) / 9, (st + 1) % 9);
     load_epilogue_consts();
     // Split last pair (a wave of 32 channels x four pixel tiles, lean epilogue without the sum): with one
     // workgroup per CU nothing hides the epilogue -- a convert, a multiply-add and a byte pack per value, a
@@ -441,7 +422,7 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
     } else {
 #pragma unroll
       for (int st = LAST0; st < 9 * PAIRS; ++st)
-        tap_mfmas(st & 1, st % 9, pair0 + PAIRS - 1, true, st + 1 < 9 * PAIRS ? PAIRS - 1 : -1, (st + 1) % 9);
+        tap_mfmas(st & 1, st % 9, PAIRS - 1, true, st + 1 < 9 * PAIRS ? PAIRS - 1 : -1, (st + 1) % 9);
     }
   } else
   for (int chunk = 0; chunk < nchunks; ++chunk) {
@@ -534,7 +515,6 @@ struct Variant {
   conv3x3v_kernel_t kernel;
   conv3x3v_kernel_t unrolled[3];   // straight-line K loop for layers of exactly 2, 4, 8 unit pairs, or null
   conv3x3v_kernel_t split[3];      // the same with the last pair split (lean epilogue without the sum), or null
-  bool sp;                         // strided pixels (its straight-line forms take one fill only)
 };
 #define V(WM, WN, TM, TN, CT, NPASS)                                                              \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
@@ -559,7 +539,7 @@ struct Variant {
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ",sp>", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, conv3x3v_unit_stride(CT * NPASS, TN, true), k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 0, true>, \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, true>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, true>, \
-     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>}, {nullptr, nullptr, nullptr}, true }
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>}, {nullptr, nullptr, nullptr} }
 const Variant kVariants[] = {
     V(2, 2, 2, 1, 128, 1),  // 0: 128 oc x  64 px, rows up to  31 cells
     V(2, 2, 2, 1, 256, 1),  // 1: 128 oc x  64 px, rows up to  95 cells
@@ -670,10 +650,8 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
   a.lean = lean_mode(a.ep, false);
   dim3 grid(8 * a.tiles_per_xcd, 1, 1);
   conv3x3v_kernel_t kernel = k.kernel;
-  // the straight-line forms: one fill holds every unit, or (plain form only) whole fills of 2, 4 or 8 pairs
-  const bool one_fill = a.units_pad == a.chunk_units;
-  if (one_fill || (a.units_pad % a.chunk_units == 0 && !k.sp)) {
-    const int pairs = a.chunk_units / 2;
+  if (a.units_pad == a.chunk_units) {   // one fill holds every unit
+    const int pairs = a.units_pad / 2;
     const int slot = pairs == 2 ? 0 : (pairs == 4 ? 1 : (pairs == 8 ? 2 : -1));
     const char *env = getenv("EHIP_CONV3X3V_UNROLL");
     if (slot >= 0 && k.unrolled[slot] && !(env && env[0] == '0')) {
@@ -683,7 +661,7 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
       // own N = 32, one workgroup per CU: 6.12 against 6.54 us)
       const char *sl = getenv("EHIP_CONV3X3V_SPLIT_LAST");
       const bool want = sl && sl[0] ? sl[0] != '0' : a.tiles <= 512;
-      if (one_fill && k.split[slot] && (a.lean & 1) && !(a.lean & 4) && want) kernel = k.split[slot];
+      if (k.split[slot] && (a.lean & 1) && !(a.lean & 4) && want) kernel = k.split[slot];
     }
   }
   if (lds_bytes > 48 * 1024) {

@@ -279,10 +279,10 @@ def test_conv3x3_virtual_rows_many_channels_restage():
 
 @pytest.mark.parametrize("unroll", ["0", "1"])
 @pytest.mark.parametrize("variant,ic", [(9, 512), (9, 768), (13, 256), (10, 1024), (12, 192), (2, 512)])
-def test_conv3x3_straight_line_over_several_fills(variant, ic, unroll, monkeypatch):
-    """more input channels than one LDS fill holds, in whole fills of 2, 4 or 8 unit pairs: the straight-line K loop
-    walks the fills (512 channels in the 128 x 128 tile: two fills of eight pairs; 768: three), and the same layers
-    with the K loop as a loop"""
+def test_conv3x3_several_fills_of_whole_pairs(variant, ic, unroll, monkeypatch):
+    """more input channels than one LDS fill holds, in whole fills of 2, 4 or 8 unit pairs (512 channels in the
+    128 x 128 tile: two fills of eight pairs; 768: three): whichever form of the K loop the launcher picks for them,
+    and the loop form forced"""
     monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", str(variant))
     monkeypatch.setenv("EHIP_CONV3X3V_UNROLL", unroll)
     res = run_and_compare(Layer(2, ic, 144, 13, k=3, pad=1, out_type=ol.S8, seed=95 + variant + ic, w_sigma=0.02))
