@@ -16,6 +16,7 @@ LIB = os.path.join(HERE, "libeuler_hip.so")
 SOURCES = [
     "ehip_gemm.hip",
     "ehip_gemm1x1.hip",
+    "ehip_gemm1x1w.hip",
     "ehip_conv3x3v.hip",
     "ehip_fewch.hip",
     "ehip_depthwise.hip",
@@ -47,6 +48,7 @@ EXTRA_FLAGS = {
     "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-pragma-unroll-threshold=1000000"],
     # the resident-tile 1x1 kernel's leading scalar arguments: preloaded as well
     "ehip_gemm1x1.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "ehip_gemm1x1w.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     # and those of the 1x1 kernels with few input channels
     "ehip_gemm.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }

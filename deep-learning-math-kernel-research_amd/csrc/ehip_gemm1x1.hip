@@ -132,20 +132,6 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(EHIP_RES_HEAD, GemmAr
   const bool dense = (geom >> 16) & 1u;   // stride 1 and the output plane is the input plane
   TRACE_POINT(0);
 
-  // ---- the accumulators start from the compensation ------------------------------------------------
-  const long long cidx = oc0 + 16 * lh;   // the lane's 16 channels of tile 0
-  v16i acc[TM][TN];
-#pragma unroll
-  for (int mt = 0; mt < TM; ++mt) {
-    v4i c4[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) c4[q] = *reinterpret_cast<const v4i *>(a.ep.comp + cidx + 32 * mt + 4 * q);
-#pragma unroll
-    for (int nt = 0; nt < TN; ++nt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = c4[v >> 2][v & 3];
-  }
-
   // ---- the whole pixel tile, all units, straight into LDS -----------------------------------------------
   // A wave-load moves 64 consecutive pixels of one unit (1 KB): lane i's 16 bytes land at the wave-uniform
   // LDS address + 16 i.  Pixel halves of 64 (P_T / 64) x units are dealt to the four waves round-robin.
@@ -223,6 +209,21 @@ __global__ __launch_bounds__(kBlock, 1) void k_gemm1x1_res(EHIP_RES_HEAD, GemmAr
   };
   if (NHWC) request_tile_nhwc();
   else if (!PIPE) request_tile();
+
+  // ---- the accumulators start from the compensation ------------------------------------------------
+  const long long cidx = oc0 + 16 * lh;   // the lane's 16 channels of tile 0
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt) {
+    v4i c4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) c4[q] = *reinterpret_cast<const v4i *>(a.ep.comp + cidx + 32 * mt + 4 * q);
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mt][nt][v] = c4[v >> 2][v & 3];
+  }
+
 
   TRACE_POINT(1);
   // ---- weights [units_pad][ocpp][16]: lane = packed row l32 of unit 2 ks + lh, tile mt 32 rows on --------

@@ -64,6 +64,7 @@ struct GemmArgs {
   long long *trace;            // development aid, normally null (see EHIP_TRACE)
   int lean;                    // set by the launcher: lean_mode() of the epilogue (0 = general epilogue)
   unsigned u1_magic;           // set by the resident-tile launcher: div_magic(units_pad + 1)
+  int wr_region, wr_stage, wr_nbuf;   // set by the weights-resident launcher: pixels per region, bytes per LDS stage, stages
 };
 
 struct Conv3x3Args {
@@ -188,6 +189,9 @@ const char *gemm_variant_name(int variant);
 int gemm1x1_res_pick(const GemmArgs &a, int nbatch);   // variant, or -1 when the layer is not one for it
 const char *gemm1x1_res_name(int variant);
 hipError_t launch_gemm1x1_res(const GemmArgs &a, int variant, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr);
+// 1x1 layers of 256 / 512 / 1024 input channels with the lean epilogue: weights resident in registers, pixels streamed
+bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch);
+hipError_t launch_gemm1x1_wres(const GemmArgs &a, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr);
 
 hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s, LaunchPlan<Conv3x3Args> *plan = nullptr);
 int conv3x3v_pick_variant(int n, int oh, int ow, int oc2);   // -1: rows too wide for every variant

@@ -240,10 +240,13 @@ int elx_conv(eld_conv_t &desc, void *output, void *input, void *weights, void *b
   }
   if (!out_on_device) {
     if (hipMemcpy(output, dout, desc.byte_sizes.output, hipMemcpyDeviceToHost) != hipSuccess) return ELX_GENERAL_ERROR;
-  } else if (desc.stream_sync) {
-    // Device tensors: the layer is ordered on the NULL stream like every later kernel or copy that touches
-    // them, so eager mode needs no host wait (a chain of layers stays asynchronous).  stream_sync asks for
-    // the wait, as it does for the reference's stream (src/elx_conv.cpp:233-236).
+  } else if (desc.eager_mode || desc.stream_sync) {
+    // Device or managed tensors.  Eager mode (the descriptor's default) returns with the result complete, as the
+    // reference's does (src/elx_conv.cpp:226-230): a host that reads a managed output, or a consumer on a
+    // non-blocking stream, may use it straight away.  A caller that chains layers on the device asks for the
+    // reference's stream mode instead (eager_mode = false): the layer is then only ordered on the NULL stream,
+    // like every later kernel or copy that touches its tensors, and stream_sync adds the wait
+    // (src/elx_conv.cpp:231-236).
     if (hipStreamSynchronize(nullptr) != hipSuccess) return ELX_GENERAL_ERROR;
   }
   return ELX_OK;

@@ -15,6 +15,8 @@
 #include <cstring>
 #include <vector>
 
+#include <hip/hip_runtime_api.h>
+
 #include "euler.hpp"
 #include "euler_reorder.hpp"
 
@@ -101,6 +103,17 @@ int main(int argc, char **argv)
   if (elx_conv(desc, ob.data(), xb.data(), wb.data(), bias.data()) != ELX_OK) return 5;
   ob = ob0;
   if (elx_conv(desc, ob.data(), xb.data(), wb.data(), bias.data()) != ELX_OK) return 5;
+  if (getenv("EULER_CHECK_MANAGED_OUTPUT")) {
+    // Eager mode (the descriptor's default) with the output in managed memory: the result must be complete when
+    // elx_conv returns, as the reference's eager mode is (src/elx_conv.cpp:226-230).  The host reads it straight
+    // after the call, with no synchronisation of its own, and that is what gets compared.
+    uint8_t *ym = nullptr;
+    if (hipMallocManaged(reinterpret_cast<void **>(&ym), ob.size()) != hipSuccess) return 8;
+    memcpy(ym, ob0.data(), ob.size());
+    if (elx_conv(desc, ym, xb.data(), wb.data(), bias.data()) != ELX_OK) return 5;
+    memcpy(ob.data(), ym, ob.size());
+    (void)hipFree(ym);
+  }
 
   std::vector<uint8_t> out((size_t)n * oc * oh * oh * osz);
   if (use_nhwc && osz == 1) reorder<uint8_t, nchw, nhwc>(out.data(), ob.data(), n, oc, oh, oh);

@@ -21,7 +21,7 @@ def from_blocked(b, c):
     return np.ascontiguousarray(b.transpose(0, 1, 4, 2, 3).reshape(n, c2 * 16, h, w)[:, :c])
 
 
-@pytest.mark.parametrize("case", [
+CASES = [
     dict(n=2, ic=64, oc=48, hw=12, k=3, pad=1, out_type=ol.U8, T=12),
     dict(n=2, ic=96, oc=64, hw=7, k=1, pad=0, out_type=ol.S8, with_sum=True),
     dict(n=1, ic=32, oc=80, hw=9, k=1, pad=0, out_type=ol.F32),
@@ -30,8 +30,11 @@ def from_blocked(b, c):
     dict(n=2, ic=32, oc=32, hw=14, k=3, pad=1, stride=2, out_type=ol.U8, depthwise=True, T=7),
     dict(n=2, ic=96, oc=64, hw=7, k=1, pad=0, out_type=ol.S8, with_sum=True, nhwc=True),
     dict(n=2, ic=3, oc=64, hw=22, k=7, pad=3, stride=2, out_type=ol.S8, nhwc=True),   # a first layer: 3-channel nhwc image
-], ids=["3x3_u8", "1x1_s8_sum", "1x1_f32", "depthwise_u8", "3x3_s2_s8", "depthwise_s2_u8", "1x1_s8_sum_nhwc",
-        "7x7_s2_3ch_nhwc"])
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=["3x3_u8", "1x1_s8_sum", "1x1_f32", "depthwise_u8", "3x3_s2_s8", "depthwise_s2_u8",
+                                              "1x1_s8_sum_nhwc", "7x7_s2_3ch_nhwc"])
 def test_elx_conv_on_host_buffers(case, tmp_path):
     assert os.path.exists(CHECK), "euler_api_check is not built (python -c 'import __graft_entry__ as g; g.build()')"
     c = dict(stride=1, with_sum=False, depthwise=False, T=0, nhwc=False)
@@ -56,6 +59,13 @@ def test_elx_conv_on_host_buffers(case, tmp_path):
     assert r.returncode == 0, "rc=%d stdout=%s stderr=%s" % (r.returncode, r.stdout, r.stderr)
     got = np.fromfile(fout, dtype=exp.dtype).reshape(exp.shape)
     assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), "%d values differ" % int((got != exp).sum())
+    if case is CASES[0] or case is CASES[1]:
+        # eager mode with a managed output: the client reads the result on the host straight after elx_conv returns
+        r = subprocess.run(args, capture_output=True, text=True, timeout=120,
+                           env=dict(os.environ, EULER_CHECK_MANAGED_OUTPUT="1"))
+        assert r.returncode == 0, "rc=%d stdout=%s stderr=%s" % (r.returncode, r.stdout, r.stderr)
+        got = np.fromfile(fout, dtype=exp.dtype).reshape(exp.shape)
+        assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), "managed output: %d values differ" % int((got != exp).sum())
 
 
 @pytest.mark.parametrize("in_type,out_type,tile,mode", [
