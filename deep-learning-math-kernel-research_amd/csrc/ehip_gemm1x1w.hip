@@ -23,7 +23,7 @@
 #ifdef EHIP_TRACE
 #define TRACE_POINT(i)                                                                             \
   do {                                                                                             \
-    if (a.trace && lane == 0) a.trace[((size_t)blockIdx.x * 4 + wave) * 16 + (i)] = wall_clock64(); \
+    if (a.trace && lane == 0) a.trace[((size_t)blockIdx.x * NW + wave) * 16 + (i)] = wall_clock64(); \
   } while (0)
 #else
 #define TRACE_POINT(i) do { } while (0)
@@ -77,8 +77,11 @@ struct PixInfo {
 #define EHIP_WRES_HEAD                                                                                                  \
   const uint8_t *in, const int8_t *w, const int *comp, int p_total, int ohw, unsigned ohw_magic, int ihw, int ic2, int ocpp, \
       unsigned geom, int ntiles_all, int nreg, int stage_bytes
-template <int NKS, int TM, int SUM>   // SUM: 0 none, 1 the old output is u8, 2 it is s8
-__global__ __launch_bounds__(kBlock, 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, GemmArgs rest)
+// NW waves per workgroup: four, two workgroups per CU; or eight in one workgroup per CU, which then share ONE copy
+// of every pixel tile (1024 input channels, where a wave can only hold the weights of 32 channels: eight waves own
+// the 256 channels that four own with fewer input channels)
+template <int NKS, int TM, int SUM, int NW>   // SUM: 0 none, 1 the old output is u8, 2 it is s8
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, GemmArgs rest)
 {
   GemmArgs a = rest;
   a.in = in; a.w = w; a.ep.comp = comp; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic;
@@ -106,7 +109,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, Gemm
   const int ntiles = tq + (reg < tr ? 1 : 0);
   if (ntiles == 0) return;
   const int p0 = tile0 * 32;
-  const int ocw = by * (4 * OCW) + wave * OCW;   // the wave's first channel
+  const int ocw = by * (NW * OCW) + wave * OCW;   // the wave's first channel
   const int oc_lane = ocw + 16 * lh;             // the lane's 16 channels of tile 0 (tile mt: + 32 mt)
   const int oc_real = a.oc2 * 16;
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds;
@@ -140,10 +143,10 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, Gemm
   const unsigned unit_stride = (unsigned)a.ihw * 16u;
 
   // tile tt of the run into stage st: k-step j's operand is one wave-load (lane = unit 2 j + lh, pixel l32)
-  // landing at st + 1 KB * j; the waves take every fourth.  With the sum, the wave's own TM cells per lane
+  // landing at st + 1 KB * j; the waves take one in NW.  With the sum, the wave's own TM cells per lane
   // follow at st + 1 KB * (NKS + TM wave + mt), lane i's at + 16 i.  A tile's loads are issued one by one (load d of
   // the wave's LPT), so that they can be spread over the k-steps of a K loop.
-  constexpr int LPT = NKS / 4 + (SUM ? TM : 0);   // loads of one wave per tile
+  constexpr int LPT = NKS / NW + (SUM ? TM : 0);   // loads of one wave per tile
   unsigned pend_in = 0, pend_out = 0, pend_sb = 0;
   auto issue_setup = [&](int tt, int st) {
     const PixInfo pi = pix_info(tt);
@@ -152,11 +155,11 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, Gemm
     pend_sb = lds_base + (unsigned)st * (unsigned)stage_bytes;
   };
   auto issue_load = [&](int d) {
-    if (d < NKS / 4) {
-      const int j = wave + 4 * d;
+    if (d < NKS / NW) {
+      const int j = wave + NW * d;
       dma16(a.in + (size_t)(2 * j) * unit_stride, pend_in, pend_sb + 1024u * (unsigned)j);
     } else if (SUM) {
-      const int mt = d - NKS / 4;
+      const int mt = d - NKS / NW;
       // (a tile of channels behind the real ones reads the cell of tile 0: any readable address will do)
       const bool ok = oc_lane + 32 * mt < oc_real;
       dma16(a.out, ok ? pend_out + mt * tile_stride : pend_out - lane_cell, pend_sb + 1024u * (unsigned)(NKS + TM * wave + mt));
@@ -168,9 +171,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, Gemm
     for (int d = 0; d < LPT; ++d) issue_load(d);
   };
 
-  // ---- prologue: the first two tiles, then the constants and the weights ------------------------------------
+  // ---- prologue: the first tile, the constants, the weights, the second tile ----------------------------------
   issue_tile(0, 0);
-  if (ntiles > 1) issue_tile(1, 1);
   TRACE_POINT(1);
 
   if (lane < OCW) {
@@ -186,6 +188,10 @@ __global__ __launch_bounds__(kBlock, 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, Gemm
   for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) areg[ks][mt] = *reinterpret_cast<const v4i *>(wb + ks * w_step + mt * 512);
+  // The second tile behind the weights: a wave's loads complete in issue order, and the first tile's K loop needs
+  // the weights, not the second tile.  (The compiler's waits for the weights then cover these few loads as well: the
+  // last k-steps of the first tile wait for the second tile, which the tile's barrier waits for anyway.)
+  if (ntiles > 1) issue_tile(1, 1);
   // the lane's constants of tile mt, channels 4 q .. 4 q + 3, out of LDS
   auto cl_read = [&](int arr, int mt, int q) -> float4 {
     return *reinterpret_cast<const float4 *>(cl_f + OCW * arr + 32 * mt + 16 * lh + 4 * q);
@@ -316,39 +322,41 @@ int wres_tm(int nks) { return nks <= 16 ? 2 : 1; }
 wres_kernel_t wres_kernel(int nks, int sum)
 {
   switch (nks * 4 + sum) {
-  case 8 * 4 + 0: return k_gemm1x1_wres<8, 2, 0>;
-  case 8 * 4 + 1: return k_gemm1x1_wres<8, 2, 1>;
-  case 8 * 4 + 2: return k_gemm1x1_wres<8, 2, 2>;
-  case 16 * 4 + 0: return k_gemm1x1_wres<16, 2, 0>;
-  case 16 * 4 + 1: return k_gemm1x1_wres<16, 2, 1>;
-  case 16 * 4 + 2: return k_gemm1x1_wres<16, 2, 2>;
-  case 32 * 4 + 0: return k_gemm1x1_wres<32, 1, 0>;
-  case 32 * 4 + 1: return k_gemm1x1_wres<32, 1, 1>;
-  case 32 * 4 + 2: return k_gemm1x1_wres<32, 1, 2>;
+  case 8 * 4 + 0: return k_gemm1x1_wres<8, 2, 0, 4>;
+  case 8 * 4 + 1: return k_gemm1x1_wres<8, 2, 1, 4>;
+  case 8 * 4 + 2: return k_gemm1x1_wres<8, 2, 2, 4>;
+  case 16 * 4 + 0: return k_gemm1x1_wres<16, 2, 0, 4>;
+  case 16 * 4 + 1: return k_gemm1x1_wres<16, 2, 1, 4>;
+  case 16 * 4 + 2: return k_gemm1x1_wres<16, 2, 2, 4>;
+  case 32 * 4 + 0: return k_gemm1x1_wres<32, 1, 0, 8>;
+  case 32 * 4 + 1: return k_gemm1x1_wres<32, 1, 1, 8>;
+  case 32 * 4 + 2: return k_gemm1x1_wres<32, 1, 2, 8>;
   }
   return nullptr;
 }
+int wres_nw(int nks) { return nks <= 16 ? 4 : 8; }
 
 // The launch geometry, or false when the layer is not one for this kernel: two workgroups per CU (80 KB of LDS
 // each) where the ring of stages then still holds three tiles or a whole run, else one per CU with all 160 KB.
 struct WresGeom {
-  int nks, tm, sum, nb, nreg, tiles, stage, nbuf;
+  int nks, tm, nw, sum, nb, nreg, tiles, stage, nbuf;
   size_t lds_bytes;
 };
 bool wres_geom(const GemmArgs &a, WresGeom &g)
 {
   g.nks = a.units_pad / 2;
   g.tm = wres_tm(g.nks);
+  g.nw = wres_nw(g.nks);
   const int lean = lean_mode(a.ep, false);
   g.sum = (lean & 4) ? (a.ep.out_type == EHIP_S8 ? 2 : 1) : 0;
-  g.nb = (a.oc2 * 16 + 128 * g.tm - 1) / (128 * g.tm);
+  g.nb = (a.oc2 * 16 + 32 * g.nw * g.tm - 1) / (32 * g.nw * g.tm);
   g.tiles = (a.p_total + 31) / 32;
-  g.stage = g.nks * 1024 + (g.sum ? 4 * g.tm * 1024 : 0);
-  const size_t cl_bytes = 4 * 3 * 32 * g.tm * 4;   // per-channel constants of the four waves
+  g.stage = g.nks * 1024 + (g.sum ? g.nw * g.tm * 1024 : 0);
+  const size_t cl_bytes = g.nw * 3 * 32 * g.tm * 4;   // per-channel constants of the waves
   int forced_slots = 0, forced_nbuf = 0;
   if (const char *env = getenv("EHIP_WRES_SLOTS")) forced_slots = atoi(env);
   if (const char *env = getenv("EHIP_WRES_NBUF")) forced_nbuf = atoi(env);
-  for (int per_cu = 2; per_cu >= 1; --per_cu) {
+  for (int per_cu = g.nw == 8 ? 1 : 2; per_cu >= 1; --per_cu) {
     const int slots = forced_slots > 0 ? forced_slots : 256 * per_cu;
     g.nreg = slots / g.nb > 0 ? slots / g.nb : 1;
     if (g.nreg > g.tiles) g.nreg = g.tiles;
@@ -378,7 +386,7 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch)
   if ((a.units_pad != 16 && a.units_pad != 32 && a.units_pad != 64) || a.ic2 != a.units_pad) return false;
   if (a.stride_h > 255 || a.stride_w > 255) return false;
   const int oc = a.oc2 * 16;
-  const int oc_wg = 128 * wres_tm(a.units_pad / 2);
+  const int oc_wg = 32 * wres_nw(a.units_pad / 2) * wres_tm(a.units_pad / 2);
   const int nb = (oc + oc_wg - 1) / oc_wg;
   if (nb >= 4096) return false;
   // fewer than three quarters of the channel blocks' rows real, or too few pixels to give every CU a run: the
@@ -390,7 +398,7 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch)
   // 512 -> 256 at 28 x 28: 11.7 vs 13.4, 256 -> 256 at 28 x 28: 8.3 vs 9.8), level or behind with shorter runs
   // (512 -> 512 at 14 x 14: 8.0 vs 7.7, 512 -> 2048 at 7 x 7: 8.2 vs 8.0) and with 1024 input channels, whose waves own
   // one tile of 32 channels (1024 -> 256 at 14 x 14: 8.6 vs 8.4, 1024 -> 1024 at 7 x 7: 8.6 vs 7.2)
-  if (!forced && (a.units_pad > 32 || (long long)((a.p_total + 31) / 32) * nb < 3 * 512)) return false;
+  if (!forced && !getenv("EHIP_WRES_TRY32") && (a.units_pad > 32 || (long long)((a.p_total + 31) / 32) * nb < 3 * 512)) return false;
   // a lane's offsets into the input and the output are 32 bits wide
   const long long n_img = a.p_total / (a.ohw > 0 ? a.ohw : 1);
   if (n_img * a.ic2 * a.ihw * 16 >= (1ll << 32) || (long long)a.p_total * a.oc2 * 16 >= (1ll << 32)) return false;
@@ -419,7 +427,7 @@ hipError_t launch_gemm1x1_wres(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gem
   p->valid = true;
   p->kernel = reinterpret_cast<void (*)(GemmArgs)>(kernel);
   p->grid = dim3(8 * g.nb * ((g.nreg + 7) / 8));
-  p->block = dim3(kBlock);
+  p->block = dim3(g.nw * 64);
   p->lds = (unsigned)g.lds_bytes;
   p->args = a;
   p->enqueue = wres_enqueue;

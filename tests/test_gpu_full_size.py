@@ -109,7 +109,37 @@ def test_configured_winograd_layer_u8_in_s8_out(key, check_images, nhwc):
     assert len(np.unique(got)) > 60       # and the s8 codes use their range
 
 
-@pytest.mark.parametrize("key", ["C2", "C3a", "C3b", "C1", "C5a"])
+@pytest.mark.parametrize("key", ["C4a", "C4b", "C4a_i8", "C4b_i8"])
+def test_benchmark_winograd_layer_with_calibrated_scales(key):
+    """The benchmark's own Winograd tensors (workloads.DeviceLayer: seeded tensors, wino_tinput_quant calibrated from
+    the transformed-input range, output scale from the fp32 reference convolution) through the oracle: the bytes
+    that bench.py times.  Every image is an independent problem: the first two are compared bit for bit."""
+    import torch
+    wl = W.WORKLOADS[key]
+    layer = W.DeviceLayer(wl)
+    d = layer.desc
+    layer.run(1)
+    torch.cuda.synchronize()
+    k = 2
+    got = host(layer.out[:k])
+    x = host(layer.x[:k])
+    pk = ol.make_params(k, wl.ic, wl.oc, wl.hw, wl.hw, 3, 3, 1, out_type=wl.out_type, in_scale=d.input_scale, with_bias=True,
+                        with_relu=True, out_scale=d.output_scale, out_z=d.output_z, wino_tile=wl.tile)
+    pk.tin_scale, pk.tin_z = d.tinput_scale, d.tinput_z
+    wb, bias = host(layer.w), host(layer.bias)
+    twq, tscale, tshift = ol.wino_prepare(pk, wb)
+    assert np.array_equal(layer.conv.query(pkg().Q_WEIGHTS_S8), twq.ravel()), "transformed weights differ"
+    tin = ol.wino_trans_input(pk, np.ascontiguousarray(x).astype(np.float32))
+    tout, _ = ol.wino_gemm(pk, tin, twq, tscale, tshift)
+    exp = ol.wino_trans_output(pk, tout, bias)
+    assert np.array_equal(bits(got), bits(exp)), "%d of %d values differ" % (int((got != exp).sum()), got.size)
+    # the calibrated transformed-input codes use their range: the scale is the one the range asks for
+    assert abs(d.tinput_scale * 255.0 - (layer.calibration["tinput_max"] - layer.calibration["tinput_min"])) < 1e-3
+    if wl.out_type == ol.S8:
+        assert got.max() >= 100   # (of two images; the calibrated scale puts the whole batch's maximum at 127)
+
+
+@pytest.mark.parametrize("key", ["C2", "C3a", "C3b", "C1", "C5a", "C5b"])
 def test_benchmark_layer_with_calibrated_scales(key):
     """The benchmark's own tensors (workloads.DeviceLayer: seeded fp32 tensors, output / sum scales calibrated
     from the fp32 reference convolution as the reference's harness does) through the oracle: same bytes, and
@@ -139,7 +169,7 @@ def test_benchmark_layer_with_calibrated_scales(key):
     elif wl.out_type == ol.U8:
         assert got.max() >= 250
     elif wl.out_type == ol.S8:
-        assert got.max() >= 120
+        assert got.max() >= 100   # (of two images; the calibrated scale puts the whole batch's maximum at 127)
         assert layer.calibration["sum_scale"] > 0
     # seeded: a second layer holds the same bytes
     again = W.DeviceLayer(wl)

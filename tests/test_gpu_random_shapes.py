@@ -46,11 +46,56 @@ def test_random_kxk(seed):
         # ask for one more output row / column: pads only at the right / bottom
         if r.integers(0, 2):
             out_hw = natural + 1
+    # the right / bottom pad that the output size implies must be k/2 - 1 or k/2 as well: the reference's c160
+    # shape set (src/elx_int8_conv_direct.cpp:66-77 with the pads of src/elx_conv.cpp:36-37); a drawn size whose
+    # implied pad is another grows until it is one of them, so that no seed ends in a refused layer
+    o = out_hw or natural
+    while max(0, (o - 1) * stride + k - hw - pad) not in (k // 2 - 1, k // 2):
+        hw += 1
+        out_hw = None
+        o = natural = (hw + 2 * pad - k) // stride + 1
+    assert reference_c160_shape_ok(k, stride, pad, hw, o)
     out_type = OUT_TYPES[int(r.integers(0, 4))]
     nhwc_in = ic % 16 == 0 and bool(r.integers(0, 2))
     nhwc_out = oc % 16 == 0 and bool(r.integers(0, 2))
     run_and_compare(Layer(int(r.integers(1, 3)), ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=seed,
                           out_hw=out_hw, in_nhwc=nhwc_in, out_nhwc=nhwc_out))
+
+
+def reference_c160_shape_ok(k, stride, pad, hw, out_hw):
+    """what the reference's direct int8 executor accepts for a square k x k layer (src/elx_int8_conv_direct.cpp:66-77):
+    3 / 5 / 7 kernels, stride 1 or 2, left / top pad and the right / bottom pad it recomputes from the output size
+    (rp = max(0, ws (ow - 1) + kw - iw - lp), src/elx_conv.cpp:36-37) all k/2 - 1 or k/2"""
+    rp = max(0, stride * (out_hw - 1) + k - hw - pad)
+    return k in (3, 5, 7) and stride in (1, 2) and pad in (k // 2 - 1, k // 2) and rp in (k // 2 - 1, k // 2)
+
+
+def test_every_refused_kxk_shape_is_one_the_reference_refuses():
+    """ehip_conv_create over seeded k x k shapes, pads and output sizes, fitting and not: wherever it answers
+    "c160: shape not supported" the reference's own shape test fails too (the library may accept more: an output
+    size that leaves input columns unused, which the reference's clamped pad turns away for 5x5 and 7x7)."""
+    from gpu_common import pkg
+    E = pkg()
+    r = _rng(900)
+    refused = accepted = 0
+    for _ in range(600):
+        k = int(r.choice([3, 5, 7]))
+        stride = int(r.choice([1, 2, 3]))
+        pad = int(r.integers(0, k // 2 + 2))
+        hw = int(r.integers(k + 1, 30))
+        natural = (hw + 2 * pad - k) // stride + 1
+        out_hw = max(1, natural + int(r.integers(-1, 2)))
+        d = E.make_desc(1, 32, 32, hw, hw, k, k, pad, stride, output_type=ol.U8)
+        d.oh = d.ow = out_hw
+        try:
+            E.Conv(d).close()
+            accepted += 1
+        except E.EulerHipError as exc:
+            if "c160: shape not supported" not in str(exc):
+                continue
+            refused += 1
+            assert not reference_c160_shape_ok(k, stride, pad, hw, out_hw), (k, stride, pad, hw, out_hw)
+    assert refused > 50 and accepted > 50
 
 
 @pytest.mark.parametrize("seed", range(24))
