@@ -72,6 +72,7 @@ def _load():
     lib.ehip_conv_prepare.argtypes = [vp, vp, vp, vp]
     lib.ehip_conv_execute.argtypes = [vp, vp, vp, vp, vp, vp]
     lib.ehip_conv_execute_repeat.argtypes = [vp, vp, vp, vp, ci, vp]
+    lib.ehip_conv_execute_stages.argtypes = [vp, vp, vp, vp, ci, ci, vp]
     lib.ehip_conv_query.argtypes = [vp, ci, vp, ctypes.POINTER(sz)]
     lib.ehip_quantize_input_u8.argtypes = [vp, vp, sz, fl, fl, vp]
     lib.ehip_wino_tinput_range.argtypes = [ctypes.POINTER(ConvDesc), vp, ctypes.POINTER(fl), ctypes.POINTER(fl)]
@@ -88,7 +89,7 @@ lib = _load()
 
 EXPORTED_SYMBOLS = (
     "ehip_init", "ehip_last_error", "ehip_conv_create", "ehip_conv_destroy", "ehip_conv_prepare",
-    "ehip_conv_execute", "ehip_conv_execute_repeat", "ehip_conv_query", "ehip_conv_kernel_name", "ehip_quantize_input_u8",
+    "ehip_conv_execute", "ehip_conv_execute_repeat", "ehip_conv_execute_stages", "ehip_conv_query", "ehip_conv_kernel_name", "ehip_quantize_input_u8",
     "ehip_wino_tinput_range", "ehip_wino_tinput_range_noalloc", "ehip_reorder_nchw_to_blocked", "ehip_reorder_blocked_to_nchw",
     "ehip_reorder_oihw_to_blocked", "ehip_ref_conv_f32_range", "ehip_calibrate_output_quant",
 )
@@ -171,6 +172,12 @@ class Conv:
 
     def execute_repeat(self, output, input, count, bias=None, stream=0):
         _check(lib.ehip_conv_execute_repeat(self._h, _ptr(output), _ptr(input), _ptr(bias), count,
+                                            ctypes.c_void_p(stream)))
+
+    def execute_stages(self, output, input, stages, count=1, bias=None, stream=0):
+        """stages of a Winograd layer on their own: mask of 1 (input transform), 2 (GEMMs, fused: + output
+        transform), 4 (stand-alone output transform)"""
+        _check(lib.ehip_conv_execute_stages(self._h, _ptr(output), _ptr(input), _ptr(bias), stages, count,
                                             ctypes.c_void_p(stream)))
 
     def query(self, what):

@@ -65,6 +65,7 @@ struct ehip_conv {
 
   // launch plans of the steady state (filled by the first execute, see LaunchPlan); the Winograd ones are
   // used only when the layer runs in one pass (no chunking)
+  int stage_mask = 7;   // Winograd: which stages execute() launches (ehip_conv_execute_stages)
   LaunchPlan<GemmArgs> plan_gemm;
   LaunchPlan<Conv3x3Args> plan_3x3;
   LaunchPlan<FewChArgs> plan_fewch;
@@ -694,8 +695,9 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       const float tin_repS = 1.0f / d.tinput_scale;
       w.mrepS = d.input_scale * tin_repS;
       w.mz = ceilf(d.tinput_z);
-      HIP_TRY(launch_wino_trans_input(w, s, one_pass ? &c->plan_wino_in : nullptr));
+      if (c->stage_mask & 1) HIP_TRY(launch_wino_trans_input(w, s, one_pass ? &c->plan_wino_in : nullptr));
       if (c->fused) {
+        if (!(c->stage_mask & 2)) continue;
         WinoFusedArgs f;
         memset(&f, 0, sizeof(f));
         f.tin = c->tin; f.tin_blocked = c->tin_blocked; f.w = c->wpacked; f.out = w.out; f.bias = w.bias;
@@ -722,8 +724,8 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
       a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
       a.in_batch_stride = (long long)c->ic2 * w.t * 16;
       a.out_batch_stride = (long long)c->oc2 * w.t * 16;
-      HIP_TRY(launch_gemm(a, c->nbatch, c->variant, s, one_pass ? &c->plan_gemm : nullptr));
-      HIP_TRY(launch_wino_trans_output(w, s, one_pass ? &c->plan_wino_out : nullptr));
+      if (c->stage_mask & 2) HIP_TRY(launch_gemm(a, c->nbatch, c->variant, s, one_pass ? &c->plan_gemm : nullptr));
+      if (c->stage_mask & 4) HIP_TRY(launch_wino_trans_output(w, s, one_pass ? &c->plan_wino_out : nullptr));
     }
     break;
   }
@@ -731,6 +733,19 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     return fail(EHIP_GENERAL_ERROR, "internal: no executor");
   }
   return EHIP_OK;
+}
+
+EHIP_API int ehip_conv_execute_stages(ehip_conv_t *c, void *output_dev, const void *input_dev, const void *bias_dev,
+                                      int stages, int count, void *hip_stream)
+{
+  if (!c || !c->prepared) return fail(EHIP_GENERAL_ERROR, "execute_stages needs a prepared handle");
+  if (c->family != FAM_WINOGRAD) return fail(EHIP_GENERAL_ERROR, "execute_stages: not a Winograd layer");
+  if (stages < 1 || stages > 7) return fail(EHIP_GENERAL_ERROR, "execute_stages: stages is a mask of 1 | 2 | 4");
+  c->stage_mask = stages;
+  int rc = EHIP_OK;
+  for (int i = 0; i < count && rc == EHIP_OK; ++i) rc = ehip_conv_execute(c, output_dev, input_dev, nullptr, bias_dev, hip_stream);
+  c->stage_mask = 7;
+  return rc;
 }
 
 EHIP_API int ehip_conv_execute_repeat(ehip_conv_t *c, void *output_dev, const void *input_dev,

@@ -128,6 +128,17 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *conv, void *output_dev, const void *
 EHIP_API int ehip_conv_execute_repeat(ehip_conv_t *conv, void *output_dev, const void *input_dev,
                                       const void *bias_dev, int count, void *hip_stream);
 
+/* The stages of a Winograd layer on their own, `count` times back to back: what the reference runs as three
+ * objects of its own, elx_conv_wino_trans_input_t::execute (src/elx_conv_wino_trans_input.cpp:599-654),
+ * elx_int8_conv_wino_gemm_t::execute (src/elx_int8_conv_wino_gemm.cpp:23-205) and
+ * elx_conv_wino_trans_output_t::execute (src/elx_conv_wino_trans_output.cpp:212-423), called one after the other by
+ * the executor (src/elx_int8_conv_wino_xopt.hpp:70-121).  `stages` is a mask: 1 = input transform into the
+ * handle's transformed-input buffer, 2 = the A x A GEMMs (in the fused schedule together with the output
+ * transform, into output_dev), 4 = the stand-alone output transform (three-kernel schedule only).  A stage reads
+ * what an earlier call's stage left in the handle's buffers.  For stage-level measurements and tests. */
+EHIP_API int ehip_conv_execute_stages(ehip_conv_t *conv, void *output_dev, const void *input_dev, const void *bias_dev,
+                                      int stages, int count, void *hip_stream);
+
 /* Copies workspace contents to a host buffer in a canonical layout (see EHIP_Q_*).  Synchronous.
  * Returns the number of bytes through *bytes when host_dst is NULL. */
 EHIP_API int ehip_conv_query(ehip_conv_t *conv, int what, void *host_dst, size_t *bytes);
