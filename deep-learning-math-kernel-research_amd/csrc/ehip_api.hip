@@ -398,10 +398,9 @@ int setup_workspace(ehip_conv *c)
     c->units_pad = up(c->ic2, gemm_variant_chunk(c->variant));
     {
       const char *env = getenv("EHIP_WINO_FUSED");
-      // the fused GEMM + output transform is built for F(4x4,3x3); the other tile sizes run the
-      // three-kernel schedule
-      // ... and so does the in-place sum (the stand-alone output transform reads the old output)
-      c->fused = !(env && env[0] == '0') && d.tile_size == 6 && !d.with_ip_sum;
+      // every tile size, with or without the in-place sum, runs the fused GEMM + output transform, as the
+      // reference's a161 schedule does (src/eld_conv.cpp:255-281); EHIP_WINO_FUSED=0 keeps the three kernels
+      c->fused = !(env && env[0] == '0');
     }
     c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
                               : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output";
@@ -412,7 +411,9 @@ int setup_workspace(ehip_conv *c)
     // (blocked: whole blocks of 32 tiles)  allocated with one pad unit behind it
     c->tin_bytes = (size_t)c->nbatch * c->ic2 * (c->tin_blocked ? up(c->t, 32) : c->t) * 16;
     c->tout_bytes = c->fused ? 16 : (size_t)c->nbatch * c->oc2 * c->t * 16 * sizeof(float);
-    if ((rc = dev_alloc(&c->tin, c->tin_bytes + (size_t)c->t * 16, true)) != EHIP_OK) return rc;
+    // (the pad: an odd unit count makes the last k-step read one unit past its position -- in the blocked layout
+    // 512 bytes past the last one, multiplied by zero weights)
+    if ((rc = dev_alloc(&c->tin, c->tin_bytes + ((size_t)c->t * 16 > 1024 ? (size_t)c->t * 16 : 1024), true)) != EHIP_OK) return rc;
     if ((rc = dev_alloc(reinterpret_cast<uint8_t **>(&c->tout), c->tout_bytes, false)) != EHIP_OK) return rc;
     break;
   }
@@ -704,7 +705,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.scale = c->scale; f.shift = c->shift; f.comp = c->comp;
         f.n = w.n; f.ic2 = c->ic2; f.units_pad = c->units_pad; f.oc2 = c->oc2; f.ocpp = c->ocpp;
         f.oh = d.oh; f.ow = d.ow; f.ht = w.ht; f.wt = w.wt; f.nt = w.nt; f.t = w.t;
-        f.with_bias = d.with_bias; f.with_relu = d.with_relu;
+        f.with_bias = d.with_bias; f.with_relu = d.with_relu; f.with_sum = d.with_ip_sum; f.tile = d.tile_size;
         f.out_type = w.out_type; f.out_repS = w.out_repS; f.out_z = w.out_z;
         f.out_nhwc = w.out_nhwc;
         f.trace = trace_buffer();

@@ -133,6 +133,8 @@ struct WinoFusedArgs {
   float out_repS, out_z;   // u8 / s8 output: 1 / output_S, ceil(output_z)
   int n, ic2, units_pad, oc2, ocpp, oh, ow, ht, wt, nt, t;
   int with_bias, with_relu;
+  int with_sum;         // in-place sum: the old output is added before the ReLU
+  int tile;             // tile size A: 6 (or 0), 5, 4
   int out_nhwc;         // output as [n][h][w][c] (c % 16 == 0)
   int nx, ny;           // set by the launcher: blocks of 32 tiles, of 64 channels
   long long *trace;     // development aid, normally null (see EHIP_TRACE)

@@ -393,7 +393,10 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
       const size_t cell = ((size_t)oh * ow_n + ow) * px + 4 * q;   // element index inside the plane
       if (OUT == EHIP_F32) {
         {   // non-temporal: 200 MB of f32 output that nothing reads back soon (C4a 287 -> 261 us); the 4-byte
-            // stores of u8 / s8 output, and the transformed input (read right after), lose with it
+            // stores of u8 / s8 output, and the transformed input (read right after), lose with it.  The
+            // 64-byte pieces (four lanes' 16 bytes) then reach memory one by one: the write counter reads 1.7 x
+            // the output against 1.25 x with plain stores, and the kernel is still the faster one (C4a 251 vs
+            // 277 us; without any output store 230 us: the write path is not what bounds it)
           typedef float v4f __attribute__((ext_vector_type(4)));
           const v4f vv = {y[0][e], y[1][e], y[2][e], y[3][e]};
           __builtin_nontemporal_store(vv, reinterpret_cast<v4f *>(static_cast<float *>(plane) + cell));
@@ -466,10 +469,15 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 //
 // Workgroups are numbered so that the channel blocks of one tile block run next to each other on
 // the same XCD (blockIdx.x % 8), where the second and later ones find the tiles in that XCD's L2.
-template <int KS>
+// A: the tile size (6, 5, 4); its A x A positions are dealt to the four waves in runs of PW = ceil(A x A / 4): nine
+// each for A = 6, four each for A = 4, and 7 + 7 + 7 + 4 for A = 5.
+// SUM: the in-place sum (a compile-time copy: as a run-time flag in the common code it cost the layers without a
+// sum 4 %, as copies behind a uniform branch twice their time -- the kernel sits at the edge of its registers).
+template <int KS, int A = 6, bool SUM = false>
 __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 {
-  extern __shared__ float4 xl[];   // [36][32 tiles][8 cells of 4 channels], cell ^ ((tile / 2) & 7)
+  constexpr int AA = A * A, PW = (AA + 3) / 4, CN = PW * 24, NJ = (CN + 63) / 64;
+  extern __shared__ float4 xl[];   // [AA][32 tiles][8 cells of 4 channels], cell ^ ((tile / 2) & 7)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   // (not through readfirstlane: with the operand addresses computed on the scalar unit the kernel measured 3 %
@@ -483,7 +491,10 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   if (bx >= a.nx) return;          // whole workgroup
   const int t0 = bx * 32, oc0 = by * 64;
   const int oc_real = a.oc2 * 16;
-  const int p0 = 9 * wave;
+  const int p0 = PW * wave;
+  // positions of this wave: all PW, except in the last wave when four runs of PW overshoot A x A (A = 5)
+  constexpr bool EVEN = 4 * PW == AA;
+  const int np = EVEN ? PW : (AA - p0 < PW ? AA - p0 : PW);
   const int nks = a.units_pad >> 1;   // k-steps (32 channels) per position
   const int nkc = nks / KS;
 
@@ -505,7 +516,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     // padded k-steps multiply zero weights: any valid cell will do (an odd unit count reads one
     // unit past the position, which is the next position or the pad unit behind the buffer)
     const int ksc = ks < ks_last ? ks : ks_last;
-    const uint8_t *pb = a.tin_blocked ? a.tin + (((long long)bx * 36 + p) * a.ic2 + 2 * ksc) * 512
+    const uint8_t *pb = a.tin_blocked ? a.tin + (((long long)bx * AA + p) * a.ic2 + 2 * ksc) * 512
                                       : a.tin + ((long long)p * a.ic2 + 2 * ksc) * a.t * 16;
     rb[slot] = *reinterpret_cast<const v4i *>(pb + b_lane);
   };
@@ -514,32 +525,33 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   // the channels at a time: 27 rows of 32 dwords, staged in the 16 KB of LDS the exchange buffer
   // leaves free.  Read from there every lane pays one LDS broadcast per constant instead of a
   // global load instruction (which costs the address path as much as a full 1 KB load).
-  float4 *cl = xl + 36 * 32 * 8 + wave * 216;
-  float4 cst[4];
+  float4 *cl = xl + AA * 32 * 8 + wave * CN;
+  float4 cst[NJ];
   auto load_consts_half = [&](int h) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       int idx = lane + 64 * j;
-      idx = idx < 216 ? idx : 215;
+      idx = idx < CN ? idx : CN - 1;
       const int row = idx >> 3, cell = idx & 7;
       const int i = row / 3, arr = row - 3 * i;
+      const int p = p0 + i < AA ? p0 + i : AA - 1;   // (a wave with fewer positions: rows nobody reads)
       const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
-      cst[j] = *reinterpret_cast<const float4 *>(src + (long long)(p0 + i) * a.ocpp + oc0 + 32 * h + 4 * cell);
+      cst[j] = *reinterpret_cast<const float4 *>(src + (long long)p * a.ocpp + oc0 + 32 * h + 4 * cell);
     }
   };
   auto store_consts_half = [&]() {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const int idx = lane + 64 * j;
-      cl[idx < 216 ? idx : 215] = cst[j];
+      cl[idx < CN ? idx : CN - 1] = cst[j];
     }
   };
   load_consts_half(0);
   store_consts_half();
 
-  v16i acc[9][2];
+  v16i acc[PW][2];
 #pragma unroll
-  for (int i = 0; i < 9; ++i)
+  for (int i = 0; i < PW; ++i)
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -548,8 +560,8 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 #pragma unroll
   for (int k = 0; k < KS; ++k) issue(k, p0, k);
 #pragma unroll
-  for (int i = 0; i < 9; ++i) {
-    for (int c = 0; c < nkc; ++c) {
+  for (int i = 0; i < PW; ++i) {
+    for (int c = 0; c < (EVEN || i < np ? nkc : 0); ++c) {
 #pragma unroll
       for (int k = 0; k < KS; ++k) {
         const v4i b = rb[k] ^ (int)0x80808080;
@@ -558,7 +570,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
         // refill the slot with the operands KS steps ahead (the very last block re-reads itself)
         int pn = p0 + i, ksn = (c + 1) * KS + k;
         if (ksn >= nks) { ksn -= nks; pn += 1; }
-        if (pn > p0 + 8) { pn = p0 + 8; ksn = nks - KS + k; }
+        if (pn > p0 + np - 1) { pn = p0 + np - 1; ksn = nks - KS + k; }
         issue(k, pn, ksn);
       }
     }
@@ -588,12 +600,13 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     };
     read_consts(0, 0);
 #pragma unroll
-    for (int i = 0; i < 9; ++i) {
+    for (int i = 0; i < PW; ++i) {
       const int p = p0 + i;
-      if (i + 1 < 9) read_consts(i + 1, (i + 1) & 1);
+      if (i + 1 < PW) read_consts(i + 1, (i + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
+        if (!EVEN && i >= np) continue;   // a position the last wave does not have
         const float4 sc = kq[i & 1][q], sh = kq[i & 1][4 + q], cf = kq[i & 1][8 + q];
         float4 r;
         r.x = __builtin_fmaf((float)(acc[i][h][4 * q + 0] + __float_as_int(cf.x)), sc.x, sh.x);
@@ -611,9 +624,9 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     TRACE_POINT(3 + 4 * h);
     const int oc = oc0 + 32 * h + 4 * q8;
     if (t < a.t && oc < oc_real) {
-      float4 m[36];
+      float4 m[AA];
 #pragma unroll
-      for (int e = 0; e < 36; ++e) m[e] = xl[(e * 32 + tile_l) * 8 + (q8 ^ ((tile_l >> 1) & 7))];
+      for (int e = 0; e < AA; ++e) m[e] = xl[(e * 32 + tile_l) * 8 + (q8 ^ ((tile_l >> 1) & 7))];
       float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
       if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
       const size_t plane = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (oc >> 4) * 16
@@ -622,14 +635,14 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
       const int q = (oc >> 2) & 3;
       TRACE_POINT(4 + 4 * h);
       if (a.out_type == EHIP_U8)
-        output_tile<EHIP_U8>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
-                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow, false, px);
+        output_tile<EHIP_U8, A>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
+                                static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow, SUM, px);
       else if (a.out_type == EHIP_S8)
-        output_tile<EHIP_S8>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
-                             static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow, false, px);
+        output_tile<EHIP_S8, A>(m, bias, a.with_bias != 0, a.with_relu != 0, a.out_repS, a.out_z,
+                                static_cast<uint8_t *>(a.out) + plane, q, th, tw, a.oh, a.ow, SUM, px);
       else
-        output_tile<EHIP_F32>(m, bias, a.with_bias != 0, a.with_relu != 0, 0.f, 0.f, static_cast<float *>(a.out) + plane, q,
-                              th, tw, a.oh, a.ow, false, px);
+        output_tile<EHIP_F32, A>(m, bias, a.with_bias != 0, a.with_relu != 0, 0.f, 0.f, static_cast<float *>(a.out) + plane, q,
+                                 th, tw, a.oh, a.ow, SUM, px);
     }
     TRACE_POINT(5 + 4 * h);
   }
@@ -688,14 +701,27 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   a.nx = (a.t + 31) / 32;
   a.ny = (a.oc2 * 16 + 63) / 64;
   const int nks = a.units_pad / 2;
-  const size_t lds = (size_t)36 * 32 * 32 * sizeof(float) + 4 * 216 * sizeof(float4);   // exchange + constants
+  const int A = a.tile ? a.tile : 6, AA = A * A;
+  const size_t lds = (size_t)AA * 32 * 32 * sizeof(float) + 4 * (size_t)((AA + 3) / 4 * 24) * sizeof(float4);   // exchange + constants
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
   // operand ring depth in k-steps.  Measured (C4a / C4b / C4a_i8 / C4b_i8, us): 8 deep 261.7 / 177.3 / 247.6 /
   // 178.6, 4 deep 250.4 / 172.8 / 241.2 / 176.5, 2 deep 286.8 / 215.6 (f32 layers)
   int ks_max = 4;
   if (const char *env = getenv("EHIP_WINO_KS")) ks_max = atoi(env);
-  void (*kernel)(WinoFusedArgs) = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8>
-      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4> : k_wino_gemm_output<2>);
+  void (*kernel)(WinoFusedArgs) = nullptr;
+#define EHIP_WF(AV, SV)                                                                                 \
+  kernel = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV>                                \
+      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4, AV, SV> : k_wino_gemm_output<2, AV, SV>)
+  if (a.with_sum) {
+    if (A == 4) EHIP_WF(4, true);
+    else if (A == 5) EHIP_WF(5, true);
+    else EHIP_WF(6, true);
+  } else {
+    if (A == 4) EHIP_WF(4, false);
+    else if (A == 5) EHIP_WF(5, false);
+    else EHIP_WF(6, false);
+  }
+#undef EHIP_WF
   if (nks % 2 != 0) return hipErrorInvalidValue;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;

@@ -227,15 +227,17 @@ def test_wino_no_bias_no_relu():
 
 
 # ---- tile sizes 4 (F(2x2,3x3)) and 5 (F(3x3,3x3)) with u8 input and every user output type ------------
+@pytest.mark.parametrize("fused", ["1", "0"])
 @pytest.mark.parametrize("tile", [4, 5])
 @pytest.mark.parametrize("out_type", [ol.F32, ol.U8, ol.S8])
 @pytest.mark.parametrize("n,ic,oc,hw,with_relu", [(2, 32, 32, 10, True), (1, 64, 80, 13, True), (1, 48, 32, 7, False),
                                                   (2, 16, 16, 4, True)])
-def test_wino_other_tiles_u8_input_quantized_output(tile, out_type, n, ic, oc, hw, with_relu):
+def test_wino_other_tiles_u8_input_quantized_output(tile, out_type, n, ic, oc, hw, with_relu, fused, monkeypatch):
     """The F(2x2,3x3) store rounds toward minus infinity, the others to nearest even; without ReLU negative
     values of a u8 output end as 255 (src/kernel/elk_conv_wino_2x2_3x3_output.hxx:142-151,
     src/kernel/elk_conv_wino_3x3_3x3_output.hxx:74-86)."""
     import torch
+    monkeypatch.setenv("EHIP_WINO_FUSED", fused)   # both schedules against the oracle: they are byte-identical
     E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=9 * n + hw + ic + out_type + tile, out_type=out_type,
                                          with_relu=with_relu, out_z=0.0 if out_type == ol.S8 else 2.4, tile=tile)
     d_x = dev(xq)
@@ -249,7 +251,7 @@ def test_wino_other_tiles_u8_input_quantized_output(tile, out_type, n, ic, oc, h
     tin, exp = _oracle_u8(p, xq, wb, bias)
     assert tin.shape[0] == tile * tile
     conv = E.Conv(d)
-    assert conv.kernel_name.endswith("k_wino_trans_output")   # three-kernel schedule
+    assert conv.kernel_name.endswith("k_wino_gemm_output" if fused == "1" else "k_wino_trans_output")
     tdt = {ol.F32: torch.float32, ol.U8: torch.uint8, ol.S8: torch.int8}[out_type]
     d_out = torch.full(exp.shape, 5, dtype=tdt, device="cuda")
     d_b = dev(bias)
@@ -285,12 +287,14 @@ def test_wino_automatic_tile_size():
 
 
 # ---- in-place sum (with_ip_sum) in the output transform ------------------------------------------------
+@pytest.mark.parametrize("fused", ["1", "0"])
 @pytest.mark.parametrize("tile", [6, 4, 5])
 @pytest.mark.parametrize("out_type", [ol.F32, ol.U8, ol.S8])
-def test_wino_with_ip_sum(tile, out_type):
+def test_wino_with_ip_sum(tile, out_type, fused, monkeypatch):
     """The old output (f32, or the u8 / s8 code as it is) is added after the output quantization and before
     the ReLU (src/kernel/elk_conv_wino_4x4_3x3_output.hxx:168-187)."""
     import torch
+    monkeypatch.setenv("EHIP_WINO_FUSED", fused)
     n, ic, oc, hw = 2, 32, 48, 11
     E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=31 + tile + out_type, out_type=out_type,
                                          out_z=0.0 if out_type == ol.S8 else 1.6, tile=tile)
@@ -309,7 +313,7 @@ def test_wino_with_ip_sum(tile, out_type):
     exp = ol.wino_trans_output(p, tout, bias, out_init=old)
     assert not np.array_equal(exp, ol.wino_trans_output(p, tout, bias))   # the sum operand matters
     conv = E.Conv(d)
-    assert conv.kernel_name.endswith("k_wino_trans_output")
+    assert conv.kernel_name.endswith("k_wino_gemm_output" if fused == "1" else "k_wino_trans_output")
     d_out = dev(old)
     d_b = dev(bias)
     conv.execute(d_out, dev(xq), dev(wb), d_b)
@@ -328,8 +332,6 @@ def test_wino_nhwc_activations(tile, out_type, with_sum, in_nhwc, out_nhwc, fuse
     Winograd transforms, src/elx_conv_wino_trans_input.cpp:226-262, src/elx_conv_wino_trans_output.cpp:136-190):
     the same values as with nChw16c, in the other layout."""
     import torch
-    if fused == "0" and (tile != 6 or with_sum):
-        pytest.skip("only the 6x6 tile without a sum has a fused schedule to switch off")
     monkeypatch.setenv("EHIP_WINO_FUSED", fused)
     n, ic, oc, hw = 2, 48, 80, 13
     E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=91 + tile + out_type, out_type=out_type,
