@@ -370,8 +370,14 @@ int setup_workspace(ehip_conv *c)
     c->T = d.flatting_t > 0 ? (d.flatting_t > d.ow ? d.ow : d.flatting_t) : 1;
     c->wtb = (d.ow + c->T - 1) / c->T;
     c->Tr = d.ow % c->T ? d.ow % c->T : c->T;
+    // what the depthwise launchers pack into 16 or 8 bits and address with 32: refused here, at setup, so that a
+    // handle that was created also executes
+    if (d.ih >= 65536 || d.iw >= 65536 || d.oh >= 65536 || d.ow >= 65536 || d.pad_t > 255 || d.pad_l > 255 ||
+        (long long)d.n * c->oc2 * d.oh * d.ow >= (1ll << 28) || (long long)d.n * c->oc2 * d.ih * d.iw >= (1ll << 28))
+      return fail(EHIP_UNIMPLEMENTED, "direct_depthwise: tensor too large");
     c->kernel_name = depthwise_mfma_applies(d.stride_h, d.oh, d.ow, d.pad_t, d.pad_l, d.output_type, d.with_relu, d.relu_lower,
-                                            d.relu_upper) ? "k_depthwise3x3_mfma" : "k_depthwise3x3_u8s8";
+                                            d.relu_upper, (long long)d.n * c->oc2, d.ih, d.iw)
+        ? "k_depthwise3x3_mfma" : "k_depthwise3x3_u8s8";
     break;
   }
   case FAM_WINOGRAD: {
@@ -381,17 +387,10 @@ int setup_workspace(ehip_conv *c)
     c->ht = (d.oh + d.tile_size - 3) / (d.tile_size - 2);
     c->wt = (d.ow + d.tile_size - 3) / (d.tile_size - 2);
     c->nt = c->ht * c->wt;
-    // The three stages can run over a few images at a time (EHIP_WINO_CHUNK) with the intermediates
-    // sized for one pass; measured on MI355X this only costs (the 256 MB memory-side cache does not
-    // keep the f32 GEMM result away from HBM), so one pass over the whole batch is the default.
-    {
-      long long cn = d.n;
-      const char *env = getenv("EHIP_WINO_CHUNK");
-      if (env && env[0]) cn = atoi(env);
-      if (cn < 1) cn = 1;
-      if (cn > d.n) cn = d.n;
-      c->chunk_n = (int)cn;
-    }
+    // One pass over the whole batch.  (Running the stages over a few images at a time, with the intermediates
+    // sized for one pass, was measured on MI355X and only costs: the 256 MB memory-side cache does not keep the
+    // intermediates away from HBM.  The pass loop of execute stays: chunk_n images per pass.)
+    c->chunk_n = d.n;
     c->t = c->nt * c->chunk_n;   // tiles per pass
     if ((long long)c->t >= (1ll << 31) / 64) return fail(EHIP_UNIMPLEMENTED, "winograd: too many tiles");
     c->variant = gemm_pick_variant(c->t, c->oc2, c->ic2, c->nbatch, 1);
@@ -404,10 +403,7 @@ int setup_workspace(ehip_conv *c)
     }
     c->kernel_name = c->fused ? std::string("k_wino_trans_input_u8 + k_wino_gemm_output")
                               : std::string("k_wino_trans_input_u8 + ") + gemm_variant_name(c->variant) + " + k_wino_trans_output";
-    {
-      const char *env = getenv("EHIP_WINO_TIN_BLOCKED");
-      c->tin_blocked = c->fused && !(env && env[0] == '0');
-    }
+    c->tin_blocked = c->fused;   // the fused schedule's layout: a workgroup's whole input is one contiguous run
     // (blocked: whole blocks of 32 tiles)  allocated with one pad unit behind it
     c->tin_bytes = (size_t)c->nbatch * c->ic2 * (c->tin_blocked ? up(c->t, 32) : c->t) * 16;
     c->tout_bytes = c->fused ? 16 : (size_t)c->nbatch * c->oc2 * c->t * 16 * sizeof(float);

@@ -630,10 +630,11 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
 hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_t s, LaunchPlan<Conv3x3Args> *plan)
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
-    plan->args.in = a0.in;
-    plan->args.out = a0.out;
+    Conv3x3Args local = plan->args;   // a copy: the kept plan is only read (executes from several threads or streams)
+    local.in = a0.in;
+    local.out = a0.out;
     // (the plan keeps this kernel's pointer under the one-argument type of its slot)
-    return conv3x3v_enqueue(reinterpret_cast<conv3x3v_kernel_t>(plan->kernel), plan->grid, plan->lds, plan->args, s);
+    return conv3x3v_enqueue(reinterpret_cast<conv3x3v_kernel_t>(plan->kernel), plan->grid, plan->lds, local, s);
   }
   const Variant &k = kVariants[variant];
   Conv3x3Args a = a0;
@@ -669,15 +670,16 @@ hipError_t launch_conv3x3v(const Conv3x3Args &a0, int n, int variant, hipStream_
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return e;
   }
-  if (plan) {
-    plan->valid = true;
+  const hipError_t e = conv3x3v_enqueue(kernel, grid, (unsigned)lds_bytes, a, s);
+  if (plan && e == hipSuccess) {   // kept only once the first launch has gone out
     plan->kernel = reinterpret_cast<void (*)(Conv3x3Args)>(kernel);
     plan->grid = grid;
     plan->block = dim3(kBlock);
     plan->lds = (unsigned)lds_bytes;
     plan->args = a;
+    plan->valid = true;
   }
-  return conv3x3v_enqueue(kernel, grid, (unsigned)lds_bytes, a, s);
+  return e;
 }
 
 }  // namespace ehip

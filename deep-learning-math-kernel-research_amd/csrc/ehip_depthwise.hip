@@ -473,14 +473,13 @@ hipError_t dw_launch(LaunchPlan<DepthwiseArgs> *plan, dw_kernel_t kernel, dim3 g
   }
   LaunchPlan<DepthwiseArgs> local;
   LaunchPlan<DepthwiseArgs> *p = plan ? plan : &local;
-  p->valid = true;
   p->kernel = reinterpret_cast<void (*)(DepthwiseArgs)>(kernel);
   p->grid = grid;
   p->block = block;
   p->lds = 0;
   p->args = a;
   p->enqueue = dw_enqueue;
-  return dw_enqueue(*p, s);
+  return plan_first_launch(p, s);
 }
 template <int RB, int S>
 dw_kernel_t kernel_rbs(int mode)
@@ -497,10 +496,16 @@ dw_kernel_t kernel_rb(int stride, int mode)
 // The matrix-core kernel: stride 1, u8 output with a ReLU inside the code range, pads 0 / 1, and a plane
 // of up to four 32-column chunks whose chunks and 8-row strips are mostly real pixels (EHIP_DW_MFMA=0 / 1
 // overrides the last condition).
-bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, int out_type, int with_relu, float lo, float hi)
+bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, int out_type, int with_relu, float lo, float hi,
+                            long long planes, int ih, int iw)
 {
   if (stride != 1 || out_type != EHIP_U8 || !with_relu || !(lo >= 0.0f && hi <= 255.0f && hi >= lo)) return false;
   if (pad_t < 0 || pad_t > 1 || pad_l < 0 || pad_l > 1 || ow > 128) return false;
+  // the kernel addresses both tensors with 32-bit byte offsets and keeps the last 64 KB of that range as "nowhere";
+  // a larger layer runs on the dot4 kernel
+  if (planes * ((oh + 7) / 8) >= (1ll << 30) || planes * ih * iw * 16 >= (1ll << 32) - 65536 ||
+      planes * oh * ow * 16 >= (1ll << 32) - 65536)
+    return false;
   if (const char *env = getenv("EHIP_DW_MFMA")) return atoi(env) != 0;
   // measured (N = 64, with non-temporal output stores): ahead of the dot4 kernel at 28, 56 and 112 columns
   // (8.8 / 13.1 / 14.2 us against 10.2 / 16.7 / 16.4 us for 256 / 128 / 32 channels), behind it on the half-empty
@@ -512,16 +517,15 @@ bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, in
 hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<DepthwiseArgs> *plan)
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
-    plan->args.in = a0.in;
-    plan->args.out = a0.out;
-    return plan_relaunch(*plan, s);
+    return plan_relaunch(*plan, [&](DepthwiseArgs &x) { x.in = a0.in; x.out = a0.out; }, s);
   }
   DepthwiseArgs a = a0;
   if (a.stride != 1 && a.stride != 2) {
     set_error("depthwise: stride must be 1 or 2");
     return hipErrorInvalidValue;
   }
-  if (depthwise_mfma_applies(a.stride, a.oh, a.ow, a.pad_t, a.pad_l, a.out_type, a.with_relu, a.lo, a.hi)) {
+  if (depthwise_mfma_applies(a.stride, a.oh, a.ow, a.pad_t, a.pad_l, a.out_type, a.with_relu, a.lo, a.hi, (long long)a.n * a.g2, a.ih,
+                             a.iw)) {
     const int nc = (a.ow + 31) / 32;
     const bool full = a.lo == 0.0f && a.hi == 255.0f;
     a.T_magic = div_magic(a.T);
@@ -536,8 +540,7 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<D
     }
     // a run of strips per workgroup, about four workgroups per CU (enough to hide a barrier and the
     // epilogue of one behind the MFMAs of another), the same run length for all so that none is the tail
-    int cus = 256 * 4;
-    if (const char *env = getenv("EHIP_DW_WGS_PER_CU")) cus = 256 * atoi(env);
+    const int cus = 256 * 4;
     int per_wg = (int)((total + cus - 1) / cus);
     if (per_wg < 1) per_wg = 1;
     a.strips_per_wg = per_wg;
@@ -553,10 +556,9 @@ hipError_t launch_depthwise(const DepthwiseArgs &a0, hipStream_t s, LaunchPlan<D
   int rb = (a.oh >= 28 && a.oh % 7 == 0) ? 7 : (a.oh >= 16 ? 4 : (a.oh >= 7 ? 2 : 1));
   // measured at N = 64: 14 x 14 planes at stride 1 want seven rows as well (512 channels: 6.05 against 7.2 us with
   // two, 6.3 with four), 56 x 56 outputs of a stride-2 layer two (64 channels 112 -> 56: 13.4 against 15.3 us with
-  // seven: 15 input rows of five pixels per lane are too many loads in flight); EHIP_DW_RB forces 1, 2, 4 or 7
+  // seven: 15 input rows of five pixels per lane are too many loads in flight)
   if (a.stride == 1 && a.oh == 14) rb = 7;
   if (a.stride == 2 && a.oh >= 56) rb = 2;
-  if (const char *env = getenv("EHIP_DW_RB")) { const int e = atoi(env); if (e == 1 || e == 2 || e == 4 || e == 7) rb = e; }
   const int ohb = (a.oh + rb - 1) / rb;
   const int wp = (a.ow + 1) / 2;
   a.lanes_per_plane = ohb * wp * 4;

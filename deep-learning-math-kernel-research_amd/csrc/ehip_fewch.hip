@@ -486,9 +486,7 @@ hipError_t launch_conv_fewch(FewChArgs &a, hipStream_t s, LaunchPlan<FewChArgs> 
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
     if (a.in_nhwc && (reinterpret_cast<uintptr_t>(a.in) & 3)) return hipErrorInvalidValue;   // aligned dword loads
-    plan->args.in = a.in;
-    plan->args.out = a.out;
-    return plan_relaunch(*plan, s);
+    return plan_relaunch(*plan, [&](FewChArgs &x) { x.in = a.in; x.out = a.out; }, s);
   }
   {
     // lean_mode() but for the per-pixel shift rows, which this kernel's lean path reads itself

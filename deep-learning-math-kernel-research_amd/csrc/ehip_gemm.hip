@@ -693,7 +693,8 @@ typedef void (*smallk_kernel_t)(EHIP_SMALLK_HEAD, GemmArgs);
 template <int KS>
 smallk_kernel_t smallk_kernel(int tnw)
 {
-  return tnw == 2 ? k_gemm_smallk_u8s8<2, KS> : k_gemm_smallk_u8s8<1, KS>;
+  (void)tnw;   // (two pixel tiles per iteration cost more in occupancy than they gain in overlap: one)
+  return k_gemm_smallk_u8s8<1, KS>;
 }
 hipError_t smallk_enqueue(const LaunchPlan<GemmArgs> &plan, hipStream_t s)
 {
@@ -710,14 +711,13 @@ hipError_t smallk_launch(LaunchPlan<GemmArgs> *plan, smallk_kernel_t kernel, dim
   if (a.stride_h > 255 || a.stride_w > 255) return hipErrorInvalidValue;   // geom's fields
   LaunchPlan<GemmArgs> local;
   LaunchPlan<GemmArgs> *p = plan ? plan : &local;
-  p->valid = true;
   p->kernel = reinterpret_cast<void (*)(GemmArgs)>(kernel);
   p->grid = grid;
   p->block = dim3(kBlock);
   p->lds = 0;
   p->args = a;
   p->enqueue = smallk_enqueue;
-  return smallk_enqueue(*p, s);
+  return plan_first_launch(p, s);
 }
 }  // namespace
 
@@ -740,14 +740,12 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
   const int groups = oc_tiles;
   a.sk_wo = groups >= 4 ? 4 : (groups >= 2 ? 2 : 1);
   const int ny = (groups + a.sk_wo - 1) / a.sk_wo;
-  int tnw = 1;   // (two pixel tiles per iteration cost more in occupancy than they gain in overlap)
-  if (const char *env = getenv("EHIP_SMALLK_TNW")) tnw = atoi(env) == 2 ? 2 : 1;
+  const int tnw = 1;   // (two pixel tiles per iteration cost more in occupancy than they gain in overlap)
   const int ntiles = (a.p_total + 32 * tnw - 1) / (32 * tnw);
   const int wpn = 4 / a.sk_wo;
   // one resident set of workgroups, so that a wave amortises its weights over many tiles
   int nx = (ntiles + wpn - 1) / wpn;
-  int wgs = 768;   // three workgroups per CU: what the register budget of the one-tile form admits, and the measured optimum
-  if (const char *env = getenv("EHIP_SMALLK_WGS")) wgs = atoi(env) > 0 ? atoi(env) : wgs;
+  const int wgs = 768;   // three workgroups per CU: what the register budget of the one-tile form admits, and the measured optimum
   const int cap = (wgs + ny - 1) / ny;
   if (nx > cap) nx = cap;
   smallk_kernel_t kernel = ks == 1 ? smallk_kernel<1>(tnw) : (ks == 2 ? smallk_kernel<2>(tnw) : smallk_kernel<4>(tnw));
@@ -757,7 +755,6 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
   // faster than one; eight tiles lose again.
   int ocw = ks == 4 ? 2 : 4;
   while (ocw > 1 && ocw > oc_tiles) ocw >>= 1;
-  if (const char *env = getenv("EHIP_SMALLK_OCW")) { const int e = atoi(env); if (e == 1 || e == 2 || (e == 4 && ks < 4)) ocw = e; }
   if (a.lean && ocw > 1) {
     const int groups2 = (oc_tiles + ocw - 1) / ocw;
     a.sk_wo = groups2 >= 4 ? 4 : (groups2 >= 2 ? 2 : 1);
@@ -766,8 +763,7 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
     const int ntiles2 = (a.p_total + 31) / 32;
     int nx2 = (ntiles2 + wpn2 - 1) / wpn2;
     // one resident set: four workgroups per CU with the weights of up to 32 channels per lane, else three
-    int wgs2 = ks == 1 ? 1024 : 768;
-    if (const char *env = getenv("EHIP_SMALLK_WGS")) wgs2 = atoi(env) > 0 ? atoi(env) : wgs2;
+    const int wgs2 = ks == 1 ? 1024 : 768;
     const int cap2 = (wgs2 + ny2 - 1) / ny2;
     if (nx2 > cap2) nx2 = cap2;
     smallk_kernel_t lk = nullptr;
@@ -788,9 +784,7 @@ hipError_t launch_gemm_smallk(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gemm
 hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t s, LaunchPlan<GemmArgs> *plan)
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
-    plan->args.in = a0.in;
-    plan->args.out = a0.out;
-    return plan_relaunch(*plan, s);
+    return plan_relaunch(*plan, [&](GemmArgs &x) { x.in = a0.in; x.out = a0.out; }, s);
   }
   if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s, plan);
   if (gemm1x1_wres_applies(a0, nbatch)) return launch_gemm1x1_wres(a0, s, plan);
@@ -805,7 +799,7 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   a.ny = (a.oc2 * 16 + k.oc_t - 1) / k.oc_t;
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8), nbatch);
   // prefetch depth: must divide the number of fills.  Measured on the configured layers depth 2 is
-  // as good as it gets (depth 4 costs registers and gains nothing); EHIP_GEMM_DEPTH overrides.
+  // as good as it gets (depth 4 costs registers and gains nothing).
   const int taps = a.kh * a.kw > 1 ? a.kh * a.kw : 1;
   a.k_real = taps * a.units_pad;   // kh x kw: units_pad is the ic2 real units of a tap
   a.k_units = up(a.k_real, k.kc);
@@ -813,8 +807,6 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   a.kw_magic = div_magic(a.kw > 0 ? a.kw : 1);
   const int nchunks = a.k_units / k.kc;
   int dl = 1;
-  const char *env = getenv("EHIP_GEMM_DEPTH");
-  if (env && env[0]) dl = atoi(env) >= 4 ? 2 : (atoi(env) >= 2 ? 1 : 0);
   if (taps > 1 && (taps > 64 || nbatch != 1)) return hipErrorInvalidValue;
   const int fmt = taps > 1 ? (a.in_nhwc ? 4 : (a.ic2 % k.kc == 0 ? 2 : 3)) : (a.in_nhwc ? 1 : 0);
   while (dl > 0 && (nchunks % (1 << dl) != 0 || !k.kernel[fmt][dl])) --dl;

@@ -416,6 +416,7 @@ int gemm1x1_res_pick(const GemmArgs &a, int nbatch)
   const char *env = getenv("EHIP_GEMM1X1_RES");
   if (env && env[0] == '0') return -1;
   if (nbatch != 1 || a.kh * a.kw > 1 || a.ep.shift_tab) return -1;
+  if (a.stride_h > 255 || a.stride_w > 255 || a.oc2 >= 4096) return -1;   // what the kernel's packed leading argument holds
   // nhwc output: through the lean epilogue only (a lane's 16 bytes are contiguous there as well; the general
   // epilogue of this kernel addresses blocked cells)
   if (a.out_nhwc && !lean_mode(a.ep, false)) return -1;
@@ -489,7 +490,6 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
   if (a.stride_h > 255 || a.stride_w > 255 || a.oc2 >= 4096) return hipErrorInvalidValue;   // geom's fields
   LaunchPlan<GemmArgs> local;
   LaunchPlan<GemmArgs> *p = plan ? plan : &local;
-  p->valid = true;
   p->kernel = reinterpret_cast<void (*)(GemmArgs)>(kernel);
   p->grid = grid;
   p->block = dim3(kBlock);
@@ -497,7 +497,7 @@ hipError_t launch_gemm1x1_res(const GemmArgs &a0, int v, hipStream_t s, LaunchPl
   p->args = a;
   p->enqueue = res_enqueue;
   p->name = k.name;   // (nhwc output: the handle could not tell at creation whether the lean epilogue applies)
-  return res_enqueue(*p, s);
+  return plan_first_launch(p, s);
 }
 
 }  // namespace ehip

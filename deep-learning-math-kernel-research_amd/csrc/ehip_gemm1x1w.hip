@@ -398,7 +398,7 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch)
   // 512 -> 256 at 28 x 28: 11.7 vs 13.4, 256 -> 256 at 28 x 28: 8.3 vs 9.8), level or behind with shorter runs
   // (512 -> 512 at 14 x 14: 8.0 vs 7.7, 512 -> 2048 at 7 x 7: 8.2 vs 8.0) and with 1024 input channels, whose waves own
   // one tile of 32 channels (1024 -> 256 at 14 x 14: 8.6 vs 8.4, 1024 -> 1024 at 7 x 7: 8.6 vs 7.2)
-  if (!forced && !getenv("EHIP_WRES_TRY32") && (a.units_pad > 32 || (long long)((a.p_total + 31) / 32) * nb < 3 * 512)) return false;
+  if (!forced && (a.units_pad > 32 || (long long)((a.p_total + 31) / 32) * nb < 3 * 512)) return false;
   // a lane's offsets into the input and the output are 32 bits wide
   const long long n_img = a.p_total / (a.ohw > 0 ? a.ohw : 1);
   if (n_img * a.ic2 * a.ihw * 16 >= (1ll << 32) || (long long)a.p_total * a.oc2 * 16 >= (1ll << 32)) return false;
@@ -424,7 +424,6 @@ hipError_t launch_gemm1x1_wres(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gem
   if (e != hipSuccess) return e;
   LaunchPlan<GemmArgs> local;
   LaunchPlan<GemmArgs> *p = plan ? plan : &local;
-  p->valid = true;
   p->kernel = reinterpret_cast<void (*)(GemmArgs)>(kernel);
   p->grid = dim3(8 * g.nb * ((g.nreg + 7) / 8));
   p->block = dim3(g.nw * 64);
@@ -432,7 +431,7 @@ hipError_t launch_gemm1x1_wres(const GemmArgs &a0, hipStream_t s, LaunchPlan<Gem
   p->args = a;
   p->enqueue = wres_enqueue;
   p->name = "k_gemm1x1_wres";
-  return wres_enqueue(*p, s);
+  return plan_first_launch(p, s);
 }
 
 }  // namespace ehip

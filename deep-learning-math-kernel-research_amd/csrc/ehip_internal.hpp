@@ -160,22 +160,41 @@ template <typename Args>
 inline hipError_t plan_launch(LaunchPlan<Args> *plan, void (*kernel)(Args), dim3 grid, dim3 block, size_t lds, const Args &a,
                               hipStream_t s)
 {
-  if (plan) {
-    plan->valid = true;
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, a);
+  const hipError_t e = hipGetLastError();
+  if (plan && e == hipSuccess) {   // kept only once the first launch has gone out
     plan->kernel = kernel;
     plan->grid = grid;
     plan->block = block;
     plan->lds = (unsigned)lds;
     plan->args = a;
+    plan->valid = true;
   }
-  hipLaunchKernelGGL(kernel, grid, block, lds, s, a);
-  return hipGetLastError();
+  return e;
 }
+// A launcher that fills a plan by hand launches through this: the plan becomes valid when the launch has gone out.
 template <typename Args>
-inline hipError_t plan_relaunch(LaunchPlan<Args> &plan, hipStream_t s)
+inline hipError_t plan_first_launch(LaunchPlan<Args> *p, hipStream_t s)
 {
-  if (plan.enqueue) return plan.enqueue(plan, s);
-  hipLaunchKernelGGL(plan.kernel, plan.grid, plan.block, plan.lds, s, plan.args);
+  hipError_t e;
+  if (p->enqueue) {
+    e = p->enqueue(*p, s);
+  } else {
+    hipLaunchKernelGGL(p->kernel, p->grid, p->block, p->lds, s, p->args);
+    e = hipGetLastError();
+  }
+  p->valid = e == hipSuccess;
+  return e;
+}
+// Later launches of a valid plan: the kept plan is only read.  The tensors of this call are patched into a COPY of
+// the argument block, so executes of one handle from several threads or streams never see each other's pointers.
+template <typename Args, typename Patch>
+inline hipError_t plan_relaunch(const LaunchPlan<Args> &plan, Patch patch, hipStream_t s)
+{
+  LaunchPlan<Args> local = plan;
+  patch(local.args);
+  if (local.enqueue) return local.enqueue(local, s);
+  hipLaunchKernelGGL(local.kernel, local.grid, local.block, local.lds, s, local.args);
   return hipGetLastError();
 }
 
@@ -203,7 +222,8 @@ const char *conv3x3v_variant_name(int variant);
 
 hipError_t launch_depthwise(const DepthwiseArgs &a, hipStream_t s, LaunchPlan<DepthwiseArgs> *plan = nullptr);
 hipError_t launch_depthwise_diag(const int8_t *wpacked, int g2n, void *diag, hipStream_t s);
-bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, int out_type, int with_relu, float lo, float hi);
+bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, int out_type, int with_relu, float lo, float hi,
+                            long long planes, int ih, int iw);
 hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
 hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);

@@ -651,8 +651,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s, LaunchPlan<WinoArgs> *plan)
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
-    plan->args.in = a0.in;
-    return plan_relaunch(*plan, s);
+    return plan_relaunch(*plan, [&](WinoArgs &x) { x.in = a0.in; }, s);
   }
   WinoArgs a = a0;
   {
@@ -673,9 +672,7 @@ hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s, LaunchPlan
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan)
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
-    plan->args.out = a.out;
-    plan->args.bias = a.bias;
-    return plan_relaunch(*plan, s);
+    return plan_relaunch(*plan, [&](WinoArgs &x) { x.out = a.out; x.bias = a.bias; }, s);
   }
   dim3 grid((a.t + 63) / 64, a.oc2);
   void (*kern)(WinoArgs) = nullptr;
@@ -693,9 +690,7 @@ hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan
 hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan)
 {
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
-    plan->args.out = a0.out;
-    plan->args.bias = a0.bias;
-    return plan_relaunch(*plan, s);
+    return plan_relaunch(*plan, [&](WinoFusedArgs &x) { x.out = a0.out; x.bias = a0.bias; }, s);
   }
   WinoFusedArgs a = a0;
   a.nx = (a.t + 31) / 32;

@@ -154,11 +154,12 @@ def test_conv1x1_weights_resident_kernel_ring_depths(nbuf, monkeypatch):
 
 
 def test_conv1x1_weights_resident_kernel_can_be_switched_off(monkeypatch):
+    # (256 -> 1024 at 14 x 14, N = 64: runs of three tiles per workgroup, the launcher's own choice)
     monkeypatch.setenv("EHIP_GEMM1X1_WRES", "0")
-    res = run_and_compare(Layer(16, 512, 256, 14, out_type=ol.S8, with_sum=True, seed=720))
+    res = run_and_compare(Layer(64, 256, 1024, 14, out_type=ol.S8, with_sum=True, seed=720))
     assert res["conv"].kernel_name != "k_gemm1x1_wres"
     monkeypatch.delenv("EHIP_GEMM1X1_WRES")
-    res = run_and_compare(Layer(16, 512, 256, 14, out_type=ol.S8, with_sum=True, seed=720))
+    res = run_and_compare(Layer(64, 256, 1024, 14, out_type=ol.S8, with_sum=True, seed=720))
     assert res["conv"].kernel_name == "k_gemm1x1_wres"
 
 
@@ -678,6 +679,17 @@ def test_setup_rejects_what_the_reference_rejects():
     conv = E.Conv(E.make_desc(1, 64, 64, 8, 8))
     with pytest.raises(E.EulerHipError):
         conv.execute(None, None)
+
+
+def test_setup_refuses_what_no_kernel_can_address():
+    """Limits of the kernels' packed arguments and 32-bit offsets are applied when the handle is created (nothing is
+    allocated yet), so that a handle that exists also executes: a depthwise layer of 2^30 output cells is refused
+    with a message, not created and then failed at every execute."""
+    E = pkg()
+    d = E.make_desc(4096, 1024, 1024, 64, 64, 3, 3, pad=1, g=1024, algorithm=E.CONV_DIRECT, flatting_t=16)
+    with pytest.raises(E.EulerHipError) as ei:
+        E.Conv(d)
+    assert ei.value.code == E.EHIP_UNIMPLEMENTED and "tensor too large" in str(ei.value)
 
 
 @pytest.mark.parametrize("kind", ["1x1 many channels", "1x1 many channels, sum, nhwc", "1x1 few channels", "1x1 few channels f32", "3x3",
