@@ -74,9 +74,11 @@ struct PixInfo {
 }  // namespace
 
 // geom = stride_h | stride_w << 8 | dense << 16 | nb << 20 (channel blocks of 4 x TM x 32)
+// (the leading arguments are what the first tile's loads and the weight loads need: they arrive in scalar registers
+// with the wave, while the rest of the argument block is still being fetched; owiw = ow | iw << 16)
 #define EHIP_WRES_HEAD                                                                                                  \
-  const uint8_t *in, const int8_t *w, const int *comp, int p_total, int ohw, unsigned ohw_magic, int ihw, int ic2, int ocpp, \
-      unsigned geom, int ntiles_all, int nreg, int stage_bytes
+  const uint8_t *in, const int8_t *w, int p_total, int ohw, unsigned ohw_magic, int ihw, int ic2, int ocpp, unsigned geom, \
+      int ntiles_all, int nreg, unsigned owiw, unsigned ow_magic
 // NW waves per workgroup: four, two workgroups per CU; or eight in one workgroup per CU, which then share ONE copy
 // of every pixel tile (1024 input channels, where a wave can only hold the weights of 32 channels: eight waves own
 // the 256 channels that four own with fewer input channels)
@@ -84,8 +86,9 @@ template <int NKS, int TM, int SUM, int NW>   // SUM: 0 none, 1 the old output i
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_WRES_HEAD, GemmArgs rest)
 {
   GemmArgs a = rest;
-  a.in = in; a.w = w; a.ep.comp = comp; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic;
-  a.ihw = ihw; a.ic2 = ic2; a.ocpp = ocpp;
+  a.in = in; a.w = w; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic;
+  a.ihw = ihw; a.ic2 = ic2; a.ocpp = ocpp; a.ow = (int)(owiw & 0xffffu); a.iw = (int)(owiw >> 16); a.ow_magic = ow_magic;
+  constexpr int stage_bytes = NKS * 1024 + (SUM ? NW * TM * 1024 : 0);
   a.stride_h = (int)(geom & 0xffu); a.stride_w = (int)((geom >> 8) & 0xffu);
   const bool dense = (geom >> 16) & 1u;
   const int nb = (int)(geom >> 20);
@@ -113,15 +116,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
   const int oc_lane = ocw + 16 * lh;             // the lane's 16 channels of tile 0 (tile mt: + 32 mt)
   const int oc_real = a.oc2 * 16;
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds;
-  const int stage_cells = stage_bytes >> 4;
-  const int nbuf = a.wr_nbuf;
+  constexpr int stage_cells = stage_bytes >> 4;
   // The weights fill the vector registers: the per-channel constants (scale, shift, compensation) of the wave's
   // channels live in a wave-private piece of LDS behind the stages, [3][OCW] dwords, channel c of the wave at
   // index c: a lane's four consecutive channels are one 16-byte read, the same for half a wave.
-  float *const cl_f = reinterpret_cast<float *>(lds + (size_t)nbuf * stage_cells) + wave * (3 * OCW);
   TRACE_POINT(0);
 
-  auto pix_info = [&](int tt) -> PixInfo {
+  auto pix_info = [&](int tt, bool with_out = true) -> PixInfo {
     PixInfo pi;
     const int gp = p0 + 32 * tt + l32;
     pi.valid = gp < a.p_total;
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
       sp = oh * a.stride_h * a.iw + (r - oh * a.ow) * a.stride_w;
     }
     pi.in_off = ((unsigned)n * (unsigned)(a.ic2 * a.ihw) + (unsigned)sp) * 16u;
-    pi.out_off = a.out_nhwc ? (unsigned)gpc * (unsigned)oc_real : ((unsigned)n * (unsigned)(a.oc2 * a.ohw) + (unsigned)r) * 16u;
+    pi.out_off = with_out ? (a.out_nhwc ? (unsigned)gpc * (unsigned)(a.oc2 * 16) : ((unsigned)n * (unsigned)(a.oc2 * a.ohw) + (unsigned)r) * 16u) : 0u;
     return pi;
   };
   // byte offset, from the pixel's out_off, of the lane's cell in the wave's tile mt
@@ -171,15 +172,17 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
     for (int d = 0; d < LPT; ++d) issue_load(d);
   };
 
-  // ---- prologue: the first tile, the constants, the weights, the second tile ----------------------------------
-  issue_tile(0, 0);
-  TRACE_POINT(1);
-
-  if (lane < OCW) {
-    cl_f[lane] = a.ep.scale[ocw + lane];
-    cl_f[OCW + lane] = a.ep.shift[ocw + lane];
-    reinterpret_cast<int *>(cl_f)[2 * OCW + lane] = a.ep.comp[ocw + lane];
+  // ---- prologue ------------------------------------------------------------------------------------------------
+  // First what the leading arguments alone can address: the first tile's pixels and the weights.  The rest of the
+  // argument block (output pointer, constants, ring depth) is still on its way from memory then.
+  {
+    const PixInfo pi = pix_info(0, false);
+    pend_in = pi.in_off + (unsigned)lh * unit_stride;
+    pend_sb = lds_base;
+#pragma unroll
+    for (int d = 0; d < NKS / NW; ++d) issue_load(d);
   }
+  TRACE_POINT(1);
   // weights [units][ocpp][16]: lane = packed row l32 of unit 2 ks + lh; tile mt 32 rows on
   const int8_t *wb = a.w + ((long long)lh * a.ocpp + ocw + l32) * 16;
   const long long w_step = (long long)a.ocpp * 32;   // two units
@@ -188,9 +191,22 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
   for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) areg[ks][mt] = *reinterpret_cast<const v4i *>(wb + ks * w_step + mt * 512);
-  // The second tile behind the weights: a wave's loads complete in issue order, and the first tile's K loop needs
-  // the weights, not the second tile.  (The compiler's waits for the weights then cover these few loads as well: the
-  // last k-steps of the first tile wait for the second tile, which the tile's barrier waits for anyway.)
+  // Then what needs the argument block: the per-channel constants (into registers now, into LDS once the weights
+  // are in: a wave's loads complete in issue order, and nothing may make the first tile's K loop wait for more than
+  // its next weights), the first tile's sum operand, the second tile.  (The compiler's waits for the weights cover
+  // the few loads it does not know of that follow them: the last k-steps of the first tile wait for the second
+  // tile, which the tile's barrier waits for anyway.)
+  const int nbuf = a.wr_nbuf;
+  float *const cl_f = reinterpret_cast<float *>(lds + (size_t)nbuf * stage_cells) + wave * (3 * OCW);
+  const int cl_idx = lane < OCW ? lane : OCW - 1;
+  const float c_sc = a.ep.scale[ocw + cl_idx];
+  const float c_sh = a.ep.shift[ocw + cl_idx];
+  const int c_comp = a.ep.comp[ocw + cl_idx];
+  if (SUM) {
+    issue_setup(0, 0);
+#pragma unroll
+    for (int d = NKS / NW; d < LPT; ++d) issue_load(d);
+  }
   if (ntiles > 1) issue_tile(1, 1);
   // the lane's constants of tile mt, channels 4 q .. 4 q + 3, out of LDS
   auto cl_read = [&](int arr, int mt, int q) -> float4 {
@@ -225,25 +241,32 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
     // tile t + nbuf - 2 goes into the stage that the barrier of tile t - 1 has freed (tile t - 2's), a load per k-step
     const bool issue = !FIRST && nbuf >= 3 && t + nbuf - 2 < ntiles;
     if (issue) issue_setup(t + nbuf - 2, st < 2 ? st + nbuf - 2 : st - 2);
-    // the accumulators start from the compensation
+    // the accumulators start from the compensation (the first tile's from zero: its constants are not in LDS yet,
+    // its epilogue adds the compensation)
     v16i acc[TM];
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const float4 c = cl_read(2, mt, q);
+        float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!FIRST) c = cl_read(2, mt, q);
         acc[mt][4 * q] = __float_as_int(c.x); acc[mt][4 * q + 1] = __float_as_int(c.y);
         acc[mt][4 * q + 2] = __float_as_int(c.z); acc[mt][4 * q + 3] = __float_as_int(c.w);
       }
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      if (ks == NKS - 2 && t + 1 < ntiles) {
-        if (FIRST) {
-          // every load the compiler knows of (weights, constants) has been consumed or is pinned here, before the
-          // first load it does not know of is issued behind them: its own waits stay exact
+      if (FIRST && ks == NKS - 2) {
+        // every load the compiler knows of (weights, constants) has been consumed or is pinned here, before the
+        // next load it does not know of is issued behind them: its own waits stay exact.  The constants go to LDS.
 #pragma unroll
-          for (int mt = 0; mt < TM; ++mt) asm volatile("" : : "v"(areg[NKS - 1][mt]), "v"(areg[NKS - 2][mt]));
+        for (int mt = 0; mt < TM; ++mt) asm volatile("" : : "v"(areg[NKS - 1][mt]), "v"(areg[NKS - 2][mt]));
+        if (lane < OCW) {
+          cl_f[lane] = c_sc;
+          cl_f[OCW + lane] = c_sh;
+          reinterpret_cast<int *>(cl_f)[2 * OCW + lane] = c_comp;
         }
+      }
+      if (ks == NKS - 2 && t + 1 < ntiles) {
         // this wave's share of tile t + 1 has landed: tiles issued behind it are t + 2 .. min(t + nbuf - 2, ntiles - 1)
         const int last = FIRST ? 1 : (t + nbuf - 2 < ntiles - 1 ? t + nbuf - 2 : ntiles - 1);
         wait_vm(LPT * (last - (t + 1) > 0 ? last - (t + 1) : 0));
@@ -274,10 +297,15 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
         const float4 s4 = cl_read(0, mt, q), h4 = cl_read(1, mt, q);
         const float sc[4] = {s4.x, s4.y, s4.z, s4.w};
         const float sh[4] = {h4.x, h4.y, h4.z, h4.w};
+        int cv[4] = {0, 0, 0, 0};
+        if (FIRST) {
+          const float4 c4 = cl_read(2, mt, q);
+          cv[0] = __float_as_int(c4.x); cv[1] = __float_as_int(c4.y); cv[2] = __float_as_int(c4.z); cv[3] = __float_as_int(c4.w);
+        }
         unsigned pk = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          float f = __builtin_fmaf((float)acc[mt][4 * q + j], sc[j], sh[j]);
+          float f = __builtin_fmaf((float)(FIRST ? acc[mt][4 * q + j] + cv[j] : acc[mt][4 * q + j]), sc[j], sh[j]);
           if (SUM) {
             const unsigned b = ((unsigned)old[q] >> (8 * j)) & 0xffu;
             const int o = SUM == 2 ? (int)(signed char)b : (int)b;
@@ -310,8 +338,8 @@ hipError_t wres_enqueue(const LaunchPlan<GemmArgs> &plan, hipStream_t s)
   const GemmArgs &a = plan.args;
   const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
   const unsigned geom = (unsigned)a.stride_h | (unsigned)a.stride_w << 8 | (dense ? 1u << 16 : 0u) | (unsigned)a.ny << 20;
-  hipLaunchKernelGGL(reinterpret_cast<wres_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.ep.comp,
-                     a.p_total, a.ohw, a.ohw_magic, a.ihw, a.ic2, a.ocpp, geom, a.wr_region, a.nx, a.wr_stage, a);
+  hipLaunchKernelGGL(reinterpret_cast<wres_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.p_total, a.ohw,
+                     a.ohw_magic, a.ihw, a.ic2, a.ocpp, geom, a.wr_region, a.nx, (unsigned)a.ow | (unsigned)a.iw << 16, a.ow_magic, a);
   return hipGetLastError();
 }
 
@@ -384,7 +412,7 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch)
   if (nbatch != 1 || a.kh * a.kw > 1 || a.ep.shift_tab || a.in_nhwc) return false;
   if (!lean_mode(a.ep, false)) return false;
   if ((a.units_pad != 16 && a.units_pad != 32 && a.units_pad != 64) || a.ic2 != a.units_pad) return false;
-  if (a.stride_h > 255 || a.stride_w > 255) return false;
+  if (a.stride_h > 255 || a.stride_w > 255 || a.ow >= 65536 || a.iw >= 65536) return false;
   const int oc = a.oc2 * 16;
   const int oc_wg = 32 * wres_nw(a.units_pad / 2) * wres_tm(a.units_pad / 2);
   const int nb = (oc + oc_wg - 1) / oc_wg;
