@@ -473,7 +473,10 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 // each for A = 6, four each for A = 4, and 7 + 7 + 7 + 4 for A = 5.
 // SUM: the in-place sum (a compile-time copy: as a run-time flag in the common code it cost the layers without a
 // sum 4 %, as copies behind a uniform branch twice their time -- the kernel sits at the edge of its registers).
-template <int KS, int A = 6, bool SUM = false>
+// NT: blocks of 32 tiles per workgroup.  Tile size 4 has 16 positions, four per wave: its accumulators for 64
+// channels x 32 tiles fill a quarter of the wave's registers, so a workgroup takes 64 tiles (a weight operand
+// then feeds two MFMAs as a tile operand does: 1 KB of operands per MFMA instead of 1.5).
+template <int KS, int A = 6, bool SUM = false, int NT = 1>
 __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 {
   constexpr int AA = A * A, PW = (AA + 3) / 4, CN = PW * 24, NJ = (CN + 63) / 64;
@@ -489,7 +492,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   const int by = seq % a.ny;
   const int bx = (seq / a.ny) * 8 + xcd;
   if (bx >= a.nx) return;          // whole workgroup
-  const int t0 = bx * 32, oc0 = by * 64;
+  const int t0 = bx * 32 * NT, oc0 = by * 64;
   const int oc_real = a.oc2 * 16;
   const int p0 = PW * wave;
   // positions of this wave: all PW, except in the last wave when four runs of PW overshoot A x A (A = 5)
@@ -501,14 +504,21 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   // operand addresses = wave-uniform pointer (scalar arithmetic) + a per-lane 32-bit offset that
   // never changes: lane = packed row / tile l32 of unit 2 * ks + lh
   const unsigned a_lane = (unsigned)(lh * a.ocpp + l32) * 16u;
-  const int tile = t0 + l32 < a.t ? t0 + l32 : a.t - 1;
   // plain layout: tile `tile` of unit lh; blocked: cell l32 of unit lh inside the block's own run (cells of
-  // tiles past the end hold nothing and are never stored)
-  const unsigned b_lane = a.tin_blocked ? (unsigned)(lh * 32 + l32) * 16u : (unsigned)(lh * a.t + tile) * 16u;
+  // tiles past the end hold nothing and are never stored; a block past the last one reads the last one)
+  unsigned b_lane[NT];
+  long long b_block[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int tile = t0 + 32 * j + l32 < a.t ? t0 + 32 * j + l32 : a.t - 1;
+    b_lane[j] = a.tin_blocked ? (unsigned)(lh * 32 + l32) * 16u : (unsigned)(lh * a.t + tile) * 16u;
+    const int nb32 = (a.t + 31) >> 5;
+    b_block[j] = bx * NT + j < nb32 ? bx * NT + j : nb32 - 1;
+  }
   const int ks_last = ((a.ic2 + 1) >> 1) - 1;   // last k-step that holds real channels
 
   TRACE_POINT(0);
-  v4i ra[KS][2], rb[KS];
+  v4i ra[KS][2], rb[KS][NT];
   auto issue = [&](int slot, int p, int ks) {
     const int8_t *pa = a.w + (((long long)p * a.units_pad + 2 * ks) * a.ocpp + oc0) * 16;
     ra[slot][0] = *reinterpret_cast<const v4i *>(pa + a_lane);
@@ -516,9 +526,12 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     // padded k-steps multiply zero weights: any valid cell will do (an odd unit count reads one
     // unit past the position, which is the next position or the pad unit behind the buffer)
     const int ksc = ks < ks_last ? ks : ks_last;
-    const uint8_t *pb = a.tin_blocked ? a.tin + (((long long)bx * AA + p) * a.ic2 + 2 * ksc) * 512
-                                      : a.tin + ((long long)p * a.ic2 + 2 * ksc) * a.t * 16;
-    rb[slot] = *reinterpret_cast<const v4i *>(pb + b_lane);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const uint8_t *pb = a.tin_blocked ? a.tin + ((b_block[j] * AA + p) * a.ic2 + 2 * ksc) * 512
+                                        : a.tin + ((long long)p * a.ic2 + 2 * ksc) * a.t * 16;
+      rb[slot][j] = *reinterpret_cast<const v4i *>(pb + b_lane[j]);
+    }
   };
 
   // Per-(position, channel) scale / shift / compensation of the wave's nine positions, one half of
@@ -549,13 +562,15 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   load_consts_half(0);
   store_consts_half();
 
-  v16i acc[PW][2];
+  v16i acc[PW][2][NT];
 #pragma unroll
   for (int i = 0; i < PW; ++i)
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][h][v] = 0;
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][h][j][v] = 0;
 
 #pragma unroll
   for (int k = 0; k < KS; ++k) issue(k, p0, k);
@@ -564,9 +579,12 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     for (int c = 0; c < (EVEN || i < np ? nkc : 0); ++c) {
 #pragma unroll
       for (int k = 0; k < KS; ++k) {
-        const v4i b = rb[k] ^ (int)0x80808080;
-        acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][0], b, acc[i][0], 0, 0, 0);
-        acc[i][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][1], b, acc[i][1], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const v4i b = rb[k][j] ^ (int)0x80808080;
+          acc[i][0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][0], b, acc[i][0][j], 0, 0, 0);
+          acc[i][1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][1], b, acc[i][1][j], 0, 0, 0);
+        }
         // refill the slot with the operands KS steps ahead (the very last block re-reads itself)
         int pn = p0 + i, ksn = (c + 1) * KS + k;
         if (ksn >= nks) { ksn -= nks; pn += 1; }
@@ -580,15 +598,17 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   TRACE_POINT(1);
   // ---- requantize, exchange, output transform ----------------------------------------------------
   const int tile_l = tid >> 3, q8 = tid & 7;
-  const int t = t0 + tile_l;
-  const int tc = t < a.t ? t : a.t - 1;
-  const int n = tc / a.nt;
-  const int rem = tc - n * a.nt;
-  const int th = rem / a.wt;
-  const int tw = rem - th * a.wt;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
-    if (h) __syncthreads();        // everyone has gathered the first half
+#pragma unroll
+   for (int j = 0; j < NT; ++j) {   // a round: 32 channels x 32 tiles through the exchange buffer
+    const int t = t0 + 32 * j + tile_l;
+    const int tc = t < a.t ? t : a.t - 1;
+    const int n = tc / a.nt;
+    const int rem = tc - n * a.nt;
+    const int th = rem / a.wt;
+    const int tw = rem - th * a.wt;
+    if (h || j) __syncthreads();   // everyone has gathered the round before
     __builtin_amdgcn_wave_barrier();
     // constants of position i + 1 are read from LDS while position i is requantized
     float4 kq[2][12];
@@ -609,16 +629,16 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
         if (!EVEN && i >= np) continue;   // a position the last wave does not have
         const float4 sc = kq[i & 1][q], sh = kq[i & 1][4 + q], cf = kq[i & 1][8 + q];
         float4 r;
-        r.x = __builtin_fmaf((float)(acc[i][h][4 * q + 0] + __float_as_int(cf.x)), sc.x, sh.x);
-        r.y = __builtin_fmaf((float)(acc[i][h][4 * q + 1] + __float_as_int(cf.y)), sc.y, sh.y);
-        r.z = __builtin_fmaf((float)(acc[i][h][4 * q + 2] + __float_as_int(cf.z)), sc.z, sh.z);
-        r.w = __builtin_fmaf((float)(acc[i][h][4 * q + 3] + __float_as_int(cf.w)), sc.w, sh.w);
+        r.x = __builtin_fmaf((float)(acc[i][h][j][4 * q + 0] + __float_as_int(cf.x)), sc.x, sh.x);
+        r.y = __builtin_fmaf((float)(acc[i][h][j][4 * q + 1] + __float_as_int(cf.y)), sc.y, sh.y);
+        r.z = __builtin_fmaf((float)(acc[i][h][j][4 * q + 2] + __float_as_int(cf.z)), sc.z, sh.z);
+        r.w = __builtin_fmaf((float)(acc[i][h][j][4 * q + 3] + __float_as_int(cf.w)), sc.w, sh.w);
         xl[(p * 32 + l32) * 8 + ((4 * lh + q) ^ ((l32 >> 1) & 7))] = r;
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_wave_barrier();
-    if (h == 0) store_consts_half();   // the wave is done with the first half's constants
+    if (h == 0 && j == NT - 1) store_consts_half();   // the wave is done with the first half's constants
     TRACE_POINT(2 + 4 * h);
     __syncthreads();
     TRACE_POINT(3 + 4 * h);
@@ -645,6 +665,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
                                  th, tw, a.oh, a.ow, SUM, px);
     }
     TRACE_POINT(5 + 4 * h);
+   }
   }
 }
 
@@ -693,10 +714,11 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
     return plan_relaunch(*plan, [&](WinoFusedArgs &x) { x.out = a0.out; x.bias = a0.bias; }, s);
   }
   WinoFusedArgs a = a0;
-  a.nx = (a.t + 31) / 32;
+  const int A = a.tile ? a.tile : 6, AA = A * A;
+  const int ntb = A == 4 ? 2 : 1;   // blocks of 32 tiles per workgroup
+  a.nx = (a.t + 32 * ntb - 1) / (32 * ntb);
   a.ny = (a.oc2 * 16 + 63) / 64;
   const int nks = a.units_pad / 2;
-  const int A = a.tile ? a.tile : 6, AA = A * A;
   const size_t lds = (size_t)AA * 32 * 32 * sizeof(float) + 4 * (size_t)((AA + 3) / 4 * 24) * sizeof(float4);   // exchange + constants
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
   // operand ring depth in k-steps.  Measured (C4a / C4b / C4a_i8 / C4b_i8, us): 8 deep 261.7 / 177.3 / 247.6 /
@@ -705,8 +727,9 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   if (const char *env = getenv("EHIP_WINO_KS")) ks_max = atoi(env);
   void (*kernel)(WinoFusedArgs) = nullptr;
 #define EHIP_WF(AV, SV)                                                                                 \
-  kernel = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV>                                \
-      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4, AV, SV> : k_wino_gemm_output<2, AV, SV>)
+  kernel = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1>               \
+      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4, AV, SV, AV == 4 ? 2 : 1>                 \
+                                       : k_wino_gemm_output<2, AV, SV, AV == 4 ? 2 : 1>)
   if (a.with_sum) {
     if (A == 4) EHIP_WF(4, true);
     else if (A == 5) EHIP_WF(5, true);
