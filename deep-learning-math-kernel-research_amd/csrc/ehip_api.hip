@@ -86,7 +86,8 @@ int fail(int code, const std::string &msg)
 
 void free_all(ehip_conv *c)
 {
-  void *ptrs[] = {c->wpacked, c->scale, c->shift, c->absmax, c->wsum, c->comp, c->tin, c->tout,
+  // (scale, shift and comp are one allocation: see setup_workspace)
+  void *ptrs[] = {c->wpacked, c->scale, c->absmax, c->wsum, c->tin, c->tout,
                   c->cls_h, c->cls_w, c->rects, c->shift_tab};
   for (void *p : ptrs)
     if (p) (void)hipFree(p);
@@ -428,11 +429,13 @@ int setup_workspace(ehip_conv *c)
   }
   c->per_oc = (size_t)c->nbatch * c->ocpp;
   if ((rc = dev_alloc(&c->wpacked, c->wpacked_bytes, true)) != EHIP_OK) return rc;
-  if ((rc = dev_alloc(&c->scale, c->per_oc, true)) != EHIP_OK) return rc;
-  if ((rc = dev_alloc(&c->shift, c->per_oc, true)) != EHIP_OK) return rc;
+  // scale, shift and compensation back to back, [3][per_oc]: a kernel can take them as one pointer among its
+  // preloaded leading arguments and ask for all three before the rest of its argument block has arrived
+  if ((rc = dev_alloc(&c->scale, 3 * c->per_oc, true)) != EHIP_OK) return rc;
+  c->shift = c->scale + c->per_oc;
+  c->comp = reinterpret_cast<int *>(c->scale + 2 * c->per_oc);
   if ((rc = dev_alloc(&c->absmax, c->per_oc, true)) != EHIP_OK) return rc;
   if ((rc = dev_alloc(&c->wsum, c->per_oc, true)) != EHIP_OK) return rc;
-  if ((rc = dev_alloc(&c->comp, c->per_oc, true)) != EHIP_OK) return rc;
   if (c->nclass > 1 && (rc = dev_alloc(&c->shift_tab, (size_t)c->nclass * c->ocpp, true)) != EHIP_OK) return rc;
   return EHIP_OK;
 }

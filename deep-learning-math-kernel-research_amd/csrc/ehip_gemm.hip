@@ -786,8 +786,8 @@ hipError_t launch_gemm(const GemmArgs &a0, int nbatch, int variant, hipStream_t 
   if (plan && plan->valid) {   // everything but the tensors is as on the first launch
     return plan_relaunch(*plan, [&](GemmArgs &x) { x.in = a0.in; x.out = a0.out; }, s);
   }
-  if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s, plan);
   if (gemm1x1_wres_applies(a0, nbatch)) return launch_gemm1x1_wres(a0, s, plan);
+  if (gemm_smallk_applies(a0.ic2, a0.kh * a0.kw, nbatch)) return launch_gemm_smallk(a0, s, plan);
   {
     const int rv = gemm1x1_res_pick(a0, nbatch);
     if (rv >= 0) return launch_gemm1x1_res(a0, rv, s, plan);

@@ -55,7 +55,7 @@ __device__ __forceinline__ void wait_vm(int n)
 #if defined(__HIP_DEVICE_COMPILE__)
 #define EHIP_W(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
   switch (n) {
-    EHIP_W(0) EHIP_W(2) EHIP_W(3) EHIP_W(4) EHIP_W(5) EHIP_W(6) EHIP_W(8) EHIP_W(9) EHIP_W(10) EHIP_W(12) EHIP_W(15)
+    EHIP_W(0) EHIP_W(1) EHIP_W(2) EHIP_W(3) EHIP_W(4) EHIP_W(5) EHIP_W(6) EHIP_W(8) EHIP_W(9) EHIP_W(10) EHIP_W(12) EHIP_W(15)
     EHIP_W(16) EHIP_W(18) EHIP_W(20) EHIP_W(24) EHIP_W(25) EHIP_W(30) EHIP_W(32) EHIP_W(36) EHIP_W(40)
     default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
   }
@@ -74,11 +74,12 @@ struct PixInfo {
 }  // namespace
 
 // geom = stride_h | stride_w << 8 | dense << 16 | nb << 20 (channel blocks of 4 x TM x 32)
-// (the leading arguments are what the first tile's loads and the weight loads need: they arrive in scalar registers
-// with the wave, while the rest of the argument block is still being fetched; owiw = ow | iw << 16)
+// (the leading arguments are what the first tile's loads, the per-channel constants and the weight loads need: they
+// arrive in scalar registers with the wave, while the rest of the argument block is still being fetched;
+// owiw = ow | iw << 16; consts = [3][ocpp]: scale, shift, compensation, one allocation)
 #define EHIP_WRES_HEAD                                                                                                  \
-  const uint8_t *in, const int8_t *w, int p_total, int ohw, unsigned ohw_magic, int ihw, int ic2, int ocpp, unsigned geom, \
-      int ntiles_all, int nreg, unsigned owiw, unsigned ow_magic
+  const uint8_t *in, const int8_t *w, const float *consts, int p_total, int ohw, unsigned ohw_magic, int ihw, int ocpp, \
+      unsigned geom, int nreg, unsigned owiw, unsigned ow_magic
 // NW waves per workgroup: four, two workgroups per CU; or eight in one workgroup per CU, which then share ONE copy
 // of every pixel tile (1024 input channels, where a wave can only hold the weights of 32 channels: eight waves own
 // the 256 channels that four own with fewer input channels)
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
 {
   GemmArgs a = rest;
   a.in = in; a.w = w; a.p_total = p_total; a.ohw = ohw; a.ohw_magic = ohw_magic;
-  a.ihw = ihw; a.ic2 = ic2; a.ocpp = ocpp; a.ow = (int)(owiw & 0xffffu); a.iw = (int)(owiw >> 16); a.ow_magic = ow_magic;
+  a.ihw = ihw; a.ic2 = 2 * NKS; a.ocpp = ocpp; a.ow = (int)(owiw & 0xffffu); a.iw = (int)(owiw >> 16); a.ow_magic = ow_magic;
   constexpr int stage_bytes = NKS * 1024 + (SUM ? NW * TM * 1024 : 0);
   a.stride_h = (int)(geom & 0xffu); a.stride_w = (int)((geom >> 8) & 0xffu);
   const bool dense = (geom >> 16) & 1u;
@@ -109,6 +110,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
   const int reg = xcd * ((nreg + 7) >> 3) + seq / nb;
   if (reg >= nreg) return;   // whole workgroup
   // runs of whole tiles: the first (ntiles_all % nreg) runs are one tile longer
+  const int ntiles_all = (p_total + 31) >> 5;
   const int tq = ntiles_all / nreg, tr = ntiles_all - tq * nreg;
   const int tile0 = reg * tq + (reg < tr ? reg : tr);
   const int ntiles = tq + (reg < tr ? 1 : 0);
@@ -184,6 +186,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
 #pragma unroll
     for (int d = 0; d < NKS / NW; ++d) issue_load(d);
   }
+  // the per-channel constants next (into registers now, into LDS once the weights are in): the first tile's epilogue
+  // is what waits for them, and behind the weights they would arrive a trip to memory later
+  const int cl_idx = lane < OCW ? lane : OCW - 1;
+  const float c_sc = consts[ocw + cl_idx];
+  const float c_sh = consts[ocpp + ocw + cl_idx];
+  const int c_comp = reinterpret_cast<const int *>(consts)[2 * ocpp + ocw + cl_idx];
   TRACE_POINT(1);
   // weights [units][ocpp][16]: lane = packed row l32 of unit 2 ks + lh; tile mt 32 rows on
   const int8_t *wb = a.w + ((long long)lh * a.ocpp + ocw + l32) * 16;
@@ -193,23 +201,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
   for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) areg[ks][mt] = *reinterpret_cast<const v4i *>(wb + ks * w_step + mt * 512);
-  // Then what needs the argument block: the per-channel constants (into registers now, into LDS once the weights
-  // are in: a wave's loads complete in issue order, and nothing may make the first tile's K loop wait for more than
-  // its next weights), the first tile's sum operand, the second tile.  (The compiler's waits for the weights cover
+  // Then what needs the argument block: the first tile's sum operand, the second tile.  (The compiler's waits for the weights cover
   // the few loads it does not know of that follow them: the last k-steps of the first tile wait for the second
   // tile, which the tile's barrier waits for anyway.)
   const int nbuf = a.wr_nbuf;
   float *const cl_f = reinterpret_cast<float *>(lds + (size_t)nbuf * stage_cells) + wave * (3 * OCW);
-  const int cl_idx = lane < OCW ? lane : OCW - 1;
-  const float c_sc = a.ep.scale[ocw + cl_idx];
-  const float c_sh = a.ep.shift[ocw + cl_idx];
-  const int c_comp = a.ep.comp[ocw + cl_idx];
   if (SUM) {
     issue_setup(0, 0);
 #pragma unroll
     for (int d = NKS / NW; d < LPT; ++d) issue_load(d);
   }
   if (ntiles > 1) issue_tile(1, 1);
+  // (the other tiles that fit in the ring are asked for from the first tile's K loop: queued here, ahead of the
+  // first loads of the CU's other workgroup, they delayed its start by more than they gained -- 256 -> 512 stride 2 at
+  // 56 x 56 13.8 against 13.4 us.  Stage nbuf - 1 stays free for the tile that the second tile's K loop asks for.)
+  const int npre = nbuf > 3 ? nbuf - 2 : 1;   // tiles 1 .. npre are in flight when the first tile ends
   // the lane's constants of tile mt, channels 4 q .. 4 q + 3, out of LDS
   auto cl_read = [&](int arr, int mt, int q) -> float4 {
     return *reinterpret_cast<const float4 *>(cl_f + OCW * arr + 32 * mt + 16 * lh + 4 * q);
@@ -267,22 +273,29 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
           cl_f[OCW + lane] = c_sh;
           reinterpret_cast<int *>(cl_f)[2 * OCW + lane] = c_comp;
         }
+        for (int tt = 2; tt <= npre && tt < ntiles; ++tt) issue_tile(tt, tt);   // (their stages have never been used)
       }
-      if (ks == NKS - 2 && t + 1 < ntiles) {
+      // (the first tile does this behind its epilogue: its second tile was asked for a moment ago and is a trip to
+      // memory away, time in which the epilogue's stores can already leave)
+      if (!FIRST && ks == NKS - 2 && t + 1 < ntiles) {
         // this wave's share of tile t + 1 has landed: tiles issued behind it are t + 2 .. min(t + nbuf - 2, ntiles - 1)
-        const int last = FIRST ? 1 : (t + nbuf - 2 < ntiles - 1 ? t + nbuf - 2 : ntiles - 1);
+        const int last = t + nbuf - 2 < ntiles - 1 ? t + nbuf - 2 : ntiles - 1;
         wait_vm(LPT * (last - (t + 1) > 0 ? last - (t + 1) : 0));
         __syncthreads();
         // everybody's share has; and nobody reads tile t - 1's stage any more
-        if (FIRST)
-          for (int tt = 2; tt < nbuf - 1 && tt < ntiles; ++tt) issue_tile(tt, tt);
       }
-      if (!FIRST && ks < LPT && issue) issue_load(ks);
+      // (all of a tile's loads go out before the k-step of the barrier, whose wait counts them: PER per k-step)
+      constexpr int PER = (LPT + NKS - 3) / (NKS - 2);
+      if (!FIRST && issue) {
+#pragma unroll
+        for (int d = ks * PER; d < (ks + 1) * PER; ++d)
+          if (d < LPT) issue_load(d);
+      }
 #pragma unroll
       for (int mt = 0; mt < TM; ++mt) {
         acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[ks][mt], bq[ks & 3], acc[mt], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (mt == 0) bq[(ks + 2) & 3] = ks + 2 < NKS ? tb[(ks + 2) * 64] : tbn[(ks + 2 - NKS) * 64];
+        if (mt == 0 && (ks + 2 < NKS || !FIRST)) bq[(ks + 2) & 3] = ks + 2 < NKS ? tb[(ks + 2) * 64] : tbn[(ks + 2 - NKS) * 64];
         if (mt == TM - 1) bq[(ks + 1) & 3] ^= (int)0x80808080;
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -333,6 +346,16 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void k_gemm1x1_wres(EHIP_
         }
       }
     }
+    if (FIRST && ntiles > 1) {
+      // the second tile: this wave's share has landed (the epilogue's stores are younger than every load issued so
+      // far and only make the wait stricter), then everybody's; its first two operands
+      const int last = npre < ntiles - 1 ? npre : ntiles - 1;
+      wait_vm(LPT * (last - 1 > 0 ? last - 1 : 0));
+      __syncthreads();
+      bq[0] = tbn[0];
+      bq[1] = tbn[64];
+      bq[0] ^= (int)0x80808080;
+    }
   };
   tile_step(std::true_type{}, 0, 0);
   TRACE_POINT(3);
@@ -352,8 +375,8 @@ hipError_t wres_enqueue(const LaunchPlan<GemmArgs> &plan, hipStream_t s)
   const GemmArgs &a = plan.args;
   const bool dense = a.stride_h == 1 && a.stride_w == 1 && a.iw == a.ow;
   const unsigned geom = (unsigned)a.stride_h | (unsigned)a.stride_w << 8 | (dense ? 1u << 16 : 0u) | (unsigned)a.ny << 20;
-  hipLaunchKernelGGL(reinterpret_cast<wres_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.p_total, a.ohw,
-                     a.ohw_magic, a.ihw, a.ic2, a.ocpp, geom, a.wr_region, a.nx, (unsigned)a.ow | (unsigned)a.iw << 16, a.ow_magic, a);
+  hipLaunchKernelGGL(reinterpret_cast<wres_kernel_t>(plan.kernel), plan.grid, plan.block, plan.lds, s, a.in, a.w, a.ep.scale, a.p_total,
+                     a.ohw, a.ohw_magic, a.ihw, a.ocpp, geom, a.nx, (unsigned)a.ow | (unsigned)a.iw << 16, a.ow_magic, a);
   return hipGetLastError();
 }
 
@@ -366,6 +389,9 @@ wres_kernel_t wres_kernel(int nks, int sum, int nw)
   (void)nw;   // (eight waves in one workgroup per CU with up to 512 input channels: measured, 14.1 against 13.1 us on the
               // 512 -> 1024 stride-2 layer; two workgroups of four waves stay)
   switch (nks * 4 + sum) {
+  case 4 * 4 + 0: return k_gemm1x1_wres<4, 2, 0, 4>;
+  case 4 * 4 + 1: return k_gemm1x1_wres<4, 2, 1, 4>;
+  case 4 * 4 + 2: return k_gemm1x1_wres<4, 2, 2, 4>;
   case 8 * 4 + 0: return k_gemm1x1_wres<8, 2, 0, 4>;
   case 8 * 4 + 1: return k_gemm1x1_wres<8, 2, 1, 4>;
   case 8 * 4 + 2: return k_gemm1x1_wres<8, 2, 2, 4>;
@@ -388,7 +414,7 @@ struct WresGeom {
 };
 bool wres_geom(const GemmArgs &a, WresGeom &g)
 {
-  g.nks = a.units_pad / 2;
+  g.nks = a.ic2 / 2;   // (the packed weights may be padded to more units: never read)
   g.tm = wres_tm(g.nks);
   g.nw = wres_nw(g.nks);
   const int lean = lean_mode(a.ep, false);
@@ -427,10 +453,12 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch)
   if (env && env[0] == '0') return false;
   if (nbatch != 1 || a.kh * a.kw > 1 || a.ep.shift_tab || a.in_nhwc) return false;
   if (!lean_mode(a.ep, false)) return false;
-  if ((a.units_pad != 16 && a.units_pad != 32 && a.units_pad != 64) || a.ic2 != a.units_pad) return false;
+  // the kernel takes the per-channel constants as ONE leading pointer: scale, shift and compensation in one allocation
+  if (a.ep.shift != a.ep.scale + a.ocpp || reinterpret_cast<const float *>(a.ep.comp) != a.ep.scale + 2 * (size_t)a.ocpp) return false;
+  if (a.ic2 != 8 && a.ic2 != 16 && a.ic2 != 32 && a.ic2 != 64) return false;
   if (a.stride_h > 255 || a.stride_w > 255 || a.ow >= 65536 || a.iw >= 65536) return false;
   const int oc = a.oc2 * 16;
-  const int oc_wg = 32 * wres_nw(a.units_pad / 2) * wres_tm(a.units_pad / 2);
+  const int oc_wg = 32 * wres_nw(a.ic2 / 2) * wres_tm(a.ic2 / 2);
   const int nb = (oc + oc_wg - 1) / oc_wg;
   if (nb >= 4096) return false;
   // fewer than three quarters of the channel blocks' rows real, or too few pixels to give every CU a run: the
@@ -442,7 +470,7 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch)
   // 512 -> 256 at 28 x 28: 11.7 vs 13.4, 256 -> 256 at 28 x 28: 8.3 vs 9.8), level or behind with shorter runs
   // (512 -> 512 at 14 x 14: 8.0 vs 7.7, 512 -> 2048 at 7 x 7: 8.2 vs 8.0) and with 1024 input channels, whose waves own
   // one tile of 32 channels (1024 -> 256 at 14 x 14: 8.6 vs 8.4, 1024 -> 1024 at 7 x 7: 8.6 vs 7.2)
-  if (!forced && (a.units_pad > 32 || (long long)((a.p_total + 31) / 32) * nb < 3 * 512)) return false;
+  if (!forced && (a.ic2 > 32 || (long long)((a.p_total + 31) / 32) * nb < 3 * 512)) return false;
   // a lane's offsets into the input and the output are 32 bits wide
   const long long n_img = a.p_total / (a.ohw > 0 ? a.ohw : 1);
   if (n_img * a.ic2 * a.ihw * 16 >= (1ll << 32) || (long long)a.p_total * a.oc2 * 16 >= (1ll << 32)) return false;

@@ -125,9 +125,10 @@ def test_conv1x1_resident_pixel_tile_kernel_nhwc_input(variant, n, ic, oc, hw, s
 
 @pytest.mark.parametrize("slots", ["", "8", "40"])
 @pytest.mark.parametrize("n,ic,oc,hw,stride", [(2, 256, 256, 14, 1), (3, 256, 80, 9, 1), (1, 512, 272, 14, 2), (2, 1024, 128, 7, 1),
-                                               (1, 512, 48, 5, 1), (3, 1024, 336, 9, 1), (5, 512, 128, 14, 1)])
+                                               (1, 512, 48, 5, 1), (3, 1024, 336, 9, 1), (5, 512, 128, 14, 1),
+                                               (3, 128, 272, 11, 1), (2, 128, 512, 14, 2)])
 def test_conv1x1_weights_resident_kernel(slots, n, ic, oc, hw, stride, monkeypatch):
-    """the 1x1 kernel with the weights in registers and the pixels streamed through a ring of LDS stages: 256 / 512 /
+    """the 1x1 kernel with the weights in registers and the pixels streamed through a ring of LDS stages: 128 / 256 / 512 /
     1024 input channels, ragged channel and pixel counts, stride 2, u8 / s8 with and without the sum, other ReLU
     bounds, blocked and nhwc output; few workgroup slots make the runs longer than the ring, so stages are reused"""
     monkeypatch.setenv("EHIP_GEMM1X1_WRES", "1")
@@ -148,7 +149,7 @@ def test_conv1x1_weights_resident_kernel_ring_depths(nbuf, monkeypatch):
     monkeypatch.setenv("EHIP_GEMM1X1_WRES", "1")
     monkeypatch.setenv("EHIP_WRES_SLOTS", "16")
     monkeypatch.setenv("EHIP_WRES_NBUF", nbuf)
-    for ic, with_sum in ((256, True), (512, False), (1024, True)):
+    for ic, with_sum in ((128, True), (256, True), (512, False), (1024, True)):
         res = run_and_compare(Layer(4, ic, 256, 14, out_type=ol.S8, with_sum=with_sum, seed=710 + ic))
         assert res["conv"].kernel_name == "k_gemm1x1_wres"
 
