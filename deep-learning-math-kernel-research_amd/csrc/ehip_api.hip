@@ -222,7 +222,10 @@ int classify(ehip_conv *c)
           d.ow == d.iw + d.pad_l + d.pad_r - 2 && d.oh == d.ih + d.pad_t + d.pad_b - 2;
       // the GEMM family walks [tap][unit] for kh x kw; it also owns the per-pixel shift that a zero
       // point with padding needs
-      c->family = (s1_3x3 && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC && d.input_fmt != EHIP_NHWC)
+      // 3x3 stride 2 runs the same kernel over four phase planes of the input (EHIP_CONV3X3V_S2=0: the GEMM form)
+      const char *s2env = getenv("EHIP_CONV3X3V_S2");
+      const bool s2_3x3 = d.kh == 3 && d.kw == 3 && d.stride_h == 2 && d.stride_w == 2 && !(s2env && s2env[0] == '0');
+      c->family = ((s1_3x3 || s2_3x3) && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC && d.input_fmt != EHIP_NHWC)
           ? FAM_CONV_3X3 : FAM_GEMM_1X1;
       {
         // at most four input channels: several pixels per operand cell, weights in registers
@@ -282,7 +285,7 @@ int setup_workspace(ehip_conv *c)
     c->nbatch = 1;
     if ((long long)(d.oh + 2) * (d.ow + 2) * (d.ow + 2) >= (1ll << 31))
       return fail(EHIP_UNIMPLEMENTED, "direct 3x3: image too large");
-    c->variant = conv3x3v_pick_variant(d.n, d.oh, d.ow, c->oc2);
+    c->variant = conv3x3v_pick_variant(d.n, d.oh, d.ow, c->oc2, d.stride_h);
     if (c->variant >= 0) {
       c->chunk_units = conv3x3v_chunk_units(c->variant, c->ic2);
       c->units_pad = up(c->ic2, c->chunk_units);
@@ -653,7 +656,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
     a.pad_t = d.pad_t; a.pad_l = d.pad_l;
     a.ic2 = c->ic2; a.units_pad = c->units_pad; a.oc2 = c->oc2; a.ocpp = c->ocpp;
     a.chunk_units = c->chunk_units;
-    a.vw = d.ow + 2;
+    a.vw = d.stride_h == 2 ? d.ow + 1 : d.ow + 2;
     a.vw_magic = div_magic(a.vw);
     a.trace = trace_buffer();
     HIP_TRY(launch_conv3x3v(a, d.n, c->variant, s, &c->plan_3x3));

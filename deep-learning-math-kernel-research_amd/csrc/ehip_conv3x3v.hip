@@ -18,6 +18,12 @@
 // -128, whose product with a weight is cancelled exactly by the 128 * sum(weights) the accumulators
 // start from, so skipped border taps of the reference and zero taps here give the same s32.
 //
+// Stride 2 (template S = 2): the staged input of a unit is de-interleaved into four phase planes,
+// plane (pr, pc)[r][c] = in[2 r + pr - pad_t][2 c + pc - pad_l], each addressed by virtual rows of VW = ow + 1
+// cells.  Tap (kh, kw) of output pixel v then reads plane (kh & 1, kw & 1) at v + (kh >> 1) * VW + (kw >> 1):
+// again one constant offset per tap, so the K loop is the stride-1 loop with another offset table, and only the
+// staging plan (which input cell goes where) differs.  One of every VW virtual pixels is a frame column.
+//
 // MFMA mapping as in the 1x1 kernel (v_mfma_i32_32x32x32_i8; A = weights in packed row order,
 // B = pixels, a lane's D = 16 consecutive output channels of one pixel).  A wave owns TM x TN tiles of 32 x 32; its
 // weight operands (9 taps x TM) live in registers and every slot is refilled with the next channel
@@ -63,10 +69,12 @@ constexpr int conv3x3v_unit_stride(int cells, int tn, bool sp)
   return r * tn;
 }
 
-template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS, bool SP, bool SL>
+template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS, bool SP, bool SL, int S>
 __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
 {
   static_assert(!SL || (PAIRS > 0 && !SP && TM == 1 && TN == 4), "split last pair: straight-line form, 32 channels x 4 tiles");
+  static_assert(S == 1 || (S == 2 && !SP && (CT * NPASS) % 4 == 0), "stride 2: four phase planes per staged unit");
+  constexpr int PS = CT * NPASS / 4;   // stride 2: staged cells per phase plane
   constexpr int OC_T = WM * TM * 32;
   constexpr int P_T = WN * TN * 32;
   constexpr int STRIDE = conv3x3v_unit_stride(CT * NPASS, TN, SP);   // LDS cells per unit
@@ -120,10 +128,21 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
   bool gin[NPASS];
 #pragma unroll
   for (int p = 0; p < NPASS; ++p) {
-    const int v = v0 + tid % CT + p * CT;
-    const int r = fastdiv(v, VW, a.vw_magic);
-    const int c = v - r * VW;
-    const int ih = r - a.pad_t, iw = c - a.pad_l;
+    int ih, iw;
+    if (S == 2) {
+      const int cell = tid % CT + p * CT;   // plane q = cell / PS, cell j of it
+      const int q = cell / PS, v = v0 + cell - q * PS;
+      const int r = fastdiv(v, VW, a.vw_magic);
+      const int c = v - r * VW;
+      ih = 2 * r + (q >> 1) - a.pad_t;
+      iw = 2 * c + (q & 1) - a.pad_l;
+    } else {
+      const int v = v0 + tid % CT + p * CT;
+      const int r = fastdiv(v, VW, a.vw_magic);
+      const int c = v - r * VW;
+      ih = r - a.pad_t;
+      iw = c - a.pad_l;
+    }
     gin[p] = ih >= 0 && ih < a.ih && iw >= 0 && iw < a.iw;
     goff[p] = gin[p] ? (ih * a.iw + iw) * 16 : 0;
   }
@@ -216,7 +235,8 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
   v4i bq[2][TN];
   auto read_b = [&](int par, int pl, int tap, int nt) {
     const v4i *tile = lds + (2 * pl + lh) * STRIDE + pw0 + l32;
-    bq[par][nt] = tile[nt * 32 + (tap / 3) * VW + tap % 3];
+    const int kh = tap / 3, kw = tap % 3;
+    bq[par][nt] = tile[nt * 32 + (S == 2 ? ((kh & 1) * 2 + (kw & 1)) * PS + (kh >> 1) * VW + (kw >> 1) : kh * VW + kw)];
   };
   // one tap of one channel pair out of operand buffer par; next_pl >= 0: the operands of (next_pl,
   // next_tap) are read into the other buffer on the way
@@ -490,14 +510,14 @@ __device__ __forceinline__ void conv3x3v_body(const Conv3x3Args &a)
 #define EHIP_CONV3X3V_HEAD                                                                                            \
   const uint8_t *in, int ih, int iw, int oh, int ow, int pad_t, int pad_l, int ic2, int chunk_units, int vw,         \
       unsigned vw_magic, int gx, int gy, int tiles, int tiles_per_xcd
-template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS = 0, bool SP = false, bool SL = false>
+template <int WM, int WN, int TM, int TN, int CT, int NPASS, int PAIRS = 0, bool SP = false, bool SL = false, int S = 1>
 __global__ __launch_bounds__(kBlock, 2) void k_conv3x3v_u8s8(EHIP_CONV3X3V_HEAD, Conv3x3Args rest)
 {
   Conv3x3Args a = rest;
   a.in = in; a.ih = ih; a.iw = iw; a.oh = oh; a.ow = ow; a.pad_t = pad_t; a.pad_l = pad_l; a.ic2 = ic2;
   a.chunk_units = chunk_units; a.vw = vw; a.vw_magic = vw_magic; a.gx = gx; a.gy = gy; a.tiles = tiles;
   a.tiles_per_xcd = tiles_per_xcd;
-  conv3x3v_body<WM, WN, TM, TN, CT, NPASS, PAIRS, SP, SL>(a);
+  conv3x3v_body<WM, WN, TM, TN, CT, NPASS, PAIRS, SP, SL, S>(a);
 }
 
 namespace {
@@ -515,31 +535,37 @@ struct Variant {
   conv3x3v_kernel_t kernel;
   conv3x3v_kernel_t unrolled[3];   // straight-line K loop for layers of exactly 2, 4, 8 unit pairs, or null
   conv3x3v_kernel_t split[3];      // the same with the last pair split (lean epilogue without the sum), or null
+  int stride;                      // 1, or 2: the staged unit is four phase planes of cells / 4 cells each
 };
 #define V(WM, WN, TM, TN, CT, NPASS)                                                              \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
-    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>, {nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr} }
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>, {nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}, 1 }
 #define VU(WM, WN, TM, TN, CT, NPASS)                                                             \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4>,  \
-     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>}, {nullptr, nullptr, nullptr} }
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>}, {nullptr, nullptr, nullptr}, 1 }
 #define VU2(WM, WN, TM, TN, CT, NPASS) /* straight-line form for two unit pairs only (64 input channels) */ \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
-    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, nullptr, nullptr}, {nullptr, nullptr, nullptr} }
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, nullptr, nullptr}, {nullptr, nullptr, nullptr}, 1 }
 #define VK(WM, WN, TM, TN, CT, NPASS)                                                             \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ">", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS>,                            \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4>,  \
      k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8>},                                               \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, false, true>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, false, true>, \
-     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, false, true>} }
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, false, true>}, 1 }
+#define V2(WM, WN, TM, TN, CT, NPASS) /* stride 2; straight-line forms for two and four unit pairs */ \
+  { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ",s2>", WM * TM * 32, WN * TN * 32, \
+    CT * NPASS, CT * NPASS, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 0, false, false, 2>,       \
+    {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, false, false, 2>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, false, false, 2>, \
+     nullptr}, {nullptr, nullptr, nullptr}, 2 }
 #define VS(WM, WN, TM, TN, CT, NPASS)                                                             \
   { "k_conv3x3v_u8s8<" #WM "," #WN "," #TM "," #TN "," #CT "," #NPASS ",sp>", WM * TM * 32, WN * TN * 32, \
     CT * NPASS, conv3x3v_unit_stride(CT * NPASS, TN, true), k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 0, true>, \
     {k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 2, true>, k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 4, true>, \
-     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>}, {nullptr, nullptr, nullptr} }
+     k_conv3x3v_u8s8<WM, WN, TM, TN, CT, NPASS, 8, true>}, {nullptr, nullptr, nullptr}, 1 }
 const Variant kVariants[] = {
     V(2, 2, 2, 1, 128, 1),  // 0: 128 oc x  64 px, rows up to  31 cells
     V(2, 2, 2, 1, 256, 1),  // 1: 128 oc x  64 px, rows up to  95 cells
@@ -561,36 +587,67 @@ const Variant kVariants[] = {
     VS(2, 2, 2, 2, 256, 1), // 17: as 2, strided pixels
     VS(4, 1, 1, 4, 256, 2), // 18: as 13, strided pixels
     VS(2, 2, 2, 4, 256, 2), // 19: 128 oc x 256 px, rows up to 127 cells, a wave = 64 oc x 128 px, strided pixels
+    V2(4, 1, 1, 2, 128, 3), // 20: stride 2, 128 oc x  64 px, output rows up to 29 pixels, every wave all pixels
+    V2(4, 1, 1, 4, 128, 5), // 21: stride 2, 128 oc x 128 px, output rows up to 29 pixels, every wave all pixels
+    V2(4, 1, 1, 2, 256, 2), // 22: stride 2, 128 oc x  64 px, output rows up to 61 pixels
+    V2(1, 4, 2, 1, 128, 5), // 23: stride 2,  64 oc x 128 px, output rows up to 29 pixels
 };
 #undef V
 #undef VU
 #undef VK
 #undef VU2
 #undef VS
+#undef V2
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLdsBudget = 64 * 1024;
 }  // namespace
 
 const char *conv3x3v_variant_name(int v) { return kVariants[v].name; }
 int conv3x3v_num_variants() { return kNumVariants; }
-bool conv3x3v_fits(int v, int ow) { return kVariants[v].p_t + 2 * (ow + 2) + 2 <= kVariants[v].cells; }
+bool conv3x3v_fits(int v, int ow, int stride)
+{
+  if (kVariants[v].stride != stride) return false;
+  if (stride == 2) return kVariants[v].p_t + (ow + 1) + 2 <= kVariants[v].cells / 4;   // a phase plane: tile + a row + a cell
+  return kVariants[v].p_t + 2 * (ow + 2) + 2 <= kVariants[v].cells;
+}
 
 // units of 16 input channels staged per LDS fill: all of them if they fit the budget
 int conv3x3v_chunk_units(int v, int ic2)
 {
+  // (stride 2: four pairs per fill, 48 to 80 KB, so that 128 / 256 / 512 input channels are whole fills)
+  if (kVariants[v].stride == 2) return ic2 < 8 ? up(ic2, 2) : 8;
   int cu = (kLdsBudget / (kVariants[v].ustride * 16)) & ~1;
   const int all = up(ic2, 2);
   return cu < all ? cu : all;
 }
 
 // -1: no variant fits the row width
-int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
+int conv3x3v_pick_variant(int n, int oh, int ow, int oc2, int stride)
 {
   const char *env = getenv("EHIP_CONV3X3V_VARIANT");
   if (env && env[0]) {
     int v = atoi(env);
-    if (v >= 0 && v < kNumVariants && conv3x3v_fits(v, ow)) return v;
+    if (v >= 0 && v < kNumVariants && conv3x3v_fits(v, ow, stride)) return v;
     return -1;
+  }
+  if (stride == 2) {
+    // fewest computed pixels first, then the chip's fill
+    int best = -1;
+    double best_score = -1;
+    for (int v = 0; v < kNumVariants; ++v) {
+      if (!conv3x3v_fits(v, ow, 2)) continue;
+      const Variant &k = kVariants[v];
+      const int oc = oc2 * 16;
+      if (oc > 64 && k.oc_t < 128) continue;
+      const int gx = (oh * (ow + 1) + k.p_t - 1) / k.p_t, gy = (oc + k.oc_t - 1) / k.oc_t;
+      const long long wgs = (long long)gx * gy * n;
+      const double util = (double)(oh * ow) / ((double)gx * k.p_t) * (double)oc / ((double)gy * k.oc_t);
+      const double fill = wgs >= 256 ? 1.0 : (double)wgs / 256.0;
+      const double big = (k.p_t >= 128 && wgs >= 440) ? 1.15 : 1.0;   // enough work: amortise the weights (as below)
+      const double score = util * fill * big;
+      if (score > best_score) { best_score = score; best = v; }
+    }
+    return best;
   }
   // Measured on MI355X (3x3 128 -> 128 @28x28, N = 32 .. 512): a workgroup's time is the time to
   // pull its weights through the CU's vector-memory path, so tiles whose four waves own disjoint
@@ -601,12 +658,12 @@ int conv3x3v_pick_variant(int n, int oh, int ow, int oc2)
   // than the 128-pixel tiles with three passes.
   const int oc = oc2 * 16, vpx = oh * (ow + 2);
   static const double pref[] = {0.80, 0.78, 0.92, 0.90, 1.0, 0.95, 1.0, 0.95, 0.85, 1.12, 0.95, 0.97, 1.14, 0.93, 0.85,
-                                0.0, 0.0, 0.0, 0.0, 0.0};
+                                0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
   int best = -1;
   double best_score = -1;
   for (int pass = 0; pass < 2 && best < 0; ++pass)   // second pass: any channel tile that fits the rows
   for (int v = 0; v < kNumVariants; ++v) {
-    if (!conv3x3v_fits(v, ow)) continue;
+    if (!conv3x3v_fits(v, ow, 1)) continue;
     const Variant &k = kVariants[v];
     if (pass == 0) {
       if (oc > 64 && k.oc_t < 128) continue;

@@ -76,7 +76,7 @@ struct Conv3x3Args {
   int pad_t, pad_l;
   int ic2, units_pad, oc2, ocpp;
   int chunk_units;      // ic2 units staged per LDS fill (even)
-  int vw;               // virtual row width ow + 2
+  int vw;               // virtual row width: ow + 2 (stride 1), ow + 1 (stride 2)
   unsigned vw_magic;    // div_magic(vw)
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
   int gx, gy, tiles, tiles_per_xcd;   // set by the launcher: pixel tiles per image, channel tiles, all tiles, ceil(tiles / 8)
@@ -215,7 +215,7 @@ bool gemm1x1_wres_applies(const GemmArgs &a, int nbatch);
 hipError_t launch_gemm1x1_wres(const GemmArgs &a, hipStream_t s, LaunchPlan<GemmArgs> *plan = nullptr);
 
 hipError_t launch_conv3x3v(const Conv3x3Args &a, int n, int variant, hipStream_t s, LaunchPlan<Conv3x3Args> *plan = nullptr);
-int conv3x3v_pick_variant(int n, int oh, int ow, int oc2);   // -1: rows too wide for every variant
+int conv3x3v_pick_variant(int n, int oh, int ow, int oc2, int stride);   // stride 1 or 2 (both directions); -1: rows too wide for every variant
 int conv3x3v_chunk_units(int variant, int ic2);
 int conv3x3v_num_variants();
 const char *conv3x3v_variant_name(int variant);

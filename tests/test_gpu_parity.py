@@ -348,6 +348,32 @@ def test_conv3x3_wide_rows():
 def test_direct_kxk_strided(out_type, n, ic, oc, hw, k, pad, stride, out_hw):
     res = run_and_compare(Layer(n, ic, oc, hw, k=k, pad=pad, stride=stride, out_type=out_type, seed=90 + k + stride,
                                 out_hw=out_hw))
+    # 3x3 stride 2 has a form of the 3x3 kernel (four phase planes of the input); the rest walks [tap][unit] in the GEMM
+    assert res["conv"].kernel_name.startswith("k_conv3x3v_u8s8" if (k, stride) == (3, 2) else "k_gemm_u8s8")
+
+
+@pytest.mark.parametrize("variant", ["", "20", "21", "22", "23"])
+@pytest.mark.parametrize("n,ic,oc,hw,pad,out_hw", [
+    (2, 128, 128, 30, 0, None),    # pre-padded input, 128 channels: the straight-line K loop of four unit pairs
+    (3, 64, 80, 15, 1, None),      # two unit pairs, ragged channels, odd size
+    (2, 256, 64, 14, 1, None),     # two fills
+    (1, 48, 272, 14, 0, 7),        # pads only right / bottom, three units
+    (2, 32, 32, 57, 1, None),      # output rows of 29 pixels: the widest the 128-pixel tiles take
+    (1, 16, 16, 8, 1, None),
+])
+def test_direct_3x3_stride2_phase_planes(variant, n, ic, oc, hw, pad, out_hw, monkeypatch):
+    """3x3 stride 2 through the 3x3 kernel: the staged input as four phase planes, every tile variant, every output type"""
+    if variant:
+        monkeypatch.setenv("EHIP_CONV3X3V_VARIANT", variant)
+    for out_type in (ol.U8, ol.S8, ol.F32, ol.S32):
+        res = run_and_compare(Layer(n, ic, oc, hw, k=3, pad=pad, stride=2, out_type=out_type, seed=95 + ic + hw + out_type,
+                                    out_hw=out_hw))
+        assert "s2" in res["conv"].kernel_name
+
+
+def test_direct_3x3_stride2_phase_planes_can_be_switched_off(monkeypatch):
+    monkeypatch.setenv("EHIP_CONV3X3V_S2", "0")
+    res = run_and_compare(Layer(2, 64, 48, 14, k=3, pad=1, stride=2, out_type=ol.S8, seed=97))
     assert res["conv"].kernel_name.startswith("k_gemm_u8s8")
 
 
@@ -459,6 +485,7 @@ def test_direct_few_input_channels_rows_too_wide_for_lds():
 @pytest.mark.parametrize("variant", range(7))
 def test_direct_3x3_stride2_every_kernel_variant(variant, monkeypatch):
     monkeypatch.setenv("EHIP_GEMM_VARIANT", str(variant))
+    monkeypatch.setenv("EHIP_CONV3X3V_S2", "0")   # the GEMM form
     run_and_compare(Layer(2, 80, 96, 13, k=3, pad=1, stride=2, out_type=ol.U8, seed=120 + variant))
 
 
