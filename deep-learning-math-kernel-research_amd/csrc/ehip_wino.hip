@@ -476,7 +476,9 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 // NT: blocks of 32 tiles per workgroup.  Tile size 4 has 16 positions, four per wave: its accumulators for 64
 // channels x 32 tiles fill a quarter of the wave's registers, so a workgroup takes 64 tiles (a weight operand
 // then feeds two MFMAs as a tile operand does: 1 KB of operands per MFMA instead of 1.5).
-template <int KS, int A = 6, bool SUM = false, int NT = 1>
+// NH: halves of 32 channels per workgroup, two unless the layer has so few tiles that 64-channel workgroups would
+// leave CUs without one (256 -> 256 at 14 x 14, N = 64: 128 workgroups of 64 channels).
+template <int KS, int A = 6, bool SUM = false, int NT = 1, int NH = 2>
 __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 {
   constexpr int AA = A * A, PW = (AA + 3) / 4, CN = PW * 24, NJ = (CN + 63) / 64;
@@ -492,7 +494,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   const int by = seq % a.ny;
   const int bx = (seq / a.ny) * 8 + xcd;
   if (bx >= a.nx) return;          // whole workgroup
-  const int t0 = bx * 32 * NT, oc0 = by * 64;
+  const int t0 = bx * 32 * NT, oc0 = by * 32 * NH;
   const int oc_real = a.oc2 * 16;
   const int p0 = PW * wave;
   // positions of this wave: all PW, except in the last wave when four runs of PW overshoot A x A (A = 5)
@@ -518,11 +520,11 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   const int ks_last = ((a.ic2 + 1) >> 1) - 1;   // last k-step that holds real channels
 
   TRACE_POINT(0);
-  v4i ra[KS][2], rb[KS][NT];
+  v4i ra[KS][NH], rb[KS][NT];
   auto issue = [&](int slot, int p, int ks) {
     const int8_t *pa = a.w + (((long long)p * a.units_pad + 2 * ks) * a.ocpp + oc0) * 16;
-    ra[slot][0] = *reinterpret_cast<const v4i *>(pa + a_lane);
-    ra[slot][1] = *reinterpret_cast<const v4i *>(pa + 512 + a_lane);
+#pragma unroll
+    for (int h = 0; h < NH; ++h) ra[slot][h] = *reinterpret_cast<const v4i *>(pa + 512 * h + a_lane);
     // padded k-steps multiply zero weights: any valid cell will do (an odd unit count reads one
     // unit past the position, which is the next position or the pad unit behind the buffer)
     const int ksc = ks < ks_last ? ks : ks_last;
@@ -562,11 +564,11 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
   load_consts_half(0);
   store_consts_half();
 
-  v16i acc[PW][2][NT];
+  v16i acc[PW][NH][NT];
 #pragma unroll
   for (int i = 0; i < PW; ++i)
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < NH; ++h)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -582,8 +584,9 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           const v4i b = rb[k][j] ^ (int)0x80808080;
-          acc[i][0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][0], b, acc[i][0][j], 0, 0, 0);
-          acc[i][1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][1], b, acc[i][1][j], 0, 0, 0);
+#pragma unroll
+          for (int h = 0; h < NH; ++h)
+            acc[i][h][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[k][h], b, acc[i][h][j], 0, 0, 0);
         }
         // refill the slot with the operands KS steps ahead (the very last block re-reads itself)
         int pn = p0 + i, ksn = (c + 1) * KS + k;
@@ -594,12 +597,12 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
     }
   }
 
-  load_consts_half(1);   // second half's constants travel while the first half is processed
+  if (NH > 1) load_consts_half(1);   // second half's constants travel while the first half is processed
   TRACE_POINT(1);
   // ---- requantize, exchange, output transform ----------------------------------------------------
   const int tile_l = tid >> 3, q8 = tid & 7;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int h = 0; h < NH; ++h) {
 #pragma unroll
    for (int j = 0; j < NT; ++j) {   // a round: 32 channels x 32 tiles through the exchange buffer
     const int t = t0 + 32 * j + tile_l;
@@ -638,7 +641,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_wave_barrier();
-    if (h == 0 && j == NT - 1) store_consts_half();   // the wave is done with the first half's constants
+    if (NH > 1 && h == 0 && j == NT - 1) store_consts_half();   // the wave is done with the first half's constants
     TRACE_POINT(2 + 4 * h);
     __syncthreads();
     TRACE_POINT(3 + 4 * h);
@@ -717,7 +720,11 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   const int A = a.tile ? a.tile : 6, AA = A * A;
   const int ntb = A == 4 ? 2 : 1;   // blocks of 32 tiles per workgroup
   a.nx = (a.t + 32 * ntb - 1) / (32 * ntb);
-  a.ny = (a.oc2 * 16 + 63) / 64;
+  // 64 channels per workgroup; 32 where that would leave a quarter of the CUs or more without a workgroup
+  int nh = 2;
+  if (ntb == 1 && (long long)a.nx * ((a.oc2 * 16 + 63) / 64) <= 192 && a.oc2 * 16 > 32) nh = 1;
+  if (const char *env = getenv("EHIP_WINO_HALVES")) if (ntb == 1 && (env[0] == '1' || env[0] == '2')) nh = env[0] - '0';
+  a.ny = (a.oc2 * 16 + 32 * nh - 1) / (32 * nh);
   const int nks = a.units_pad / 2;
   const size_t lds = (size_t)AA * 32 * 32 * sizeof(float) + 4 * (size_t)((AA + 3) / 4 * 24) * sizeof(float4);   // exchange + constants
   dim3 grid(8 * a.ny * ((a.nx + 7) / 8));
@@ -726,10 +733,15 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   int ks_max = 4;
   if (const char *env = getenv("EHIP_WINO_KS")) ks_max = atoi(env);
   void (*kernel)(WinoFusedArgs) = nullptr;
+#define EHIP_WF1(AV, SV, NHV)                                                                          \
+  kernel = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1, NHV>          \
+      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4, AV, SV, AV == 4 ? 2 : 1, NHV>            \
+                                       : k_wino_gemm_output<2, AV, SV, AV == 4 ? 2 : 1, NHV>)
 #define EHIP_WF(AV, SV)                                                                                 \
-  kernel = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1>               \
-      : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4, AV, SV, AV == 4 ? 2 : 1>                 \
-                                       : k_wino_gemm_output<2, AV, SV, AV == 4 ? 2 : 1>)
+  do {                                                                                                  \
+    if (AV != 4 && nh == 1) EHIP_WF1(AV, SV, (AV != 4 ? 1 : 2));                                        \
+    else EHIP_WF1(AV, SV, 2);                                                                           \
+  } while (0)
   if (a.with_sum) {
     if (A == 4) EHIP_WF(4, true);
     else if (A == 5) EHIP_WF(5, true);
@@ -740,6 +752,7 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
     else EHIP_WF(6, false);
   }
 #undef EHIP_WF
+#undef EHIP_WF1
   if (nks % 2 != 0) return hipErrorInvalidValue;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;

@@ -108,6 +108,15 @@ def test_wino_fused_every_operand_ring_depth(ring, monkeypatch):
     _fused(2, 256, 80, 9)
 
 
+@pytest.mark.parametrize("halves", ["1", "2"])
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 256, 80, 9), (1, 64, 144, 13), (3, 32, 64, 7)])
+def test_wino_fused_channels_per_workgroup(halves, n, ic, oc, hw, monkeypatch):
+    """the fused kernel with workgroups of 32 channels (what layers of few tiles get, so that every CU has a
+    workgroup) and of 64; ragged channel counts leave the last workgroup partly past the real channels"""
+    monkeypatch.setenv("EHIP_WINO_HALVES", halves)
+    _fused(n, ic, oc, hw)
+
+
 def _fused(n, ic, oc, hw):
     import torch
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
