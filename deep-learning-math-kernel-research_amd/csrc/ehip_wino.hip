@@ -478,7 +478,10 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_output(WinoArgs a)
 // then feeds two MFMAs as a tile operand does: 1 KB of operands per MFMA instead of 1.5).
 // NH: halves of 32 channels per workgroup, two unless the layer has so few tiles that 64-channel workgroups would
 // leave CUs without one (256 -> 256 at 14 x 14, N = 64: 128 workgroups of 64 channels).
-template <int KS, int A = 6, bool SUM = false, int NT = 1, int NH = 2>
+// NKSF: 0, or the k-steps of a position when they are fewer than the ring is deep (64 / 128 input channels: 2 / 4).
+// The ring then runs ahead over the wave's positions as one flat sequence of steps -- with a ring of one position
+// every position costs a trip to memory (64 -> 64: 36 MFMAs per wave in 16 K clocks).
+template <int KS, int A = 6, bool SUM = false, int NT = 1, int NH = 2, int NKSF = 0>
 __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 {
   constexpr int AA = A * A, PW = (AA + 3) / 4, CN = PW * 24, NJ = (CN + 63) / 64;
@@ -574,6 +577,28 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][h][j][v] = 0;
 
+  if constexpr (NKSF > 0) {
+    // flat: step s = k-step s % NKSF of position s / NKSF, slot s % KS, refilled with step s + KS (positions past the
+    // wave's last one -- tile size 5, last wave -- repeat it: their accumulators are never read)
+    auto issue_step = [&](int slot, int sn) {
+      int pi = sn / NKSF;
+      pi = pi < np ? pi : np - 1;
+      issue(slot, p0 + pi, sn % NKSF);
+    };
+#pragma unroll
+    for (int k = 0; k < KS; ++k) issue_step(k, k);
+#pragma unroll
+    for (int s = 0; s < PW * NKSF; ++s) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const v4i b = rb[s % KS][j] ^ (int)0x80808080;
+#pragma unroll
+        for (int h = 0; h < NH; ++h)
+          acc[s / NKSF][h][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ra[s % KS][h], b, acc[s / NKSF][h][j], 0, 0, 0);
+      }
+      if (s + KS < PW * NKSF) issue_step(s % KS, s + KS);
+    }
+  } else {
 #pragma unroll
   for (int k = 0; k < KS; ++k) issue(k, p0, k);
 #pragma unroll
@@ -595,6 +620,7 @@ __global__ __launch_bounds__(kBlock, 1) void k_wino_gemm_output(WinoFusedArgs a)
         issue(k, pn, ksn);
       }
     }
+  }
   }
 
   if (NH > 1) load_consts_half(1);   // second half's constants travel while the first half is processed
@@ -732,9 +758,13 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   // 178.6, 4 deep 250.4 / 172.8 / 241.2 / 176.5, 2 deep 286.8 / 215.6 (f32 layers)
   int ks_max = 4;
   if (const char *env = getenv("EHIP_WINO_KS")) ks_max = atoi(env);
+  bool flat = true;   // 64 / 128 input channels: the ring runs ahead over positions
+  if (const char *env = getenv("EHIP_WINO_FLAT")) flat = env[0] != '0';
   void (*kernel)(WinoFusedArgs) = nullptr;
 #define EHIP_WF1(AV, SV, NHV)                                                                          \
-  kernel = (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1, NHV>          \
+  kernel = (nks == 2 && flat) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1, NHV, 2>                  \
+      : (nks == 4 && flat) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1, NHV, 4>                     \
+      : (nks % 8 == 0 && ks_max >= 8) ? k_wino_gemm_output<8, AV, SV, AV == 4 ? 2 : 1, NHV>          \
       : ((nks % 4 == 0 && ks_max >= 4) ? k_wino_gemm_output<4, AV, SV, AV == 4 ? 2 : 1, NHV>            \
                                        : k_wino_gemm_output<2, AV, SV, AV == 4 ? 2 : 1, NHV>)
 #define EHIP_WF(AV, SV)                                                                                 \

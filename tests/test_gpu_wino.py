@@ -117,6 +117,29 @@ def test_wino_fused_channels_per_workgroup(halves, n, ic, oc, hw, monkeypatch):
     _fused(n, ic, oc, hw)
 
 
+@pytest.mark.parametrize("flat", ["0", "1"])
+@pytest.mark.parametrize("tile", [6, 5, 4])
+@pytest.mark.parametrize("ic", [64, 128, 48])
+def test_wino_fused_few_input_channels(flat, tile, ic, monkeypatch):
+    """64 / 128 input channels (2 / 4 k-steps per position): the operand ring running ahead over the positions as one
+    flat sequence of steps, and filled position by position; 48 channels (padded to 64) as well"""
+    monkeypatch.setenv("EHIP_WINO_FLAT", flat)
+    import torch
+    E, p, d, xq, wb, bias = make_wino_u8(2, ic, 80, 13, seed=31 + tile + ic, out_type=ol.S8, tile=tile)
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    _, exp = _oracle_u8(p, xq, wb, bias)
+    conv = E.Conv(d)
+    assert conv.kernel_name.endswith("k_wino_gemm_output")
+    d_b = dev(bias)
+    d_out = torch.zeros(exp.shape, dtype=torch.int8, device="cuda")
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, dev(xq), None, d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
 def _fused(n, ic, oc, hw):
     import torch
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
