@@ -377,7 +377,8 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
       if (with_bias) r = r + b;
       if (OUT != EHIP_F32) r = __builtin_fmaf(r, repS, z);
       if (with_sum) r = r + old[k][e];
-      if (with_relu) r = r > 0.0f ? r : 0.0f;
+      // (u8 / s8 output: the ReLU is part of the clamp in front of the byte pack below)
+      if (with_relu && OUT == EHIP_F32) r = r > 0.0f ? r : 0.0f;
       y[k][e] = r;
     }
   }
@@ -403,6 +404,17 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
         }
       } else {
         unsigned o = 0u;
+        if (with_relu) {
+          // ReLU and the type's upper bound in one clamp (a NaN comes out of it as 0, like out of the ReLU's
+          // comparison); what is left of the conversion -- rounding to nearest even, or the floor of F(2x2,3x3)
+          // first -- is the byte pack's own, and floor and clamp commute
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            float r = __builtin_amdgcn_fmed3f(y[k][e], 0.0f, OUT == EHIP_S8 ? 127.0f : 255.0f);
+            if (A == 4) r = __builtin_floorf(r);
+            o = __builtin_amdgcn_cvt_pk_u8_f32(r, k, o);
+          }
+        } else
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const float r = y[k][e];
