@@ -374,7 +374,10 @@ __device__ __forceinline__ void output_tile(const float4 *m, const float4 &bias,
 #pragma unroll
     for (int e = 0; e < M * M; ++e) {
       float r = o[e];
-      if (with_bias) r = r + b;
+      // (the caller passes a zero bias when the layer has none; adding it anyway can only turn a -0.0 into +0.0, which
+      // the output quantization's multiply-add maps to the same value -- so only f32 output needs the condition,
+      // which otherwise costs a select per value)
+      if (OUT != EHIP_F32 || with_bias) r = r + b;
       if (OUT != EHIP_F32) r = __builtin_fmaf(r, repS, z);
       if (with_sum) r = r + old[k][e];
       // (u8 / s8 output: the ReLU is part of the clamp in front of the byte pack below)
