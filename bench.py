@@ -260,15 +260,7 @@ def cpu_baseline(wl, budget_s=12.0):
     threads = int(lib.orc_num_threads())
     model, logical, physical, smt = host_cpus()
     wino = wl.algorithm == E.CONV_WINOGRAD
-    if wl.in_z != 0.0 or (wl.nhwc_in and wl.ic <= 4):
-        # a first layer as the reference's tuned runs feed it (scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh:12):
-        # a compact three-channel nhwc image with zero point 128.  The oracle computes such a layer for the parity
-        # tests pixel class by pixel class (the shift depends on which taps fall inside the image), on channels
-        # padded to 16: a checker, not the reference's loop nest over three channels, and timing it would quote a
-        # CPU rate the reference does not have.
-        return {"value": None, "unit": "TOPS", "cores": 0, "kind": "port",
-                "sample": "not timed: the oracle's path for a three-channel image with an input zero point is a per-class "
-                          "checker over channels padded to 16, not a port of the reference's first-layer loop nest"}
+    first = wl.in_z != 0.0 or (wl.nhwc_in and wl.ic <= 4)
     # a first guess of one pass: ~1 TOPS per 8 VNNI threads for the direct nests, far less for the others
     n = wl.n
     rate = (0.12 if vnni else 0.004) * threads * (0.05 if wl.depthwise else (0.3 if wino else 1.0)) * 1e12
@@ -280,7 +272,7 @@ def cpu_baseline(wl, budget_s=12.0):
     p = ol.make_params(n, wl.ic, wl.oc, wl.hw, wl.hw, wl.k, wl.k, wl.pad, wl.stride, g=g, out_type=wl.out_type,
                        with_sum=wl.with_sum, out_scale=0.02, sum_scale=0.7 if wl.with_sum else 0.0, relu_hi=relu_hi,
                        T=wl.T, out_hw=(wl.oh, wl.oh), pad_tl=wl.pad, wino_tile=wl.tile if wino else 0,
-                       in_scale=1.0 if wl.in_type == E.F32 else 1.0 / 255.0)
+                       in_scale=1.0 if wl.in_type == E.F32 else 1.0 / 255.0, in_z=wl.in_z)
     b = rng.normal(0, 0.01, ol.up16(wl.oc)).astype(np.float32)
     out = np.zeros((n, oc2, wl.oh, wl.oh, 16), ol.NP_OF[wl.out_type])
     if wl.with_sum:
@@ -302,6 +294,23 @@ def cpu_baseline(wl, budget_s=12.0):
             lib.orc_wino_gemm(pp, ol.ptr(tin), ol.ptr(twq), ol.ptr(tscale), ol.ptr(tshift), ol.ptr(tout), None)
             lib.orc_wino_trans_output(pp, ol.ptr(tout), ol.ptr(b), ol.ptr(out))
         nest = "Winograd input transform + u8 x s8 GEMM + output transform"
+    elif first:
+        # A first layer as the reference's tuned runs feed it (scripts/best_configs/resnetv1_5-n64-clx-1s-int8.sh:12):
+        # three channels, input zero point 128, so the shift of a pixel depends on which taps fall inside the image.
+        # The oracle runs it as the same k x k nest over one 16-channel unit (the image's channels padded to 16 --
+        # the reference pads three to four, a quarter of these multiplies) with a shift row per pixel.
+        x = rng.integers(0, 256, (n, ic2, wl.hw, wl.hw, 16)).astype(np.uint8)
+        x[..., wl.ic:] = 0
+        w = rng.normal(0, wl.w_sigma, (wl.oc, wl.ic, wl.k, wl.k)).astype(np.float32)
+        wb = ol.weights_to_blocked(w)
+        wq, scale, shift, _ = ol.direct_prepare(p, wb, b)
+        smap = np.zeros((wl.oh, wl.oh, ol.up16(wl.oc)), np.float32)
+        assert lib.orc_direct_border_shifts(ctypes.byref(p), ol.ptr(wb), ol.ptr(b), ol.ptr(smap)) == 0
+        args = (ctypes.byref(p), ol.ptr(x), ol.ptr(wq), ol.ptr(scale), ol.ptr(smap), ol.ptr(out), None)
+
+        def one_pass():
+            assert lib.orc_direct_execute_border(*args) == 0
+        nest = "direct %dx%d nest over the image's channels padded to 16, a shift row per pixel," % (wl.k, wl.k)
     elif wl.depthwise:
         x = rng.integers(0, 256, (n, ic2, wl.hw, wl.hw, 16)).astype(np.uint8)
         w = rng.normal(0, wl.w_sigma, (wl.ic, 1, 3, 3)).astype(np.float32)
