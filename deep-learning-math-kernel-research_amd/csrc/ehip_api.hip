@@ -224,7 +224,9 @@ int classify(ehip_conv *c)
       // point with padding needs
       // 3x3 stride 2 runs the same kernel over four phase planes of the input (EHIP_CONV3X3V_S2=0: the GEMM form)
       const char *s2env = getenv("EHIP_CONV3X3V_S2");
-      const bool s2_3x3 = d.kh == 3 && d.kw == 3 && d.stride_h == 2 && d.stride_w == 2 && !(s2env && s2env[0] == '0');
+      // (its staging plan holds a cell's byte offset inside one image plane in 31 bits)
+      const bool s2_3x3 = d.kh == 3 && d.kw == 3 && d.stride_h == 2 && d.stride_w == 2 && !(s2env && s2env[0] == '0') &&
+          (long long)d.ih * d.iw * 16 < (1ll << 31);
       c->family = ((s1_3x3 || s2_3x3) && !(d.input_z != 0.0f && padded) && d.output_fmt != EHIP_NHWC && d.input_fmt != EHIP_NHWC)
           ? FAM_CONV_3X3 : FAM_GEMM_1X1;
       {
