@@ -21,6 +21,7 @@ SOURCES = [
     "ehip_fewch.hip",
     "ehip_depthwise.hip",
     "ehip_wino.hip",
+    "ehip_wino_lanes.hip",
     "ehip_prepare.hip",
     "ehip_harness.hip",
     "ehip_api.hip",
@@ -48,6 +49,8 @@ EXTRA_FLAGS = {
     "ehip_conv3x3v.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-pragma-unroll-threshold=1000000"],
     # the resident-tile 1x1 kernel's leading scalar arguments: preloaded as well
     "ehip_gemm1x1.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    # the Winograd kernel whose requantized values take the accumulators' place in the vector registers
+    "ehip_wino_lanes.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "ehip_gemm1x1w.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16", "-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     # and those of the 1x1 kernels with few input channels
     "ehip_gemm.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],

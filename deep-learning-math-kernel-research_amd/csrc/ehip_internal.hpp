@@ -227,6 +227,9 @@ bool depthwise_mfma_applies(int stride, int oh, int ow, int pad_t, int pad_l, in
 hipError_t launch_wino_trans_input(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
 hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan<WinoArgs> *plan = nullptr);
 hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);
+// at most 256 input channels, u8 / s8 output: the form without an exchange between GEMMs and transform (ehip_wino_lanes.hip)
+bool wino_lanes_applies(const WinoFusedArgs &a);
+hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);
 // min / max of the transformed input: partials = 2 * a.ic2 dwords of device scratch, result = two floats
 // of device memory (min, max); three launches on `s`, nothing else
 hipError_t launch_wino_range(const WinoArgs &a, int ic_real, unsigned *partials, float *minmax_out_dev, hipStream_t s);

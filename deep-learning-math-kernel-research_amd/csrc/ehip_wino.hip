@@ -776,6 +776,7 @@ hipError_t launch_wino_gemm_output(const WinoFusedArgs &a0, hipStream_t s, Launc
   }
   WinoFusedArgs a = a0;
   const int A = a.tile ? a.tile : 6, AA = A * A;
+  if (wino_lanes_applies(a)) return launch_wino_gemm_output_lanes(a, s, plan);
   const int ntb = A == 4 ? 2 : 1;   // blocks of 32 tiles per workgroup
   a.nx = (a.t + 32 * ntb - 1) / (32 * ntb);
   // 64 channels per workgroup; 32 where that would leave a quarter of the CUs or more without a workgroup

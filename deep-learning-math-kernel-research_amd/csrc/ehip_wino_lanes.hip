@@ -1,0 +1,235 @@
+// Winograd GEMMs + output transform for layers with at most 256 input channels and u8 / s8 output: the form whose
+// lanes own a tile x four channels at every position, so that nothing is exchanged between the GEMMs and the transform.
+//
+// Replaces, for those layers, elx_int8_conv_wino_gemm_t::execute + trans_output as the reference's fused schedule
+// runs them per thread (a161, src/elx_int8_conv_wino_xopt.hpp:21-179; src/elx_int8_conv_wino_gemm.cpp:23-205,
+// src/elx_conv_wino_trans_output.cpp:212-423).
+//
+// A file of its own because it is compiled with the accumulators of the matrix instructions in the ordinary vector
+// registers (-amdgpu-mfma-vgpr-form): the requantized values then take the accumulators' place and two workgroups
+// fit on a CU, where the general kernel of ehip_wino.hip needs the accumulation registers for its 288 accumulators.
+#include "ehip_internal.hpp"
+#include "ehip_wino_tiles.hpp"
+
+namespace ehip {
+
+namespace {
+
+__device__ __forceinline__ float comp_of(const float4 &v, int k) { return k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w)); }
+
+// output_tile for u8 / s8 output with few registers: one channel at a time, its bytes packed into the pixels' dwords
+// as they come (16 dwords live instead of 4 x 16 floats; the old output of the in-place sum stays packed as well).
+// Same operations in the same order per value as output_tile.
+template <int OUT, int A>
+__device__ __forceinline__ void output_tile_packed(const float4 *m, const float4 &bias, bool with_relu, float repS, float z,
+                                                   uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, bool with_sum,
+                                                   int px)
+{
+  static_assert(OUT == EHIP_U8 || OUT == EHIP_S8, "quantized output");
+  constexpr int AA = A * A, M = A - 2;
+  unsigned pk[M * M], old[M * M];
+#pragma unroll
+  for (int e = 0; e < M * M; ++e) pk[e] = 0u;
+  if (with_sum) {
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+      for (int j = 0; j < M; ++j) {
+        const int oh = M * th + i, ow = M * tw + j;
+        const bool in = oh < oh_n && ow < ow_n;
+        const size_t cell = in ? ((size_t)oh * ow_n + ow) * px + 4 * q : 0;
+        old[M * i + j] = *reinterpret_cast<const unsigned *>(plane + cell);
+      }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float f[AA], o[M * M];
+#pragma unroll
+    for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
+    wino::tile_output<A>(f, o);
+    const float b = comp_of(bias, k);
+#pragma unroll
+    for (int e = 0; e < M * M; ++e) {
+      float r = o[e] + b;
+      r = __builtin_fmaf(r, repS, z);
+      if (with_sum) {
+        const unsigned ob = (old[e] >> (8 * k)) & 0xffu;
+        r = r + (OUT == EHIP_U8 ? (float)ob : (float)(int)(signed char)ob);
+      }
+      if (with_relu) {
+        r = __builtin_amdgcn_fmed3f(r, 0.0f, OUT == EHIP_S8 ? 127.0f : 255.0f);
+        if (A == 4) r = __builtin_floorf(r);
+        pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r, k, pk[e]);
+      } else if (A == 4) {
+        const float fl = __builtin_floorf(r);
+        if (OUT == EHIP_U8) pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r >= 0.0f ? fl : 300.0f, k, pk[e]);
+        else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(fl)) & 0xffu) << (8 * k);
+      } else {
+        if (OUT == EHIP_U8) pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r >= -0.5f ? r : 300.0f, k, pk[e]);
+        else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
+      }
+    }
+    // (one channel after the other: interleaved, the four transforms' intermediates do not fit the registers)
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    const int oh = M * th + i;
+    if (oh >= oh_n) break;
+#pragma unroll
+    for (int j = 0; j < M; ++j) {
+      const int ow = M * tw + j;
+      if (ow >= ow_n) break;
+      *reinterpret_cast<unsigned *>(plane + ((size_t)oh * ow_n + ow) * px + 4 * q) = pk[M * i + j];
+    }
+  }
+}
+
+}  // namespace
+
+// The general kernel (k_wino_gemm_output, ehip_wino.hip) keeps 64 channels x 32 tiles x all positions in its four waves'
+// registers, one wave per SIMD, and passes the results through 144 KB of LDS to the transform; with few input channels
+// it is all output phase (64 -> 64: 37 K of a workgroup's 47 K clocks).
+// Here v_mfma_i32_16x16x64_i8 makes the GEMM's own result layout the transform's: a lane of the 16 x 16 result holds
+// four consecutive packed rows = four consecutive output channels of ONE tile, so with all A x A positions of its 16
+// channels x 16 tiles in one wave (4 accumulator registers per position) every lane already owns the A x A values
+// of one tile x four channels -- requantization, Y = At M A and the store happen in the lane, with no exchange, no
+// barrier, and two to three workgroups per CU to hide each other's latencies.  The price is the operand stream:
+// 2 KB per 16 x 16 x 64 MFMA, which only so short a K loop can afford.
+// Workgroup = 32 channels x 32 tiles (one block of the blocked tinput); wave = (half of the channels, half of the
+// tiles); NKS = k-steps of 64 channels per position (1, 2 or 4).
+template <int A, bool SUM, int NKS>
+__global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedArgs a)
+{
+  constexpr int AA = A * A, D = 8, STEPS = AA * NKS;
+  extern __shared__ float4 cl[];   // [AA][3][8 quads of the workgroup's 32 channels]: scale, shift, compensation
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, g = lane >> 4;
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int by = seq % a.ny;
+  const int bx = (seq / a.ny) * 8 + xcd;
+  if (bx >= a.nx) return;          // whole workgroup
+  const int oc0 = by * 32;
+  const int r0 = (wave & 1) * 16;          // the wave's packed rows inside the group of 32
+  const int th16 = (wave >> 1) * 16;       // its tiles inside the block of 32
+  const int oc_real = a.oc2 * 16;
+
+  // constants of the workgroup's channels, once: 24 cells of four channels per position
+  for (int idx = tid; idx < AA * 24; idx += kBlock) {
+    const int p = idx / 24, rem = idx - 24 * p, arr = rem >> 3, cell = rem & 7;
+    const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
+    cl[idx] = *reinterpret_cast<const float4 *>(src + (long long)p * a.ocpp + oc0 + 4 * cell);
+  }
+
+  // operands: lane = packed row / tile l16 of unit 4 ks + g, one 16-byte cell each; a wave-uniform base per step plus
+  // one 32-bit offset per lane (as 64-bit pointers per lane the unrolled loop's 72 addresses fill the register file)
+  const unsigned a_off = (unsigned)(g * a.ocpp + oc0 + r0 + l16) * 16u;
+  const long long w_pos = (long long)a.units_pad * a.ocpp * 16, w_ks = (long long)4 * a.ocpp * 16;
+  const uint8_t *tbase = a.tin + (long long)bx * AA * a.ic2 * 512;
+  const long long t_pos = (long long)a.ic2 * 512;
+  unsigned b_off[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    // units past the last real one multiply zero weights: any valid cell will do
+    int u = 4 * ks + g;
+    u = u < a.ic2 ? u : a.ic2 - 1;
+    b_off[ks] = (unsigned)(u * 512 + (th16 + l16) * 16);
+  }
+  v4i ra[D], rb[D];
+  auto issue = [&](int slot, int sn) {
+    const int p = sn / NKS, ks = sn - NKS * p;
+    const int8_t *wp = a.w + p * w_pos + ks * w_ks;      // wave-uniform
+    const uint8_t *tp = tbase + p * t_pos;               // wave-uniform
+    ra[slot] = *reinterpret_cast<const v4i *>(wp + a_off);
+    rb[slot] = *reinterpret_cast<const v4i *>(tp + b_off[ks]);
+  };
+  v4i acc[AA];
+#pragma unroll
+  for (int e = 0; e < AA; ++e) acc[e] = v4i{0, 0, 0, 0};
+#pragma unroll
+  for (int k = 0; k < D; ++k)
+    if (k < STEPS) issue(k, k);
+#pragma unroll
+  for (int sn = 0; sn < STEPS; ++sn) {
+    const v4i b = rb[sn % D] ^ (int)0x80808080;
+    acc[sn / NKS] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ra[sn % D], b, acc[sn / NKS], 0, 0, 0);
+    if (sn + D < STEPS) issue(sn % D, sn + D);
+    __builtin_amdgcn_sched_barrier(0);   // (the loads stay where the ring puts them: hoisted, they spill)
+  }
+  __syncthreads();   // the constants are in LDS
+
+  // the lane's channels: packed rows r0 + 4 g .. + 3 of the group hold channels 16 (g & 1) + 4 (r0 / 8 + g / 2) + j
+  const int quad = 4 * (g & 1) + (r0 >> 3) + (g >> 1);   // cell of four channels inside the group of 32
+  const int oc = oc0 + 4 * quad;
+  const int t = bx * 32 + th16 + l16;
+  if (t >= a.t || oc >= oc_real) return;
+  float4 m[AA];
+  int cq = quad;   // (the constants' cell, re-derived group by group: see below)
+#pragma unroll
+  for (int e = 0; e < AA; ++e) {
+    const float4 sc = cl[e * 24 + cq], sh = cl[e * 24 + 8 + cq], cf = cl[e * 24 + 16 + cq];
+    m[e].x = __builtin_fmaf((float)(acc[e][0] + __float_as_int(cf.x)), sc.x, sh.x);
+    m[e].y = __builtin_fmaf((float)(acc[e][1] + __float_as_int(cf.y)), sc.y, sh.y);
+    m[e].z = __builtin_fmaf((float)(acc[e][2] + __float_as_int(cf.z)), sc.z, sh.z);
+    m[e].w = __builtin_fmaf((float)(acc[e][3] + __float_as_int(cf.w)), sc.w, sh.w);
+    // (four positions' constants in flight at a time: the compiler would read all 108 cells first and spill the
+    // accumulators to make room, so the next group's address is made to depend on this group's last result)
+    // (and every value is pinned where it is computed: sunk towards their use, the values leave their constants live)
+    asm volatile("" : "+v"(m[e].x), "+v"(m[e].y), "+v"(m[e].z), "+v"(m[e].w));
+    if ((e & 3) == 3) asm volatile("" : "+v"(cq) : "v"(m[e].w));
+  }
+  const int n = t / a.nt;
+  const int rem = t - n * a.nt;
+  const int th = rem / a.wt;
+  const int tw = rem - th * a.wt;
+  float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
+  const size_t plane = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (oc >> 4) * 16
+                                  : ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 16;
+  const int px = a.out_nhwc ? a.oc2 * 16 : 16;
+  const int q = (oc >> 2) & 3;
+  // (u8 / s8 output only: the launcher keeps f32 output, whose four channels of a pixel leave as one 16-byte store
+  // and would need all of them in registers at once, on the general form)
+  if (a.out_type == EHIP_U8)
+    output_tile_packed<EHIP_U8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + plane, q,
+                                   th, tw, a.oh, a.ow, SUM, px);
+  else
+    output_tile_packed<EHIP_S8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + plane, q,
+                                   th, tw, a.oh, a.ow, SUM, px);
+}
+
+bool wino_lanes_applies(const WinoFusedArgs &a)
+{
+  const char *env = getenv("EHIP_WINO_LANES");
+  const int nks64 = (a.ic2 + 3) / 4;
+  // Measured at N = 64, u8 in / s8 out, against the general kernel (fused stage, us): 64 -> 64 at 56 x 56 28.5 vs 34.1, at
+  // 224 x 224 370 vs 459; 128 -> 128 at 112 x 112 238 vs 300; 128 -> 256 at 56 x 56 107 vs 133; 256 -> 256 at 56 x 56 164 vs 171;
+  // 512 -> 512 at 28 x 28 (eight k-steps per position, 288 unrolled steps) 648 vs 134: up to 256 input channels.
+  return a.tin_blocked && (nks64 <= 2 || nks64 == 4) && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && a.out_type != EHIP_F32 &&
+      !(env && env[0] == '0');
+}
+
+hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a0, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan)
+{
+  WinoFusedArgs a = a0;
+  const int A = a.tile ? a.tile : 6, AA = A * A;
+  const int nks64 = (a.ic2 + 3) / 4;
+  a.nx = (a.t + 31) / 32;
+  a.ny = (a.oc2 * 16 + 31) / 32;
+  void (*kernel)(WinoFusedArgs) = nullptr;
+#define EHIP_WL(AV)                                                                                                    \
+  kernel = a.with_sum ? (nks64 == 1 ? k_wino_gemm_output_lanes<AV, true, 1>                                             \
+                                    : (nks64 == 2 ? k_wino_gemm_output_lanes<AV, true, 2> : k_wino_gemm_output_lanes<AV, true, 4>)) \
+                      : (nks64 == 1 ? k_wino_gemm_output_lanes<AV, false, 1>                                            \
+                                    : (nks64 == 2 ? k_wino_gemm_output_lanes<AV, false, 2> : k_wino_gemm_output_lanes<AV, false, 4>))
+  if (A == 4) EHIP_WL(4);
+  else if (A == 5) EHIP_WL(5);
+  else EHIP_WL(6);
+#undef EHIP_WL
+  const size_t lds = (size_t)AA * 24 * sizeof(float4);
+  return plan_launch(plan, kernel, dim3(8 * a.ny * ((a.nx + 7) / 8)), dim3(kBlock), lds, a, s);
+}
+
+}  // namespace ehip

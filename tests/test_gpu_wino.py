@@ -140,6 +140,32 @@ def test_wino_fused_few_input_channels(flat, tile, ic, monkeypatch):
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
+@pytest.mark.parametrize("lanes", ["1", "0"])
+@pytest.mark.parametrize("tile", [6, 5, 4])
+@pytest.mark.parametrize("out_type", [ol.U8, ol.S8])
+@pytest.mark.parametrize("n,ic,oc,hw,with_relu", [(2, 64, 80, 13, True), (1, 128, 48, 9, False), (3, 256, 32, 7, True),
+                                                  (1, 48, 144, 28, True), (2, 192, 64, 10, True)])
+def test_wino_fused_lanes_form(lanes, tile, out_type, n, ic, oc, hw, with_relu, monkeypatch):
+    """up to 256 input channels with u8 / s8 output: the fused stage whose lanes own a tile x four channels at every
+    position (16 x 16 x 64 matrix instruction, no exchange through LDS), and the general form on the same layers; one,
+    two and four k-steps of 64 channels per position, channel counts that leave units, rows and tiles unused"""
+    import torch
+    monkeypatch.setenv("EHIP_WINO_LANES", lanes)
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=41 + tile + ic + out_type, out_type=out_type, tile=tile,
+                                         with_relu=with_relu, out_z=0.0 if out_type == ol.S8 else 2.4)
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    _, exp = _oracle_u8(p, xq, wb, bias)
+    conv = E.Conv(d)
+    d_b = dev(bias)
+    d_out = torch.zeros(exp.shape, dtype=torch.uint8 if out_type == ol.U8 else torch.int8, device="cuda")
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, dev(xq), None, d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
 def _fused(n, ic, oc, hw):
     import torch
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
