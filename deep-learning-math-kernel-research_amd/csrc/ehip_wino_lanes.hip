@@ -116,13 +116,6 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
   const int th16 = (wave >> 1) * 16;       // its tiles inside the block of 32
   const int oc_real = a.oc2 * 16;
 
-  // constants of the workgroup's channels, once: 24 cells of four channels per position
-  for (int idx = tid; idx < AA * 24; idx += kBlock) {
-    const int p = idx / 24, rem = idx - 24 * p, arr = rem >> 3, cell = rem & 7;
-    const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
-    cl[idx] = *reinterpret_cast<const float4 *>(src + (long long)p * a.ocpp + oc0 + 4 * cell);
-  }
-
   // operands: lane = packed row / tile l16 of unit 4 ks + g, one 16-byte cell each; a wave-uniform base per step plus
   // one 32-bit offset per lane (as 64-bit pointers per lane the unrolled loop's 72 addresses fill the register file)
   const unsigned a_off = (unsigned)(g * a.ocpp + oc0 + r0 + l16) * 16u;
@@ -145,12 +138,38 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
     ra[slot] = *reinterpret_cast<const v4i *>(wp + a_off);
     rb[slot] = *reinterpret_cast<const v4i *>(tp + b_off[ks]);
   };
-  v4i acc[AA];
-#pragma unroll
-  for (int e = 0; e < AA; ++e) acc[e] = v4i{0, 0, 0, 0};
+  // the first operands are requested before anything else; the constants of the workgroup's channels (24 cells of
+  // four channels per position) travel behind them, all of a thread's loads before its first store
 #pragma unroll
   for (int k = 0; k < D; ++k)
     if (k < STEPS) issue(k, k);
+  {
+    constexpr int NC = (AA * 24 + kBlock - 1) / kBlock;
+    float4 cst[NC];
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      int idx = tid + j * kBlock;
+      idx = idx < AA * 24 ? idx : AA * 24 - 1;
+      const int p = idx / 24, rem = idx - 24 * p, arr = rem >> 3, cell = rem & 7;
+      const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
+      cst[j] = *reinterpret_cast<const float4 *>(src + (long long)p * a.ocpp + oc0 + 4 * cell);
+    }
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      const int idx = tid + j * kBlock;
+      if (idx < AA * 24) cl[idx] = cst[j];
+    }
+  }
+  __syncthreads();   // the constants are in LDS
+  // the lane's channels: packed rows r0 + 4 g .. + 3 of the group hold channels 16 (g & 1) + 4 (r0 / 8 + g / 2) + j
+  const int quad = 4 * (g & 1) + (r0 >> 3) + (g >> 1);   // cell of four channels inside the group of 32
+  // the accumulators start from the compensation 128 * sum(weights) of their (position, channel)
+  v4i acc[AA];
+#pragma unroll
+  for (int e = 0; e < AA; ++e) {
+    const float4 cf = cl[e * 24 + 16 + quad];
+    acc[e] = v4i{__float_as_int(cf.x), __float_as_int(cf.y), __float_as_int(cf.z), __float_as_int(cf.w)};
+  }
 #pragma unroll
   for (int sn = 0; sn < STEPS; ++sn) {
     const v4i b = rb[sn % D] ^ (int)0x80808080;
@@ -158,10 +177,6 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
     if (sn + D < STEPS) issue(sn % D, sn + D);
     __builtin_amdgcn_sched_barrier(0);   // (the loads stay where the ring puts them: hoisted, they spill)
   }
-  __syncthreads();   // the constants are in LDS
-
-  // the lane's channels: packed rows r0 + 4 g .. + 3 of the group hold channels 16 (g & 1) + 4 (r0 / 8 + g / 2) + j
-  const int quad = 4 * (g & 1) + (r0 >> 3) + (g >> 1);   // cell of four channels inside the group of 32
   const int oc = oc0 + 4 * quad;
   const int t = bx * 32 + th16 + l16;
   if (t >= a.t || oc >= oc_real) return;
@@ -169,11 +184,11 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
   int cq = quad;   // (the constants' cell, re-derived group by group: see below)
 #pragma unroll
   for (int e = 0; e < AA; ++e) {
-    const float4 sc = cl[e * 24 + cq], sh = cl[e * 24 + 8 + cq], cf = cl[e * 24 + 16 + cq];
-    m[e].x = __builtin_fmaf((float)(acc[e][0] + __float_as_int(cf.x)), sc.x, sh.x);
-    m[e].y = __builtin_fmaf((float)(acc[e][1] + __float_as_int(cf.y)), sc.y, sh.y);
-    m[e].z = __builtin_fmaf((float)(acc[e][2] + __float_as_int(cf.z)), sc.z, sh.z);
-    m[e].w = __builtin_fmaf((float)(acc[e][3] + __float_as_int(cf.w)), sc.w, sh.w);
+    const float4 sc = cl[e * 24 + cq], sh = cl[e * 24 + 8 + cq];
+    m[e].x = __builtin_fmaf((float)acc[e][0], sc.x, sh.x);
+    m[e].y = __builtin_fmaf((float)acc[e][1], sc.y, sh.y);
+    m[e].z = __builtin_fmaf((float)acc[e][2], sc.z, sh.z);
+    m[e].w = __builtin_fmaf((float)acc[e][3], sc.w, sh.w);
     // (four positions' constants in flight at a time: the compiler would read all 108 cells first and spill the
     // accumulators to make room, so the next group's address is made to depend on this group's last result)
     // (and every value is pinned where it is computed: sunk towards their use, the values leave their constants live)
