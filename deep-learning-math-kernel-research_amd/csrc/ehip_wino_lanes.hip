@@ -10,6 +10,7 @@
 // fit on a CU, where the general kernel of ehip_wino.hip needs the accumulation registers for its 288 accumulators.
 #include "ehip_internal.hpp"
 #include "ehip_wino_tiles.hpp"
+#include <type_traits>
 
 namespace ehip {
 
@@ -17,61 +18,58 @@ namespace {
 
 __device__ __forceinline__ float comp_of(const float4 &v, int k) { return k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w)); }
 
-// output_tile for u8 / s8 output with few registers: one channel at a time, its bytes packed into the pixels' dwords
-// as they come (16 dwords live instead of 4 x 16 floats; the old output of the in-place sum stays packed as well).
-// Same operations in the same order per value as output_tile.
+// The pieces of output_tile for u8 / s8 output with few registers: one channel at a time, its bytes packed into the
+// pixels' dwords as they come (16 dwords live instead of 4 x 16 floats; the old output of the in-place sum stays packed
+// as well).  Same operations in the same order per value as output_tile.
+template <int A>
+__device__ __forceinline__ void load_old(unsigned *old, const uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, int px)
+{
+  constexpr int M = A - 2;
+#pragma unroll
+  for (int i = 0; i < M; ++i)
+#pragma unroll
+    for (int j = 0; j < M; ++j) {
+      const int oh = M * th + i, ow = M * tw + j;
+      const bool in = oh < oh_n && ow < ow_n;
+      const size_t cell = in ? ((size_t)oh * ow_n + ow) * px + 4 * q : 0;
+      old[M * i + j] = *reinterpret_cast<const unsigned *>(plane + cell);
+    }
+}
+
+// channel k of the lane's four: bias, output scale, old output, ReLU, rounding, byte k of the pixels' dwords
 template <int OUT, int A>
-__device__ __forceinline__ void output_tile_packed(const float4 *m, const float4 &bias, bool with_relu, float repS, float z,
-                                                   uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, bool with_sum,
-                                                   int px)
+__device__ __forceinline__ void pack_channel(const float *o, float b, int k, bool with_relu, float repS, float z, bool with_sum,
+                                             const unsigned *old, unsigned *pk)
 {
   static_assert(OUT == EHIP_U8 || OUT == EHIP_S8, "quantized output");
-  constexpr int AA = A * A, M = A - 2;
-  unsigned pk[M * M], old[M * M];
+  constexpr int M = A - 2;
 #pragma unroll
-  for (int e = 0; e < M * M; ++e) pk[e] = 0u;
-  if (with_sum) {
-#pragma unroll
-    for (int i = 0; i < M; ++i)
-#pragma unroll
-      for (int j = 0; j < M; ++j) {
-        const int oh = M * th + i, ow = M * tw + j;
-        const bool in = oh < oh_n && ow < ow_n;
-        const size_t cell = in ? ((size_t)oh * ow_n + ow) * px + 4 * q : 0;
-        old[M * i + j] = *reinterpret_cast<const unsigned *>(plane + cell);
-      }
-  }
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    float f[AA], o[M * M];
-#pragma unroll
-    for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
-    wino::tile_output<A>(f, o);
-    const float b = comp_of(bias, k);
-#pragma unroll
-    for (int e = 0; e < M * M; ++e) {
-      float r = o[e] + b;
-      r = __builtin_fmaf(r, repS, z);
-      if (with_sum) {
-        const unsigned ob = (old[e] >> (8 * k)) & 0xffu;
-        r = r + (OUT == EHIP_U8 ? (float)ob : (float)(int)(signed char)ob);
-      }
-      if (with_relu) {
-        r = __builtin_amdgcn_fmed3f(r, 0.0f, OUT == EHIP_S8 ? 127.0f : 255.0f);
-        if (A == 4) r = __builtin_floorf(r);
-        pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r, k, pk[e]);
-      } else if (A == 4) {
-        const float fl = __builtin_floorf(r);
-        if (OUT == EHIP_U8) pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r >= 0.0f ? fl : 300.0f, k, pk[e]);
-        else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(fl)) & 0xffu) << (8 * k);
-      } else {
-        if (OUT == EHIP_U8) pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r >= -0.5f ? r : 300.0f, k, pk[e]);
-        else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
-      }
+  for (int e = 0; e < M * M; ++e) {
+    float r = o[e] + b;
+    r = __builtin_fmaf(r, repS, z);
+    if (with_sum) {
+      const unsigned ob = (old[e] >> (8 * k)) & 0xffu;
+      r = r + (OUT == EHIP_U8 ? (float)ob : (float)(int)(signed char)ob);
     }
-    // (one channel after the other: interleaved, the four transforms' intermediates do not fit the registers)
-    __builtin_amdgcn_sched_barrier(0);
+    if (with_relu) {
+      r = __builtin_amdgcn_fmed3f(r, 0.0f, OUT == EHIP_S8 ? 127.0f : 255.0f);
+      if (A == 4) r = __builtin_floorf(r);
+      pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r, k, pk[e]);
+    } else if (A == 4) {
+      const float fl = __builtin_floorf(r);
+      if (OUT == EHIP_U8) pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r >= 0.0f ? fl : 300.0f, k, pk[e]);
+      else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(fl)) & 0xffu) << (8 * k);
+    } else {
+      if (OUT == EHIP_U8) pk[e] = __builtin_amdgcn_cvt_pk_u8_f32(r >= -0.5f ? r : 300.0f, k, pk[e]);
+      else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
+    }
   }
+}
+
+template <int A>
+__device__ __forceinline__ void store_packed(const unsigned *pk, uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, int px)
+{
+  constexpr int M = A - 2;
 #pragma unroll
   for (int i = 0; i < M; ++i) {
     const int oh = M * th + i;
@@ -83,6 +81,37 @@ __device__ __forceinline__ void output_tile_packed(const float4 *m, const float4
       *reinterpret_cast<unsigned *>(plane + ((size_t)oh * ow_n + ow) * px + 4 * q) = pk[M * i + j];
     }
   }
+}
+
+template <int OUT, int A>
+__device__ __forceinline__ void output_tile_packed(const float4 *m, const float4 &bias, bool with_relu, float repS, float z,
+                                                   uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, bool with_sum,
+                                                   int px)
+{
+  constexpr int AA = A * A, M = A - 2;
+  unsigned pk[M * M], old[M * M];
+#pragma unroll
+  for (int e = 0; e < M * M; ++e) pk[e] = 0u;
+  if (with_sum) load_old<A>(old, plane, q, th, tw, oh_n, ow_n, px);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float f[AA], o[M * M];
+#pragma unroll
+    for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
+    wino::tile_output<A>(f, o);
+    pack_channel<OUT, A>(o, comp_of(bias, k), k, with_relu, repS, z, with_sum, old, pk);
+    // (one channel after the other: interleaved, the four transforms' intermediates do not fit the registers)
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  store_packed<A>(pk, plane, q, th, tw, oh_n, ow_n, px);
+}
+
+// the one-dimensional output transform of tile sizes 6 and 5
+template <int A>
+__device__ __forceinline__ void out_1d(const float *f, float *o)
+{
+  if (A == 6) wino::out6_1d(f, o);
+  else wino::out5_1d(f, o);
 }
 
 }  // namespace
@@ -215,6 +244,246 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
                                    th, tw, a.oh, a.ow, SUM, px);
 }
 
+// The same lanes, weights resident: with at most 128 input channels the packed weights of 16 channels at every position
+// fit the LDS twice over (36 or 72 KB a workgroup), so a workgroup = 16 channels x 64 tiles stages them once and then
+// walks over blocks of 64 tiles: the operand stream from L2 is the transformed input alone (half of what the form
+// above requests per MFMA), every wave has tiles of its own (nothing is requested twice inside a workgroup), and the
+// ring of input operands runs on from one block of tiles to the next, so the first operands of the next block travel
+// while this one's output transform keeps the vector units busy.  No barrier after the staging.
+// a.nx = blocks of 64 tiles, a.ny = groups of 16 packed rows; grid = 8 XCDs x a.ny x slots, a slot walks over the
+// blocks slot * 8 + xcd, + 8 * slots, ...
+template <int A, bool SUM, int NKS>
+__global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoFusedArgs a)
+{
+  constexpr int AA = A * A, STEPS = AA * NKS;
+  constexpr int D = A == 6 ? (SUM ? 6 : 12) : (A == 5 ? 5 : 8);   // divides STEPS: a ring slot holds the same steps in every block
+  static_assert(STEPS % D == 0, "ring");
+  extern __shared__ float4 lds[];
+  v4i *wl = reinterpret_cast<v4i *>(lds);   // [STEPS][4 units][16 packed rows] cells of 16 bytes
+  float4 *cl = lds + STEPS * 64;            // [AA][3][4 quads of the workgroup's 16 rows]: scale, shift, compensation
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, g = lane >> 4;
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int by = seq % a.ny;
+  const int slot = seq / a.ny;
+  const int item_step = 8 * (int)(gridDim.x / (8u * a.ny));
+  int item = slot * 8 + xcd;
+  if (item >= a.nx) return;          // whole workgroup
+  // the workgroup's 16 channels are one block of the output: of the group of 32 packed rows (row 8 gq + 4 h + j holds
+  // channel 16 h + 4 gq + j) it takes the rows of half h, gathered so that MFMA row 4 gq + j is channel 16 h + 4 gq + j
+  // and the four lanes of a tile write the 16 bytes of a pixel's channel block together
+  const int oc0 = (by >> 1) * 32, h = by & 1;
+  const int oc_real = a.oc2 * 16;
+  const int nblk = (a.t + 31) >> 5;
+
+  const long long t_pos = (long long)a.ic2 * 512;
+  const long long t_blk = t_pos * AA;
+  unsigned b_off[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    // units past the last real one multiply zero weights: any valid cell will do
+    int u = 4 * ks + g;
+    u = u < a.ic2 ? u : a.ic2 - 1;
+    b_off[ks] = (unsigned)(u * 512 + ((wave & 1) * 16 + l16) * 16);
+  }
+  // the wave's block of 32 tiles inside the item (the last item of an odd count has one block only: its upper waves
+  // read the lower block again and store nothing)
+  auto base_of = [&](int it) {
+    int blk = 2 * it + (wave >> 1);
+    blk = blk < nblk ? blk : nblk - 1;
+    return a.tin + blk * t_blk;      // wave-uniform
+  };
+  v4i rb[D];
+  // step sn = (column i, row r, k-step ks) in that order; its position is A r + i (tile size 4: one group, in order)
+  auto issue = [&](int rs, int sn, const uint8_t *tb) {
+    const int ks = sn % NKS, pr = sn / NKS;
+    const int p = A == 4 ? pr : A * (pr % A) + pr / A;
+    rb[rs] = *reinterpret_cast<const v4i *>(tb + p * t_pos + b_off[ks]);
+  };
+  const uint8_t *tb = base_of(item);
+#pragma unroll
+  for (int k = 0; k < D; ++k) issue(k, k, tb);
+  {
+    // the weights: per (step, unit) 16 rows x 16 bytes = 256 contiguous bytes of [pos][unit][OCpp][16]
+    constexpr int NP = (STEPS * 64 + kBlock - 1) / kBlock;
+    const long long w_pos = (long long)a.units_pad * a.ocpp * 16;
+    v4i tmp[NP];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      int idx = tid + j * kBlock;
+      idx = idx < STEPS * 64 ? idx : STEPS * 64 - 1;
+      const int chunk = idx >> 4, cell = idx & 15;
+      const int sn = chunk >> 2, u = chunk & 3;
+      const int p = sn / NKS, ks = sn - NKS * p;
+      tmp[j] = *reinterpret_cast<const v4i *>(a.w + p * w_pos +
+                                              ((long long)(4 * ks + u) * a.ocpp + oc0 + 8 * (cell >> 2) + 4 * h + (cell & 3)) * 16);
+    }
+    constexpr int NC = (AA * 12 + kBlock - 1) / kBlock;
+    float4 cst[NC];
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      int idx = tid + j * kBlock;
+      idx = idx < AA * 12 ? idx : AA * 12 - 1;
+      const int p = idx / 12, rem = idx - 12 * p, arr = rem >> 2, gq = rem & 3;
+      const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
+      cst[j] = *reinterpret_cast<const float4 *>(src + (long long)p * a.ocpp + oc0 + 16 * h + 4 * gq);
+    }
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      const int idx = tid + j * kBlock;
+      if (idx < STEPS * 64) wl[idx] = tmp[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      const int idx = tid + j * kBlock;
+      if (idx < AA * 12) cl[idx] = cst[j];
+    }
+  }
+  const int oc = oc0 + 16 * h + 4 * g;   // the lane's four channels
+  const bool oc_ok = oc < oc_real;
+  float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (a.with_bias && oc_ok) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
+  const int px = a.out_nhwc ? a.oc2 * 16 : 16;
+  const int q = (oc >> 2) & 3;
+  __syncthreads();   // weights and constants are in LDS; the waves run on their own from here
+  // the lane's cells as opaque bases: every read below is base + immediate offset (left to itself the compiler folds
+  // the constants' place behind the weights into each address, beyond the offset field, one register per cell)
+  int wla = g * 16 + l16, clg = STEPS * 64 + g;   // cells of 16 bytes from the start of the LDS
+  asm volatile("" : "+v"(wla), "+v"(clg));
+  // Tile sizes 6 and 5: Y = At M A one dimension at a time.  The steps run column by column of M (positions A r + i,
+  // r = 0 .. A - 1): a column's A positions are multiplied, requantized and taken through the first one-dimensional
+  // transform at once, which leaves (A - 2) values per column and channel -- so a lane keeps 4 x (A - 2) x A floats and
+  // one column of accumulators instead of all A x A positions, and the vector work of one column runs while the
+  // operands of the next ones travel.  Tile size 4 (a two-dimensional formula in the reference) keeps its 16 positions.
+  constexpr int M = A - 2;
+  constexpr int NCOL = A == 4 ? 1 : A;      // groups of positions that are finished together
+  constexpr int PER = AA / NCOL;            // positions per group
+  // the weights of step sn: cell offset of its (position, k-step)
+  auto wcell = [](int sn) {
+    const int ks = sn % NKS, pr = sn / NKS;
+    const int p = A == 4 ? pr : A * (pr % A) + pr / A;
+    return (p * NKS + ks) * 64;
+  };
+  for (;;) {
+    const int next = item + item_step;
+    const bool more = next < a.nx;                      // wave-uniform
+    const uint8_t *tbn = base_of(more ? next : item);   // (the last block's tail requests its own head again: unused)
+    const int t = item * 64 + wave * 16 + l16;
+    const bool valid = t < a.t && oc_ok;
+    // (lanes without a tile or channel of their own take part with tile 0 / channel 0 and store nothing)
+    const int tc = valid ? t : 0, occ = valid ? oc : 0;
+    const int n = tc / a.nt;
+    const int rem = tc - n * a.nt;
+    const int th = rem / a.wt;
+    const int tw = rem - th * a.wt;
+    uint8_t *plane = static_cast<uint8_t *>(a.out) +
+        (a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (occ >> 4) * 16 : ((size_t)n * a.oc2 + (occ >> 4)) * a.oh * a.ow * 16);
+    float T[4][M][A == 4 ? 1 : A];   // first-stage results [channel][row][column]
+    float4 m4[A == 4 ? AA : 1];      // tile size 4: the requantized positions
+    unsigned old[M * M];
+    v4i ra[3];
+    ra[0] = wl[wla + wcell(0)];
+    ra[1] = wl[wla + wcell(1)];
+#pragma unroll
+    for (int i = 0; i < NCOL; ++i) {
+      if (SUM && i == NCOL - 1) load_old<A>(old, plane, q, th, tw, a.oh, a.ow, px);
+      // the accumulators start from the compensation 128 * sum(weights) of their (position, channel)
+      v4i acc[PER];
+#pragma unroll
+      for (int r = 0; r < PER; ++r) {
+        const int p = NCOL == 1 ? r : A * r + i;
+        const float4 cf = lds[clg + p * 12 + 8];
+        acc[r] = v4i{__float_as_int(cf.x), __float_as_int(cf.y), __float_as_int(cf.z), __float_as_int(cf.w)};
+      }
+#pragma unroll
+      for (int r = 0; r < PER; ++r)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          const int sn = (i * PER + r) * NKS + ks;
+          if (sn + 2 < STEPS) ra[(sn + 2) % 3] = wl[wla + wcell(sn + 2)];   // the weights of the step after next
+          const v4i b = rb[sn % D] ^ (int)0x80808080;
+          acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ra[sn % 3], b, acc[r], 0, 0, 0);
+          if (sn + D < STEPS) issue(sn % D, sn + D, tb);
+          else issue(sn % D, sn + D - STEPS, tbn);
+          __builtin_amdgcn_sched_barrier(0);   // (the loads stay where the ring puts them: hoisted, they spill)
+        }
+      float4 mc[PER];
+#pragma unroll
+      for (int r = 0; r < PER; ++r) {
+        const int p = NCOL == 1 ? r : A * r + i;
+        const float4 sc = lds[clg + p * 12], sh = lds[clg + p * 12 + 4];
+        mc[r].x = __builtin_fmaf((float)acc[r][0], sc.x, sh.x);
+        mc[r].y = __builtin_fmaf((float)acc[r][1], sc.y, sh.y);
+        mc[r].z = __builtin_fmaf((float)acc[r][2], sc.z, sh.z);
+        mc[r].w = __builtin_fmaf((float)acc[r][3], sc.w, sh.w);
+        // (pinned where it is computed: the compiler would read every constant first)
+        asm volatile("" : "+v"(mc[r].x), "+v"(mc[r].y), "+v"(mc[r].z), "+v"(mc[r].w));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (NCOL == 1) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) m4[NCOL == 1 ? r : 0] = mc[r];
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float f[PER], o[M];
+#pragma unroll
+          for (int r = 0; r < PER; ++r) f[r] = comp_of(mc[r], k);
+          out_1d<A>(f, o);
+#pragma unroll
+          for (int r = 0; r < M; ++r) {
+            // (pinned: left to the compiler the transform moves to the end and the requantized column stays live)
+            asm volatile("" : "+v"(o[r]));
+            T[k][r][NCOL == 1 ? 0 : i] = o[r];
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    unsigned pk[M * M];
+#pragma unroll
+    for (int e = 0; e < M * M; ++e) pk[e] = 0u;
+    // second dimension, output scale, rounding and packing, one channel after the other (interleaved, the four
+    // transforms' intermediates do not fit the registers); output type and ReLU are chosen once per block of tiles
+    auto finish = [&](auto out_c, auto relu_c) {
+      constexpr int OUT = decltype(out_c)::value;
+      constexpr bool RELU = decltype(relu_c)::value;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float y[M * M];
+        if (NCOL == 1) {
+          float f[AA];
+#pragma unroll
+          for (int e = 0; e < AA; ++e) f[e] = comp_of(m4[NCOL == 1 ? e : 0], k);
+          wino::tile_output<A>(f, y);
+        } else {
+#pragma unroll
+          for (int r = 0; r < M; ++r) out_1d<A>(T[k][r], &y[M * r]);
+        }
+        pack_channel<OUT, A>(y, comp_of(bias, k), k, RELU, a.out_repS, a.out_z, SUM, old, pk);
+#pragma unroll
+        for (int e = 0; e < M * M; ++e) asm volatile("" : "+v"(pk[e]));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    using U8C = std::integral_constant<int, EHIP_U8>;
+    using S8C = std::integral_constant<int, EHIP_S8>;
+    if (a.out_type == EHIP_U8) {
+      if (a.with_relu) finish(U8C{}, std::true_type{});
+      else finish(U8C{}, std::false_type{});
+    } else {
+      if (a.with_relu) finish(S8C{}, std::true_type{});
+      else finish(S8C{}, std::false_type{});
+    }
+    if (valid) store_packed<A>(pk, plane, q, th, tw, a.oh, a.ow, px);
+    if (!more) break;
+    item = next;
+    tb = tbn;
+  }
+}
+
 bool wino_lanes_applies(const WinoFusedArgs &a)
 {
   const char *env = getenv("EHIP_WINO_LANES");
@@ -231,9 +500,31 @@ hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a0, hipStream_t s,
   WinoFusedArgs a = a0;
   const int A = a.tile ? a.tile : 6, AA = A * A;
   const int nks64 = (a.ic2 + 3) / 4;
+  void (*kernel)(WinoFusedArgs) = nullptr;
+  const char *env = getenv("EHIP_WINO_LANES_WRES");
+  if (nks64 <= 2 && !(env && env[0] == '0')) {
+    // weights resident: blocks of 64 tiles, groups of 16 packed rows, two workgroups per CU walking over the blocks
+    a.nx = (a.t + 63) / 64;
+    a.ny = 2 * ((a.oc2 * 16 + 31) / 32);
+    int slots = 64 / a.ny;   // 8 XCDs x ny x slots ~ 512 workgroups
+    if (const char *sl = getenv("EHIP_WINO_LANES_SLOTS")) slots = atoi(sl);   // (fewer: more blocks of tiles per workgroup)
+    slots = slots < 1 ? 1 : slots;
+    const int need = (a.nx + 7) / 8;
+    slots = slots < need ? slots : need;
+#define EHIP_WLR(AV)                                                                                                   \
+  kernel = a.with_sum ? (nks64 == 1 ? k_wino_gemm_output_lanes_wres<AV, true, 1> : k_wino_gemm_output_lanes_wres<AV, true, 2>) \
+                      : (nks64 == 1 ? k_wino_gemm_output_lanes_wres<AV, false, 1> : k_wino_gemm_output_lanes_wres<AV, false, 2>)
+    if (A == 4) EHIP_WLR(4);
+    else if (A == 5) EHIP_WLR(5);
+    else EHIP_WLR(6);
+#undef EHIP_WLR
+    const size_t lds = (size_t)AA * nks64 * 1024 + (size_t)AA * 12 * sizeof(float4);
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    return plan_launch(plan, kernel, dim3(8 * a.ny * slots), dim3(kBlock), lds, a, s);
+  }
   a.nx = (a.t + 31) / 32;
   a.ny = (a.oc2 * 16 + 31) / 32;
-  void (*kernel)(WinoFusedArgs) = nullptr;
 #define EHIP_WL(AV)                                                                                                    \
   kernel = a.with_sum ? (nks64 == 1 ? k_wino_gemm_output_lanes<AV, true, 1>                                             \
                                     : (nks64 == 2 ? k_wino_gemm_output_lanes<AV, true, 2> : k_wino_gemm_output_lanes<AV, true, 4>)) \

@@ -166,6 +166,43 @@ def test_wino_fused_lanes_form(lanes, tile, out_type, n, ic, oc, hw, with_relu, 
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
+@pytest.mark.parametrize("slots", ["1", ""])
+@pytest.mark.parametrize("wres", ["1", "0"])
+@pytest.mark.parametrize("tile", [6, 5, 4])
+@pytest.mark.parametrize("out_type,with_sum", [(ol.U8, 0), (ol.S8, 1), (ol.U8, 1)])
+@pytest.mark.parametrize("n,ic,oc,hw,with_relu", [(5, 64, 48, 64, True), (1, 128, 32, 36, False), (2, 48, 16, 40, True),
+                                                  (3, 128, 80, 30, True)])
+def test_wino_fused_lanes_weights_resident(slots, wres, tile, out_type, with_sum, n, ic, oc, hw, with_relu, monkeypatch):
+    """at most 128 input channels with u8 / s8 output: workgroups that keep the weights of 16 channels in LDS and walk
+    over blocks of 64 tiles, the operand ring running on from one block into the next (one workgroup per XCD and
+    channel block, so that every workgroup takes several blocks, and the default grid); an odd number of blocks of 32
+    tiles, channels and tiles that leave lanes unused, the in-place sum; and the form that streams both operands"""
+    import torch
+    monkeypatch.setenv("EHIP_WINO_LANES_WRES", wres)
+    if slots:
+        monkeypatch.setenv("EHIP_WINO_LANES_SLOTS", slots)
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=57 + tile + ic + out_type, out_type=out_type, tile=tile,
+                                         with_relu=with_relu, out_z=0.0 if out_type == ol.S8 else 1.6)
+    p.with_sum = with_sum
+    d.with_ip_sum = with_sum
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    rng = np.random.default_rng(91 + tile + hw)
+    shape = (n, ol.up16(oc) // 16, hw, hw, 16)
+    old = rng.integers(-30 if out_type == ol.S8 else 0, 60, shape).astype(ol.NP_OF[out_type])
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xq.astype(f32)), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias, out_init=old if with_sum else None)
+    conv = E.Conv(d)
+    d_out = dev(old)
+    d_b = dev(bias)
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, dev(xq), None, d_b)
+    torch.cuda.synchronize()
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
 def _fused(n, ic, oc, hw):
     import torch
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
