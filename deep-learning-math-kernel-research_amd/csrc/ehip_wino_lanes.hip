@@ -106,6 +106,60 @@ __device__ __forceinline__ void output_tile_packed(const float4 *m, const float4
   store_packed<A>(pk, plane, q, th, tw, oh_n, ow_n, px);
 }
 
+// 4 x 4 transpose of dwords between four registers and the four 16-lane rows of a wave: register j of row g becomes
+// register g of row j (v_permlane32_swap exchanges the upper rows of one register with the lower rows of another,
+// v_permlane16_swap the odd rows with the even ones).  All lanes take part.
+__device__ __forceinline__ void rows_transpose(unsigned &x0, unsigned &x1, unsigned &x2, unsigned &x3)
+{
+  auto a = __builtin_amdgcn_permlane32_swap(x0, x2, false, false);
+  auto b = __builtin_amdgcn_permlane32_swap(x1, x3, false, false);
+  auto c = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+  auto d = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+  x0 = c[0];
+  x1 = c[1];
+  x2 = d[0];
+  x3 = d[1];
+}
+
+// Output by whole cells of 16 channels: the four lanes of a tile (rows g = 0 .. 3 of the wave, four channels each) hold
+// the 16 bytes of every pixel between them; after the transpose the lane of row g holds the whole cell of the pixel in
+// column g of the tile's row i and writes it with one 16-byte store (a wave then covers 16 tiles x 4 pixels of an
+// image row = up to 1 KB in one piece, where dword stores leave 16 pieces of 16 bytes per instruction).
+// block: the tile's image and channel block; ok: the tile exists.  Called by all lanes.
+template <int A>
+__device__ __forceinline__ void store_cells(const unsigned *pk, uint8_t *block, int g, bool ok, int th, int tw, int oh_n, int ow_n,
+                                            int px)
+{
+  constexpr int M = A - 2;
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    unsigned c0 = pk[M * i], c1 = pk[M * i + 1], c2 = M > 2 ? pk[M * i + (M > 2 ? 2 : 0)] : 0u, c3 = M > 3 ? pk[M * i + (M > 3 ? 3 : 0)] : 0u;
+    rows_transpose(c0, c1, c2, c3);
+    const int oh = M * th + i, ow = M * tw + g;
+    if (ok && g < M && oh < oh_n && ow < ow_n)
+      *reinterpret_cast<uint4 *>(block + ((size_t)oh * ow_n + ow) * px) = make_uint4(c0, c1, c2, c3);
+  }
+}
+
+// the old output of the in-place sum the same way round: cells in, the lane's four channels of every pixel out
+template <int A>
+__device__ __forceinline__ void load_old_cells(unsigned *old, const uint8_t *block, int g, int th, int tw, int oh_n, int ow_n, int px)
+{
+  constexpr int M = A - 2;
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    const int oh = M * th + i, ow = M * tw + g;
+    const bool in = g < M && oh < oh_n && ow < ow_n;
+    const uint4 c = *reinterpret_cast<const uint4 *>(block + (in ? ((size_t)oh * ow_n + ow) * px : 0));
+    unsigned c0 = c.x, c1 = c.y, c2 = c.z, c3 = c.w;
+    rows_transpose(c0, c1, c2, c3);
+    old[M * i] = c0;
+    old[M * i + 1] = c1;
+    if (M > 2) old[M * i + (M > 2 ? 2 : 0)] = c2;
+    if (M > 3) old[M * i + (M > 3 ? 3 : 0)] = c3;
+  }
+}
+
 // the one-dimensional output transform of tile sizes 6 and 5
 template <int A>
 __device__ __forceinline__ void out_1d(const float *f, float *o)
@@ -346,7 +400,6 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
   float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
   if (a.with_bias && oc_ok) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
   const int px = a.out_nhwc ? a.oc2 * 16 : 16;
-  const int q = (oc >> 2) & 3;
   __syncthreads();   // weights and constants are in LDS; the waves run on their own from here
   // the lane's cells as opaque bases: every read below is base + immediate offset (left to itself the compiler folds
   // the constants' place behind the weights into each address, beyond the offset field, one register per cell)
@@ -388,7 +441,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
     ra[1] = wl[wla + wcell(1)];
 #pragma unroll
     for (int i = 0; i < NCOL; ++i) {
-      if (SUM && i == NCOL - 1) load_old<A>(old, plane, q, th, tw, a.oh, a.ow, px);
+      if (SUM && i == NCOL - 1) load_old_cells<A>(old, plane, g, th, tw, a.oh, a.ow, px);
       // the accumulators start from the compensation 128 * sum(weights) of their (position, channel)
       v4i acc[PER];
 #pragma unroll
@@ -477,7 +530,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
       if (a.with_relu) finish(S8C{}, std::true_type{});
       else finish(S8C{}, std::false_type{});
     }
-    if (valid) store_packed<A>(pk, plane, q, th, tw, a.oh, a.ow, px);
+    store_cells<A>(pk, plane, g, valid, th, tw, a.oh, a.ow, px);
     if (!more) break;
     item = next;
     tb = tbn;
