@@ -21,21 +21,6 @@ __device__ __forceinline__ float comp_of(const float4 &v, int k) { return k == 0
 // The pieces of output_tile for u8 / s8 output with few registers: one channel at a time, its bytes packed into the
 // pixels' dwords as they come (16 dwords live instead of 4 x 16 floats; the old output of the in-place sum stays packed
 // as well).  Same operations in the same order per value as output_tile.
-template <int A>
-__device__ __forceinline__ void load_old(unsigned *old, const uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, int px)
-{
-  constexpr int M = A - 2;
-#pragma unroll
-  for (int i = 0; i < M; ++i)
-#pragma unroll
-    for (int j = 0; j < M; ++j) {
-      const int oh = M * th + i, ow = M * tw + j;
-      const bool in = oh < oh_n && ow < ow_n;
-      const size_t cell = in ? ((size_t)oh * ow_n + ow) * px + 4 * q : 0;
-      old[M * i + j] = *reinterpret_cast<const unsigned *>(plane + cell);
-    }
-}
-
 // channel k of the lane's four: bias, output scale, old output, ReLU, rounding, byte k of the pixels' dwords
 template <int OUT, int A>
 __device__ __forceinline__ void pack_channel(const float *o, float b, int k, bool with_relu, float repS, float z, bool with_sum,
@@ -64,46 +49,6 @@ __device__ __forceinline__ void pack_channel(const float *o, float b, int k, boo
       else pk[e] |= ((unsigned)ssat8(cvt_s32_rne(r)) & 0xffu) << (8 * k);
     }
   }
-}
-
-template <int A>
-__device__ __forceinline__ void store_packed(const unsigned *pk, uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, int px)
-{
-  constexpr int M = A - 2;
-#pragma unroll
-  for (int i = 0; i < M; ++i) {
-    const int oh = M * th + i;
-    if (oh >= oh_n) break;
-#pragma unroll
-    for (int j = 0; j < M; ++j) {
-      const int ow = M * tw + j;
-      if (ow >= ow_n) break;
-      *reinterpret_cast<unsigned *>(plane + ((size_t)oh * ow_n + ow) * px + 4 * q) = pk[M * i + j];
-    }
-  }
-}
-
-template <int OUT, int A>
-__device__ __forceinline__ void output_tile_packed(const float4 *m, const float4 &bias, bool with_relu, float repS, float z,
-                                                   uint8_t *plane, int q, int th, int tw, int oh_n, int ow_n, bool with_sum,
-                                                   int px)
-{
-  constexpr int AA = A * A, M = A - 2;
-  unsigned pk[M * M], old[M * M];
-#pragma unroll
-  for (int e = 0; e < M * M; ++e) pk[e] = 0u;
-  if (with_sum) load_old<A>(old, plane, q, th, tw, oh_n, ow_n, px);
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    float f[AA], o[M * M];
-#pragma unroll
-    for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
-    wino::tile_output<A>(f, o);
-    pack_channel<OUT, A>(o, comp_of(bias, k), k, with_relu, repS, z, with_sum, old, pk);
-    // (one channel after the other: interleaved, the four transforms' intermediates do not fit the registers)
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  store_packed<A>(pk, plane, q, th, tw, oh_n, ow_n, px);
 }
 
 // 4 x 4 transpose of dwords between four registers and the four 16-lane rows of a wave: register j of row g becomes
@@ -160,6 +105,31 @@ __device__ __forceinline__ void load_old_cells(unsigned *old, const uint8_t *blo
   }
 }
 
+// All positions of the lane's tile x four channels -> the output: Y = At M A channel by channel, packed, and written by
+// whole cells.  Called by all lanes of the wave (ok: the lane's tile and channels exist).
+template <int OUT, int A>
+__device__ __forceinline__ void output_tile_packed(const float4 *m, const float4 &bias, bool with_relu, float repS, float z,
+                                                   uint8_t *block, int g, bool ok, int th, int tw, int oh_n, int ow_n,
+                                                   bool with_sum, int px)
+{
+  constexpr int AA = A * A, M = A - 2;
+  unsigned pk[M * M], old[M * M];
+#pragma unroll
+  for (int e = 0; e < M * M; ++e) pk[e] = 0u;
+  if (with_sum) load_old_cells<A>(old, block, g, th, tw, oh_n, ow_n, px);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float f[AA], o[M * M];
+#pragma unroll
+    for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
+    wino::tile_output<A>(f, o);
+    pack_channel<OUT, A>(o, comp_of(bias, k), k, with_relu, repS, z, with_sum, old, pk);
+    // (one channel after the other: interleaved, the four transforms' intermediates do not fit the registers)
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  store_cells<A>(pk, block, g, ok, th, tw, oh_n, ow_n, px);
+}
+
 // the one-dimensional output transform of tile sizes 6 and 5
 template <int A>
 __device__ __forceinline__ void out_1d(const float *f, float *o)
@@ -195,13 +165,15 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
   const int bx = (seq / a.ny) * 8 + xcd;
   if (bx >= a.nx) return;          // whole workgroup
   const int oc0 = by * 32;
-  const int r0 = (wave & 1) * 16;          // the wave's packed rows inside the group of 32
+  // the wave's 16 channels are one block of the output: of the group of 32 packed rows (row 8 gq + 4 h + j holds
+  // channel 16 h + 4 gq + j) it takes the rows of half h, gathered so that MFMA row 4 gq + j is channel 16 h + 4 gq + j
+  const int h = wave & 1;
   const int th16 = (wave >> 1) * 16;       // its tiles inside the block of 32
   const int oc_real = a.oc2 * 16;
 
   // operands: lane = packed row / tile l16 of unit 4 ks + g, one 16-byte cell each; a wave-uniform base per step plus
   // one 32-bit offset per lane (as 64-bit pointers per lane the unrolled loop's 72 addresses fill the register file)
-  const unsigned a_off = (unsigned)(g * a.ocpp + oc0 + r0 + l16) * 16u;
+  const unsigned a_off = (unsigned)(g * a.ocpp + oc0 + 8 * (l16 >> 2) + 4 * h + (l16 & 3)) * 16u;
   const long long w_pos = (long long)a.units_pad * a.ocpp * 16, w_ks = (long long)4 * a.ocpp * 16;
   const uint8_t *tbase = a.tin + (long long)bx * AA * a.ic2 * 512;
   const long long t_pos = (long long)a.ic2 * 512;
@@ -244,8 +216,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
     }
   }
   __syncthreads();   // the constants are in LDS
-  // the lane's channels: packed rows r0 + 4 g .. + 3 of the group hold channels 16 (g & 1) + 4 (r0 / 8 + g / 2) + j
-  const int quad = 4 * (g & 1) + (r0 >> 3) + (g >> 1);   // cell of four channels inside the group of 32
+  const int quad = 4 * h + g;   // the lane's four channels: cell inside the group of 32
   // the accumulators start from the compensation 128 * sum(weights) of their (position, channel)
   v4i acc[AA];
 #pragma unroll
@@ -262,7 +233,8 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
   }
   const int oc = oc0 + 4 * quad;
   const int t = bx * 32 + th16 + l16;
-  if (t >= a.t || oc >= oc_real) return;
+  // (lanes without a tile or channel of their own take part with tile 0 / channel 0 and store nothing)
+  const bool valid = t < a.t && oc < oc_real;
   float4 m[AA];
   int cq = quad;   // (the constants' cell, re-derived group by group: see below)
 #pragma unroll
@@ -278,24 +250,24 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
     asm volatile("" : "+v"(m[e].x), "+v"(m[e].y), "+v"(m[e].z), "+v"(m[e].w));
     if ((e & 3) == 3) asm volatile("" : "+v"(cq) : "v"(m[e].w));
   }
-  const int n = t / a.nt;
-  const int rem = t - n * a.nt;
+  const int tc = valid ? t : 0, occ = valid ? oc : 0;
+  const int n = tc / a.nt;
+  const int rem = tc - n * a.nt;
   const int th = rem / a.wt;
   const int tw = rem - th * a.wt;
   float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
-  const size_t plane = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (oc >> 4) * 16
-                                  : ((size_t)n * a.oc2 + (oc >> 4)) * a.oh * a.ow * 16;
+  if (a.with_bias) bias = *reinterpret_cast<const float4 *>(a.bias + occ);
+  const size_t block = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (occ >> 4) * 16
+                                  : ((size_t)n * a.oc2 + (occ >> 4)) * a.oh * a.ow * 16;
   const int px = a.out_nhwc ? a.oc2 * 16 : 16;
-  const int q = (oc >> 2) & 3;
   // (u8 / s8 output only: the launcher keeps f32 output, whose four channels of a pixel leave as one 16-byte store
   // and would need all of them in registers at once, on the general form)
   if (a.out_type == EHIP_U8)
-    output_tile_packed<EHIP_U8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + plane, q,
-                                   th, tw, a.oh, a.ow, SUM, px);
+    output_tile_packed<EHIP_U8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + block, g,
+                                   valid, th, tw, a.oh, a.ow, SUM, px);
   else
-    output_tile_packed<EHIP_S8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + plane, q,
-                                   th, tw, a.oh, a.ow, SUM, px);
+    output_tile_packed<EHIP_S8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + block, g,
+                                   valid, th, tw, a.oh, a.ow, SUM, px);
 }
 
 // The same lanes, weights resident: with at most 128 input channels the packed weights of 16 channels at every position
