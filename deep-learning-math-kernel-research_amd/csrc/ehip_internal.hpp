@@ -114,7 +114,7 @@ struct WinoArgs {
   int n, ic2, oc2, ih, iw, oh, ow, ht, wt, nt, t, pad_t, pad_l;
   int tile;             // tile size A: 6 (or 0) = F(4x4,3x3), 4 = F(2x2,3x3), 5 = F(3x3,3x3); 36 below reads A * A
   int nblocks, items_per_xcd;   // set by the input-transform launcher: blocks of 64 tiles; ceil(blocks x units / 8)
-  int buf_gather;       // set by the input-transform launcher: the input is below 4 GB, gather with buffer loads
+  int buf_gather;       // set by the input-transform launcher: the input is below 4 GB, gather with buffer loads (2: u8 input by whole cells)
   float mrepS, mz;      // input_S / tinput_S, ceil(tinput_z)
   int with_bias, with_relu;
   int with_sum;         // in-place sum: the old output is added before the ReLU (stand-alone output transform only)

@@ -59,11 +59,36 @@ __device__ __forceinline__ void buffer_load_cell(BufferRsrc r, unsigned off, uns
 {
   v = __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
 }
+__device__ __forceinline__ void buffer_load_cell(BufferRsrc r, unsigned off, uint4 &v)
+{
+  typedef unsigned v4u __attribute__((ext_vector_type(4)));
+  const v4u x = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
+  v = make_uint4(x.x, x.y, x.z, x.w);
+}
+// 4 x 4 transpose of dwords between four registers and the four lanes of a quad (lanes 4 n .. 4 n + 3): register j of
+// lane q becomes register q of lane j.  Two exchanges, with the neighbour (lane ^ 1) and across (lane ^ 2); in each a lane
+// sends the register its partner lacks and takes the partner's in its place.
+__device__ __forceinline__ void quad_transpose(unsigned &x0, unsigned &x1, unsigned &x2, unsigned &x3, int lane)
+{
+  const bool odd = (lane & 1) != 0, hi = (lane & 2) != 0;
+  {
+    const unsigned r01 = __builtin_amdgcn_mov_dpp(odd ? x0 : x1, 0xB1, 0xf, 0xf, true);   // quad_perm [1, 0, 3, 2]
+    const unsigned r23 = __builtin_amdgcn_mov_dpp(odd ? x2 : x3, 0xB1, 0xf, 0xf, true);
+    if (odd) { x0 = r01; x2 = r23; } else { x1 = r01; x3 = r23; }
+  }
+  {
+    const unsigned r02 = __builtin_amdgcn_mov_dpp(hi ? x0 : x2, 0x4E, 0xf, 0xf, true);    // quad_perm [2, 3, 0, 1]
+    const unsigned r13 = __builtin_amdgcn_mov_dpp(hi ? x1 : x3, 0x4E, 0xf, 0xf, true);
+    if (hi) { x0 = r02; x1 = r13; } else { x2 = r02; x3 = r13; }
+  }
+}
 #else
 typedef int BufferRsrc;
 __device__ inline BufferRsrc make_rsrc(const void *, unsigned) { return 0; }
 __device__ inline void buffer_load_cell(BufferRsrc, unsigned, float4 &v) { v = float4(); }
 __device__ inline void buffer_load_cell(BufferRsrc, unsigned, unsigned &v) { v = 0u; }
+__device__ inline void buffer_load_cell(BufferRsrc, unsigned, uint4 &v) { v = uint4(); }
+__device__ inline void quad_transpose(unsigned &, unsigned &, unsigned &, unsigned &, int) {}
 #endif
 
 __device__ __forceinline__ float comp_of(const float4 &v, int k)
@@ -165,6 +190,45 @@ __device__ __forceinline__ void gather_tile_buf(const WinoArgs &a, const TileCoo
     }
 }
 
+// u8 input below 4 GB, by whole cells: the four lanes of a tile (one channel quad each) share the tile's pixels out
+// between them -- lane q loads the 16 bytes (all four quads) of pixels q, 4 + q, 8 + q, ... -- and a transpose inside
+// the quad hands every lane its own quad of four pixels at a time.  A wave's load then covers 16 tiles x four
+// neighbouring pixels = up to 1 KB in lane order, a quarter of the load instructions and of the cache lines looked up
+// per byte (one dword per lane and pixel looks up a 64-byte line for 16 bytes).  Cells of the zero frame are sent
+// to an offset outside the buffer, as in gather_tile_buf.
+template <int A>
+__device__ __forceinline__ void gather_tile_wide(const WinoArgs &a, const TileCoord &c, int c2, int q, unsigned *d)
+{
+  constexpr int AA = A * A;
+  const unsigned pc = a.in_nhwc ? (unsigned)a.ic2 : 1u;   // cells between neighbouring pixels
+  const unsigned cells = (unsigned)a.n * a.ic2 * a.ih * a.iw;
+  const BufferRsrc rin = make_rsrc(a.in, cells * 16u);
+  const unsigned plane = a.in_nhwc ? (unsigned)c.n * a.ih * a.iw * pc + c2 : ((unsigned)c.n * a.ic2 + c2) * a.ih * a.iw;
+  constexpr int NK = (AA + 3) / 4;
+  uint4 v[NK];
+  // every load first (offsets without a branch), then the exchanges
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    const int e = 4 * k + q;       // the lane's pixel of this group
+    const int i = e / A, j = e - A * i;
+    const int h = c.h0 + i, w = c.w0 + j;
+    const bool ok = e < AA && (unsigned)h < (unsigned)a.ih && (unsigned)w < (unsigned)a.iw;
+    const unsigned off = (plane + (unsigned)(h * a.iw + w) * pc) * 16u;
+    buffer_load_cell(rin, ok ? off : 0xffffff00u, v[k]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    quad_transpose(v[k].x, v[k].y, v[k].z, v[k].w, q);
+    d[4 * k] = v[k].x;
+    if (4 * k + 1 < AA) d[4 * k + 1 < AA ? 4 * k + 1 : 0] = v[k].y;
+    if (4 * k + 2 < AA) d[4 * k + 2 < AA ? 4 * k + 2 : 0] = v[k].z;
+    if (4 * k + 3 < AA) d[4 * k + 3 < AA ? 4 * k + 3 : 0] = v[k].w;
+  }
+}
+template <int A>
+__device__ __forceinline__ void gather_tile_wide(const WinoArgs &, const TileCoord &, int, int, float4 *) {}   // (u8 input only)
+
 }  // namespace
 
 // block: 64 consecutive tiles x 4 channel quads of one 16-channel unit.  Work items are numbered tile
@@ -178,6 +242,7 @@ template <typename Cell, int A = 6>
 __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
 {
   constexpr int AA = A * A;
+  constexpr bool kCodes = sizeof(Cell) == sizeof(unsigned);
   const int q = threadIdx.x & 3;
   const int item = (blockIdx.x & 7) * a.items_per_xcd + (blockIdx.x >> 3);
   if (item >= a.nblocks * a.ic2) return;   // whole workgroup
@@ -188,7 +253,8 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   if (t >= a.t) return;
   const TileCoord c = tile_coord<A>(a, t);
   Cell d[AA];
-  if (a.buf_gather) gather_tile_buf<A>(a, c, c2, q, d);
+  if (kCodes && a.buf_gather == 2) gather_tile_wide<A>(a, c, c2, q, d);
+  else if (a.buf_gather) gather_tile_buf<A>(a, c, c2, q, d);
   else gather_tile<A>(a, c, c2, q, d);
   unsigned packed[AA];
   // mixed: the wave holds interior and rim tiles -- the per-lane, branch-free form of the transform.
@@ -201,7 +267,6 @@ __global__ __launch_bounds__(kBlock) void k_wino_trans_input_u8(WinoArgs a)
   // u8 user input: the codes are finite, so with finite quantization constants no NaN can arise and ONE running
   // float minimum (an instruction per two values) says whether anything fell below -0.5; constants that are not
   // finite send every wave to the exact form.
-  constexpr bool kCodes = sizeof(Cell) == sizeof(unsigned);
   const bool odd_consts = !(__builtin_fabsf(a.mrepS) <= 3.402823466e38f) || !(__builtin_fabsf(a.mz) <= 3.402823466e38f);
   auto channels = [&](bool mixed, bool watch) {
     unsigned seen_u = 0u;
@@ -740,6 +805,8 @@ hipError_t launch_wino_trans_input(const WinoArgs &a0, hipStream_t s, LaunchPlan
     const unsigned long long bytes = (unsigned long long)a.n * a.ic2 * a.ih * a.iw * 16 * (a.in_u8 ? 1 : 4);
     const char *env = getenv("EHIP_WINO_BUF_GATHER");
     a.buf_gather = bytes <= 0xffffff00ull && !(env && env[0] == '0');
+    const char *wide = getenv("EHIP_WINO_WIDE_GATHER");
+    if (a.buf_gather && a.in_u8 && !(wide && wide[0] == '0')) a.buf_gather = 2;   // whole cells and a transpose inside the quad
   }
   a.nblocks = (a.t + 63) / 64;
   a.items_per_xcd = (int)(((long long)a.nblocks * a.ic2 + 7) / 8);
