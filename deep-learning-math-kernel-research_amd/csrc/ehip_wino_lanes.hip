@@ -130,6 +130,44 @@ __device__ __forceinline__ void output_tile_packed(const float4 *m, const float4
   store_cells<A>(pk, block, g, ok, th, tw, oh_n, ow_n, px);
 }
 
+// f32 output (no output scale, no in-place sum here): bias and ReLU as output_tile applies them, and the lane's four
+// channels of every pixel leave as one 16-byte store (the four lanes of a tile write the 64 bytes of a pixel's block).
+// y: [channel][pixel]; block: the tile's image and channel block, in floats.
+template <int A>
+__device__ __forceinline__ void finish_channel_f32(float *y, float b, bool with_bias, bool with_relu)
+{
+  constexpr int M = A - 2;
+#pragma unroll
+  for (int e = 0; e < M * M; ++e) {
+    float r = y[e];
+    if (with_bias) r = r + b;
+    if (with_relu) r = r > 0.0f ? r : 0.0f;
+    y[e] = r;
+  }
+}
+template <int A>
+__device__ __forceinline__ void store_f32(const float (*y)[(A - 2) * (A - 2)], float *block, int g, bool ok, int th, int tw, int oh_n,
+                                          int ow_n, int px)
+{
+  constexpr int M = A - 2;
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  if (!ok) return;
+#pragma unroll
+  for (int i = 0; i < M; ++i) {
+    const int oh = M * th + i;
+    if (oh >= oh_n) break;
+#pragma unroll
+    for (int j = 0; j < M; ++j) {
+      const int ow = M * tw + j;
+      if (ow >= ow_n) break;
+      const int e = M * i + j;
+      const v4f vv = {y[0][e], y[1][e], y[2][e], y[3][e]};
+      // (non-temporal: output that nothing reads back soon)
+      __builtin_nontemporal_store(vv, reinterpret_cast<v4f *>(block + ((size_t)oh * ow_n + ow) * px + 4 * g));
+    }
+  }
+}
+
 // the one-dimensional output transform of tile sizes 6 and 5
 template <int A>
 __device__ __forceinline__ void out_1d(const float *f, float *o)
@@ -260,8 +298,24 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
   const size_t block = a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (occ >> 4) * 16
                                   : ((size_t)n * a.oc2 + (occ >> 4)) * a.oh * a.ow * 16;
   const int px = a.out_nhwc ? a.oc2 * 16 : 16;
-  // (u8 / s8 output only: the launcher keeps f32 output, whose four channels of a pixel leave as one 16-byte store
-  // and would need all of them in registers at once, on the general form)
+  if (!SUM && a.out_type == EHIP_F32) {
+    // channel by channel: a channel's requantized positions die as its 16 outputs are born
+    constexpr int M = A - 2;
+    float y[4][M * M];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float f[AA];
+#pragma unroll
+      for (int e = 0; e < AA; ++e) f[e] = comp_of(m[e], k);
+      wino::tile_output<A>(f, y[k]);
+      finish_channel_f32<A>(y[k], comp_of(bias, k), a.with_bias != 0, a.with_relu != 0);
+#pragma unroll
+      for (int e = 0; e < M * M; ++e) asm volatile("" : "+v"(y[k][e]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    store_f32<A>(y, static_cast<float *>(a.out) + block, g, valid, th, tw, a.oh, a.ow, px);
+    return;
+  }
   if (a.out_type == EHIP_U8)
     output_tile_packed<EHIP_U8, A>(m, bias, a.with_relu != 0, a.out_repS, a.out_z, static_cast<uint8_t *>(a.out) + block, g,
                                    valid, th, tw, a.oh, a.ow, SUM, px);
@@ -495,14 +549,36 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
     };
     using U8C = std::integral_constant<int, EHIP_U8>;
     using S8C = std::integral_constant<int, EHIP_S8>;
-    if (a.out_type == EHIP_U8) {
-      if (a.with_relu) finish(U8C{}, std::true_type{});
-      else finish(U8C{}, std::false_type{});
+    if (!SUM && a.out_type == EHIP_F32) {
+      float y[4][M * M];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (NCOL == 1) {
+          float f[AA];
+#pragma unroll
+          for (int e = 0; e < AA; ++e) f[e] = comp_of(m4[NCOL == 1 ? e : 0], k);
+          wino::tile_output<A>(f, y[k]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < M; ++r) out_1d<A>(T[k][r], &y[k][M * r]);
+        }
+        finish_channel_f32<A>(y[k], comp_of(bias, k), a.with_bias != 0, a.with_relu != 0);
+#pragma unroll
+        for (int e = 0; e < M * M; ++e) asm volatile("" : "+v"(y[k][e]));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // (plane: the block's offset in elements, worked out on the byte pointer)
+      store_f32<A>(y, static_cast<float *>(a.out) + (plane - static_cast<uint8_t *>(a.out)), g, valid, th, tw, a.oh, a.ow, px);
     } else {
-      if (a.with_relu) finish(S8C{}, std::true_type{});
-      else finish(S8C{}, std::false_type{});
+      if (a.out_type == EHIP_U8) {
+        if (a.with_relu) finish(U8C{}, std::true_type{});
+        else finish(U8C{}, std::false_type{});
+      } else {
+        if (a.with_relu) finish(S8C{}, std::true_type{});
+        else finish(S8C{}, std::false_type{});
+      }
+      store_cells<A>(pk, plane, g, valid, th, tw, a.oh, a.ow, px);
     }
-    store_cells<A>(pk, plane, g, valid, th, tw, a.oh, a.ow, px);
     if (!more) break;
     item = next;
     tb = tbn;
@@ -516,7 +592,7 @@ bool wino_lanes_applies(const WinoFusedArgs &a)
   // Measured at N = 64, u8 in / s8 out, against the general kernel (fused stage, us): 64 -> 64 at 56 x 56 28.5 vs 34.1, at
   // 224 x 224 370 vs 459; 128 -> 128 at 112 x 112 238 vs 300; 128 -> 256 at 56 x 56 107 vs 133; 256 -> 256 at 56 x 56 164 vs 171;
   // 512 -> 512 at 28 x 28 (eight k-steps per position, 288 unrolled steps) 648 vs 134: up to 256 input channels.
-  return a.tin_blocked && (nks64 <= 2 || nks64 == 4) && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && a.out_type != EHIP_F32 &&
+  return a.tin_blocked && (nks64 <= 2 || nks64 == 4) && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && !(a.out_type == EHIP_F32 && a.with_sum) &&
       !(env && env[0] == '0');
 }
 
