@@ -81,8 +81,13 @@ __device__ __forceinline__ void store_cells(const unsigned *pk, uint8_t *block, 
     unsigned c0 = pk[M * i], c1 = pk[M * i + 1], c2 = M > 2 ? pk[M * i + (M > 2 ? 2 : 0)] : 0u, c3 = M > 3 ? pk[M * i + (M > 3 ? 3 : 0)] : 0u;
     rows_transpose(c0, c1, c2, c3);
     const int oh = M * th + i, ow = M * tw + g;
-    if (ok && g < M && oh < oh_n && ow < ow_n)
-      *reinterpret_cast<uint4 *>(block + ((size_t)oh * ow_n + ow) * px) = make_uint4(c0, c1, c2, c3);
+    if (ok && g < M && oh < oh_n && ow < ow_n) {
+      // (non-temporal: the output would only push the transformed input, which the other channel blocks' workgroups
+      // still read, out of the L2 -- 128 -> 128 at 112 x 112: 130 -> 100 us)
+      typedef unsigned v4u __attribute__((ext_vector_type(4)));
+      const v4u vv = {c0, c1, c2, c3};
+      __builtin_nontemporal_store(vv, reinterpret_cast<v4u *>(block + ((size_t)oh * ow_n + ow) * px));
+    }
   }
 }
 
