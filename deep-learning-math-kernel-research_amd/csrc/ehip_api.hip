@@ -714,6 +714,9 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.out_nhwc = w.out_nhwc;
         f.trace = trace_buffer();
         HIP_TRY(launch_wino_gemm_output(f, s, one_pass ? &c->plan_wino_fused : nullptr));
+        // (which form of the fused stage runs is the launcher's choice: known from the first execute on)
+        if (c->plan_wino_fused.name && c->kernel_name.find(c->plan_wino_fused.name) == std::string::npos)
+          c->kernel_name = std::string("k_wino_trans_input_u8 + ") + c->plan_wino_fused.name;
         continue;
       }
       GemmArgs a;

@@ -627,7 +627,9 @@ hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a0, hipStream_t s,
     const size_t lds = (size_t)AA * nks64 * 1024 + (size_t)AA * 12 * sizeof(float4);
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    return plan_launch(plan, kernel, dim3(8 * a.ny * slots), dim3(kBlock), lds, a, s);
+    const hipError_t rc = plan_launch(plan, kernel, dim3(8 * a.ny * slots), dim3(kBlock), lds, a, s);
+    if (plan && rc == hipSuccess) plan->name = "k_wino_gemm_output_lanes_wres";
+    return rc;
   }
   a.nx = (a.t + 31) / 32;
   a.ny = (a.oc2 * 16 + 31) / 32;
@@ -641,7 +643,9 @@ hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a0, hipStream_t s,
   else EHIP_WL(6);
 #undef EHIP_WL
   const size_t lds = (size_t)AA * 24 * sizeof(float4);
-  return plan_launch(plan, kernel, dim3(8 * a.ny * ((a.nx + 7) / 8)), dim3(kBlock), lds, a, s);
+  const hipError_t rc = plan_launch(plan, kernel, dim3(8 * a.ny * ((a.nx + 7) / 8)), dim3(kBlock), lds, a, s);
+  if (plan && rc == hipSuccess) plan->name = "k_wino_gemm_output_lanes";
+  return rc;
 }
 
 }  // namespace ehip
