@@ -143,7 +143,8 @@ EHIP_API int ehip_conv_execute_stages(ehip_conv_t *conv, void *output_dev, const
  * Returns the number of bytes through *bytes when host_dst is NULL. */
 EHIP_API int ehip_conv_query(ehip_conv_t *conv, int what, void *host_dst, size_t *bytes);
 
-/* Name of the kernel variant execute() launches (for profiles), and its launch geometry. */
+/* Name of the kernel variant execute() launches (for profiles), and its launch geometry.  Where the launcher chooses
+ * between forms of a kernel (epilogue forms, the fused Winograd stage), the name is final after the first execute. */
 EHIP_API const char *ehip_conv_kernel_name(ehip_conv_t *conv);
 
 /* Replaces the harness-side fp32 -> u8 activation quantization
