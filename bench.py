@@ -74,6 +74,51 @@ def _hip_events():
     return _HIP_EVENTS[0]
 
 
+def chained_network(layers, batches):
+    """The layers of a network in order, `count` executes of each, as one sequence per batch on one stream: timed as
+    `batches` sequences enqueued launch by launch, and as the same number of replays of a HIP graph that holds one
+    sequence.  Every kernel then follows a different kernel with different tensors, as in a model run.  The graph's
+    last replay must leave the same bytes in every layer's output as the last eager sequence."""
+    import torch
+    s = torch.cuda.Stream()
+    def sequence(stream):
+        for count, l in layers:
+            l.conv.execute_repeat(l.out, l.x, count, bias=l.bias, stream=stream)
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(batches):
+            fn()
+        torch.cuda.synchronize()   # (a replay runs on the current stream, the sequences on s)
+        return (time.perf_counter() - t0) / batches
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < max(PREHEAT_S, 0.02):   # also the first execute of every handle: its launch plans
+        sequence(s.cuda_stream)
+        s.synchronize()
+    eager = timed(lambda: sequence(s.cuda_stream))
+    # outputs of layers with the in-place sum change with every execute: compare from a common state
+    def snapshot():
+        return [l.out.clone() for _, l in layers]
+    def restore(state):
+        for (_, l), o in zip(layers, state):
+            l.out.copy_(o)
+    start = snapshot()
+    sequence(s.cuda_stream)
+    s.synchronize()
+    want = snapshot()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        sequence(torch.cuda.current_stream().cuda_stream)
+    restore(start)
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    same = all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(snapshot(), want))
+    graph = timed(g.replay)
+    return {"batches": batches, "eager_ms_per_batch": round(eager * 1e3, 4), "graph_ms_per_batch": round(graph * 1e3, 4),
+            "graph_images_per_s": round(64 / graph, 1), "graph_replay_matches_eager": bool(same)}
+
+
 def measure(layer, steps, warmup):
     """(wall seconds per step, HIP-event seconds per step).  Both regions hold exactly `steps`
     executions enqueued back to back on the stream the kernels run on (the default stream).
@@ -377,6 +422,11 @@ def main():
                     help="with --network: run the 3x3 stride-1 layers with CONV_DIRECT instead of the Winograd "
                          "algorithm the reference's scripts ask for (on this GPU the direct kernel is the faster one; "
                          "its results are the reference's DIRECT results, not its Winograd results)")
+    ap.add_argument("--chained", action="store_true",
+                    help="with --network: besides the sum of the layers' own times, run the whole list of layers in order "
+                         "as ONE sequence per batch -- enqueued launch by launch on a stream, and replayed from a HIP "
+                         "graph of the same launches -- so that every kernel follows a different one (cold caches, "
+                         "launch gaps between unlike kernels); all layers' tensors stay resident")
     ap.add_argument("--preheat-ms", type=float, default=100.0,
                     help="untimed run of the layer before the warmup steps, so that the GPU is at its running clocks "
                          "(profiler runs pass a small value to keep their traces short)")
@@ -469,6 +519,7 @@ def main():
     if args.network:
         net = W.NETWORKS[args.network]
         rows, total_s, total_ops = [], 0.0, 0.0
+        kept = []
         for count, w2 in net:
             if args.direct3x3 and w2.algorithm == E.CONV_WINOGRAD:
                 w2 = W.Workload(w2.key, "3x3 direct %d->%d @%d u8->s8" % (w2.ic, w2.oc, w2.hw), w2.n, w2.ic, w2.oc, w2.hw, k=3,
@@ -480,8 +531,14 @@ def main():
             # the FC layers are configured with n = 1 over 8 x 8 "pixels" = one row per image of the batch
             total_s += count * wall2
             total_ops += count * w2.ops()
+            if args.chained:
+                kept.append((count, l2))
+                continue
             del l2
             torch.cuda.empty_cache()
+        chained = None
+        if args.chained:
+            chained = chained_network(kept, 20 if total_s > 1e-3 else 50)
         print(json.dumps({"metric": "network_conv_layers_images_per_s", "network": args.network,
                           "three_by_three": "direct" if args.direct3x3 else "as configured by the reference's script",
                           "value": round(64 / total_s, 1), "unit": "images/s", "batch": 64,
@@ -489,7 +546,7 @@ def main():
                           "effective_tops": round(total_ops / total_s / 1e12, 1), "data": "synthetic",
                           "note": "sum over the network's convolution layers of count x time of one execute, each "
                                   "layer timed back to back on its own device-resident tensors; pooling, residual "
-                                  "adds and softmax are not part of the library", "layers": rows}))
+                                  "adds and softmax are not part of the library", "chained": chained, "layers": rows}))
         return
 
     wl = W.WORKLOADS[args.workload]
