@@ -203,6 +203,48 @@ def test_wino_fused_lanes_weights_resident(slots, wres, tile, out_type, with_sum
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
+@pytest.mark.parametrize("out_type", [ol.S8, ol.F32])
+@pytest.mark.parametrize("n,ic,oc,hw", [(8, 64, 64, 224), (16, 128, 128, 112), (16, 256, 256, 56)])
+def test_wino_fused_forms_agree_at_full_size(out_type, n, ic, oc, hw, monkeypatch):
+    """the VGG layers at their real planes (a share of the batch), where the weights-resident workgroups take many blocks
+    of tiles each: the three forms of the fused stage -- lanes with resident weights, lanes with both operands streamed,
+    the general kernel -- written independently of each other, leave the same bytes (each is pinned against the oracle
+    at sizes the oracle finishes in seconds by the tests above)"""
+    import torch
+    E = pkg()
+    g = torch.Generator(device="cuda").manual_seed(1234 + ic + hw)
+    x = torch.randint(0, 256, (n, ic // 16, hw, hw, 16), dtype=torch.uint8, device="cuda", generator=g)
+    w = (torch.randn((oc // 16, ic // 16, 3, 3, 16, 16), device="cuda", generator=g) * 0.02).float()
+    bias = (torch.randn(oc, device="cuda", generator=g) * 0.01).float()
+    out_scale = 4.0 * 0.02 * np.sqrt(9 * ic / 3.0) / 127.0
+    d = E.make_desc(n, ic, oc, hw, hw, 3, 3, 1, algorithm=E.CONV_WINOGRAD, input_type=E.U8, output_type=out_type,
+                    with_bias=True, with_relu=True, input_quant=(1.0 / 255.0, 0.0), tile_size=6, execution_mode=0xa161,
+                    wino_tinput_quant=(22.0 / 255.0, 104.0), output_quant=(out_scale, 0.0))
+    outs = {}
+    for name, env in (("resident", {}), ("streamed", {"EHIP_WINO_LANES_WRES": "0"}), ("general", {"EHIP_WINO_LANES": "0"})):
+        for k in ("EHIP_WINO_LANES_WRES", "EHIP_WINO_LANES"):
+            monkeypatch.delenv(k, raising=False)
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        conv = E.Conv(d)
+        out = torch.zeros((n, oc // 16, hw, hw, 16), dtype=torch.float32 if out_type == ol.F32 else torch.int8, device="cuda")
+        conv.prepare(w, bias)
+        conv.execute(out, x, None, bias)
+        torch.cuda.synchronize()
+        outs[name] = (out, conv.kernel_name)
+        del conv
+    if ic <= 128:
+        assert outs["resident"][1].endswith("k_wino_gemm_output_lanes_wres")
+    assert outs["streamed"][1].endswith("k_wino_gemm_output_lanes")
+    assert outs["general"][1].endswith("k_wino_gemm_output")
+    ref = outs["general"][0]
+    assert int((ref.view(torch.uint8) != 0).sum()) > ref.numel() // 8   # (not a layer of zeros)
+    for name in ("resident", "streamed"):
+        got = outs[name][0]
+        assert torch.equal(got.view(torch.uint8), ref.view(torch.uint8)), "%s differs from the general kernel at %d values" % (
+            name, int((got != ref).sum()))
+
+
 def _fused(n, ic, oc, hw):
     import torch
     E, p, d, xb, wb, bias = make_wino(n, ic, oc, hw, seed=n * 10 + hw + ic)
