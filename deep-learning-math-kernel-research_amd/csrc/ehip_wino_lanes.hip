@@ -1,5 +1,5 @@
-// Winograd GEMMs + output transform for layers with at most 256 input channels and u8 / s8 output: the form whose
-// lanes own a tile x four channels at every position, so that nothing is exchanged between the GEMMs and the transform.
+// Winograd GEMMs + output transform for layers with at most 256 input channels: the form whose lanes own a tile x four
+// channels at every position, so that nothing is exchanged through LDS between the GEMMs and the transform.
 //
 // Replaces, for those layers, elx_int8_conv_wino_gemm_t::execute + trans_output as the reference's fused schedule
 // runs them per thread (a161, src/elx_int8_conv_wino_xopt.hpp:21-179; src/elx_int8_conv_wino_gemm.cpp:23-205,
@@ -18,10 +18,10 @@ namespace {
 
 __device__ __forceinline__ float comp_of(const float4 &v, int k) { return k == 0 ? v.x : (k == 1 ? v.y : (k == 2 ? v.z : v.w)); }
 
-// The pieces of output_tile for u8 / s8 output with few registers: one channel at a time, its bytes packed into the
-// pixels' dwords as they come (16 dwords live instead of 4 x 16 floats; the old output of the in-place sum stays packed
-// as well).  Same operations in the same order per value as output_tile.
-// channel k of the lane's four: bias, output scale, old output, ReLU, rounding, byte k of the pixels' dwords
+// The pieces of output_tile (ehip_wino.hip) for u8 / s8 output with few registers: one channel at a time, its bytes
+// packed into the pixels' dwords as they come (16 dwords live instead of 4 x 16 floats; the old output of the in-place
+// sum stays packed as well).  Same operations in the same order per value as output_tile.
+// pack_channel: channel k of the lane's four -- bias, output scale, old output, ReLU, rounding, byte k of the dwords.
 template <int OUT, int A>
 __device__ __forceinline__ void pack_channel(const float *o, float b, int k, bool with_relu, float repS, float z, bool with_sum,
                                              const unsigned *old, unsigned *pk)
@@ -187,11 +187,12 @@ __device__ __forceinline__ void out_1d(const float *f, float *o)
 // registers, one wave per SIMD, and passes the results through 144 KB of LDS to the transform; with few input channels
 // it is all output phase (64 -> 64: 37 K of a workgroup's 47 K clocks).
 // Here v_mfma_i32_16x16x64_i8 makes the GEMM's own result layout the transform's: a lane of the 16 x 16 result holds
-// four consecutive packed rows = four consecutive output channels of ONE tile, so with all A x A positions of its 16
+// four consecutive rows = four consecutive output channels of ONE tile, so with all A x A positions of its 16
 // channels x 16 tiles in one wave (4 accumulator registers per position) every lane already owns the A x A values
-// of one tile x four channels -- requantization, Y = At M A and the store happen in the lane, with no exchange, no
-// barrier, and two to three workgroups per CU to hide each other's latencies.  The price is the operand stream:
-// 2 KB per 16 x 16 x 64 MFMA, which only so short a K loop can afford.
+// of one tile x four channels -- requantization and Y = At M A happen in the lane, with no exchange through LDS, no
+// barrier, and two workgroups per CU to hide each other's latencies; only the finished bytes are transposed between the
+// wave's rows, for stores of whole cells.  The price is the operand stream: 2 KB per 16 x 16 x 64 MFMA, which only so
+// short a K loop can afford.
 // Workgroup = 32 channels x 32 tiles (one block of the blocked tinput); wave = (half of the channels, half of the
 // tiles); NKS = k-steps of 64 channels per position (1, 2 or 4).
 template <int A, bool SUM, int NKS>
