@@ -338,9 +338,10 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
 // while this one's output transform keeps the vector units busy.  No barrier after the staging.
 // a.nx = blocks of 64 tiles, a.ny = groups of 16 packed rows; grid = 8 XCDs x a.ny x slots, a slot walks over the
 // blocks slot * 8 + xcd, + 8 * slots, ...
-template <int A, bool SUM, int NKS>
-__global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoFusedArgs a)
+template <int A, bool SUM, int NKS, int NW = 4>
+__global__ __launch_bounds__(64 * NW, 2) void k_wino_gemm_output_lanes_wres(WinoFusedArgs a)
 {
+  constexpr int TB = 64 * NW;   // threads; a block of tiles of the workgroup = 16 NW tiles = NW / 2 blocks of 32
   constexpr int AA = A * A, STEPS = AA * NKS;
   constexpr int D = A == 6 ? (SUM ? 6 : 12) : (A == 5 ? 5 : 8);   // divides STEPS: a ring slot holds the same steps in every block
   static_assert(STEPS % D == 0, "ring");
@@ -377,7 +378,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
   // the wave's block of 32 tiles inside the item (the last item of an odd count has one block only: its upper waves
   // read the lower block again and store nothing)
   auto base_of = [&](int it) {
-    int blk = 2 * it + (wave >> 1);
+    int blk = (NW / 2) * it + (wave >> 1);
     blk = blk < nblk ? blk : nblk - 1;
     return a.tin + blk * t_blk;      // wave-uniform
   };
@@ -393,12 +394,12 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
   for (int k = 0; k < D; ++k) issue(k, k, tb);
   {
     // the weights: per (step, unit) 16 rows x 16 bytes = 256 contiguous bytes of [pos][unit][OCpp][16]
-    constexpr int NP = (STEPS * 64 + kBlock - 1) / kBlock;
+    constexpr int NP = (STEPS * 64 + TB - 1) / TB;
     const long long w_pos = (long long)a.units_pad * a.ocpp * 16;
     v4i tmp[NP];
 #pragma unroll
     for (int j = 0; j < NP; ++j) {
-      int idx = tid + j * kBlock;
+      int idx = tid + j * TB;
       idx = idx < STEPS * 64 ? idx : STEPS * 64 - 1;
       const int chunk = idx >> 4, cell = idx & 15;
       const int sn = chunk >> 2, u = chunk & 3;
@@ -406,11 +407,11 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
       tmp[j] = *reinterpret_cast<const v4i *>(a.w + p * w_pos +
                                               ((long long)(4 * ks + u) * a.ocpp + oc0 + 8 * (cell >> 2) + 4 * h + (cell & 3)) * 16);
     }
-    constexpr int NC = (AA * 12 + kBlock - 1) / kBlock;
+    constexpr int NC = (AA * 12 + TB - 1) / TB;
     float4 cst[NC];
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-      int idx = tid + j * kBlock;
+      int idx = tid + j * TB;
       idx = idx < AA * 12 ? idx : AA * 12 - 1;
       const int p = idx / 12, rem = idx - 12 * p, arr = rem >> 2, gq = rem & 3;
       const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
@@ -418,12 +419,12 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
     }
 #pragma unroll
     for (int j = 0; j < NP; ++j) {
-      const int idx = tid + j * kBlock;
+      const int idx = tid + j * TB;
       if (idx < STEPS * 64) wl[idx] = tmp[j];
     }
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-      const int idx = tid + j * kBlock;
+      const int idx = tid + j * TB;
       if (idx < AA * 12) cl[idx] = cst[j];
     }
   }
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
     const int next = item + item_step;
     const bool more = next < a.nx;                      // wave-uniform
     const uint8_t *tbn = base_of(more ? next : item);   // (the last block's tail requests its own head again: unused)
-    const int t = item * 64 + wave * 16 + l16;
+    const int t = item * (16 * NW) + wave * 16 + l16;
     const bool valid = t < a.t && oc_ok;
     // (lanes without a tile or channel of their own take part with tile 0 / channel 0 and store nothing)
     const int tc = valid ? t : 0, occ = valid ? oc : 0;
@@ -591,6 +592,29 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes_wres(WinoF
   }
 }
 
+namespace {
+template <int A, bool SUM>
+auto pick_wres_nks(int nks64, int nw) -> void (*)(WinoFusedArgs)
+{
+  switch (nks64) {
+    case 1: return k_wino_gemm_output_lanes_wres<A, SUM, 1>;
+    case 2: return k_wino_gemm_output_lanes_wres<A, SUM, 2>;
+    case 3: return nw == 8 ? k_wino_gemm_output_lanes_wres<A, SUM, 3, 8> : k_wino_gemm_output_lanes_wres<A, SUM, 3>;
+    case 4: return nw == 8 ? k_wino_gemm_output_lanes_wres<A, SUM, 4, 8> : k_wino_gemm_output_lanes_wres<A, SUM, 4>;
+    case 8:
+      if (A == 4) return nw == 8 ? k_wino_gemm_output_lanes_wres<4, SUM, 8, 8> : k_wino_gemm_output_lanes_wres<4, SUM, 8>;
+      return nullptr;
+    default: return nullptr;
+  }
+}
+auto pick_wres(int A, bool sum, int nks64, int nw) -> void (*)(WinoFusedArgs)
+{
+  if (A == 4) return sum ? pick_wres_nks<4, true>(nks64, nw) : pick_wres_nks<4, false>(nks64, nw);
+  if (A == 5) return sum ? pick_wres_nks<5, true>(nks64, nw) : pick_wres_nks<5, false>(nks64, nw);
+  return sum ? pick_wres_nks<6, true>(nks64, nw) : pick_wres_nks<6, false>(nks64, nw);
+}
+}  // namespace
+
 bool wino_lanes_applies(const WinoFusedArgs &a)
 {
   const char *env = getenv("EHIP_WINO_LANES");
@@ -598,7 +622,10 @@ bool wino_lanes_applies(const WinoFusedArgs &a)
   // Measured at N = 64, u8 in / s8 out, against the general kernel (fused stage, us): 64 -> 64 at 56 x 56 28.5 vs 34.1, at
   // 224 x 224 370 vs 459; 128 -> 128 at 112 x 112 238 vs 300; 128 -> 256 at 56 x 56 107 vs 133; 256 -> 256 at 56 x 56 164 vs 171;
   // 512 -> 512 at 28 x 28 (eight k-steps per position, 288 unrolled steps) 648 vs 134: up to 256 input channels.
-  return a.tin_blocked && (nks64 <= 2 || nks64 == 4) && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && !(a.out_type == EHIP_F32 && a.with_sum) &&
+  const int A = a.tile ? a.tile : 6;
+  // the weights of 16 channels at every position must fit the LDS (the streamed form: 1, 2 or 4 k-steps)
+  const bool fits = nks64 <= 4 || (A == 4 && nks64 == 8);
+  return a.tin_blocked && fits && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && !(a.out_type == EHIP_F32 && a.with_sum) &&
       !(env && env[0] == '0');
 }
 
@@ -609,26 +636,28 @@ hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a0, hipStream_t s,
   const int nks64 = (a.ic2 + 3) / 4;
   void (*kernel)(WinoFusedArgs) = nullptr;
   const char *env = getenv("EHIP_WINO_LANES_WRES");
-  if (nks64 <= 2 && !(env && env[0] == '0')) {
-    // weights resident: blocks of 64 tiles, groups of 16 packed rows, two workgroups per CU walking over the blocks
-    a.nx = (a.t + 63) / 64;
+  if (!(env && env[0] == '0') || nks64 == 3 || nks64 > 4) {   // (the streamed form below has 1, 2 and 4 k-steps only)
+    // weights resident: the weights of 16 channels in LDS, workgroups walking over blocks of tiles.  Up to 128 input
+    // channels: four waves, 64 tiles a block, two workgroups per CU; 256: the weights fill the LDS (tile size 6: 147 KB),
+    // one workgroup per CU, of eight waves (128 tiles a block) so that every SIMD still has two
+    const size_t lds = (size_t)AA * nks64 * 1024 + (size_t)AA * 12 * sizeof(float4);
+    const int per_cu = 2 * lds <= 160 * 1024 ? 2 : 1;
+    const char *wv = getenv("EHIP_WINO_LANES_WAVES");
     a.ny = 2 * ((a.oc2 * 16 + 31) / 32);
-    int slots = 64 / a.ny;   // 8 XCDs x ny x slots ~ 512 workgroups
+    // (eight waves where that still gives every CU a workgroup: 256 -> 256 at 56 x 56 104 -> 89 us, at 14 x 14 14.5 -> 15.8 us)
+    int nw = per_cu == 1 && (long long)((a.t + 127) / 128) * a.ny >= 256 ? 8 : 4;
+    if (wv) nw = wv[0] == '8' && nks64 >= 3 ? 8 : 4;
+    a.nx = (a.t + 16 * nw - 1) / (16 * nw);
+    int slots = 32 * per_cu / a.ny;   // 8 XCDs x ny x slots ~ 256 workgroups per workgroup a CU holds
     if (const char *sl = getenv("EHIP_WINO_LANES_SLOTS")) slots = atoi(sl);   // (fewer: more blocks of tiles per workgroup)
     slots = slots < 1 ? 1 : slots;
     const int need = (a.nx + 7) / 8;
     slots = slots < need ? slots : need;
-#define EHIP_WLR(AV)                                                                                                   \
-  kernel = a.with_sum ? (nks64 == 1 ? k_wino_gemm_output_lanes_wres<AV, true, 1> : k_wino_gemm_output_lanes_wres<AV, true, 2>) \
-                      : (nks64 == 1 ? k_wino_gemm_output_lanes_wres<AV, false, 1> : k_wino_gemm_output_lanes_wres<AV, false, 2>)
-    if (A == 4) EHIP_WLR(4);
-    else if (A == 5) EHIP_WLR(5);
-    else EHIP_WLR(6);
-#undef EHIP_WLR
-    const size_t lds = (size_t)AA * nks64 * 1024 + (size_t)AA * 12 * sizeof(float4);
+    kernel = pick_wres(A, a.with_sum != 0, nks64, nw);
+    if (!kernel) return hipErrorInvalidValue;
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    const hipError_t rc = plan_launch(plan, kernel, dim3(8 * a.ny * slots), dim3(kBlock), lds, a, s);
+    const hipError_t rc = plan_launch(plan, kernel, dim3(8 * a.ny * slots), dim3(64 * nw), lds, a, s);
     if (plan && rc == hipSuccess) plan->name = "k_wino_gemm_output_lanes_wres";
     return rc;
   }

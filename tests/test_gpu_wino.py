@@ -203,6 +203,44 @@ def test_wino_fused_lanes_weights_resident(slots, wres, tile, out_type, with_sum
     assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
 
 
+@pytest.mark.parametrize("waves", ["4", "8"])
+@pytest.mark.parametrize("slots", ["1", ""])
+@pytest.mark.parametrize("tile", [6, 5, 4])
+@pytest.mark.parametrize("out_type,with_sum", [(ol.S8, 0), (ol.U8, 1), (ol.F32, 0)])
+@pytest.mark.parametrize("n,ic,oc,hw", [(2, 256, 48, 30), (1, 192, 32, 36), (3, 512, 32, 18)])
+def test_wino_fused_lanes_weights_resident_many_channels(waves, slots, tile, out_type, with_sum, n, ic, oc, hw, monkeypatch):
+    """192 / 256 input channels (three / four k-steps of 64 per position; 512 with tile size 4): the weights of 16
+    channels fill most of the LDS, one workgroup per CU, of four or of eight waves (64 / 128 tiles a block)"""
+    import torch
+    if ic == 512 and tile != 4:
+        pytest.skip("the weights of 16 channels x 512 inputs fit the LDS with tile size 4 only")
+    monkeypatch.setenv("EHIP_WINO_LANES_WAVES", waves)
+    if slots:
+        monkeypatch.setenv("EHIP_WINO_LANES_SLOTS", slots)
+    E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=63 + tile + ic + out_type, out_type=out_type, tile=tile,
+                                         out_z=0.0 if out_type != ol.U8 else 1.6)
+    p.with_sum = with_sum
+    d.with_ip_sum = with_sum
+    p.tin_scale, p.tin_z = 22.0 / 255.0, 104.0
+    d.tinput_scale, d.tinput_z = p.tin_scale, p.tin_z
+    rng = np.random.default_rng(93 + tile + hw)
+    shape = (n, ol.up16(oc) // 16, hw, hw, 16)
+    old = (rng.normal(0, 0.05, shape).astype(f32) if out_type == ol.F32 else
+           rng.integers(-30 if out_type == ol.S8 else 0, 60, shape).astype(ol.NP_OF[out_type]))
+    twq, tscale, tshift = ol.wino_prepare(p, wb)
+    tout, _ = ol.wino_gemm(p, ol.wino_trans_input(p, xq.astype(f32)), twq, tscale, tshift)
+    exp = ol.wino_trans_output(p, tout, bias, out_init=old if with_sum else None)
+    conv = E.Conv(d)
+    d_out = dev(old)
+    d_b = dev(bias)
+    conv.prepare(dev(wb), d_b)
+    conv.execute(d_out, dev(xq), None, d_b)
+    torch.cuda.synchronize()
+    assert conv.kernel_name.endswith("k_wino_gemm_output_lanes_wres")
+    got = host(d_out)
+    assert np.array_equal(bits(got), bits(exp)), "output differs at %d of %d" % (int((got != exp).sum()), got.size)
+
+
 @pytest.mark.parametrize("out_type", [ol.S8, ol.F32])
 @pytest.mark.parametrize("n,ic,oc,hw", [(8, 64, 64, 224), (16, 128, 128, 112), (16, 256, 256, 56)])
 def test_wino_fused_forms_agree_at_full_size(out_type, n, ic, oc, hw, monkeypatch):
