@@ -413,6 +413,10 @@ int setup_workspace(ehip_conv *c)
     // (blocked: whole blocks of 32 tiles)  allocated with one pad unit behind it
     c->tin_bytes = (size_t)c->nbatch * c->ic2 * (c->tin_blocked ? up(c->t, 32) : c->t) * 16;
     c->tout_bytes = c->fused ? 16 : (size_t)c->nbatch * c->oc2 * c->t * 16 * sizeof(float);
+    if (c->fused) {   // (the fused stage's own parking space, where its kernel asks for one)
+      const size_t park = wino_lanes_tpart_bytes(d.tile_size, c->ic2, c->oc2, c->t);
+      if (park > c->tout_bytes) c->tout_bytes = park;
+    }
     // (the pad: an odd unit count makes the last k-step read one unit past its position -- in the blocked layout
     // 512 bytes past the last one, multiplied by zero weights)
     if ((rc = dev_alloc(&c->tin, c->tin_bytes + ((size_t)c->t * 16 > 1024 ? (size_t)c->t * 16 : 1024), true)) != EHIP_OK) return rc;
@@ -712,6 +716,7 @@ EHIP_API int ehip_conv_execute(ehip_conv_t *c, void *output_dev, const void *inp
         f.with_bias = d.with_bias; f.with_relu = d.with_relu; f.with_sum = d.with_ip_sum; f.tile = d.tile_size;
         f.out_type = w.out_type; f.out_repS = w.out_repS; f.out_z = w.out_z;
         f.out_nhwc = w.out_nhwc;
+        f.tpart = c->tout_bytes > 16 ? reinterpret_cast<float4 *>(c->tout) : nullptr;
         f.trace = trace_buffer();
         HIP_TRY(launch_wino_gemm_output(f, s, one_pass ? &c->plan_wino_fused : nullptr));
         // (which form of the fused stage runs is the launcher's choice: known from the first execute on)

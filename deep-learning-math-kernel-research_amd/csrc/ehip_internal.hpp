@@ -137,6 +137,7 @@ struct WinoFusedArgs {
   int tile;             // tile size A: 6 (or 0), 5, 4
   int out_nhwc;         // output as [n][h][w][c] (c % 16 == 0)
   int nx, ny;           // set by the launcher: blocks of 32 tiles, of 64 channels
+  float4 *tpart;        // first-stage results parked between the two passes of the 512-channel lanes kernel (wino_lanes_tpart_bytes)
   long long *trace;     // development aid, normally null (see EHIP_TRACE)
 };
 
@@ -229,6 +230,8 @@ hipError_t launch_wino_trans_output(const WinoArgs &a, hipStream_t s, LaunchPlan
 hipError_t launch_wino_gemm_output(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);
 // at most 256 input channels, u8 / s8 output: the form without an exchange between GEMMs and transform (ehip_wino_lanes.hip)
 bool wino_lanes_applies(const WinoFusedArgs &a);
+// device memory the lanes kernel needs besides the tensors (0 for most layers): a.tpart
+size_t wino_lanes_tpart_bytes(int tile, int ic2, int oc2, int t);
 hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a, hipStream_t s, LaunchPlan<WinoFusedArgs> *plan = nullptr);
 // min / max of the transformed input: partials = 2 * a.ic2 dwords of device scratch, result = two floats
 // of device memory (min, max); three launches on `s`, nothing else

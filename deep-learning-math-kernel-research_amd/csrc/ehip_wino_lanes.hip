@@ -593,6 +593,262 @@ __global__ __launch_bounds__(64 * NW, 2) void k_wino_gemm_output_lanes_wres(Wino
 }
 
 namespace {
+// second dimension of Y = At M A from the first-stage results T[channel][row][column], then output scale, rounding,
+// packing and the store by cells (u8 / s8), or bias / ReLU and the 16-byte stores of f32 output: what the kernel above
+// does at the end of a block of tiles, for the kernel below
+template <int A, bool SUM>
+__device__ __forceinline__ void finish_columns(const WinoFusedArgs &a, float (&T)[4][A - 2][A], const unsigned *old, const float4 &bias,
+                                               uint8_t *plane, int g, bool valid, int th, int tw, int px)
+{
+  constexpr int M = A - 2;
+  if (!SUM && a.out_type == EHIP_F32) {
+    float y[4][M * M];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+#pragma unroll
+      for (int r = 0; r < M; ++r) out_1d<A>(T[k][r], &y[k][M * r]);
+      finish_channel_f32<A>(y[k], comp_of(bias, k), a.with_bias != 0, a.with_relu != 0);
+#pragma unroll
+      for (int e = 0; e < M * M; ++e) asm volatile("" : "+v"(y[k][e]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    store_f32<A>(y, static_cast<float *>(a.out) + (plane - static_cast<uint8_t *>(a.out)), g, valid, th, tw, a.oh, a.ow, px);
+    return;
+  }
+  unsigned pk[M * M];
+#pragma unroll
+  for (int e = 0; e < M * M; ++e) pk[e] = 0u;
+  auto finish = [&](auto out_c, auto relu_c) {
+    constexpr int OUT = decltype(out_c)::value;
+    constexpr bool RELU = decltype(relu_c)::value;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float y[M * M];
+#pragma unroll
+      for (int r = 0; r < M; ++r) out_1d<A>(T[k][r], &y[M * r]);
+      pack_channel<OUT, A>(y, comp_of(bias, k), k, RELU, a.out_repS, a.out_z, SUM, old, pk);
+#pragma unroll
+      for (int e = 0; e < M * M; ++e) asm volatile("" : "+v"(pk[e]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using U8C = std::integral_constant<int, EHIP_U8>;
+  using S8C = std::integral_constant<int, EHIP_S8>;
+  if (a.out_type == EHIP_U8) {
+    if (a.with_relu) finish(U8C{}, std::true_type{});
+    else finish(U8C{}, std::false_type{});
+  } else {
+    if (a.with_relu) finish(S8C{}, std::true_type{});
+    else finish(S8C{}, std::false_type{});
+  }
+  store_cells<A>(pk, plane, g, valid, th, tw, a.oh, a.ow, px);
+}
+}  // namespace
+
+// 512 input channels (tile sizes 6 and 5): the weights of 16 channels at every position are 295 / 205 KB, twice the LDS,
+// but those of HALF the columns of M fit.  The workgroup (one per CU) therefore walks over its blocks of tiles twice:
+// with the weights of the first columns it leaves the first-stage results of those columns -- (A - 2) floats per
+// column and channel, a third of what the positions themselves would be -- in a.tpart, then stages the other columns'
+// weights, walks again and finishes every block with both halves in hand.  What a lane parks it reads back itself,
+// 16 bytes per lane and value in lane order.
+// a.tpart: [a.ny][a.nx][NW][(A - 2) x C0][64 lanes] float4, C0 = columns of the first pass (wino_lanes_tpart_bytes).
+template <int A, bool SUM, int NKS, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void k_wino_gemm_output_lanes_wres2(WinoFusedArgs a)
+{
+  static_assert(A == 6 || A == 5, "tile sizes with a column-wise transform");
+  constexpr int TB = 64 * NW;
+  constexpr int AA = A * A, M = A - 2;
+  constexpr int C0 = (A + 1) / 2, C1 = A - C0;               // columns of the two passes
+  constexpr int STEPS0 = C0 * A * NKS;
+  constexpr int D = A == 6 ? (SUM ? 6 : 12) : 5;             // divides the steps of both passes
+  static_assert(STEPS0 % D == 0 && (C1 * A * NKS) % D == 0, "ring");
+  extern __shared__ float4 lds[];
+  v4i *wl = reinterpret_cast<v4i *>(lds);   // [steps of the pass][4 units][16 packed rows] cells of 16 bytes
+  float4 *cl = lds + STEPS0 * 64;           // [AA][3][4 quads of the workgroup's 16 rows]: scale, shift, compensation
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, g = lane >> 4;
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int by = seq % a.ny;
+  const int slot = seq / a.ny;
+  const int item_step = 8 * (int)(gridDim.x / (8u * a.ny));
+  const int item0 = slot * 8 + xcd;
+  if (item0 >= a.nx) return;          // whole workgroup
+  const int oc0 = (by >> 1) * 32, h = by & 1;   // (the workgroup's 16 channels: see the kernel above)
+  const int oc_real = a.oc2 * 16;
+  const int nblk = (a.t + 31) >> 5;
+  const long long t_pos = (long long)a.ic2 * 512;
+  const long long t_blk = t_pos * AA;
+  unsigned b_off[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    int u = 4 * ks + g;
+    u = u < a.ic2 ? u : a.ic2 - 1;
+    b_off[ks] = (unsigned)(u * 512 + ((wave & 1) * 16 + l16) * 16);
+  }
+  auto base_of = [&](int it) {
+    int blk = (NW / 2) * it + (wave >> 1);
+    blk = blk < nblk ? blk : nblk - 1;
+    return a.tin + blk * t_blk;      // wave-uniform
+  };
+  const int oc = oc0 + 16 * h + 4 * g;   // the lane's four channels
+  const bool oc_ok = oc < oc_real;
+  float4 bias = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (a.with_bias && oc_ok) bias = *reinterpret_cast<const float4 *>(a.bias + oc);
+  const int px = a.out_nhwc ? a.oc2 * 16 : 16;
+  int wla = g * 16 + l16, clg = STEPS0 * 64 + g;   // the lane's cells of 16 bytes from the start of the LDS, opaque
+  asm volatile("" : "+v"(wla), "+v"(clg));
+  v4i rb[D];
+
+  auto run_pass = [&](auto qc) {
+    constexpr int Q = decltype(qc)::value;
+    constexpr int CB = Q == 0 ? 0 : C0, CN = Q == 0 ? C0 : C1, STEPS = CN * A * NKS;
+    // step sn of the pass = (column CB + i, row r, k-step ks) in that order; its position is A r + CB + i
+    auto pos_of = [](int sn) { const int pr = sn / NKS; return A * (pr % A) + CB + pr / A; };
+    auto issue = [&](int rs, int sn, const uint8_t *tb) {
+      rb[rs] = *reinterpret_cast<const v4i *>(tb + pos_of(sn) * t_pos + b_off[sn % NKS]);
+    };
+    int item = item0;
+    const uint8_t *tb = base_of(item);
+#pragma unroll
+    for (int k = 0; k < D; ++k) issue(k, k, tb);
+    if (Q > 0) __syncthreads();   // every wave has left the first pass's weights
+    {
+      constexpr int NP = (STEPS * 64 + TB - 1) / TB;
+      const long long w_pos = (long long)a.units_pad * a.ocpp * 16;
+      v4i tmp[NP];
+#pragma unroll
+      for (int j = 0; j < NP; ++j) {
+        int idx = tid + j * TB;
+        idx = idx < STEPS * 64 ? idx : STEPS * 64 - 1;
+        const int chunk = idx >> 4, cell = idx & 15;
+        const int sn = chunk >> 2, u = chunk & 3;
+        // (runtime step -> position: the same map as pos_of)
+        const int pr = sn / NKS, ks = sn - NKS * pr;
+        const int pp = A * (pr % A) + CB + pr / A;
+        tmp[j] = *reinterpret_cast<const v4i *>(a.w + pp * w_pos +
+                                                ((long long)(4 * ks + u) * a.ocpp + oc0 + 8 * (cell >> 2) + 4 * h + (cell & 3)) * 16);
+      }
+      constexpr int NC = Q == 0 ? (AA * 12 + TB - 1) / TB : 1;
+      float4 cst[NC];
+      if (Q == 0) {
+#pragma unroll
+        for (int j = 0; j < NC; ++j) {
+          int idx = tid + j * TB;
+          idx = idx < AA * 12 ? idx : AA * 12 - 1;
+          const int p = idx / 12, rem = idx - 12 * p, arr = rem >> 2, gq = rem & 3;
+          const float *src = arr == 0 ? a.scale : (arr == 1 ? a.shift : reinterpret_cast<const float *>(a.comp));
+          cst[j] = *reinterpret_cast<const float4 *>(src + (long long)p * a.ocpp + oc0 + 16 * h + 4 * gq);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < NP; ++j) {
+        const int idx = tid + j * TB;
+        if (idx < STEPS * 64) wl[idx] = tmp[j];
+      }
+      if (Q == 0) {
+#pragma unroll
+        for (int j = 0; j < NC; ++j) {
+          const int idx = tid + j * TB;
+          if (idx < AA * 12) cl[idx] = cst[j];
+        }
+      }
+    }
+    __syncthreads();   // the pass's weights (and the constants) are in LDS; the waves run on their own from here
+    for (;;) {
+      const int next = item + item_step;
+      const bool more = next < a.nx;                      // wave-uniform
+      const uint8_t *tbn = base_of(more ? next : item);   // (the last block's tail requests its own head again: unused)
+      const int t = item * (16 * NW) + wave * 16 + l16;
+      const bool valid = t < a.t && oc_ok;
+      const int tc = valid ? t : 0, occ = valid ? oc : 0;
+      const int n = tc / a.nt;
+      const int rem = tc - n * a.nt;
+      const int th = rem / a.wt;
+      const int tw = rem - th * a.wt;
+      uint8_t *plane = static_cast<uint8_t *>(a.out) +
+          (a.out_nhwc ? (size_t)n * a.oh * a.ow * a.oc2 * 16 + (occ >> 4) * 16 : ((size_t)n * a.oc2 + (occ >> 4)) * a.oh * a.ow * 16);
+      // the lane's parked values of this block: [row][column of the first pass], one float4 (four channels) each
+      float4 *park = a.tpart + ((((size_t)by * a.nx + item) * NW + wave) * (M * C0)) * 64 + lane;
+      float T[4][M][A];
+      unsigned old[M * M];
+      if (Q == 1) {
+#pragma unroll
+        for (int r = 0; r < M; ++r)
+#pragma unroll
+          for (int i = 0; i < C0; ++i) {
+            const float4 v = park[(size_t)(r * C0 + i) * 64];
+            T[0][r][i] = v.x; T[1][r][i] = v.y; T[2][r][i] = v.z; T[3][r][i] = v.w;
+          }
+      }
+      v4i ra[3];
+      ra[0] = wl[wla + 0];
+      ra[1] = wl[wla + 64];
+#pragma unroll
+      for (int i = 0; i < CN; ++i) {
+        if (SUM && Q == 1 && i == CN - 1) load_old_cells<A>(old, plane, g, th, tw, a.oh, a.ow, px);
+        v4i acc[A];
+#pragma unroll
+        for (int r = 0; r < A; ++r) {
+          const float4 cf = lds[clg + (A * r + CB + i) * 12 + 8];
+          acc[r] = v4i{__float_as_int(cf.x), __float_as_int(cf.y), __float_as_int(cf.z), __float_as_int(cf.w)};
+        }
+#pragma unroll
+        for (int r = 0; r < A; ++r)
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            const int sn = (i * A + r) * NKS + ks;
+            if (sn + 2 < STEPS) ra[(sn + 2) % 3] = wl[wla + (sn + 2) * 64];   // the weights of the step after next
+            const v4i b = rb[sn % D] ^ (int)0x80808080;
+            acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ra[sn % 3], b, acc[r], 0, 0, 0);
+            if (sn + D < STEPS) issue(sn % D, sn + D, tb);
+            else issue(sn % D, sn + D - STEPS, tbn);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        float4 mc[A];
+#pragma unroll
+        for (int r = 0; r < A; ++r) {
+          const int p = A * r + CB + i;
+          const float4 sc = lds[clg + p * 12], sh = lds[clg + p * 12 + 4];
+          mc[r].x = __builtin_fmaf((float)acc[r][0], sc.x, sh.x);
+          mc[r].y = __builtin_fmaf((float)acc[r][1], sc.y, sh.y);
+          mc[r].z = __builtin_fmaf((float)acc[r][2], sc.z, sh.z);
+          mc[r].w = __builtin_fmaf((float)acc[r][3], sc.w, sh.w);
+          asm volatile("" : "+v"(mc[r].x), "+v"(mc[r].y), "+v"(mc[r].z), "+v"(mc[r].w));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float f[A], o[M];
+#pragma unroll
+          for (int r = 0; r < A; ++r) f[r] = comp_of(mc[r], k);
+          out_1d<A>(f, o);
+#pragma unroll
+          for (int r = 0; r < M; ++r) {
+            asm volatile("" : "+v"(o[r]));
+            T[k][r][CB + i] = o[r];
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (Q == 0) {
+          // the column's results are parked as they come
+#pragma unroll
+          for (int r = 0; r < M; ++r)
+            park[(size_t)(r * C0 + i) * 64] = make_float4(T[0][r][i], T[1][r][i], T[2][r][i], T[3][r][i]);
+        }
+      }
+      if (Q == 1) finish_columns<A, SUM>(a, T, old, bias, plane, g, valid, th, tw, px);
+      if (!more) break;
+      item = next;
+      tb = tbn;
+    }
+  };
+  run_pass(std::integral_constant<int, 0>{});
+  run_pass(std::integral_constant<int, 1>{});
+}
+
+namespace {
 template <int A, bool SUM>
 auto pick_wres_nks(int nks64, int nw) -> void (*)(WinoFusedArgs)
 {
@@ -603,7 +859,8 @@ auto pick_wres_nks(int nks64, int nw) -> void (*)(WinoFusedArgs)
     case 4: return nw == 8 ? k_wino_gemm_output_lanes_wres<A, SUM, 4, 8> : k_wino_gemm_output_lanes_wres<A, SUM, 4>;
     case 8:
       if (A == 4) return nw == 8 ? k_wino_gemm_output_lanes_wres<4, SUM, 8, 8> : k_wino_gemm_output_lanes_wres<4, SUM, 8>;
-      return nullptr;
+      // (two passes over half of the columns each)
+      return nw == 8 ? k_wino_gemm_output_lanes_wres2<A == 4 ? 6 : A, SUM, 8, 8> : k_wino_gemm_output_lanes_wres2<A == 4 ? 6 : A, SUM, 8, 4>;
     default: return nullptr;
   }
 }
@@ -615,6 +872,18 @@ auto pick_wres(int A, bool sum, int nks64, int nw) -> void (*)(WinoFusedArgs)
 }
 }  // namespace
 
+size_t wino_lanes_tpart_bytes(int tile, int ic2, int oc2, int t)
+{
+  const int A = tile ? tile : 6, nks64 = (ic2 + 3) / 4;
+  if (A == 4 || nks64 != 8) return 0;
+  const char *env = getenv("EHIP_WINO_LANES");
+  if (env && env[0] == '0') return 0;
+  // per tile and group of 16 channels: (A - 2) rows x the first pass's columns x 16 channels x 4 bytes (four lanes with
+  // a float4 each); tiles in whole blocks of 128, channel groups of whole 32s
+  const size_t per_tile = (size_t)(A - 2) * ((A + 1) / 2) * 64;
+  return (size_t)2 * ((oc2 * 16 + 31) / 32) * ((t + 127) / 128 * 128) * per_tile;
+}
+
 bool wino_lanes_applies(const WinoFusedArgs &a)
 {
   const char *env = getenv("EHIP_WINO_LANES");
@@ -624,7 +893,8 @@ bool wino_lanes_applies(const WinoFusedArgs &a)
   // 512 -> 512 at 28 x 28 (eight k-steps per position, 288 unrolled steps) 648 vs 134: up to 256 input channels.
   const int A = a.tile ? a.tile : 6;
   // the weights of 16 channels at every position must fit the LDS (the streamed form: 1, 2 or 4 k-steps)
-  const bool fits = nks64 <= 4 || (A == 4 && nks64 == 8);
+  // (tile sizes 6 and 5 with 512 channels: half the columns at a time, results parked in a.tpart)
+  const bool fits = nks64 <= 4 || (A == 4 && nks64 == 8) || (A != 4 && nks64 == 8 && a.tpart != nullptr);
   return a.tin_blocked && fits && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && !(a.out_type == EHIP_F32 && a.with_sum) &&
       !(env && env[0] == '0');
 }
@@ -640,7 +910,8 @@ hipError_t launch_wino_gemm_output_lanes(const WinoFusedArgs &a0, hipStream_t s,
     // weights resident: the weights of 16 channels in LDS, workgroups walking over blocks of tiles.  Up to 128 input
     // channels: four waves, 64 tiles a block, two workgroups per CU; 256: the weights fill the LDS (tile size 6: 147 KB),
     // one workgroup per CU, of eight waves (128 tiles a block) so that every SIMD still has two
-    const size_t lds = (size_t)AA * nks64 * 1024 + (size_t)AA * 12 * sizeof(float4);
+    const bool two_pass = A != 4 && nks64 == 8;   // the weights of half the columns at a time
+    const size_t lds = (two_pass ? (size_t)((A + 1) / 2) * A : (size_t)AA) * nks64 * 1024 + (size_t)AA * 12 * sizeof(float4);
     const int per_cu = 2 * lds <= 160 * 1024 ? 2 : 1;
     const char *wv = getenv("EHIP_WINO_LANES_WAVES");
     a.ny = 2 * ((a.oc2 * 16 + 31) / 32);
