@@ -872,10 +872,24 @@ auto pick_wres(int A, bool sum, int nks64, int nw) -> void (*)(WinoFusedArgs)
 }
 }  // namespace
 
-size_t wino_lanes_tpart_bytes(int tile, int ic2, int oc2, int t)
+namespace {
+// 512 input channels with tile size 6 or 5, two passes with resident weights: pays when a workgroup has at least two
+// blocks of 128 tiles to walk over (N = 64, fused stage: 512 -> 512 at 28 x 28 134 -> 113 us, at 14 x 14 36.6 -> 42.8 us,
+// at 7 x 7 26.5 -> 31.2 us), else the general kernel stays
+bool two_pass_pays(int tile, int ic2, int oc2, int t)
 {
   const int A = tile ? tile : 6, nks64 = (ic2 + 3) / 4;
-  if (A == 4 || nks64 != 8) return 0;
+  if (A == 4 || nks64 != 8) return false;
+  if (const char *env = getenv("EHIP_WINO_LANES_TWO_PASS")) return env[0] != '0';   // (1: also for the small layers)
+  const long long ny = 2 * ((oc2 * 16 + 31) / 32);
+  return (long long)((t + 127) / 128) * ny >= 512;
+}
+}  // namespace
+
+size_t wino_lanes_tpart_bytes(int tile, int ic2, int oc2, int t)
+{
+  const int A = tile ? tile : 6;
+  if (!two_pass_pays(tile, ic2, oc2, t)) return 0;
   const char *env = getenv("EHIP_WINO_LANES");
   if (env && env[0] == '0') return 0;
   // per tile and group of 16 channels: (A - 2) rows x the first pass's columns x 16 channels x 4 bytes (four lanes with
@@ -894,7 +908,7 @@ bool wino_lanes_applies(const WinoFusedArgs &a)
   const int A = a.tile ? a.tile : 6;
   // the weights of 16 channels at every position must fit the LDS (the streamed form: 1, 2 or 4 k-steps)
   // (tile sizes 6 and 5 with 512 channels: half the columns at a time, results parked in a.tpart)
-  const bool fits = nks64 <= 4 || (A == 4 && nks64 == 8) || (A != 4 && nks64 == 8 && a.tpart != nullptr);
+  const bool fits = nks64 <= 4 || (A == 4 && nks64 == 8) || (two_pass_pays(a.tile, a.ic2, a.oc2, a.t) && a.tpart != nullptr);
   return a.tin_blocked && fits && a.units_pad % 4 == 0 && a.units_pad >= 4 * nks64 && !(a.out_type == EHIP_F32 && a.with_sum) &&
       !(env && env[0] == '0');
 }

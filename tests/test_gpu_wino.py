@@ -214,6 +214,7 @@ def test_wino_fused_lanes_weights_resident_many_channels(waves, slots, tile, out
     same, with tile sizes 6 and 5 two passes over half of the columns each, the first pass's results parked in memory"""
     import torch
     monkeypatch.setenv("EHIP_WINO_LANES_WAVES", waves)
+    monkeypatch.setenv("EHIP_WINO_LANES_TWO_PASS", "1")   # (by itself the library keeps so small a layer on the general kernel)
     if slots:
         monkeypatch.setenv("EHIP_WINO_LANES_SLOTS", slots)
     E, p, d, xq, wb, bias = make_wino_u8(n, ic, oc, hw, seed=63 + tile + ic + out_type, out_type=out_type, tile=tile,
