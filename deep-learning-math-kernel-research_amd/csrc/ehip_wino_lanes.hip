@@ -1,5 +1,6 @@
-// Winograd GEMMs + output transform for layers with at most 256 input channels: the form whose lanes own a tile x four
-// channels at every position, so that nothing is exchanged through LDS between the GEMMs and the transform.
+// Winograd GEMMs + output transform, the form whose lanes own a tile x four channels at every position, so that nothing
+// is exchanged through LDS between the GEMMs and the transform: with the weights of 16 channels resident in LDS (up to
+// 256 input channels in one pass, 512 in two) or with both operands streamed (up to 256).
 //
 // Replaces, for those layers, elx_int8_conv_wino_gemm_t::execute + trans_output as the reference's fused schedule
 // runs them per thread (a161, src/elx_int8_conv_wino_xopt.hpp:21-179; src/elx_int8_conv_wino_gemm.cpp:23-205,
@@ -331,12 +332,12 @@ __global__ __launch_bounds__(kBlock, 2) void k_wino_gemm_output_lanes(WinoFusedA
 }
 
 // The same lanes, weights resident: with at most 128 input channels the packed weights of 16 channels at every position
-// fit the LDS twice over (36 or 72 KB a workgroup), so a workgroup = 16 channels x 64 tiles stages them once and then
-// walks over blocks of 64 tiles: the operand stream from L2 is the transformed input alone (half of what the form
+// fit the LDS twice over (36 or 72 KB a workgroup; with 192 / 256 channels once: NW = 4 or 8 waves, one workgroup per
+// CU), so a workgroup = 16 channels x 16 NW tiles stages them once and then walks over blocks of that many tiles: the operand stream from L2 is the transformed input alone (half of what the form
 // above requests per MFMA), every wave has tiles of its own (nothing is requested twice inside a workgroup), and the
 // ring of input operands runs on from one block of tiles to the next, so the first operands of the next block travel
 // while this one's output transform keeps the vector units busy.  No barrier after the staging.
-// a.nx = blocks of 64 tiles, a.ny = groups of 16 packed rows; grid = 8 XCDs x a.ny x slots, a slot walks over the
+// a.nx = blocks of 16 NW tiles, a.ny = groups of 16 packed rows; grid = 8 XCDs x a.ny x slots, a slot walks over the
 // blocks slot * 8 + xcd, + 8 * slots, ...
 template <int A, bool SUM, int NKS, int NW = 4>
 __global__ __launch_bounds__(64 * NW, 2) void k_wino_gemm_output_lanes_wres(WinoFusedArgs a)
