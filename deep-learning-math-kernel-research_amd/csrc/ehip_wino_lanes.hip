@@ -883,6 +883,8 @@ bool two_pass_pays(int tile, int ic2, int oc2, int t)
   if (A == 4 || nks64 != 8) return false;
   if (const char *env = getenv("EHIP_WINO_LANES_TWO_PASS")) return env[0] != '0';   // (1: also for the small layers)
   const long long ny = 2 * ((oc2 * 16 + 31) / 32);
+  // (and the parking space stays below 1 GB: beyond, the general kernel)
+  if (ny * ((t + 127) / 128 * 128) * (long long)(A - 2) * ((A + 1) / 2) * 64 > (1ll << 30)) return false;
   return (long long)((t + 127) / 128) * ny >= 512;
 }
 }  // namespace
